@@ -1,0 +1,153 @@
+/* llmops_hip.h -- C ABI of the gfx950 (MI355X) implementation of the Q4_1 fully-connected path
+ * and of the KV-cache attention op that wraps it.
+ *
+ * Every entry point replaces one function the reference binds into its `llmops` Python module
+ * (PYBIND11_MODULE, /root/reference/ops/main.cpp:62-179); the citation beside each declaration
+ * names that function.  A binding layer (pybind11, ctypes, cgo ...) passes plain device
+ * pointers and sizes; no framework types cross this boundary.
+ *
+ * Conventions
+ *  - All data pointers are DEVICE pointers on the current HIP device unless marked host.
+ *  - Tensors are dense row-major with the reference's shapes and dtypes.
+ *  - `stream` is a hipStream_t passed as void* (NULL = the default stream).  Calls only enqueue
+ *    work; they never synchronise and never allocate device memory.
+ *  - Every function returns 0 on success and a non-zero LLMOPS_E* code on failure; the message
+ *    is available from llmops_last_error() (thread local).  Argument validation mirrors the
+ *    reference's ASSERTs (ops/tensor.hpp:20-36) and happens before anything is enqueued.
+ *  - group_k is 32 or 128 (the reference fixes it at compile time, ops/op_fc.hpp:109; here it
+ *    is a run-time argument recoverable from the packed tensor's last dimension).
+ *
+ * Packed weight format == the reference's q4_1_block<G> (ops/op_fc.hpp:14-62), byte for byte:
+ *   int8 [ceil(N/32)][ceil(K/G)][ (G/8)*128 nibble bytes | 32 x fp16 d | 32 x fp16 m ]
+ *   element (k,n) of a block: byte (k>>3)*128 + n*4 + (k&3), high nibble iff (k>>2)&1.
+ */
+#ifndef LLMOPS_HIP_H
+#define LLMOPS_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define LLMOPS_OK 0
+#define LLMOPS_EINVAL 1   /* bad argument (shape, group size, null pointer, misalignment) */
+#define LLMOPS_EWORKSPACE 2 /* workspace too small */
+#define LLMOPS_EHIP 3     /* a HIP runtime call or kernel launch failed */
+
+#define LLMOPS_CACHE_F32 0
+#define LLMOPS_CACHE_F16 1
+
+typedef void* llmops_stream_t;
+
+const char* llmops_last_error(void);
+int llmops_abi_version(void);
+
+/* bytes of one packed block for group_k (640 / 2176); 0 if group_k is not supported */
+int64_t llmops_q4a_block_bytes(int group_k);
+
+/* ------------------------------------------------------------------------------------------
+ * Q4_1 weight packing
+ * ------------------------------------------------------------------------------------------ */
+
+/* offline_FC_quant_Q4A (ops/op_fc.hpp:151-219, bound at ops/main.cpp:158).
+ * wei fp32 [N,K], row stride `ld` elements -> weiq int8 [ceil(N/32), ceil(K/G), blk(G)].
+ * Byte-exact with the reference for every real (n,k); nibbles of padded rows (n >= N), which the
+ * reference leaves uninitialised, are written as 0. */
+int llmops_offline_FC_quant_Q4A(const float* wei, int64_t N, int64_t K, int64_t ld, int group_k,
+                                int8_t* weiq, llmops_stream_t stream);
+
+/* offline_FC_dequant_Q4A (ops/op_fc.hpp:124-149, ops/main.cpp:159).
+ * weiq [Ng,Kg,blk] -> out fp32 [Ng*32, Kg*G] = fp32(d)*q + fp32(m). */
+int llmops_offline_FC_dequant_Q4A(const int8_t* weiq, int64_t Ng, int64_t Kg, int group_k,
+                                  float* out, llmops_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Q8 dynamic activation quantization
+ * ------------------------------------------------------------------------------------------ */
+
+/* FC_dynamic_quantize_x (ops/op_fc.hpp:221-272; get_amax ops/utils.hpp:177-197, quant_row_q8_0
+ * ops/utils.hpp:200-220).  x fp32 [rows,K] -> xq int8 [rows,Kg*G] (round half to even, zero
+ * padded), xd fp32 [rows,Kg] = amax/127, gsum fp32 [rows,Kg] = left-to-right fp32 sum of the raw
+ * group.  All three outputs are bit-exact with the reference.  Requires K % 8 == 0. */
+int llmops_FC_dynamic_quantize_x(const float* x, int64_t rows, int64_t K, int group_k, int8_t* xq,
+                                 float* xd, float* gsum, llmops_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Q4_1 x Q8 fully connected
+ * ------------------------------------------------------------------------------------------ */
+
+/* workspace bytes llmops_fc_Q4A needs for these sizes (activation codes, split-K partial sums and
+ * arrival counters).  The first LLMOPS_FC_COUNTER_BYTES bytes of the workspace must be zero when
+ * the library first sees it; the library leaves them zero after every call.  One workspace must
+ * not be shared by calls that can overlap on the device. */
+#define LLMOPS_FC_COUNTER_BYTES 65536
+size_t llmops_fc_Q4A_workspace_bytes(int64_t rows, int64_t K, int64_t Ng, int64_t Kg, int group_k);
+
+/* fc_Q4A (ops/op_fc.hpp:286-426, bound at ops/main.cpp:160).
+ * x fp32 [rows,K] (rows = B*M), weiq [Ng,Kg,blk] -> y fp32 [rows,N]:
+ *   y[r,n] = sum_kb  fp32(d[n,kb])*dx[r,kb] * float(acc[r,n,kb]) + fp32(m[n,kb])*gsum[r,kb]
+ * with acc the exact int32 dot product of 4-bit codes and int8 activation codes.  rows <= 8 runs
+ * the HBM-streaming dot4 kernel, larger row counts the int8 MFMA kernel.  Requires K == Kg*G
+ * (every shape the reference is used with); N may be any value in (Ng*32-32, Ng*32]. */
+int llmops_fc_Q4A(const float* x, int64_t rows, int64_t K, const int8_t* weiq, int64_t Ng, int64_t Kg,
+                  int group_k, int64_t N, float* y, void* workspace, size_t workspace_bytes,
+                  llmops_stream_t stream);
+
+/* The integer core of fc_Q4A on its own (ops/op_fc.hpp:337-363): acc int32 [rows, Ng*32, Kg].
+ * `use_mfma` selects which of the two production inner loops computes it (0 = dot4 streaming
+ * kernel, 1 = int8 MFMA kernel) so that both can be checked bit-for-bit. */
+int llmops_fc_Q4A_partials(const int8_t* xq, int64_t rows, const int8_t* weiq, int64_t Ng, int64_t Kg,
+                           int group_k, int32_t* acc, int use_mfma, llmops_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Rotary embedding, KV cache, attention
+ * ------------------------------------------------------------------------------------------ */
+
+/* rope_embed (ops/op_attn.hpp:44-94, ops/main.cpp:152): in place on x fp32 [B,H,L,S];
+ * pairs (i, i+half) for i < half rotated by inv_freq[i]*(position_id+l); dims >= 2*half untouched. */
+int llmops_rope_embed(float* x, int64_t B, int64_t H, int64_t L, int64_t S, const float* inv_freq,
+                      int64_t half, int position_id, llmops_stream_t stream);
+
+/* workspace bytes for llmops_attention_rope (split-KV partial results) */
+size_t llmops_attention_workspace_bytes(int64_t B, int64_t qL, int64_t H, int64_t S, int64_t maxlen);
+
+/* attention_rope2 / attention_rope (ops/op_attn.hpp:721-1029 and :518-718; ops/main.cpp:154-155;
+ * same contract).  q,k,v fp32 [B,qL,H*S]; kv_cache [planes,B,H,maxlen,S] in fp32
+ * (LLMOPS_CACHE_F32, the reference's layout) or fp16 (LLMOPS_CACHE_F16, an extension: fp32 math
+ * on fp16-rounded K/V); slots int32 [qL] (device).  Effects: q,k rotated in place (k stays
+ * rotated), k,v rows written to cache[2*layer_id+{0,1}, b, h, slots[p], :], and q overwritten by
+ * softmax((q.K^T)/sqrt(S) with in-chunk causal mask via slots) . V over
+ * kvLen = min(position_id+qL, maxlen) cache rows. */
+int llmops_attention_rope(float* q, float* k, const float* v, int64_t B, int64_t qL, int64_t H, int64_t S,
+                          const float* inv_freq, int64_t half, void* kv_cache, int cache_dtype,
+                          int64_t planes, int64_t maxlen, const int32_t* slots, int position_id,
+                          int layer_id, void* workspace, size_t workspace_bytes, llmops_stream_t stream);
+
+/* softmax (ops/op_misc.hpp:183-194, ops/utils.hpp:484-490): in place over rows of length K */
+int llmops_softmax(float* x, int64_t rows, int64_t K, llmops_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Neighbours needed for one decode step (ops/op_misc.hpp, ops/op_embedding.hpp)
+ * ------------------------------------------------------------------------------------------ */
+
+/* rmsnorm (ops/op_misc.hpp:142-181): x[r,:] *= rsqrt(mean(x[r,:]^2)+eps) * w, in place */
+int llmops_rmsnorm(float* x, int64_t rows, int64_t hidden, const float* w, float eps, llmops_stream_t stream);
+/* iadd / imul (ops/op_misc.hpp:55-107): a (+|*)= b; b is [rows,inner] or, if b_is_row, [inner] */
+int llmops_iadd(float* a, const float* b, int64_t rows, int64_t inner, int b_is_row, llmops_stream_t stream);
+int llmops_imul(float* a, const float* b, int64_t rows, int64_t inner, int b_is_row, llmops_stream_t stream);
+/* itrans "silu" (ops/op_misc.hpp:127-138): a = a * sigmoid(a), in place */
+int llmops_itrans_silu(float* a, int64_t n, llmops_stream_t stream);
+/* embedding_q8c_quant_w (ops/op_embedding.hpp:51-78): w fp32 [V,E] -> q int8 [V,E], scales [V] */
+int llmops_embedding_q8c_quant_w(const float* w, int64_t V, int64_t E, int8_t* q, float* scales, llmops_stream_t stream);
+/* embedding_q8c (ops/op_embedding.hpp:108-137): out[i,:] = scales[ids[i]] * q[ids[i],:]; ids int64 */
+int llmops_embedding_q8c(float* out, const int64_t* ids, int64_t n, const int8_t* q, const float* scales,
+                         int64_t V, int64_t E, llmops_stream_t stream);
+/* embedding (ops/op_embedding.hpp:24-49): out[i,:] = w[ids[i],:]; ids int64 */
+int llmops_embedding(float* out, const int64_t* ids, int64_t n, const float* w, int64_t V, int64_t E, llmops_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LLMOPS_HIP_H */

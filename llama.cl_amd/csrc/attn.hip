@@ -1,0 +1,336 @@
+// Rotary embedding, KV-cache update and attention over the cache
+// (attention_rope2 / attention_rope, /root/reference/ops/op_attn.hpp:721-1029 and :518-718).
+//
+// Three launches per call:
+//   1. attn_prep_kernel   rotate q and k in place (rope_embed, ops/op_attn.hpp:44-94), write the
+//                         rotated k and the v rows into the cache at slots[p] (:764-773), and
+//                         record which cache rows were written by which token of this call.
+//   2. attn_split_kernel  split-KV attention: one workgroup per (b, h, query, chunk of C cache
+//                         rows) streams its K and V rows exactly once with 16-byte loads (all
+//                         issued before the first use so a whole chunk is in flight), computes
+//                         the chunk's scores, their max, exp and sum, and the chunk's weighted
+//                         V sum.  Chunks make up for the low head count (B*H = 32 in decode).
+//   3. attn_merge_kernel  merges the chunks of a query with the usual max/sum rescaling and
+//                         overwrites q with the result (:1018-1025).
+// The cache element type is fp32 (reference layout) or fp16 (all arithmetic still fp32).
+//
+// In-chunk causal mask (:1007-1011): for query token pq, cache row slots[p'] is excluded for
+// every p' in (pq, qL).  Excluded rows get weight exactly 0, as the reference's exp() returns 0
+// for lowest()-max.
+#include <float.h>
+
+#include "common.h"
+
+namespace llmops {
+
+// ---- rope ------------------------------------------------------------------------------------
+// theta = inv_freq[i] * (float)pos, cosf/sinf in fp32 (CosSin_cache::update, ops/op_attn.hpp:25-32)
+__device__ __forceinline__ void rope_pair(float& x0, float& x1, float inv_freq, int pos) {
+    const float xita = inv_freq * (float)pos;
+    const float c = cosf(xita), s = sinf(xita);
+    const float y0 = c * x0 - s * x1;
+    const float y1 = s * x0 + c * x1;
+    x0 = y0;
+    x1 = y1;
+}
+
+// x [B,H,L,S] in place; one thread per rotated pair
+__global__ void rope_kernel(float* __restrict__ x, int64_t BH, int64_t L, int64_t S, const float* __restrict__ inv_freq,
+                            int64_t half, int position_id) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= BH * L * half) return;
+    const int64_t p = i % half, l = (i / half) % L, bh = i / (half * L);
+    float* px = x + (bh * L + l) * S;
+    float x0 = px[p], x1 = px[p + half];
+    rope_pair(x0, x1, inv_freq[p], (int)l + position_id);
+    px[p] = x0;
+    px[p + half] = x1;
+}
+
+template <typename T>
+__device__ __forceinline__ void store_cache(T* dst, float v);
+template <>
+__device__ __forceinline__ void store_cache<float>(float* dst, float v) {
+    *dst = v;
+}
+template <>
+__device__ __forceinline__ void store_cache<__half>(__half* dst, float v) {
+    *dst = __float2half_rn(v);
+}
+
+// q,k,v [B,qL,H,S].  One workgroup per (b, l, h); thread i handles element i (and i+half).
+template <typename T>
+__global__ void attn_prep_kernel(float* __restrict__ q, float* __restrict__ k, const float* __restrict__ v, int64_t qL,
+                                 int64_t H, int64_t S, const float* __restrict__ inv_freq, int64_t half,
+                                 T* __restrict__ kc, T* __restrict__ vc, int64_t maxlen, const int32_t* __restrict__ slots,
+                                 int position_id, int32_t* __restrict__ row_token) {
+    const int64_t h = blockIdx.x % H, l = (blockIdx.x / H) % qL, b = blockIdx.x / (H * qL);
+    const int64_t base = ((b * qL + l) * H + h) * S;
+    const int slot = slots[l];
+    T* kdst = kc + ((b * H + h) * maxlen + slot) * S;
+    T* vdst = vc + ((b * H + h) * maxlen + slot) * S;
+    if (blockIdx.x < qL && threadIdx.x == 0) row_token[slots[blockIdx.x]] = (int32_t)blockIdx.x;
+    for (int64_t i = threadIdx.x; i < S; i += blockDim.x) {
+        if (i < half) {
+            float q0 = q[base + i], q1 = q[base + i + half];
+            float k0 = k[base + i], k1 = k[base + i + half];
+            const float f = inv_freq[i];
+            rope_pair(q0, q1, f, (int)l + position_id);
+            rope_pair(k0, k1, f, (int)l + position_id);
+            q[base + i] = q0;
+            q[base + i + half] = q1;
+            k[base + i] = k0;
+            k[base + i + half] = k1;
+            store_cache(kdst + i, k0);
+            store_cache(kdst + i + half, k1);
+        } else if (i >= 2 * half) {
+            store_cache(kdst + i, k[base + i]);
+        }
+        store_cache(vdst + i, v[base + i]);
+    }
+}
+
+__global__ void fill_i32_kernel(int32_t* p, int64_t n, int32_t v) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = v;
+}
+
+// ---- split-KV attention ----------------------------------------------------------------------
+__device__ __forceinline__ float4 load4(const float* p) { return *reinterpret_cast<const float4*>(p); }
+__device__ __forceinline__ float4 load4(const __half* p) {
+    const uint2 u = *reinterpret_cast<const uint2*>(p);
+    const __half2 a = *reinterpret_cast<const __half2*>(&u.x), b = *reinterpret_cast<const __half2*>(&u.y);
+    const float2 fa = __half22float2(a), fb = __half22float2(b);
+    return make_float4(fa.x, fa.y, fb.x, fb.y);
+}
+
+// Per-chunk record in the workspace: [max, sum, out[S]]
+// Workgroup = 4 waves; wave w owns rows w*PW .. w*PW+PW-1 of the chunk (C = 4*PW rows);
+// lane = 32*hf + e: row parity hf, elements 4e..4e+3 (S == 128).
+template <typename T, int PW>
+__global__ __launch_bounds__(256) void attn_split_kernel(const float* __restrict__ q, const T* __restrict__ kc,
+                                                          const T* __restrict__ vc, int64_t qL, int64_t H, int64_t maxlen,
+                                                          int64_t kvLen, const int32_t* __restrict__ row_token,
+                                                          float* __restrict__ part, int nchunks) {
+    constexpr int S = 128, C = 4 * PW, NL = PW / 2;
+    __shared__ float sc[C];
+    __shared__ float osh[4][2][S];
+    __shared__ float stat[2];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int hf = lane >> 5, e = lane & 31;
+    const int chunk = blockIdx.x % nchunks;
+    const int64_t bhq = blockIdx.x / nchunks;  // ((b*H)+h)*qL + pq
+    const int64_t pq = bhq % qL, h = (bhq / qL) % H, b = bhq / (qL * H);
+    const int64_t p0 = (int64_t)chunk * C;
+    const T* kbase = kc + (b * H + h) * maxlen * S;
+    const T* vbase = vc + (b * H + h) * maxlen * S;
+
+    // issue every K and V load of this wave before anything is consumed
+    float4 kv[NL], vv[NL];
+#pragma unroll
+    for (int i = 0; i < NL; i++) {
+        const int64_t p = p0 + wave * PW + i * 2 + hf;
+        const int64_t pc = p < kvLen ? p : kvLen - 1;
+        kv[i] = load4(kbase + pc * S + e * 4);
+        vv[i] = load4(vbase + pc * S + e * 4);
+    }
+    const float4 qv = load4(q + ((b * qL + pq) * H + h) * S + e * 4);
+    const float d_scale = 1.0f / sqrtf((float)S);
+
+#pragma unroll
+    for (int i = 0; i < NL; i++) {
+        float s = qv.x * kv[i].x;
+        s = fmaf(qv.y, kv[i].y, s);
+        s = fmaf(qv.z, kv[i].z, s);
+        s = fmaf(qv.w, kv[i].w, s);
+#pragma unroll
+        for (int o = 16; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
+        const int r = wave * PW + i * 2 + hf;
+        const int64_t p = p0 + r;
+        bool live = p < kvLen;
+        if (live && qL > 1) live = !(row_token[p] > (int32_t)pq);  // written by a later token of this call
+        if (e == 0) sc[r] = live ? s * d_scale : -FLT_MAX;
+    }
+    __syncthreads();
+    if (wave == 0) {
+        float v = lane < C ? sc[lane] : -FLT_MAX;
+        const float mx = wave_max(v);
+        // a row counts only if it is live; a chunk with no live row reports sum 0
+        float ex = (lane < C && v != -FLT_MAX) ? expf(v - mx) : 0.0f;
+        if (lane < C) sc[lane] = ex;
+        const float sum = wave_sum(ex);
+        if (lane == 0) {
+            stat[0] = mx;
+            stat[1] = sum;
+        }
+    }
+    __syncthreads();
+    float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+    for (int i = 0; i < NL; i++) {
+        const float w = sc[wave * PW + i * 2 + hf];
+        o.x = fmaf(w, vv[i].x, o.x);
+        o.y = fmaf(w, vv[i].y, o.y);
+        o.z = fmaf(w, vv[i].z, o.z);
+        o.w = fmaf(w, vv[i].w, o.w);
+    }
+    *reinterpret_cast<float4*>(&osh[wave][hf][e * 4]) = o;
+    __syncthreads();
+    float* rec = part + ((int64_t)bhq * nchunks + chunk) * (S + 2);
+    if (threadIdx.x < S) {
+        float a = 0.0f;
+#pragma unroll
+        for (int w = 0; w < 4; w++) a += osh[w][0][threadIdx.x] + osh[w][1][threadIdx.x];
+        rec[2 + threadIdx.x] = a;
+    }
+    if (threadIdx.x == 0) {
+        rec[0] = stat[0];
+        rec[1] = stat[1];
+    }
+}
+
+// out[b,pq,h,:] = sum_c exp(m_c - M) * o_c / sum_c exp(m_c - M) * s_c ; 128 threads per query
+__global__ __launch_bounds__(128) void attn_merge_kernel(float* __restrict__ q, const float* __restrict__ part, int64_t qL,
+                                                          int64_t H, int nchunks) {
+    constexpr int S = 128;
+    const int64_t bhq = blockIdx.x;
+    const int64_t pq = bhq % qL, h = (bhq / qL) % H, b = bhq / (qL * H);
+    const float* rec = part + (int64_t)bhq * nchunks * (S + 2);
+    float M = -FLT_MAX;
+    for (int c = 0; c < nchunks; c++) M = fmaxf(M, rec[(int64_t)c * (S + 2)]);
+    float den = 0.0f, num = 0.0f;
+    for (int c = 0; c < nchunks; c++) {
+        const float* r = rec + (int64_t)c * (S + 2);
+        const float sum = r[1];
+        if (sum == 0.0f) continue;
+        const float sc = expf(r[0] - M);
+        den = fmaf(sc, sum, den);
+        num = fmaf(sc, r[2 + threadIdx.x], num);
+    }
+    q[((b * qL + pq) * H + h) * S + threadIdx.x] = num * (1.0f / den);
+}
+
+// ---- softmax op (ops/op_misc.hpp:183-194): one workgroup per row ------------------------------
+__global__ __launch_bounds__(256) void softmax_kernel(float* __restrict__ x, int64_t K) {
+    __shared__ float red[4];
+    float* row = x + (int64_t)blockIdx.x * K;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    float mx = -FLT_MAX;
+    for (int64_t i = threadIdx.x; i < K; i += 256) mx = fmaxf(mx, row[i]);
+    mx = wave_max(mx);
+    if (lane == 0) red[wave] = mx;
+    __syncthreads();
+    mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    __syncthreads();
+    float sum = 0.0f;
+    for (int64_t i = threadIdx.x; i < K; i += 256) {
+        const float ex = expf(row[i] - mx);
+        row[i] = ex;
+        sum += ex;
+    }
+    sum = wave_sum(sum);
+    if (lane == 0) red[wave] = sum;
+    __syncthreads();
+    const float scale = 1.0f / (((red[0] + red[1]) + red[2]) + red[3]);
+    for (int64_t i = threadIdx.x; i < K; i += 256) row[i] *= scale;
+}
+
+static inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+static int pick_pw(int64_t bhq, int64_t kvLen) {
+    // smallest chunk count that still gives ~1024 workgroups; chunk = 4*PW rows
+    for (int pw : {16, 8, 4}) {
+        const int64_t chunks = (kvLen + 4 * pw - 1) / (4 * pw);
+        if (bhq * chunks >= 1024 || pw == 4) return pw;
+    }
+    return 4;
+}
+
+}  // namespace llmops
+
+using namespace llmops;
+
+extern "C" int llmops_rope_embed(float* x, int64_t B, int64_t H, int64_t L, int64_t S, const float* inv_freq,
+                                 int64_t half, int position_id, llmops_stream_t stream) {
+    LLMOPS_REQUIRE(x != nullptr && inv_freq != nullptr);
+    LLMOPS_REQUIRE(B > 0 && H > 0 && L > 0 && S > 0 && half > 0 && 2 * half <= S);
+    const int64_t total = B * H * L * half;
+    rope_kernel<<<(unsigned)((total + 255) / 256), 256, 0, as_stream(stream)>>>(x, B * H, L, S, inv_freq, half, position_id);
+    LLMOPS_LAUNCH_CHECK();
+    return LLMOPS_OK;
+}
+
+extern "C" size_t llmops_attention_workspace_bytes(int64_t B, int64_t qL, int64_t H, int64_t S, int64_t maxlen) {
+    if (B <= 0 || qL <= 0 || H <= 0 || S <= 0 || maxlen <= 0) return 0;
+    // pick_pw() uses 64-row chunks unless that gives fewer than 1024 workgroups, and the finer
+    // chunkings it then falls back to stay below 2048 workgroups
+    const int64_t bhq = B * H * qL;
+    int64_t records = bhq * ((maxlen + 63) / 64);
+    if (records < 2048) records = 2048;
+    return align_up((size_t)maxlen * sizeof(int32_t), 256) + (size_t)records * (S + 2) * sizeof(float);
+}
+
+template <typename T>
+static int attention_impl(float* q, float* k, const float* v, int64_t B, int64_t qL, int64_t H, int64_t S,
+                          const float* inv_freq, int64_t half, T* cache, int64_t maxlen, const int32_t* slots,
+                          int position_id, int layer_id, void* workspace, hipStream_t st) {
+    T* kc = cache + (int64_t)(2 * layer_id + 0) * B * H * maxlen * S;
+    T* vc = cache + (int64_t)(2 * layer_id + 1) * B * H * maxlen * S;
+    int32_t* row_token = reinterpret_cast<int32_t*>(workspace);
+    float* part = reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(workspace) + align_up((size_t)maxlen * 4, 256));
+    if (qL > 1) {
+        fill_i32_kernel<<<(unsigned)((maxlen + 255) / 256), 256, 0, st>>>(row_token, maxlen, -1);
+        LLMOPS_LAUNCH_CHECK();
+    }
+    attn_prep_kernel<T><<<(unsigned)(B * qL * H), 64, 0, st>>>(q, k, v, qL, H, S, inv_freq, half, kc, vc, maxlen, slots,
+                                                              position_id, row_token);
+    LLMOPS_LAUNCH_CHECK();
+    int64_t kvLen = (int64_t)position_id + qL;
+    if (kvLen > maxlen) kvLen = maxlen;
+    const int64_t bhq = B * H * qL;
+    const int pw = pick_pw(bhq, kvLen);
+    const int nchunks = (int)((kvLen + 4 * pw - 1) / (4 * pw));
+    const unsigned grid = (unsigned)(bhq * nchunks);
+    if (pw == 16)
+        attn_split_kernel<T, 16><<<grid, 256, 0, st>>>(q, kc, vc, qL, H, maxlen, kvLen, row_token, part, nchunks);
+    else if (pw == 8)
+        attn_split_kernel<T, 8><<<grid, 256, 0, st>>>(q, kc, vc, qL, H, maxlen, kvLen, row_token, part, nchunks);
+    else
+        attn_split_kernel<T, 4><<<grid, 256, 0, st>>>(q, kc, vc, qL, H, maxlen, kvLen, row_token, part, nchunks);
+    LLMOPS_LAUNCH_CHECK();
+    attn_merge_kernel<<<(unsigned)bhq, 128, 0, st>>>(q, part, qL, H, nchunks);
+    LLMOPS_LAUNCH_CHECK();
+    return LLMOPS_OK;
+}
+
+extern "C" int llmops_attention_rope(float* q, float* k, const float* v, int64_t B, int64_t qL, int64_t H, int64_t S,
+                                     const float* inv_freq, int64_t half, void* kv_cache, int cache_dtype,
+                                     int64_t planes, int64_t maxlen, const int32_t* slots, int position_id,
+                                     int layer_id, void* workspace, size_t workspace_bytes, llmops_stream_t stream) {
+    LLMOPS_REQUIRE(q != nullptr && k != nullptr && v != nullptr && inv_freq != nullptr && kv_cache != nullptr);
+    LLMOPS_REQUIRE(slots != nullptr && workspace != nullptr);
+    LLMOPS_REQUIRE(B > 0 && qL > 0 && H > 0 && maxlen > 0);
+    LLMOPS_REQUIRE(S == 128);  // head size of every supported model shape (the reference needs S % 16 == 0)
+    LLMOPS_REQUIRE(half > 0 && 2 * half <= S);
+    LLMOPS_REQUIRE(layer_id >= 0 && 2 * (int64_t)layer_id + 1 < planes);
+    LLMOPS_REQUIRE(position_id >= 0);
+    LLMOPS_REQUIRE(cache_dtype == LLMOPS_CACHE_F32 || cache_dtype == LLMOPS_CACHE_F16);
+    LLMOPS_REQUIRE(aligned(q, 16) && aligned(kv_cache, 16) && aligned(workspace, 256));
+    LLMOPS_REQUIRE(B * H * qL * ((maxlen + 63) / 64) < ((int64_t)1 << 31));
+    const size_t need = llmops_attention_workspace_bytes(B, qL, H, S, maxlen);
+    if (workspace_bytes < need)
+        return fail(LLMOPS_EWORKSPACE, "attention_rope needs %zu workspace bytes, got %zu", need, workspace_bytes);
+    hipStream_t st = as_stream(stream);
+    if (cache_dtype == LLMOPS_CACHE_F32)
+        return attention_impl<float>(q, k, v, B, qL, H, S, inv_freq, half, reinterpret_cast<float*>(kv_cache), maxlen, slots,
+                                     position_id, layer_id, workspace, st);
+    return attention_impl<__half>(q, k, v, B, qL, H, S, inv_freq, half, reinterpret_cast<__half*>(kv_cache), maxlen, slots,
+                                  position_id, layer_id, workspace, st);
+}
+
+extern "C" int llmops_softmax(float* x, int64_t rows, int64_t K, llmops_stream_t stream) {
+    LLMOPS_REQUIRE(x != nullptr && rows > 0 && K > 0 && rows < ((int64_t)1 << 31));
+    softmax_kernel<<<(unsigned)rows, 256, 0, as_stream(stream)>>>(x, K);
+    LLMOPS_LAUNCH_CHECK();
+    return LLMOPS_OK;
+}

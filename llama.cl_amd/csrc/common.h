@@ -1,0 +1,74 @@
+// Shared host/device helpers for the gfx950 llmops kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include <stdint.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <string>
+
+#include "../../include/llmops_hip.h"
+
+namespace llmops {
+
+constexpr int kGroupN = 32;   // columns per packed strip (q4_1_block::group_n, ops/op_fc.hpp:17)
+constexpr int kRowBytes = 128;  // one k8-row of a block: 32 columns x 4 bytes
+
+__host__ __device__ constexpr int64_t block_bytes(int G) { return (int64_t)(G / 8) * kRowBytes + 64 + 64; }
+
+// ---- error reporting ------------------------------------------------------------------------
+std::string& last_error();
+int fail(int code, const char* fmt, ...);
+
+#define LLMOPS_REQUIRE(cond)                                                                        \
+    do {                                                                                            \
+        if (!(cond)) return ::llmops::fail(LLMOPS_EINVAL, "assert %s failed at %s:%d", #cond, __FILE__, __LINE__); \
+    } while (0)
+
+#define LLMOPS_HIP_CHECK(expr)                                                                      \
+    do {                                                                                            \
+        hipError_t e_ = (expr);                                                                     \
+        if (e_ != hipSuccess)                                                                       \
+            return ::llmops::fail(LLMOPS_EHIP, "%s failed: %s at %s:%d", #expr, hipGetErrorString(e_), __FILE__, __LINE__); \
+    } while (0)
+
+#define LLMOPS_LAUNCH_CHECK() LLMOPS_HIP_CHECK(hipGetLastError())
+
+inline hipStream_t as_stream(llmops_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
+inline bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
+inline bool valid_group(int g) { return g == 32 || g == 128; }
+
+// ---- device helpers -------------------------------------------------------------------------
+#if defined(__HIPCC__)
+
+// fp16 bits <-> fp32, IEEE round-to-nearest-even (v_cvt_f16_f32 / v_cvt_f32_f16)
+__device__ __forceinline__ uint16_t f32_to_f16_bits(float f) { return __half_as_ushort(__float2half_rn(f)); }
+__device__ __forceinline__ float f16_bits_to_f32(uint16_t h) { return __half2float(__ushort_as_half(h)); }
+
+// signed 4 x int8 dot product with int32 accumulate (v_dot4_i32_i8)
+__device__ __forceinline__ int dot4(int a, int b, int c) { return __builtin_amdgcn_sdot4(a, b, c, false); }
+
+// 8 packed 4-bit codes in one dword (low nibbles = k 0..3, high nibbles = k 4..7 of one column)
+// against 8 int8 activation codes (xlo = k 0..3, xhi = k 4..7)
+__device__ __forceinline__ int dot8_q4(uint32_t w, int xlo, int xhi, int acc) {
+    acc = dot4((int)(w & 0x0F0F0F0Fu), xlo, acc);
+    acc = dot4((int)((w >> 4) & 0x0F0F0F0Fu), xhi, acc);
+    return acc;
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    return v;
+}
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+
+#endif  // __HIPCC__
+
+}  // namespace llmops

@@ -1,0 +1,91 @@
+// C ABI of the Q4_1 x Q8 fully-connected op: argument checks, workspace layout and dispatch
+// between the dot4 streaming kernel (few rows) and the int8 MFMA kernel (many rows).
+#include "common.h"
+
+namespace llmops {
+
+constexpr int kMaxGemvRows = 8;
+
+int launch_quant_x(const float* x, int64_t rows, int64_t K, int group_k, int8_t* xq, float* xd, float* gsum,
+                   hipStream_t stream);
+size_t gemv_workspace_bytes(int64_t rows, int64_t Ng, int64_t Kg, int G);
+int launch_gemv(const uint8_t* w, const int8_t* xq, const float* xd, const float* gs, float* y, float* part,
+                unsigned* counters, int64_t rows, int64_t Ng, int64_t Kg, int G, int64_t N, hipStream_t st);
+int launch_gemv_partials(const uint8_t* w, const int8_t* xq, int32_t* acc, int64_t rows, int64_t Ng, int64_t Kg, int G,
+                         hipStream_t st);
+size_t gemm_workspace_bytes(int64_t rows, int64_t Ng, int64_t Kg);
+int launch_gemm(const uint8_t* w, const int8_t* xq, const float* xd, const float* gs, float* y, float* part,
+                int64_t rows, int64_t Ng, int64_t Kg, int G, int64_t N, hipStream_t st);
+int launch_gemm_partials(const uint8_t* w, const int8_t* xq, int32_t* acc, int64_t rows, int64_t Ng, int64_t Kg, int G,
+                         hipStream_t st);
+
+static inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+struct FcWorkspace {
+    size_t off_xq, off_xd, off_gs, off_part, total;
+};
+
+static FcWorkspace fc_layout(int64_t rows, int64_t Ng, int64_t Kg, int G) {
+    FcWorkspace w;
+    size_t o = LLMOPS_FC_COUNTER_BYTES;
+    w.off_xq = o;
+    o = align_up(o + (size_t)rows * Kg * G, 256);
+    w.off_xd = o;
+    o = align_up(o + (size_t)rows * Kg * sizeof(float), 256);
+    w.off_gs = o;
+    o = align_up(o + (size_t)rows * Kg * sizeof(float), 256);
+    w.off_part = o;
+    o = align_up(o + (rows <= kMaxGemvRows ? gemv_workspace_bytes(rows, Ng, Kg, G) : gemm_workspace_bytes(rows, Ng, Kg)), 256);
+    w.total = o;
+    return w;
+}
+
+}  // namespace llmops
+
+using namespace llmops;
+
+extern "C" size_t llmops_fc_Q4A_workspace_bytes(int64_t rows, int64_t K, int64_t Ng, int64_t Kg, int group_k) {
+    (void)K;
+    if (!valid_group(group_k) || rows <= 0 || Ng <= 0 || Kg <= 0) return 0;
+    return fc_layout(rows, Ng, Kg, group_k).total;
+}
+
+extern "C" int llmops_fc_Q4A(const float* x, int64_t rows, int64_t K, const int8_t* weiq, int64_t Ng, int64_t Kg,
+                             int group_k, int64_t N, float* y, void* workspace, size_t workspace_bytes,
+                             llmops_stream_t stream) {
+    LLMOPS_REQUIRE(valid_group(group_k));
+    LLMOPS_REQUIRE(x != nullptr && weiq != nullptr && y != nullptr && workspace != nullptr);
+    LLMOPS_REQUIRE(rows > 0 && K > 0 && Ng > 0 && Kg > 0);
+    LLMOPS_REQUIRE(K == Kg * group_k);  // the reference reads past K otherwise (ops/op_fc.hpp:184)
+    LLMOPS_REQUIRE(N > (Ng - 1) * kGroupN && N <= Ng * kGroupN);
+    LLMOPS_REQUIRE(Ng * kGroupN <= LLMOPS_FC_COUNTER_BYTES / 4 * kGroupN);
+    LLMOPS_REQUIRE(Ng * 64 < ((int64_t)1 << 31));
+    LLMOPS_REQUIRE(aligned(weiq, 16) && aligned(workspace, 256));
+    const FcWorkspace lay = fc_layout(rows, Ng, Kg, group_k);
+    if (workspace_bytes < lay.total)
+        return fail(LLMOPS_EWORKSPACE, "fc_Q4A needs %zu workspace bytes, got %zu", lay.total, workspace_bytes);
+    uint8_t* ws = reinterpret_cast<uint8_t*>(workspace);
+    unsigned* counters = reinterpret_cast<unsigned*>(ws);
+    int8_t* xq = reinterpret_cast<int8_t*>(ws + lay.off_xq);
+    float* xd = reinterpret_cast<float*>(ws + lay.off_xd);
+    float* gs = reinterpret_cast<float*>(ws + lay.off_gs);
+    float* part = reinterpret_cast<float*>(ws + lay.off_part);
+    hipStream_t st = as_stream(stream);
+    int rc = launch_quant_x(x, rows, K, group_k, xq, xd, gs, st);
+    if (rc) return rc;
+    const uint8_t* w = reinterpret_cast<const uint8_t*>(weiq);
+    if (rows <= kMaxGemvRows) return launch_gemv(w, xq, xd, gs, y, part, counters, rows, Ng, Kg, group_k, N, st);
+    return launch_gemm(w, xq, xd, gs, y, part, rows, Ng, Kg, group_k, N, st);
+}
+
+extern "C" int llmops_fc_Q4A_partials(const int8_t* xq, int64_t rows, const int8_t* weiq, int64_t Ng, int64_t Kg,
+                                      int group_k, int32_t* acc, int use_mfma, llmops_stream_t stream) {
+    LLMOPS_REQUIRE(valid_group(group_k));
+    LLMOPS_REQUIRE(xq != nullptr && weiq != nullptr && acc != nullptr);
+    LLMOPS_REQUIRE(rows > 0 && Ng > 0 && Kg > 0);
+    LLMOPS_REQUIRE(aligned(weiq, 16) && aligned(xq, 16));
+    LLMOPS_REQUIRE(Ng * Kg < ((int64_t)1 << 31));
+    const uint8_t* w = reinterpret_cast<const uint8_t*>(weiq);
+    if (use_mfma) return launch_gemm_partials(w, xq, acc, rows, Ng, Kg, group_k, as_stream(stream));
+    return launch_gemv_partials(w, xq, acc, rows, Ng, Kg, group_k, as_stream(stream));
+}

@@ -1,0 +1,275 @@
+// Q4_1 x Q8 fully-connected product for many activation rows (prefill): int8 MFMA.
+//
+// A wavefront owns two adjacent strips (64 output columns) and RT tiles of 16 activation rows.
+// Operand layout of v_mfma_i32_16x16x{64,32}_i8: lane = 16*g + jj; the A lane holds row jj,
+// the B lane holds column jj, both for the same set of k-values chosen by g.  The packed
+// format gives, per 16-byte load, 4 adjacent columns x 8 k-values of one k8-row.  So lane
+// (g, jj) loads the k8-rows that belong to g for columns 4*(jj&7)..+3 of strip (jj>>3); dword c
+// of that load is the lane's B operand for MFMA number c, whose 16 tile columns are
+// { strip (jj>>3), column 4*(jj&7)+c }.  Unpacking is two ANDs and a shift per dword; nothing is
+// shuffled between lanes and the weights never pass through LDS.
+//   G=128: one MFMA 16x16x64 covers 8 k8-rows (g owns rows 2g,2g+1 = 16 consecutive k);
+//          two of them make one k-group.
+//   G=32 : one MFMA 16x16x32 covers the group's 4 k8-rows (g owns row g = 8 consecutive k).
+// After every k-group the int32 tile is folded into fp32 accumulators:
+//   f += (d[n]*dx[row]) * float(acc) ; f += m[n]*gsum[row]        (fc_Q4A,
+//   /root/reference/ops/op_fc.hpp:381-412; min term is m * raw group sum).
+// Result tile layout of the 16x16 MFMAs: lane holds column jj, rows 4*g+v in register v.
+#include "common.h"
+
+namespace llmops {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ uint32_t lo4(uint32_t w) { return w & 0x0F0F0F0Fu; }
+__device__ __forceinline__ uint32_t hi4(uint32_t w) { return (w >> 4) & 0x0F0F0F0Fu; }
+
+template <int G>
+struct GemmTraits;
+template <>
+struct GemmTraits<128> {
+    static constexpr int kSteps = 2;  // MFMAs per k-group
+};
+template <>
+struct GemmTraits<32> {
+    static constexpr int kSteps = 1;
+};
+
+// acc[t][c] += A(row tile t) x B(column set c) over one k-group
+template <int G, int RT>
+__device__ __forceinline__ void mma_group(const uint8_t* blk, const int8_t* const xrow[RT], int64_t kofs, int g, int q,
+                                          v4i acc[RT][4]) {
+    if (G == 128) {
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            const uint4 wa = *reinterpret_cast<const uint4*>(blk + h * 1024 + (2 * g) * kRowBytes + q * 16);
+            const uint4 wb = *reinterpret_cast<const uint4*>(blk + h * 1024 + (2 * g + 1) * kRowBytes + q * 16);
+            const uint32_t* pa = reinterpret_cast<const uint32_t*>(&wa);
+            const uint32_t* pb = reinterpret_cast<const uint32_t*>(&wb);
+            v4i b[4];
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+                b[c][0] = (int)lo4(pa[c]);
+                b[c][1] = (int)hi4(pa[c]);
+                b[c][2] = (int)lo4(pb[c]);
+                b[c][3] = (int)hi4(pb[c]);
+            }
+#pragma unroll
+            for (int t = 0; t < RT; t++) {
+                const v4i a = *reinterpret_cast<const v4i*>(xrow[t] + kofs + h * 64 + g * 16);
+#pragma unroll
+                for (int c = 0; c < 4; c++) acc[t][c] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b[c], acc[t][c], 0, 0, 0);
+            }
+        }
+    } else {
+        const uint4 wa = *reinterpret_cast<const uint4*>(blk + g * kRowBytes + q * 16);
+        const uint32_t* pa = reinterpret_cast<const uint32_t*>(&wa);
+        long b[4];
+#pragma unroll
+        for (int c = 0; c < 4; c++) b[c] = (long)(((uint64_t)hi4(pa[c]) << 32) | (uint64_t)lo4(pa[c]));
+#pragma unroll
+        for (int t = 0; t < RT; t++) {
+            const long a = *reinterpret_cast<const long*>(xrow[t] + kofs + g * 8);
+#pragma unroll
+            for (int c = 0; c < 4; c++) acc[t][c] = __builtin_amdgcn_mfma_i32_16x16x32_i8(a, b[c], acc[t][c], 0, 0, 0);
+        }
+    }
+}
+
+// grid: x = ceil(pairs/4) (4 waves = 4 strip pairs per workgroup), y = row blocks of RT*16, z = k splits
+template <int G, int RT>
+__global__ __launch_bounds__(256) void fc_gemm_kernel(const uint8_t* __restrict__ weiq, const int8_t* __restrict__ xq,
+                                                       const float* __restrict__ xd, const float* __restrict__ gs,
+                                                       float* __restrict__ out, int Ng, int Kg, int64_t ldo, int64_t N,
+                                                       int rows, int kb_per_split, int64_t split_stride) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int g = lane >> 4, jj = lane & 15, q = jj & 7, sp = jj >> 3;
+    const int pair = blockIdx.x * 4 + wave;
+    if (pair * 2 >= Ng) return;
+    const int strip = pair * 2 + sp;
+    const bool strip_ok = strip < Ng;
+    const int strip_c = strip_ok ? strip : Ng - 1;
+    const int row0 = blockIdx.y * (RT * 16);
+    const int kb0 = blockIdx.z * kb_per_split, kb1 = min(Kg, kb0 + kb_per_split);
+    const int64_t Kp = (int64_t)Kg * G;
+    const uint8_t* sbase = weiq + (int64_t)strip_c * Kg * block_bytes(G);
+
+    const int8_t* xrow[RT];
+    int vrow[RT][4];  // clamped global row of result register v
+#pragma unroll
+    for (int t = 0; t < RT; t++) {
+        xrow[t] = xq + (int64_t)min(rows - 1, row0 + t * 16 + jj) * Kp;
+#pragma unroll
+        for (int v = 0; v < 4; v++) vrow[t][v] = min(rows - 1, row0 + t * 16 + g * 4 + v);
+    }
+
+    float f[RT][4][4];
+#pragma unroll
+    for (int t = 0; t < RT; t++)
+#pragma unroll
+        for (int c = 0; c < 4; c++)
+#pragma unroll
+            for (int v = 0; v < 4; v++) f[t][c][v] = 0.0f;
+
+    for (int kb = kb0; kb < kb1; kb++) {
+        const uint8_t* blk = sbase + (int64_t)kb * block_bytes(G);
+        v4i acc[RT][4];
+#pragma unroll
+        for (int t = 0; t < RT; t++)
+#pragma unroll
+            for (int c = 0; c < 4; c++) acc[t][c] = v4i{0, 0, 0, 0};
+        mma_group<G, RT>(blk, xrow, (int64_t)kb * G, g, q, acc);
+
+        const uint2 dh = *reinterpret_cast<const uint2*>(blk + (G / 8) * kRowBytes + q * 8);
+        const uint2 mh = *reinterpret_cast<const uint2*>(blk + (G / 8) * kRowBytes + 64 + q * 8);
+        float d[4], m[4];
+        d[0] = f16_bits_to_f32((uint16_t)(dh.x & 0xFFFFu));
+        d[1] = f16_bits_to_f32((uint16_t)(dh.x >> 16));
+        d[2] = f16_bits_to_f32((uint16_t)(dh.y & 0xFFFFu));
+        d[3] = f16_bits_to_f32((uint16_t)(dh.y >> 16));
+        m[0] = f16_bits_to_f32((uint16_t)(mh.x & 0xFFFFu));
+        m[1] = f16_bits_to_f32((uint16_t)(mh.x >> 16));
+        m[2] = f16_bits_to_f32((uint16_t)(mh.y & 0xFFFFu));
+        m[3] = f16_bits_to_f32((uint16_t)(mh.y >> 16));
+#pragma unroll
+        for (int t = 0; t < RT; t++)
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                const float dx = xd[(int64_t)vrow[t][v] * Kg + kb];
+                const float gsum = gs[(int64_t)vrow[t][v] * Kg + kb];
+#pragma unroll
+                for (int c = 0; c < 4; c++) {
+                    f[t][c][v] = fmaf(d[c] * dx, (float)acc[t][c][v], f[t][c][v]);
+                    f[t][c][v] = fmaf(m[c], gsum, f[t][c][v]);
+                }
+            }
+    }
+
+    if (!strip_ok) return;
+    float* o = out + (int64_t)blockIdx.z * split_stride;
+    const int64_t n0 = (int64_t)strip * kGroupN + q * 4;
+#pragma unroll
+    for (int t = 0; t < RT; t++)
+#pragma unroll
+        for (int v = 0; v < 4; v++) {
+            const int row = row0 + t * 16 + g * 4 + v;
+            if (row >= rows) continue;
+#pragma unroll
+            for (int c = 0; c < 4; c++)
+                if (n0 + c < N) o[(int64_t)row * ldo + n0 + c] = f[t][c][v];
+        }
+}
+
+// y[row][n] = sum over splits (index order) of part[s][row][n]
+__global__ void gemm_reduce_kernel(const float* __restrict__ part, float* __restrict__ y, int64_t rows, int64_t N,
+                                   int64_t ldp, int64_t split_stride, int S) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= rows * N) return;
+    const int64_t r = i / N, n = i % N;
+    float a = 0.0f;
+    for (int s = 0; s < S; s++) a += part[(int64_t)s * split_stride + r * ldp + n];
+    y[i] = a;
+}
+
+// Integer core only, through the same mma_group: acc[row][n][kb]
+template <int G>
+__global__ __launch_bounds__(256) void fc_gemm_partials_kernel(const uint8_t* __restrict__ weiq,
+                                                                const int8_t* __restrict__ xq, int32_t* __restrict__ out,
+                                                                int Ng, int Kg, int rows) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int g = lane >> 4, jj = lane & 15, q = jj & 7, sp = jj >> 3;
+    const int pair = blockIdx.x * 4 + wave;
+    if (pair * 2 >= Ng) return;
+    const int strip = pair * 2 + sp;
+    const bool strip_ok = strip < Ng;
+    const int strip_c = strip_ok ? strip : Ng - 1;
+    const int row0 = blockIdx.y * 16;
+    const int kb = blockIdx.z;
+    const int64_t Kp = (int64_t)Kg * G;
+    const int64_t Np = (int64_t)Ng * kGroupN;
+    const uint8_t* blk = weiq + ((int64_t)strip_c * Kg + kb) * block_bytes(G);
+    const int8_t* xrow[1] = {xq + (int64_t)min(rows - 1, row0 + jj) * Kp};
+    v4i acc[1][4];
+#pragma unroll
+    for (int c = 0; c < 4; c++) acc[0][c] = v4i{0, 0, 0, 0};
+    mma_group<G, 1>(blk, xrow, (int64_t)kb * G, g, q, acc);
+    if (!strip_ok) return;
+#pragma unroll
+    for (int v = 0; v < 4; v++) {
+        const int row = row0 + g * 4 + v;
+        if (row >= rows) continue;
+#pragma unroll
+        for (int c = 0; c < 4; c++) out[((int64_t)row * Np + strip * kGroupN + q * 4 + c) * Kg + kb] = acc[0][c][v];
+    }
+}
+
+struct GemmPlan {
+    int RT, S, kb_per_split;
+};
+
+static GemmPlan plan_gemm(int64_t rows, int64_t Ng, int64_t Kg) {
+    GemmPlan p;
+    p.RT = rows > 32 ? 4 : (rows > 16 ? 2 : 1);
+    const int64_t row_blocks = (rows + p.RT * 16 - 1) / (p.RT * 16);
+    const int64_t waves = ((Ng + 1) / 2) * row_blocks;
+    int S = (int)((2048 + waves - 1) / waves);  // aim for >= 2048 wavefronts
+    if (S > Kg) S = (int)Kg;
+    if (S < 1) S = 1;
+    p.kb_per_split = (int)((Kg + S - 1) / S);
+    p.S = (int)((Kg + p.kb_per_split - 1) / p.kb_per_split);
+    return p;
+}
+
+size_t gemm_workspace_bytes(int64_t rows, int64_t Ng, int64_t Kg) {
+    const GemmPlan p = plan_gemm(rows, Ng, Kg);
+    return p.S > 1 ? (size_t)p.S * rows * Ng * kGroupN * sizeof(float) : 0;
+}
+
+template <int G, int RT>
+static void launch_gemm_t(const uint8_t* w, const int8_t* xq, const float* xd, const float* gs, float* out, int64_t Ng,
+                          int64_t Kg, int64_t ldo, int64_t N, int64_t rows, const GemmPlan& p, int64_t split_stride,
+                          hipStream_t st) {
+    dim3 grid((unsigned)(((Ng + 1) / 2 + 3) / 4), (unsigned)((rows + RT * 16 - 1) / (RT * 16)), (unsigned)p.S);
+    fc_gemm_kernel<G, RT><<<grid, 256, 0, st>>>(w, xq, xd, gs, out, (int)Ng, (int)Kg, ldo, N, (int)rows, p.kb_per_split,
+                                                split_stride);
+}
+
+int launch_gemm(const uint8_t* w, const int8_t* xq, const float* xd, const float* gs, float* y, float* part,
+                int64_t rows, int64_t Ng, int64_t Kg, int G, int64_t N, hipStream_t st) {
+    const GemmPlan p = plan_gemm(rows, Ng, Kg);
+    const int64_t Np = Ng * kGroupN;
+    float* out = p.S > 1 ? part : y;
+    const int64_t ldo = p.S > 1 ? Np : N;
+    const int64_t ss = rows * Np;
+#define LLMOPS_GEMM_CASE(GG, RR) launch_gemm_t<GG, RR>(w, xq, xd, gs, out, Ng, Kg, ldo, p.S > 1 ? Np : N, rows, p, ss, st)
+    if (G == 128) {
+        if (p.RT == 4) LLMOPS_GEMM_CASE(128, 4);
+        else if (p.RT == 2) LLMOPS_GEMM_CASE(128, 2);
+        else LLMOPS_GEMM_CASE(128, 1);
+    } else {
+        if (p.RT == 4) LLMOPS_GEMM_CASE(32, 4);
+        else if (p.RT == 2) LLMOPS_GEMM_CASE(32, 2);
+        else LLMOPS_GEMM_CASE(32, 1);
+    }
+#undef LLMOPS_GEMM_CASE
+    LLMOPS_LAUNCH_CHECK();
+    if (p.S > 1) {
+        const int64_t total = rows * N;
+        gemm_reduce_kernel<<<(unsigned)((total + 255) / 256), 256, 0, st>>>(part, y, rows, N, Np, ss, p.S);
+        LLMOPS_LAUNCH_CHECK();
+    }
+    return LLMOPS_OK;
+}
+
+int launch_gemm_partials(const uint8_t* w, const int8_t* xq, int32_t* acc, int64_t rows, int64_t Ng, int64_t Kg, int G,
+                         hipStream_t st) {
+    dim3 grid((unsigned)(((Ng + 1) / 2 + 3) / 4), (unsigned)((rows + 15) / 16), (unsigned)Kg);
+    if (G == 128)
+        fc_gemm_partials_kernel<128><<<grid, 256, 0, st>>>(w, xq, acc, (int)Ng, (int)Kg, (int)rows);
+    else
+        fc_gemm_partials_kernel<32><<<grid, 256, 0, st>>>(w, xq, acc, (int)Ng, (int)Kg, (int)rows);
+    LLMOPS_LAUNCH_CHECK();
+    return LLMOPS_OK;
+}
+
+}  // namespace llmops

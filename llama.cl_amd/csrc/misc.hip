@@ -1,0 +1,142 @@
+// Element-wise and row-wise neighbours of the FC/attention path that one decode step needs
+// (/root/reference/ops/op_misc.hpp, ops/op_embedding.hpp).  All fp32, all in place like the
+// reference; each is a single bandwidth-trivial launch.
+#include "common.h"
+
+namespace llmops {
+
+// rmsnorm (ops/op_misc.hpp:142-181): one workgroup per row
+__global__ __launch_bounds__(256) void rmsnorm_kernel(float* __restrict__ x, int64_t hidden, const float* __restrict__ w,
+                                                       float eps) {
+    __shared__ float red[4];
+    float* row = x + (int64_t)blockIdx.x * hidden;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    float ss = 0.0f;
+    for (int64_t i = threadIdx.x; i < hidden; i += 256) ss = fmaf(row[i], row[i], ss);
+    ss = wave_sum(ss);
+    if (lane == 0) red[wave] = ss;
+    __syncthreads();
+    const float rms = (((red[0] + red[1]) + red[2]) + red[3]) / (float)hidden;
+    const float rs = 1.0f / sqrtf(rms + eps);
+    for (int64_t i = threadIdx.x; i < hidden; i += 256) row[i] = row[i] * rs * w[i];
+}
+
+template <bool MUL>
+__global__ void ibinary_kernel(float* __restrict__ a, const float* __restrict__ b, int64_t total, int64_t inner,
+                               int b_is_row) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    const float bv = b[b_is_row ? i % inner : i];
+    a[i] = MUL ? a[i] * bv : a[i] + bv;
+}
+
+// itrans "silu" (ops/op_misc.hpp:127-138): x * 1/(1+exp(-x)), exact reciprocal
+__global__ void silu_kernel(float* __restrict__ a, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const float v = a[i];
+    a[i] = v * (1.0f / (1.0f + expf(-v)));
+}
+
+// embedding_q8c_quant_w (ops/op_embedding.hpp:51-78): per-row amax/127 scale, RNE int8 codes
+__global__ __launch_bounds__(256) void emb_quant_kernel(const float* __restrict__ w, int64_t E, int8_t* __restrict__ q,
+                                                         float* __restrict__ scales) {
+    __shared__ float red[4];
+    const float* row = w + (int64_t)blockIdx.x * E;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    float amax = 0.0f;
+    for (int64_t i = threadIdx.x; i < E; i += 256) amax = fmaxf(amax, fabsf(row[i]));
+    amax = wave_max(amax);
+    if (lane == 0) red[wave] = amax;
+    __syncthreads();
+    amax = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    const float d = amax / 127.0f;
+    const float id = (d != 0.0f) ? (1.0f / d) : 0.0f;
+    if (threadIdx.x == 0) scales[blockIdx.x] = d;
+    const int64_t vec = E & ~(int64_t)7;  // the reference's scalar tail rounds half away (ops/utils.hpp:217-219)
+    for (int64_t i = threadIdx.x; i < E; i += 256) {
+        const float t = row[i] * id;
+        float r = (i < vec) ? rintf(t) : roundf(t);
+        r = fminf(127.0f, fmaxf(-128.0f, r));
+        q[(int64_t)blockIdx.x * E + i] = (t != t) ? (int8_t)-128 : (int8_t)(int)r;
+    }
+}
+
+// embedding_q8c (ops/op_embedding.hpp:81-137): out[i,:] = scales[id] * q[id,:]
+__global__ void emb_q8c_kernel(float* __restrict__ out, const int64_t* __restrict__ ids, const int8_t* __restrict__ q,
+                               const float* __restrict__ scales, int64_t E) {
+    const int64_t id = ids[blockIdx.x];
+    const float s = scales[id];
+    for (int64_t e = threadIdx.x; e < E; e += blockDim.x) out[(int64_t)blockIdx.x * E + e] = s * (float)q[id * E + e];
+}
+
+// embedding (ops/op_embedding.hpp:24-49): out[i,:] = w[ids[i],:]
+__global__ void emb_kernel(float* __restrict__ out, const int64_t* __restrict__ ids, const float* __restrict__ w, int64_t E) {
+    const int64_t id = ids[blockIdx.x];
+    for (int64_t e = threadIdx.x; e < E; e += blockDim.x) out[(int64_t)blockIdx.x * E + e] = w[id * E + e];
+}
+
+}  // namespace llmops
+
+using namespace llmops;
+
+extern "C" int llmops_rmsnorm(float* x, int64_t rows, int64_t hidden, const float* w, float eps, llmops_stream_t stream) {
+    LLMOPS_REQUIRE(x != nullptr && w != nullptr && rows > 0 && hidden > 0 && rows < ((int64_t)1 << 31));
+    rmsnorm_kernel<<<(unsigned)rows, 256, 0, as_stream(stream)>>>(x, hidden, w, eps);
+    LLMOPS_LAUNCH_CHECK();
+    return LLMOPS_OK;
+}
+
+static int ibinary(bool mul, float* a, const float* b, int64_t rows, int64_t inner, int b_is_row, llmops_stream_t stream) {
+    LLMOPS_REQUIRE(a != nullptr && b != nullptr && rows > 0 && inner > 0);
+    const int64_t total = rows * inner;
+    LLMOPS_REQUIRE((total + 255) / 256 < ((int64_t)1 << 31));
+    const unsigned grid = (unsigned)((total + 255) / 256);
+    if (mul)
+        ibinary_kernel<true><<<grid, 256, 0, as_stream(stream)>>>(a, b, total, inner, b_is_row);
+    else
+        ibinary_kernel<false><<<grid, 256, 0, as_stream(stream)>>>(a, b, total, inner, b_is_row);
+    LLMOPS_LAUNCH_CHECK();
+    return LLMOPS_OK;
+}
+
+extern "C" int llmops_iadd(float* a, const float* b, int64_t rows, int64_t inner, int b_is_row, llmops_stream_t stream) {
+    return ibinary(false, a, b, rows, inner, b_is_row, stream);
+}
+extern "C" int llmops_imul(float* a, const float* b, int64_t rows, int64_t inner, int b_is_row, llmops_stream_t stream) {
+    return ibinary(true, a, b, rows, inner, b_is_row, stream);
+}
+
+extern "C" int llmops_itrans_silu(float* a, int64_t n, llmops_stream_t stream) {
+    LLMOPS_REQUIRE(a != nullptr && n > 0 && (n + 255) / 256 < ((int64_t)1 << 31));
+    silu_kernel<<<(unsigned)((n + 255) / 256), 256, 0, as_stream(stream)>>>(a, n);
+    LLMOPS_LAUNCH_CHECK();
+    return LLMOPS_OK;
+}
+
+extern "C" int llmops_embedding_q8c_quant_w(const float* w, int64_t V, int64_t E, int8_t* q, float* scales,
+                                            llmops_stream_t stream) {
+    LLMOPS_REQUIRE(w != nullptr && q != nullptr && scales != nullptr && V > 0 && E > 0 && V < ((int64_t)1 << 31));
+    emb_quant_kernel<<<(unsigned)V, 256, 0, as_stream(stream)>>>(w, E, q, scales);
+    LLMOPS_LAUNCH_CHECK();
+    return LLMOPS_OK;
+}
+
+extern "C" int llmops_embedding_q8c(float* out, const int64_t* ids, int64_t n, const int8_t* q, const float* scales,
+                                    int64_t V, int64_t E, llmops_stream_t stream) {
+    (void)V;
+    LLMOPS_REQUIRE(out != nullptr && ids != nullptr && q != nullptr && scales != nullptr && n > 0 && E > 0);
+    LLMOPS_REQUIRE(n < ((int64_t)1 << 31));
+    emb_q8c_kernel<<<(unsigned)n, 256, 0, as_stream(stream)>>>(out, ids, q, scales, E);
+    LLMOPS_LAUNCH_CHECK();
+    return LLMOPS_OK;
+}
+
+extern "C" int llmops_embedding(float* out, const int64_t* ids, int64_t n, const float* w, int64_t V, int64_t E,
+                                llmops_stream_t stream) {
+    (void)V;
+    LLMOPS_REQUIRE(out != nullptr && ids != nullptr && w != nullptr && n > 0 && E > 0 && n < ((int64_t)1 << 31));
+    emb_kernel<<<(unsigned)n, 256, 0, as_stream(stream)>>>(out, ids, w, E);
+    LLMOPS_LAUNCH_CHECK();
+    return LLMOPS_OK;
+}

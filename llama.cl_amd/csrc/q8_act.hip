@@ -1,0 +1,104 @@
+// Per-group Q8 dynamic activation quantization (FC_dynamic_quantize_x,
+// /root/reference/ops/op_fc.hpp:221-272).
+//
+// One wavefront quantizes one (row, k-group): the lanes hold the group's G floats in registers,
+// the absolute maximum is a wave reduction (order independent, hence exact), codes are
+// v_rndne (round half to even, like vroundps imm 0 in ops/utils.hpp:207) saturated to int8, and
+// the raw group sum is accumulated left to right from lane registers so that it carries the
+// same rounding as the reference's scalar loop (ops/op_fc.hpp:262-268).
+#include "common.h"
+
+namespace llmops {
+
+__device__ __forceinline__ float lane_value(float v, int lane) {
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), lane));
+}
+
+__device__ __forceinline__ int q8_code(float v, float id) {
+    const float t = v * id;
+    if (t != t) return -128;  // cvtps2dq(NaN) = INT_MIN, which the saturating packs turn into -128
+    return (int)fminf(127.0f, fmaxf(-128.0f, rintf(t)));
+}
+
+template <int G>
+__global__ __launch_bounds__(256) void quant_x_kernel(const float* __restrict__ x, int64_t rows, int64_t K, int64_t Kg,
+                                                       int8_t* __restrict__ xq, float* __restrict__ xd,
+                                                       float* __restrict__ gsum) {
+    constexpr int E = (G >= 64) ? G / 64 : 1;  // elements per lane
+    constexpr int LANES = G / E;               // lanes that hold data
+    const int lane = threadIdx.x & 63;
+    const int64_t item = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (item >= rows * Kg) return;  // whole wave leaves together
+    const int64_t r = item / Kg, kb = item % Kg;
+    const float* raw = x + r * K + kb * G;
+    const int64_t left = K - kb * G;
+    const int len = (int)(left < G ? left : G);
+
+    float v[E];
+#pragma unroll
+    for (int j = 0; j < E; j++) {
+        const int e = lane * E + j;
+        v[j] = (lane < LANES && e < len) ? raw[e] : 0.0f;
+    }
+    float amax = 0.0f;
+#pragma unroll
+    for (int j = 0; j < E; j++) amax = fmaxf(amax, fabsf(v[j]));
+    amax = wave_max(amax);
+    const float d = amax / 127.0f;
+    const float id = (d != 0.0f) ? (1.0f / d) : 0.0f;
+
+    if (lane < LANES) {
+        int8_t* q = xq + (r * Kg + kb) * G + lane * E;
+        if (E == 2) {
+            const uint32_t c0 = (uint32_t)q8_code(v[0], id) & 0xFFu;
+            const uint32_t c1 = (uint32_t)q8_code(v[E - 1], id) & 0xFFu;
+            const int e = lane * E;
+            // padding beyond len is zero (ops/op_fc.hpp:259-261)
+            *reinterpret_cast<uint16_t*>(q) = (uint16_t)((e < len ? c0 : 0u) | ((e + 1 < len ? c1 : 0u) << 8));
+        } else {
+            q[0] = (lane < len) ? (int8_t)q8_code(v[0], id) : (int8_t)0;
+        }
+    }
+
+    // left-to-right fp32 sum of the raw group, computed redundantly by every lane
+    float s = 0.0f;
+#pragma unroll
+    for (int i = 0; i < G; i++) {
+        if (i < len) s += lane_value(v[i % E], i / E);
+    }
+    if (lane == 0) {
+        xd[r * Kg + kb] = d;
+        gsum[r * Kg + kb] = s;
+    }
+}
+
+}  // namespace llmops
+
+using namespace llmops;
+
+namespace llmops {
+// shared with fc.hip
+int launch_quant_x(const float* x, int64_t rows, int64_t K, int group_k, int8_t* xq, float* xd, float* gsum,
+                   hipStream_t stream) {
+    const int64_t Kg = (K + group_k - 1) / group_k;
+    const int64_t items = rows * Kg;
+    const unsigned grid = (unsigned)((items + 3) / 4);
+    if (group_k == 32)
+        quant_x_kernel<32><<<grid, 256, 0, stream>>>(x, rows, K, Kg, xq, xd, gsum);
+    else
+        quant_x_kernel<128><<<grid, 256, 0, stream>>>(x, rows, K, Kg, xq, xd, gsum);
+    LLMOPS_LAUNCH_CHECK();
+    return LLMOPS_OK;
+}
+}  // namespace llmops
+
+extern "C" int llmops_FC_dynamic_quantize_x(const float* x, int64_t rows, int64_t K, int group_k, int8_t* xq,
+                                            float* xd, float* gsum, llmops_stream_t stream) {
+    LLMOPS_REQUIRE(valid_group(group_k));
+    LLMOPS_REQUIRE(x != nullptr && xq != nullptr && xd != nullptr && gsum != nullptr);
+    LLMOPS_REQUIRE(rows > 0 && K > 0 && (K % 8) == 0);
+    LLMOPS_REQUIRE(aligned(xq, 2));
+    const int64_t Kg = (K + group_k - 1) / group_k;
+    LLMOPS_REQUIRE(rows * Kg < ((int64_t)1 << 33));
+    return launch_quant_x(x, rows, K, group_k, xq, xd, gsum, as_stream(stream));
+}

@@ -1,0 +1,309 @@
+"""``llmops`` for MI355X -- drop-in for the reference's pybind11 module of the same name
+(``PYBIND11_MODULE(llmops, m)``, /root/reference/ops/main.cpp:62-179).
+
+Same op names, argument order, shapes, dtypes and in-place behaviour as the reference; the tensor
+type at the boundary is a ``torch.Tensor`` on the HIP device instead of the reference's own
+``llmops.tensor``.  Every op enqueues hand-written gfx950 kernels from ``libllmops_hip.so`` on the
+current torch stream.  There is no CPU or eager fallback: a missing library or a host tensor
+raises.
+
+Differences a caller can see:
+* The k-group size is a run-time choice (``group_k=32|128`` on ``offline_FC_quant_Q4A``, or
+  ``set_default_group_k``) instead of a compile-time constant (ops/op_fc.hpp:109); the other ops
+  recover it from the packed tensor's last dimension (640 -> 32, 2176 -> 128).
+* ``attention_rope[2]`` also accepts a float16 ``kv_cache`` (fp32 math on fp16-rounded K/V).
+* Errors are ``RuntimeError`` with the failed condition, like the reference's ``ASSERT``.
+"""
+import ctypes
+
+import torch
+
+from . import _lib
+
+__all__ = [
+    "offline_FC_quant_Q4A", "offline_FC_dequant_Q4A", "fc_Q4A", "FC_dynamic_quantize_x", "fc_Q4A_partials",
+    "attention_rope", "attention_rope2", "rope_embed", "softmax", "rmsnorm", "iadd", "imul", "itrans", "clone",
+    "empty", "ones", "embedding", "embedding_q8c_quant_w", "embedding_q8c", "tensor_pool", "set_default_group_k",
+    "group_k_of",
+]
+
+_default_group_k = 32  # the reference's compiled-in default (ops/op_fc.hpp:109)
+_workspaces = {}
+
+
+def set_default_group_k(g):
+    global _default_group_k
+    _require(g in (32, 128), "group_k in (32, 128)")
+    _default_group_k = g
+
+
+def _require(cond, what):
+    if not cond:
+        raise RuntimeError(f"assert {what} failed")
+
+
+def _ptr(t):
+    return ctypes.c_void_p(t.data_ptr())
+
+
+def _stream(t):
+    return ctypes.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+
+
+def _dev(t, dtype, rank=None, name="tensor"):
+    _require(isinstance(t, torch.Tensor), f"{name} is a torch.Tensor")
+    _require(t.is_cuda, f"{name} is on the HIP device (llmops has no CPU path)")
+    _require(t.dtype == dtype, f"{name}.is<{dtype}>")
+    if rank is not None:
+        _require(t.dim() == rank, f"{name}.rank == {rank}")
+    _require(t.is_contiguous(), f"{name}.is_dense()")
+
+
+def _workspace(device, nbytes):
+    """Persistent per-device scratch.  Its first bytes hold the split-K arrival counters, which
+    must start at zero and which the kernels leave at zero."""
+    key = (device.type, device.index)
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < nbytes:
+        size = max(int(nbytes), 16 << 20)
+        ws = torch.zeros(size, dtype=torch.uint8, device=device)
+        _workspaces[key] = ws
+    return ws
+
+
+def group_k_of(weiq):
+    bb = weiq.shape[-1]
+    g = (bb - 128) // 16
+    _require(g in (32, 128) and (g // 8) * 128 + 128 == bb, "weiq.size(2) == sizeof(q4_block)")
+    return g
+
+
+# ---- Q4_1 fully connected ---------------------------------------------------------------------
+def offline_FC_quant_Q4A(wei, group_k=None):
+    """fp32 [N,K] -> int8 [ceil(N/32), ceil(K/G), blk(G)] (ops/op_fc.hpp:151-219)."""
+    g = _default_group_k if group_k is None else group_k
+    _require(g in (32, 128), "group_k in (32, 128)")
+    _require(isinstance(wei, torch.Tensor) and wei.is_cuda, "wei is on the HIP device (llmops has no CPU path)")
+    _require(wei.dtype == torch.float32 and wei.dim() == 2, "wei.is<float>(2)")
+    _require(wei.stride(1) == 1, "wei inner dimension is contiguous")
+    N, K = wei.shape
+    lib = _lib.load()
+    Ng, Kg = -(-N // 32), -(-K // g)
+    out = torch.empty((Ng, Kg, lib.llmops_q4a_block_bytes(g)), dtype=torch.int8, device=wei.device)
+    _lib.check(lib.llmops_offline_FC_quant_Q4A(_ptr(wei), N, K, wei.stride(0), g, _ptr(out), _stream(wei)))
+    return out
+
+
+def offline_FC_dequant_Q4A(weiq):
+    """int8 [Ng,Kg,blk] -> fp32 [Ng*32, Kg*G] (ops/op_fc.hpp:124-149)."""
+    _dev(weiq, torch.int8, 3, "weiq")
+    g = group_k_of(weiq)
+    Ng, Kg, _ = weiq.shape
+    out = torch.empty((Ng * 32, Kg * g), dtype=torch.float32, device=weiq.device)
+    _lib.check(_lib.load().llmops_offline_FC_dequant_Q4A(_ptr(weiq), Ng, Kg, g, _ptr(out), _stream(weiq)))
+    return out
+
+
+def FC_dynamic_quantize_x(input, group_k):
+    """fp32 [..,K] -> (xq int8 [..,Kg*G], xd fp32 [..,Kg], gsum fp32 [..,Kg]) (ops/op_fc.hpp:221-272)."""
+    _dev(input, torch.float32, None, "input")
+    _require(group_k in (32, 128), "group_k in (32, 128)")
+    K = input.shape[-1]
+    lead = tuple(input.shape[:-1])
+    rows = input.numel() // K
+    Kg = -(-K // group_k)
+    xq = torch.empty(lead + (Kg * group_k,), dtype=torch.int8, device=input.device)
+    xd = torch.empty(lead + (Kg,), dtype=torch.float32, device=input.device)
+    gs = torch.empty(lead + (Kg,), dtype=torch.float32, device=input.device)
+    _lib.check(_lib.load().llmops_FC_dynamic_quantize_x(_ptr(input), rows, K, group_k, _ptr(xq), _ptr(xd), _ptr(gs),
+                                                       _stream(input)))
+    return xq, xd, gs
+
+
+def fc_Q4A(input, weiq, N):
+    """fp32 [B,M,K] x packed [Ng,Kg,blk] -> fp32 [B,M,N] (ops/op_fc.hpp:286-426)."""
+    _dev(input, torch.float32, 3, "input")
+    _dev(weiq, torch.int8, 3, "wei_quantized")
+    g = group_k_of(weiq)
+    B, M, K = input.shape
+    Ng, Kg, _ = weiq.shape
+    rows = B * M
+    lib = _lib.load()
+    need = lib.llmops_fc_Q4A_workspace_bytes(rows, K, Ng, Kg, g)
+    ws = _workspace(input.device, need)
+    out = torch.empty((B, M, int(N)), dtype=torch.float32, device=input.device)
+    _lib.check(lib.llmops_fc_Q4A(_ptr(input), rows, K, _ptr(weiq), Ng, Kg, g, int(N), _ptr(out), _ptr(ws), ws.numel(),
+                                 _stream(input)))
+    return out
+
+
+def fc_Q4A_partials(xq, weiq, use_mfma=False):
+    """The exact int32 core of fc_Q4A: int8 [..,Kg*G] x packed -> int32 [.., Ng*32, Kg]."""
+    _dev(xq, torch.int8, None, "xq")
+    _dev(weiq, torch.int8, 3, "wei_quantized")
+    g = group_k_of(weiq)
+    Ng, Kg, _ = weiq.shape
+    _require(xq.shape[-1] == Kg * g, "xq.size(-1) == Kgroups * group_k")
+    lead = tuple(xq.shape[:-1])
+    rows = xq.numel() // (Kg * g)
+    acc = torch.empty(lead + (Ng * 32, Kg), dtype=torch.int32, device=xq.device)
+    _lib.check(_lib.load().llmops_fc_Q4A_partials(_ptr(xq), rows, _ptr(weiq), Ng, Kg, g, _ptr(acc), int(bool(use_mfma)),
+                                                  _stream(xq)))
+    return acc
+
+
+# ---- attention --------------------------------------------------------------------------------
+def rope_embed(x, inv_freq, position_id):
+    """In place on fp32 [B,H,L,S] (ops/op_attn.hpp:44-94)."""
+    _dev(x, torch.float32, 4, "x")
+    _dev(inv_freq, torch.float32, 1, "inv_freq")
+    B, H, L, S = x.shape
+    _lib.check(_lib.load().llmops_rope_embed(_ptr(x), B, H, L, S, _ptr(inv_freq), inv_freq.shape[0], int(position_id),
+                                            _stream(x)))
+
+
+def attention_rope2(q, k, v, inv_freq, kv_cache, kvc_slots, position_id, layer_id):
+    """q,k,v fp32 [B,qL,H*S]; kv_cache [2*layers,B,H,maxlen,S]; kvc_slots int32 [qL].
+    In place: q <- attention output, k <- rotated k, cache rows updated (ops/op_attn.hpp:721-1029)."""
+    _dev(q, torch.float32, 3, "q")
+    _dev(k, torch.float32, 3, "k")
+    _dev(v, torch.float32, 3, "v")
+    _require(isinstance(kv_cache, torch.Tensor) and kv_cache.is_cuda and kv_cache.dim() == 5 and kv_cache.is_contiguous(),
+             "kv_cache.is<float>(5)")
+    _require(kv_cache.dtype in (torch.float32, torch.float16), "kv_cache.is<float>(5)")
+    _dev(kvc_slots, torch.int32, 1, "kvc_slots")
+    _dev(inv_freq, torch.float32, 1, "inv_freq")
+    B, qL, _ = q.shape
+    planes, Bc, H, maxlen, S = kv_cache.shape
+    _require(Bc == B, "kv_cache.size(1) == B")
+    for t, n in ((q, "q"), (k, "k"), (v, "v")):
+        _require(tuple(t.shape) == (B, qL, H * S), f"{n}.is({{B, qL, H * S}})")
+    _require(tuple(kvc_slots.shape) == (qL,), "kvc_slots.is({qL})")
+    lib = _lib.load()
+    need = lib.llmops_attention_workspace_bytes(B, qL, H, S, maxlen)
+    ws = _workspace(q.device, _lib_fc_counter_bytes() + need)
+    wptr = ctypes.c_void_p(ws.data_ptr() + _lib_fc_counter_bytes())
+    dt = 0 if kv_cache.dtype == torch.float32 else 1
+    _lib.check(lib.llmops_attention_rope(_ptr(q), _ptr(k), _ptr(v), B, qL, H, S, _ptr(inv_freq), inv_freq.shape[0],
+                                         _ptr(kv_cache), dt, planes, maxlen, _ptr(kvc_slots), int(position_id),
+                                         int(layer_id), wptr, ws.numel() - _lib_fc_counter_bytes(), _stream(q)))
+
+
+# the reference exports two kernels with one contract (ops/main.cpp:154-155)
+attention_rope = attention_rope2
+
+
+def _lib_fc_counter_bytes():
+    return 65536  # LLMOPS_FC_COUNTER_BYTES: keep other ops off the FC arrival counters
+
+
+def softmax(x):
+    """In place over the last dimension (ops/op_misc.hpp:183-194)."""
+    _dev(x, torch.float32, None, "input")
+    K = x.shape[-1]
+    _lib.check(_lib.load().llmops_softmax(_ptr(x), x.numel() // K, K, _stream(x)))
+
+
+# ---- neighbours -------------------------------------------------------------------------------
+def rmsnorm(input, weight, variance_epsilon):
+    _dev(input, torch.float32, 3, "input")
+    _dev(weight, torch.float32, 1, "weight")
+    hidden = weight.shape[0]
+    _require(input.shape[-1] == hidden, "input.size(-1) == hidden_states")
+    _lib.check(_lib.load().llmops_rmsnorm(_ptr(input), input.numel() // hidden, hidden, _ptr(weight),
+                                         float(variance_epsilon), _stream(input)))
+
+
+def _ibinary(fn, a, b):
+    _dev(a, torch.float32, None, "a")
+    _dev(b, torch.float32, None, "b")
+    _require(b.dim() == 1 or b.dim() == a.dim(), "b.is<float>(1) || b.is<float>(a.rank())")
+    _require(b.shape[-1] == a.shape[-1], "b.size(-1) == a.size(-1)")
+    if b.dim() == a.dim() and a.dim() != 1:
+        _require(tuple(b.shape) == tuple(a.shape), "b.shape() == a.shape()")
+    inner = a.shape[-1]
+    _lib.check(fn(_ptr(a), _ptr(b), a.numel() // inner, inner, int(b.dim() == 1), _stream(a)))
+
+
+def iadd(a, b):
+    _ibinary(_lib.load().llmops_iadd, a, b)
+
+
+def imul(a, b):
+    _ibinary(_lib.load().llmops_imul, a, b)
+
+
+def itrans(a, op):
+    _dev(a, torch.float32, None, "a")
+    _require(op == "silu", "false")  # the reference ASSERT(false)s on any other op (ops/op_misc.hpp:139)
+    _lib.check(_lib.load().llmops_itrans_silu(_ptr(a), a.numel(), _stream(a)))
+
+
+def clone(t):
+    _require(isinstance(t, torch.Tensor) and t.is_cuda and t.is_contiguous(), "d_rank == old.m_rank")
+    return t.clone()
+
+
+def empty(*shape, device="cuda"):
+    return torch.empty(shape, dtype=torch.float32, device=device)
+
+
+def ones(*shape, device="cuda"):
+    return torch.ones(shape, dtype=torch.float32, device=device)
+
+
+def _ids(input):
+    _require(isinstance(input, torch.Tensor) and input.is_cuda and input.is_contiguous(), "input is on the HIP device")
+    _require(input.dtype in (torch.int32, torch.int64), "input.is<int32_t>() || input.is<int64_t>()")
+    return input if input.dtype == torch.int64 else input.to(torch.int64)
+
+
+def embedding(output, input, weight):
+    _dev(weight, torch.float32, 2, "weight")
+    _dev(output, torch.float32, None, "output")
+    ids = _ids(input)
+    V, E = weight.shape
+    _require(tuple(output.shape) == tuple(input.shape) + (E,), "infer_shape() == output.shape()")
+    _lib.check(_lib.load().llmops_embedding(_ptr(output), _ptr(ids), ids.numel(), _ptr(weight), V, E, _stream(output)))
+
+
+def embedding_q8c_quant_w(input):
+    _dev(input, torch.float32, 2, "input")
+    V, E = input.shape
+    q = torch.empty((V, E), dtype=torch.int8, device=input.device)
+    s = torch.empty((V,), dtype=torch.float32, device=input.device)
+    _lib.check(_lib.load().llmops_embedding_q8c_quant_w(_ptr(input), V, E, _ptr(q), _ptr(s), _stream(input)))
+    return [q, s]
+
+
+def embedding_q8c(output, input, weight, scales):
+    _dev(weight, torch.int8, 2, "weight")
+    _dev(scales, torch.float32, 1, "scales")
+    _dev(output, torch.float32, None, "output")
+    ids = _ids(input)
+    V, E = weight.shape
+    _require(tuple(output.shape) == tuple(input.shape) + (E,), "infer_shape() == output.shape()")
+    _lib.check(_lib.load().llmops_embedding_q8c(_ptr(output), _ptr(ids), ids.numel(), _ptr(weight), _ptr(scales), V, E,
+                                               _stream(output)))
+
+
+class PoolAllocator:
+    """The reference pools small host buffers per thread (ops/tensor.hpp:47-197); device memory here
+    comes from torch's caching allocator, so these are the no-ops a caller of
+    ``tensor_pool().clear()`` (chatllama/main.py:332-334) expects to exist."""
+
+    def set_policy(self, pol):
+        pass
+
+    def summary(self, verbose):
+        return "PoolAllocator: device memory is managed by the torch caching allocator"
+
+    def clear(self):
+        pass
+
+
+_pool = PoolAllocator()
+
+
+def tensor_pool():
+    return _pool

@@ -307,9 +307,23 @@ class Reference:
             raise ValueError("Reference.fc needs N % 32 == 0 (the reference overruns its output otherwise)")
         return y[0] if x.ndim == 2 else y
 
+    def _warm_rope_table(self, f):
+        """Grow the reference's static cos/sin table past 1 MiB on first use.  Smaller tables come
+        from its thread-local buffer pool, whose deleter runs after the pool itself has been
+        destroyed at process exit (static vs thread-local destruction order) and corrupts the
+        heap; buffers of 1 MiB and more are plain malloc/free (ops/tensor.hpp:164-196)."""
+        if getattr(self, "_warmed", False):
+            return
+        half = f.shape[0]
+        pos = -(-(1 << 20) // (8 * half))
+        dummy = np.zeros((1, 1, 1, 2 * half), dtype=np.float32)
+        self._chk(self.lib.ref_rope_embed(_p(dummy), _i64(1), _i64(1), _i64(1), _i64(2 * half), _p(f), _i64(half), _int(pos)))
+        self._warmed = True
+
     def rope(self, x, inv_freq, position_id):
         x = _c32(x).copy()
         f = _c32(inv_freq)
+        self._warm_rope_table(f)
         B, H, L, S = x.shape
         self._chk(self.lib.ref_rope_embed(_p(x), _i64(B), _i64(H), _i64(L), _i64(S), _p(f), _i64(f.shape[0]), _int(position_id)))
         return x
@@ -321,6 +335,7 @@ class Reference:
         s = np.ascontiguousarray(slots, dtype=np.int32)
         B, qL, HS = q.shape
         planes, _, H, maxlen, S = cache.shape
+        self._warm_rope_table(f)
         self._chk(self.lib.ref_attention_rope(_int(version), _p(q), _p(k), _p(v), _i64(B), _i64(qL), _i64(H), _i64(S),
                                               _p(f), _i64(f.shape[0]), _p(cache), _i64(planes), _i64(maxlen), _p(s),
                                               _int(position_id), _int(layer_id)))

@@ -1,0 +1,96 @@
+"""No-GPU checks of the C-ABI library: it loads, exports every symbol the header declares, and
+rejects bad arguments before touching the device."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from conftest import ROOT
+
+HEADER = os.path.join(ROOT, "include", "llmops_hip.h")
+LIB = os.path.join(ROOT, "llama.cl_amd", "llmops", "libllmops_hip.so")
+
+
+def declared_symbols():
+    src = open(HEADER).read()
+    src = re.sub(r"/\*.*?\*/", "", src, flags=re.S)
+    return sorted(set(re.findall(r"\b(llmops_[A-Za-z0-9_]+)\s*\(", src)))
+
+
+@pytest.fixture(scope="module")
+def lib():
+    if not os.path.exists(LIB):
+        pytest.fail(f"{LIB} not built: run `python llama.cl_amd/build.py`")
+    return ctypes.CDLL(LIB)
+
+
+def test_header_declares_the_path():
+    names = declared_symbols()
+    for must in ("llmops_offline_FC_quant_Q4A", "llmops_offline_FC_dequant_Q4A", "llmops_FC_dynamic_quantize_x",
+                 "llmops_fc_Q4A", "llmops_fc_Q4A_partials", "llmops_attention_rope", "llmops_rope_embed", "llmops_softmax"):
+        assert must in names
+
+
+def test_library_exports_every_declared_symbol(lib):
+    missing = [n for n in declared_symbols() if not hasattr(lib, n)]
+    assert not missing, missing
+
+
+def test_python_binding_covers_every_declared_symbol():
+    from llmops import _lib
+    assert sorted(_lib.SIGNATURES) == declared_symbols()
+    _lib.load()
+
+
+def test_block_bytes(lib):
+    lib.llmops_q4a_block_bytes.restype = ctypes.c_int64
+    assert lib.llmops_q4a_block_bytes(32) == 640      # ops/op_fc.hpp:22-24 with G=32
+    assert lib.llmops_q4a_block_bytes(128) == 2176
+    assert lib.llmops_q4a_block_bytes(64) == 0
+
+
+def test_argument_validation_without_device(lib):
+    """Validation mirrors the reference's ASSERTs and runs before any HIP call, so it works with no GPU."""
+    lib.llmops_last_error.restype = ctypes.c_char_p
+    i64, vp = ctypes.c_int64, ctypes.c_void_p
+    rc = lib.llmops_offline_FC_quant_Q4A(vp(16), i64(32), i64(64), i64(64), 64, vp(16), vp(0))
+    assert rc == 1 and b"valid_group" in lib.llmops_last_error()
+    rc = lib.llmops_fc_Q4A(vp(256), i64(1), i64(100), vp(256), i64(1), i64(1), 128, i64(32), vp(256), vp(256),
+                           ctypes.c_size_t(1 << 20), vp(0))
+    assert rc == 1 and b"K == Kg * group_k" in lib.llmops_last_error()
+    lib.llmops_fc_Q4A_workspace_bytes.restype = ctypes.c_size_t
+    need = lib.llmops_fc_Q4A_workspace_bytes(i64(1), i64(4096), i64(128), i64(32), 128)
+    assert need > 65536
+    rc = lib.llmops_fc_Q4A(vp(256), i64(1), i64(4096), vp(256), i64(128), i64(32), 128, i64(4096), vp(256), vp(256),
+                           ctypes.c_size_t(1024), vp(0))
+    assert rc == 2 and b"workspace" in lib.llmops_last_error()
+    rc = lib.llmops_attention_rope(vp(256), vp(256), vp(256), i64(1), i64(1), i64(32), i64(64), vp(256), i64(32), vp(256), 0,
+                                   i64(2), i64(16), vp(256), 0, 0, vp(256), ctypes.c_size_t(1 << 30), vp(0))
+    assert rc == 1 and b"S == 128" in lib.llmops_last_error()
+
+
+def test_python_ops_refuse_host_tensors():
+    """The product path has no CPU fallback: host tensors raise instead of being computed elsewhere."""
+    import torch
+    import llmops
+    with pytest.raises(RuntimeError, match="HIP device"):
+        llmops.offline_FC_quant_Q4A(torch.zeros(32, 128))
+    with pytest.raises(RuntimeError, match="HIP device"):
+        llmops.fc_Q4A(torch.zeros(1, 1, 128), torch.zeros(1, 1, 2176, dtype=torch.int8), 32)
+
+
+def test_kvcache_slot_manager():
+    """KVCache.prepare mirrors chatllama/main.py:60-125: ring buffer, protected system slots, early stop."""
+    import torch
+    from llmops.opset import KVCache
+    cfg = {"layer_num": 1, "head_num": 1, "head_size": 128}
+    kv = KVCache(cfg, 1, 8, False, device="cpu")
+    assert kv.prepare(3, -1, -1) and kv.slots.tolist() == [0, 1, 2] and kv.position_id == 0      # system prompt
+    assert kv.prepare(2, 1, 0) and kv.slots.tolist() == [3, 4] and kv.position_id == 3
+    assert kv.prepare(3, 2, 0) and kv.slots.tolist() == [5, 6, 7] and kv.cur_kv_len == 8
+    # wraps around, skipping the protected system slots 0..2; sentence 1 may be overwritten
+    assert kv.prepare(2, 3, 0) and kv.slots.tolist() == [3, 4] and kv.position_id == 8
+    # sentence 2 holds the instruction: asked to fail rather than overwrite it
+    assert not kv.prepare(1, 4, 2)
+    assert kv.cur_kv_len == 8 and kv.slots.dtype == torch.int32

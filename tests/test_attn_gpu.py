@@ -1,0 +1,184 @@
+"""GPU parity of rope / KV-cache update / attention and of the small neighbour ops.
+fp32 outputs: max|err|/max|ref| <= 1e-3 against the reference-made golden vectors and the oracle."""
+import numpy as np
+import pytest
+import torch
+
+from conftest import load_golden, max_rel_err
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-3
+
+
+@pytest.fixture(scope="module")
+def ops():
+    import llmops
+    return llmops
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def host(t):
+    return t.cpu().numpy()
+
+
+def run_attention(ops, g, cache_dtype=torch.float32, fn="attention_rope2"):
+    q, k, v = dev(g["q"]), dev(g["k"]), dev(g["v"])
+    cache = dev(g["cache"]).to(cache_dtype)
+    getattr(ops, fn)(q, k, v, dev(g["inv_freq"]), cache, dev(g["slots"]), int(g["position_id"]), int(g["layer_id"]))
+    return host(q), host(k), host(cache.float())
+
+
+@pytest.mark.parametrize("name", ["attn_decode", "attn_decode_wrap", "attn_chunk", "attn_prefill"])
+@pytest.mark.parametrize("fn", ["attention_rope2", "attention_rope"])
+def test_attention_golden_fp32(ops, name, fn):
+    g = load_golden(name + ".npz")
+    out, k_rot, cache = run_attention(ops, g, fn=fn)
+    assert max_rel_err(out, g["out"]) <= TOL
+    assert max_rel_err(out, g["out"]) <= 1e-5
+    assert np.abs(k_rot - g["k_rot"]).max() <= 1e-5          # k is left rotated in place
+    assert np.abs(cache - g["cache_after"]).max() <= 1e-5
+    layer = int(g["layer_id"])
+    other = np.ones(cache.shape[0], bool)
+    other[2 * layer:2 * layer + 2] = False
+    assert np.array_equal(cache[other], g["cache"][other])   # other layers' planes untouched
+    B, qL, HS = g["q"].shape
+    H, S = cache.shape[2], cache.shape[4]
+    for l, s in enumerate(g["slots"]):                        # rows written == rotated k / raw v, bit for bit
+        assert np.array_equal(cache[2 * layer, :, :, s].reshape(B, HS), k_rot[:, l])
+        assert np.array_equal(cache[2 * layer + 1, :, :, s].reshape(B, HS), g["v"][:, l])
+    rows = np.ones(cache.shape[3], bool)
+    rows[g["slots"]] = False
+    assert np.array_equal(cache[2 * layer:2 * layer + 2][:, :, :, rows], g["cache"][2 * layer:2 * layer + 2][:, :, :, rows])
+
+
+@pytest.mark.parametrize("name", ["attn_decode", "attn_chunk"])
+def test_attention_fp16_cache(ops, orc, name):
+    """fp16 KV cache is an extension: target = fp32 math on the fp16-rounded cache (new rows included)."""
+    g = load_golden(name + ".npz")
+    out, k_rot, cache = run_attention(ops, g, cache_dtype=torch.float16)
+    g16 = dict(g)
+    g16["cache"] = g["cache"].astype(np.float16).astype(np.float32)
+    # the oracle writes fp32 k,v rows into the cache; round them as the fp16 cache does before attending
+    _, k_ref, cache_ref = orc.attention(g["q"], g["k"], g["v"], g["inv_freq"], g16["cache"], g["slots"],
+                                        int(g["position_id"]), int(g["layer_id"]))
+    cache_ref = cache_ref.astype(np.float16).astype(np.float32)
+    assert np.abs(cache - cache_ref).max() <= 2e-3           # one fp16 ulp at |x| < 4 on the rotated rows
+    # attend over the rounded cache: re-run the oracle with the new rows already in place and k,v equal to them
+    B, qL, HS = g["q"].shape
+    layer = int(g["layer_id"])
+    kr = np.stack([cache_ref[2 * layer, :, :, s].reshape(B, HS) for s in g["slots"]], 1)
+    vr = np.stack([cache_ref[2 * layer + 1, :, :, s].reshape(B, HS) for s in g["slots"]], 1)
+    # feed the already rotated q and zero frequencies so the oracle leaves q,k as given
+    zero_f = np.zeros_like(g["inv_freq"])
+    q_in = _rotated_q(orc, g)
+    want = orc.attention(q_in, kr, vr, zero_f, cache_ref, g["slots"], int(g["position_id"]), layer)[0]
+    assert max_rel_err(out, want) <= TOL
+
+
+def _rotated_q(orc, g):
+    B, qL, HS = g["q"].shape
+    H = g["cache"].shape[2]
+    S = HS // H
+    q4 = g["q"].reshape(B, qL, H, S).transpose(0, 2, 1, 3).copy()
+    return orc.rope(q4, g["inv_freq"], int(g["position_id"])).transpose(0, 2, 1, 3).reshape(B, qL, HS).copy()
+
+
+@pytest.mark.parametrize("kv", [256, 2048])
+@pytest.mark.parametrize("cache_dtype", [torch.float32, torch.float16])
+def test_attention_config4_vs_oracle(ops, orc, kv, cache_dtype):
+    """BASELINE config 4: 32 heads x 128, rope base 10000 over 128 dims, one query token, kv-len 256 / 2048."""
+    rng = np.random.default_rng(kv)
+    B, H, S, layers = 1, 32, 128, 2
+    q, k, v = (rng.standard_normal((B, 1, H * S)).astype(np.float32) for _ in range(3))
+    cache = rng.standard_normal((2 * layers, B, H, kv, S)).astype(np.float32)
+    if cache_dtype == torch.float16:
+        cache = cache.astype(np.float16).astype(np.float32)
+    inv_freq = (1.0 / (10000.0 ** (np.arange(0, S, 2, dtype=np.float32) / np.float32(S)))).astype(np.float32)
+    slots = np.array([kv - 1], np.int32)
+    g = dict(q=q, k=k, v=v, cache=cache, inv_freq=inv_freq, slots=slots, position_id=kv - 1, layer_id=1)
+    out, k_rot, cache_after = run_attention(ops, g, cache_dtype=cache_dtype)
+    want, k_ref, cache_ref = orc.attention(q, k, v, inv_freq, cache, slots, kv - 1, 1)
+    tol = TOL if cache_dtype == torch.float32 else 3e-3   # fp16 rounding of the one new K/V row (extension, no reference)
+    assert max_rel_err(out, want) <= tol
+    if cache_dtype == torch.float32:
+        assert max_rel_err(out, want) <= 1e-5
+        assert np.abs(k_rot - k_ref).max() <= 1e-4        # position 2047: fp32 sin/cos argument reduction differs slightly
+        assert np.abs(cache_after - cache_ref).max() <= 1e-4
+
+
+def test_attention_kvlen_sweep(ops, orc):
+    """Odd and tiny kv lengths (the reference's own sweep uses 30+1, 31+1, 1022..1026) and every chunking."""
+    rng = np.random.default_rng(3)
+    B, H, S, maxlen = 1, 4, 128, 1100
+    inv_freq = (1.0 / (10000.0 ** (np.arange(0, 64, 2, dtype=np.float32) / np.float32(64)))).astype(np.float32)
+    cache = rng.standard_normal((2, B, H, maxlen, S)).astype(np.float32)
+    for past in (0, 1, 15, 16, 30, 31, 63, 64, 65, 511, 1022, 1023, 1025):
+        q, k, v = (rng.standard_normal((B, 1, H * S)).astype(np.float32) for _ in range(3))
+        slots = np.array([past], np.int32)
+        g = dict(q=q, k=k, v=v, cache=cache, inv_freq=inv_freq, slots=slots, position_id=past, layer_id=0)
+        out, _, _ = run_attention(ops, g)
+        want = orc.attention(q, k, v, inv_freq, cache, slots, past, 0)[0]
+        assert max_rel_err(out, want) <= 1e-5, past
+
+
+def test_attention_prefill_chunks_vs_oracle(ops, orc):
+    rng = np.random.default_rng(4)
+    B, H, S, maxlen = 2, 3, 128, 96
+    inv_freq = (1.0 / (10000.0 ** (np.arange(0, S, 2, dtype=np.float32) / np.float32(S)))).astype(np.float32)
+    cache = rng.standard_normal((4, B, H, maxlen, S)).astype(np.float32)
+    for past, qL in ((0, 33), (40, 7), (90, 20)):   # the last one wraps the ring buffer
+        q, k, v = (rng.standard_normal((B, qL, H * S)).astype(np.float32) for _ in range(3))
+        slots = ((past + np.arange(qL)) % maxlen).astype(np.int32)
+        g = dict(q=q, k=k, v=v, cache=cache, inv_freq=inv_freq, slots=slots, position_id=past, layer_id=1)
+        out, k_rot, cache_after = run_attention(ops, g)
+        want, k_ref, cache_ref = orc.attention(q, k, v, inv_freq, cache, slots, past, 1)
+        assert max_rel_err(out, want) <= 1e-5, (past, qL)
+        assert np.abs(cache_after - cache_ref).max() <= 1e-5
+
+
+def test_rope_and_softmax_golden(ops):
+    g = load_golden("misc.npz")
+    x = dev(g["rope_x"])
+    ops.rope_embed(x, dev(g["rope_inv_freq"]), 16)
+    assert np.abs(host(x) - g["rope_out"]).max() <= 1e-5     # ops/test_ops.py:211
+    assert np.array_equal(host(x)[..., 64:], g["rope_x"][..., 64:])
+    s = dev(g["sm_in"])
+    ops.softmax(s)
+    assert np.allclose(host(s), g["sm"], rtol=1e-5, atol=1e-8)
+    lit = dev(g["lit"][None])
+    ops.softmax(lit)
+    assert np.allclose(host(lit)[0], g["sm_lit"], rtol=1e-5, atol=1e-8) and host(lit)[0, -1] == 0.0
+    big = torch.rand(7, 12, 3, 69, device="cuda") - 0.5      # ops/test_ops.py:170
+    want = torch.softmax(big, -1)
+    ops.softmax(big)
+    assert torch.allclose(big, want, rtol=1e-5, atol=1e-8)
+
+
+def test_neighbours_golden(ops):
+    g = load_golden("misc.npz")
+    x = dev(g["x"])
+    ops.rmsnorm(x, dev(g["wn"]), 1e-5)
+    assert np.allclose(host(x), g["rms"], rtol=1e-5, atol=1e-6)
+    x = dev(g["x"])
+    ops.itrans(x, "silu")
+    assert np.allclose(host(x), g["silu"], rtol=1e-3, atol=1e-6)   # the reference itself is ~3e-4 off (rcpps)
+    assert np.allclose(host(x), g["x"] / (1 + np.exp(-g["x"].astype(np.float64))), rtol=1e-6, atol=1e-7)
+    a = dev(g["x"])
+    ops.iadd(a, dev(g["x"][:, ::-1].copy()))
+    assert np.array_equal(host(a), g["iadd"])
+    a = dev(g["x"])
+    ops.imul(a, dev(g["wn"]))
+    assert np.array_equal(host(a), g["imul_row"])
+    q, s = ops.embedding_q8c_quant_w(dev(g["emb"]))
+    assert np.array_equal(host(q), g["eq"]) and np.array_equal(host(s).view(np.uint32), g["es"].view(np.uint32))
+    out = ops.empty(2, 3, 64)
+    ops.embedding_q8c(out, dev(g["ids"]), q, s)
+    assert np.array_equal(host(out), g["emb_out"])
+    out = ops.empty(2, 3, 64)
+    ops.embedding(out, dev(g["ids"]), dev(g["emb"]))
+    assert np.array_equal(host(out), g["emb"][g["ids"]])
+    with pytest.raises(RuntimeError):
+        ops.itrans(x, "gelu")

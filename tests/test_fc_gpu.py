@@ -1,0 +1,207 @@
+"""GPU parity of the Q4_1 FC path against the oracle and the committed golden vectors, through
+the `llmops` module (ctypes -> C ABI -> HIP kernels).  Bit-exact: packed bytes, Q8 codes, scales,
+group sums, int32 partial sums.  fp32 outputs: max|err|/max|ref| <= 1e-3 (the stated contract;
+observed errors are ~1e-6)."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from conftest import load_golden, max_rel_err
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-3
+
+
+@pytest.fixture(scope="module")
+def ops():
+    import llmops
+    return llmops
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def host(t):
+    return t.cpu().numpy()
+
+
+# ---- packing ------------------------------------------------------------------------------------
+@pytest.mark.parametrize("G", [32, 128])
+def test_pack_golden(ops, G):
+    g = load_golden(f"fc_g{G}.npz")
+    wq = ops.offline_FC_quant_Q4A(dev(g["w"]), G)
+    assert np.array_equal(host(wq), g["wq"])
+    assert np.array_equal(host(ops.offline_FC_dequant_Q4A(wq)).view(np.uint32), g["dq"].view(np.uint32))
+
+
+@pytest.mark.parametrize("G", [32, 128])
+@pytest.mark.parametrize("N,K", [(4096, 4096), (352, 11008), (100, 1024)])
+def test_pack_random_vs_oracle(ops, orc, G, N, K):
+    rng = np.random.default_rng(N + K + G)
+    w = (rng.standard_normal((N, K)) * 0.02).astype(np.float32)
+    w[1, :G] = 0.5                      # constant group
+    w[2, :4] = [0.0, 15.0, 2.5, 3.5]    # half-away ties when it spans the group range
+    w[3, :G] = np.where(rng.random(G) < 0.5, 0.0, -0.0)  # zero group with mixed signs: sign of m follows first element
+    wq = host(ops.offline_FC_quant_Q4A(dev(w), G))
+    want = orc.quant_w(w, G)
+    assert wq.shape == want.shape
+    assert np.array_equal(wq, want)    # includes zero nibbles / zero d,m of padded rows when N % 32 != 0
+    assert np.array_equal(host(ops.offline_FC_dequant_Q4A(dev(want))).view(np.uint32), orc.dequant_w(want).view(np.uint32))
+
+
+def test_pack_row_stride(ops, orc):
+    w = (np.random.default_rng(5).standard_normal((64, 640)) * 0.02).astype(np.float32)
+    view = dev(w)[:, :512]             # row stride 640, inner contiguous
+    assert np.array_equal(host(ops.offline_FC_quant_Q4A(view, 128)), orc.quant_w(w[:, :512], 128))
+
+
+# ---- activation quantization --------------------------------------------------------------------
+@pytest.mark.parametrize("G", [32, 128])
+def test_quant_x_golden(ops, G):
+    g = load_golden(f"fc_g{G}.npz")
+    xq, xd, gs = ops.FC_dynamic_quantize_x(dev(g["x"]), G)
+    assert np.array_equal(host(xq), g["xq"])
+    assert np.array_equal(host(xd).view(np.uint32), g["xd"].view(np.uint32))
+    assert np.array_equal(host(gs).view(np.uint32), g["gsum"].view(np.uint32))
+
+
+@pytest.mark.parametrize("G", [32, 128])
+@pytest.mark.parametrize("rows,K", [(1, 4096), (17, 11008), (2048, 4096)])
+def test_quant_x_random_vs_oracle(ops, orc, G, rows, K):
+    rng = np.random.default_rng(rows + K)
+    x = rng.standard_normal((rows, K)).astype(np.float32)
+    x[0, :8] = [127, 2.5, 3.5, -2.5, -3.5, 0.5, 1.5, -0.5]
+    x[0, 8:G] = 0
+    if rows > 1:
+        x[1, G:2 * G] = 0
+    xq, xd, gs = ops.FC_dynamic_quantize_x(dev(x), G)
+    wq, wd, wg = orc.quant_x(x, G)
+    assert np.array_equal(host(xq), wq)
+    assert np.array_equal(host(xd).view(np.uint32), wd.view(np.uint32))
+    assert np.array_equal(host(gs).view(np.uint32), wg.view(np.uint32))
+    assert list(host(xq)[0, :8]) == [127, 2, 4, -2, -4, 0, 2, 0]
+
+
+# ---- int32 partial sums -------------------------------------------------------------------------
+@pytest.mark.parametrize("G", [32, 128])
+@pytest.mark.parametrize("mfma", [False, True])
+@pytest.mark.parametrize("rows,N,K", [(1, 4096, 4096), (3, 352, 2048), (17, 96, 1024), (40, 32, 384)])
+def test_partials_bit_exact(ops, orc, G, mfma, rows, N, K):
+    rng = np.random.default_rng(rows * 7 + G)
+    wq = orc.quant_w((rng.standard_normal((N, K)) * 0.02).astype(np.float32), G)
+    xq = rng.integers(-127, 128, (rows, K)).astype(np.int8)
+    xq[0, :G] = -127
+    got = host(ops.fc_Q4A_partials(dev(xq), dev(wq), use_mfma=mfma))
+    assert np.array_equal(got, orc.fc_partials(xq, wq))
+
+
+@pytest.mark.parametrize("G", [32, 128])
+@pytest.mark.parametrize("mfma", [False, True])
+def test_partials_extreme_codes(ops, orc, G, mfma):
+    w = np.full((32, 2 * G), 15.0, np.float32)
+    w[:, 0::G] = 0.0
+    wq = orc.quant_w(w, G)
+    xq = np.full((2, 2 * G), -127, np.int8)
+    xq[1] = 127
+    got = host(ops.fc_Q4A_partials(dev(xq), dev(wq), use_mfma=mfma))
+    assert got.min() == -(G - 1) * 15 * 127 and got.max() == (G - 1) * 15 * 127
+    assert np.array_equal(got, orc.fc_partials(xq, wq))
+
+
+# ---- fp32 output --------------------------------------------------------------------------------
+@pytest.mark.parametrize("G", [32, 128])
+def test_fc_golden(ops, G):
+    g = load_golden(f"fc_g{G}.npz")
+    y = host(ops.fc_Q4A(dev(g["x"][None]), dev(g["wq"]), g["y"].shape[-1]))[0]
+    assert max_rel_err(y, g["y"]) <= TOL
+    for r in range(y.shape[0]):          # row by row too: rows differ in magnitude by 1e20
+        assert max_rel_err(y[r], g["y"][r]) <= TOL
+
+
+@pytest.mark.parametrize("G", [32, 128])
+@pytest.mark.parametrize("B,M", [(1, 1), (1, 2), (1, 4), (1, 7), (2, 17), (1, 64), (1, 130)])
+def test_fc_closed_form_exact(ops, G, B, M):
+    """ops/test_ops.py:106-149 (B=2, M=17, N=K=4096 there): every value exactly representable, so
+    the result must EQUAL x @ W.T whatever the accumulation order."""
+    N = K = 4096 if M <= 17 else 1024
+    x, w = oracle.closed_form_fc_inputs(B * M, N, K, seed=M)
+    wq = ops.offline_FC_quant_Q4A(dev(w), G)
+    assert np.array_equal(host(ops.offline_FC_dequant_Q4A(wq)), w)
+    y = host(ops.fc_Q4A(dev(x.reshape(B, M, K)), wq, N))
+    want = (x.astype(np.float64) @ w.astype(np.float64).T).astype(np.float32).reshape(B, M, N)
+    assert np.array_equal(y, want)
+
+
+CONFIG_SHAPES = [  # (G, N, K) of BASELINE configs 1 and 2
+    (32, 4096, 4096), (128, 4096, 4096), (128, 11008, 4096), (128, 4096, 11008),
+]
+
+
+@pytest.mark.parametrize("G,N,K", CONFIG_SHAPES)
+@pytest.mark.parametrize("M", [1, 3, 8, 16, 48])
+def test_fc_baseline_shapes_vs_oracle(ops, orc, G, N, K, M):
+    rng = np.random.default_rng(G + N + K + M)
+    w = (rng.standard_normal((N, K)) * 0.02).astype(np.float32)
+    x = rng.standard_normal((1, M, K)).astype(np.float32)
+    wq = orc.quant_w(w, G)
+    want = orc.fc(x, wq, N)
+    dwq, dx = dev(wq), dev(x)
+    y1 = host(ops.fc_Q4A(dx, dwq, N))
+    assert max_rel_err(y1, want) <= TOL
+    assert max_rel_err(y1, want) <= 1e-5   # what the kernels actually achieve
+    y2 = host(ops.fc_Q4A(dx, dwq, N))      # split-K partial sums are combined in a fixed order
+    assert np.array_equal(y1.view(np.uint32), y2.view(np.uint32))
+
+
+def test_fc_odd_N_and_fused_strips(ops, orc):
+    """N not a multiple of 32 (stores are clipped) and row-wise concatenation of packed tensors
+    (q/k/v fused into one launch) give the concatenated outputs."""
+    rng = np.random.default_rng(77)
+    K = 1024
+    x = rng.standard_normal((1, 2, K)).astype(np.float32)
+    w = (rng.standard_normal((100, K)) * 0.02).astype(np.float32)
+    wq = orc.quant_w(w, 128)
+    assert max_rel_err(host(ops.fc_Q4A(dev(x), dev(wq), 100)), orc.fc(x, wq, 100)) <= 1e-5
+    ws = [(rng.standard_normal((n, K)) * 0.02).astype(np.float32) for n in (64, 96, 32)]
+    packed = [orc.quant_w(a, 128) for a in ws]
+    fused = np.concatenate(packed, axis=0)
+    y = host(ops.fc_Q4A(dev(x), dev(fused), 192))
+    want = np.concatenate([orc.fc(x, p, a.shape[0]) for p, a in zip(packed, ws)], axis=-1)
+    assert max_rel_err(y, want) <= 1e-5
+
+
+def test_fc_size_independent_properties(ops):
+    """Full-size (lm_head-like) checks that need no CPU reference: a scaled one-hot activation
+    reads back one dequantized weight column, and the op is homogeneous in powers of two."""
+    G, N, K = 128, 55296, 4096
+    gen = torch.Generator(device="cpu").manual_seed(5)
+    w = (torch.randn(N, K, generator=gen) * 0.02).cuda()
+    wq = ops.offline_FC_quant_Q4A(w, G)
+    dq = ops.offline_FC_dequant_Q4A(wq)
+    for k in (0, 1234, K - 1):
+        x = torch.zeros(1, 1, K, device="cuda")
+        x[0, 0, k] = 127.0                      # dx = 1, code 127, gsum = 127
+        y = ops.fc_Q4A(x, wq, N)[0, 0]
+        assert torch.allclose(y, 127.0 * dq[:, k], rtol=1e-6, atol=1e-6)
+    x = torch.randn(1, 1, K, generator=gen).cuda()
+    y1 = ops.fc_Q4A(x, wq, N)
+    y2 = ops.fc_Q4A(x * 4.0, wq, N)            # scaling by 2^k is exact through every step
+    assert torch.equal(y1 * 4.0, y2)
+    assert (y1 - torch.nn.functional.linear(x, dq[:N])).abs().max() / y1.abs().max() < 2e-2  # Q8 activation error only
+
+
+def test_fc_argument_errors(ops):
+    x = torch.zeros(1, 1, 256, device="cuda")
+    wq = torch.zeros(1, 2, 2176, dtype=torch.int8, device="cuda")
+    with pytest.raises(RuntimeError):
+        ops.fc_Q4A(x[0], wq, 32)                                   # rank 2 input (ops/op_fc.hpp:287)
+    with pytest.raises(RuntimeError):
+        ops.fc_Q4A(x, wq.to(torch.float32), 32)                    # wrong dtype (ops/op_fc.hpp:288)
+    with pytest.raises(RuntimeError):
+        ops.fc_Q4A(torch.zeros(1, 1, 128, device="cuda"), wq, 32)  # K != Kg*G
+    with pytest.raises(RuntimeError):
+        ops.fc_Q4A(x, torch.zeros(1, 2, 1000, dtype=torch.int8, device="cuda"), 32)  # not a block size
+    with pytest.raises(RuntimeError):
+        ops.offline_FC_quant_Q4A(torch.zeros(4, 4, 4, device="cuda"))               # rank 3 weight (ops/op_fc.hpp:152)
