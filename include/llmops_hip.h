@@ -95,6 +95,13 @@ int llmops_fc_Q4A(const float* x, int64_t rows, int64_t K, const int8_t* weiq, i
                   int group_k, int64_t N, float* y, void* workspace, size_t workspace_bytes,
                   llmops_stream_t stream);
 
+/* The second half of fc_Q4A on its own (ops/op_fc.hpp:318-423): the product for activations that
+ * llmops_FC_dynamic_quantize_x has already quantized (xq int8 [rows,Kg*G], xd and gsum fp32
+ * [rows,Kg]).  llmops_fc_Q4A == llmops_FC_dynamic_quantize_x into the workspace + this. */
+int llmops_fc_Q4A_prequantized(const int8_t* xq, const float* xd, const float* gsum, int64_t rows,
+                               const int8_t* weiq, int64_t Ng, int64_t Kg, int group_k, int64_t N, float* y,
+                               void* workspace, size_t workspace_bytes, llmops_stream_t stream);
+
 /* The integer core of fc_Q4A on its own (ops/op_fc.hpp:337-363): acc int32 [rows, Ng*32, Kg].
  * `use_mfma` selects which of the two production inner loops computes it (0 = dot4 streaming
  * kernel, 1 = int8 MFMA kernel) so that both can be checked bit-for-bit. */

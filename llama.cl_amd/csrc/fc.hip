@@ -58,7 +58,7 @@ extern "C" int llmops_fc_Q4A(const float* x, int64_t rows, int64_t K, const int8
     LLMOPS_REQUIRE(rows > 0 && K > 0 && Ng > 0 && Kg > 0);
     LLMOPS_REQUIRE(K == Kg * group_k);  // the reference reads past K otherwise (ops/op_fc.hpp:184)
     LLMOPS_REQUIRE(N > (Ng - 1) * kGroupN && N <= Ng * kGroupN);
-    LLMOPS_REQUIRE(Ng * kGroupN <= LLMOPS_FC_COUNTER_BYTES / 4 * kGroupN);
+    LLMOPS_REQUIRE(Ng <= LLMOPS_FC_COUNTER_BYTES / 4);
     LLMOPS_REQUIRE(Ng * 64 < ((int64_t)1 << 31));
     LLMOPS_REQUIRE(aligned(weiq, 16) && aligned(workspace, 256));
     const FcWorkspace lay = fc_layout(rows, Ng, Kg, group_k);
@@ -76,6 +76,28 @@ extern "C" int llmops_fc_Q4A(const float* x, int64_t rows, int64_t K, const int8
     const uint8_t* w = reinterpret_cast<const uint8_t*>(weiq);
     if (rows <= kMaxGemvRows) return launch_gemv(w, xq, xd, gs, y, part, counters, rows, Ng, Kg, group_k, N, st);
     return launch_gemm(w, xq, xd, gs, y, part, rows, Ng, Kg, group_k, N, st);
+}
+
+extern "C" int llmops_fc_Q4A_prequantized(const int8_t* xq, const float* xd, const float* gsum, int64_t rows,
+                                          const int8_t* weiq, int64_t Ng, int64_t Kg, int group_k, int64_t N, float* y,
+                                          void* workspace, size_t workspace_bytes, llmops_stream_t stream) {
+    LLMOPS_REQUIRE(valid_group(group_k));
+    LLMOPS_REQUIRE(xq != nullptr && xd != nullptr && gsum != nullptr && weiq != nullptr && y != nullptr);
+    LLMOPS_REQUIRE(workspace != nullptr);
+    LLMOPS_REQUIRE(rows > 0 && Ng > 0 && Kg > 0);
+    LLMOPS_REQUIRE(N > (Ng - 1) * kGroupN && N <= Ng * kGroupN);
+    LLMOPS_REQUIRE(Ng <= LLMOPS_FC_COUNTER_BYTES / 4);
+    LLMOPS_REQUIRE(aligned(weiq, 16) && aligned(xq, 16) && aligned(workspace, 256));
+    const FcWorkspace lay = fc_layout(rows, Ng, Kg, group_k);
+    if (workspace_bytes < lay.total)
+        return fail(LLMOPS_EWORKSPACE, "fc_Q4A needs %zu workspace bytes, got %zu", lay.total, workspace_bytes);
+    uint8_t* ws = reinterpret_cast<uint8_t*>(workspace);
+    float* part = reinterpret_cast<float*>(ws + lay.off_part);
+    const uint8_t* w = reinterpret_cast<const uint8_t*>(weiq);
+    hipStream_t st = as_stream(stream);
+    if (rows <= kMaxGemvRows)
+        return launch_gemv(w, xq, xd, gsum, y, part, reinterpret_cast<unsigned*>(ws), rows, Ng, Kg, group_k, N, st);
+    return launch_gemm(w, xq, xd, gsum, y, part, rows, Ng, Kg, group_k, N, st);
 }
 
 extern "C" int llmops_fc_Q4A_partials(const int8_t* xq, int64_t rows, const int8_t* weiq, int64_t Ng, int64_t Kg,

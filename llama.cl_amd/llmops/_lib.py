@@ -21,6 +21,8 @@ SIGNATURES = {
     "llmops_FC_dynamic_quantize_x": (c_int, [c_ptr, c_i64, c_i64, c_int, c_ptr, c_ptr, c_ptr, c_ptr]),
     "llmops_fc_Q4A_workspace_bytes": (c_size, [c_i64, c_i64, c_i64, c_i64, c_int]),
     "llmops_fc_Q4A": (c_int, [c_ptr, c_i64, c_i64, c_ptr, c_i64, c_i64, c_int, c_i64, c_ptr, c_ptr, c_size, c_ptr]),
+    "llmops_fc_Q4A_prequantized": (c_int, [c_ptr, c_ptr, c_ptr, c_i64, c_ptr, c_i64, c_i64, c_int, c_i64, c_ptr, c_ptr,
+                                           c_size, c_ptr]),
     "llmops_fc_Q4A_partials": (c_int, [c_ptr, c_i64, c_ptr, c_i64, c_i64, c_int, c_ptr, c_int, c_ptr]),
     "llmops_rope_embed": (c_int, [c_ptr, c_i64, c_i64, c_i64, c_i64, c_ptr, c_i64, c_int, c_ptr]),
     "llmops_attention_workspace_bytes": (c_size, [c_i64, c_i64, c_i64, c_i64, c_i64]),
