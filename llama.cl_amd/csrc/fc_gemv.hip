@@ -175,20 +175,26 @@ __global__ __launch_bounds__(256) void fc_gemv_kernel(const uint8_t* __restrict_
         if (tr < MT && tr < rows && n < N) y[(int64_t)tr * N + n] = v;
         return;
     }
-    if (tr < MT && tr < rows) part[((int64_t)s * rows + tr) * Np + n] = v;
-    __threadfence();  // publish this workgroup's partial sums device-wide
+    // Cross-workgroup hand-off without cache-wide fences: partial sums are written and read with
+    // device-scope (write-through / cache-bypassing) accesses, and the arrival counter is a
+    // device-scope atomic.  __syncthreads() waits for this workgroup's stores to be acknowledged
+    // before thread 0 announces the arrival.  (A __threadfence() here makes every workgroup
+    // write back and invalidate its whole L2 slice, which costs far more than the kernel itself.)
+    if (tr < MT && tr < rows)
+        __hip_atomic_store(&part[((int64_t)s * rows + tr) * Np + n], v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the write-through stores above have been acknowledged
     __syncthreads();
-    if (threadIdx.x == 0) ticket_sh = atomicAdd(&counters[nb], 1u);
+    if (threadIdx.x == 0)
+        ticket_sh = __hip_atomic_fetch_add(&counters[nb], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __syncthreads();
     if (ticket_sh != (unsigned)(S - 1)) return;
-    __threadfence();  // the last arrival observes every other workgroup's partial sums
     if (tr < MT && tr < rows && n < N) {
         float acc = 0.0f;
         for (int i = 0; i < S; i++)
             acc += __hip_atomic_load(&part[((int64_t)i * rows + tr) * Np + n], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         y[(int64_t)tr * N + n] = acc;
     }
-    if (threadIdx.x == 0) counters[nb] = 0;  // ready for the next launch
+    if (threadIdx.x == 0) __hip_atomic_store(&counters[nb], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // next launch
 }
 
 // Integer core only: acc[r][n][kb] (int32).  One wavefront per step, same loads and same dot
