@@ -41,13 +41,20 @@ def fc_bytes(N, K, M=1, g=G):
     return -(-N // 32) * -(-K // g) * blk_bytes(g) + 4 * M * K + 4 * M * N
 
 
+# launch plan of the decode step: packed tensors of FCs that share their input are concatenated
+# along N (the packed format is [strip][k-block][bytes], so this is a plain torch.cat), which
+# turns q|k|v and gate|up into one launch each: same bytes, same outputs, fewer launches
+FUSED_PLAN = [("qkv", ("q", "k", "v")), ("o", ("o",)), ("gate_up", ("gate", "up")), ("down", ("down",))]
+UNFUSED_PLAN = [(n, (n,)) for n, _, _ in LAYER_FCS]
+SHAPE = {n: (N, K) for n, N, K in LAYER_FCS}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU (the path is data-parallel per GPU; multi-GPU sharding is design "
@@ -62,60 +69,73 @@ def main():
     torch.cuda.set_device(dev)
     gen = torch.Generator(device="cpu").manual_seed(2)
 
-    # ---- synthetic weights: pack once per shape on the device, then make every layer distinct ----
+    # ---- synthetic weights: quantize+pack once per FC on the device, then make every layer distinct ----
     t0 = time.time()
     packed = {}
     for name, N, K in LAYER_FCS:
         w = (torch.randn(N, K, generator=gen) * 0.02).to(dev)
         packed[name] = llmops.offline_FC_quant_Q4A(w, G)
         del w
-    weights = []  # weights[layer][i] distinct device tensors
-    for layer in range(LAYERS):
-        row = []
-        for name, N, K in LAYER_FCS:
-            base = packed[name]
+
+    def layer_weights(plan, layer):
+        out = []
+        for _, parts in plan:
+            t = torch.cat([packed[p] for p in parts], dim=0) if len(parts) > 1 else packed[parts[0]]
             # rolling the strips makes each layer's bytes distinct without re-quantizing 32 times
-            row.append(torch.roll(base, shifts=layer + 1, dims=0).contiguous() if layer else base)
-        weights.append(row)
+            out.append(torch.roll(t, shifts=layer + 1, dims=0).contiguous())
+        return out
+
     xs = {K: torch.randn(1, 1, K, generator=gen).to(dev) for K in (4096, 11008)}
-    torch.cuda.synchronize()
-    setup_s = time.time() - t0
-
     step_bytes = LAYERS * sum(fc_bytes(N, K) for _, N, K in LAYER_FCS)
-    n_fc = LAYERS * len(LAYER_FCS)
-
-    def run_step():
-        for layer in range(LAYERS):
-            for (name, N, K), wq in zip(LAYER_FCS, weights[layer]):
-                llmops.fc_Q4A(xs[K], wq, N)
-
-    # ---- whole-job timing ------------------------------------------------------------------------
     stream = torch.cuda.Stream()
+    results = {}
     with torch.cuda.stream(stream):
-        run_step()  # loads code objects, sizes the workspace
-        torch.cuda.synchronize()
-        graph = None
-        if not args.no_graph:
+        for label, plan in (("fused", FUSED_PLAN), ("unfused", UNFUSED_PLAN)):
+            weights = [layer_weights(plan, layer) for layer in range(LAYERS)]
+            dims = [(sum(SHAPE[p][0] for p in parts), SHAPE[parts[0]][1]) for _, parts in plan]
+            torch.cuda.synchronize()
+
+            def run_step():
+                for layer in range(LAYERS):
+                    for (N, K), wq in zip(dims, weights[layer]):
+                        llmops.fc_Q4A(xs[K], wq, N)
+
+            run_step()  # loads code objects, sizes the workspace
+            torch.cuda.synchronize()
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph, stream=stream):
                 run_step()
-        step = graph.replay if graph is not None else run_step
-        for _ in range(args.warmup):
-            step()
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(args.steps):
-            step()
-        torch.cuda.synchronize()
-        dt = time.perf_counter() - t0
-    ms_per_step = dt / args.steps * 1e3
-    value = step_bytes / (dt / args.steps) / 1e9
+            for _ in range(args.warmup):
+                graph.replay()
+            torch.cuda.synchronize()
+            # wall clock for `value`, HIP events on the launch stream for the kernel's average duration
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            t1 = time.perf_counter()
+            e0.record(stream)
+            for _ in range(args.steps):
+                graph.replay()
+            e1.record(stream)
+            torch.cuda.synchronize()
+            dt = time.perf_counter() - t1
+            results[label] = {"ms_per_step": dt / args.steps * 1e3, "event_ms_per_step": e0.elapsed_time(e1) / args.steps,
+                              "launches": LAYERS * len(plan)}
+            if label == "fused":
+                per_shape = measure_shapes(torch, llmops, plan, dims, weights, xs, stream)
+            del weights, graph
+        floor_us = dispatch_floor(torch, stream)
+    setup_s = time.time() - t0
 
-    # ---- dominant kernel: fc_gemv_kernel<128,1>, HIP events around back-to-back launches -----------
-    # Events are recorded on the stream the kernels run on.  The activation is quantized once up
-    # front; the timed launches are the streaming kernel alone, cycling the 32 distinct weight sets.
-    roof = measure_gemv(torch, llmops, weights, xs, stream)
-
+    main_r = results["fused"]
+    value = step_bytes / (main_r["ms_per_step"] * 1e-3) / 1e9
+    avg_us = main_r["event_ms_per_step"] * 1e3 / main_r["launches"]
+    achieved = step_bytes / (main_r["event_ms_per_step"] * 1e-3) / 1e9
+    roof = {"bound": "hbm", "kernel": "fc_gemv_fused_kernel<128,1,16,1>", "achieved": round(achieved, 1),
+            "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+            "avg_launch_us": round(avg_us, 3), "launches_per_step": main_r["launches"],
+            "bytes_per_launch_avg": int(step_bytes / main_r["launches"]), "per_shape": per_shape,
+            "dispatch_floor_us": round(floor_us, 3),
+            "timing": "HIP events on the launch stream around the timed graph replays; every node of the graph is this "
+                      "kernel, so the average includes the dispatch gap between dependent launches (dispatch_floor_us)"}
     out = {
         "metric": "Q4_1 FC decode GB/s (% HBM peak); ms/token Llama-7B shape @ kv-len 2048",
         "value": round(value, 2),
@@ -123,16 +143,20 @@ def main():
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
-        "ms_per_step": round(ms_per_step, 4),
+        "ms_per_step": round(main_r["ms_per_step"], 4),
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "int8xint4->int32, fp32 scale/accumulate",
+        "dtype": "int8 x int4 -> int32 dot, fp32 scales and accumulation",
         "data": "synthetic",
-        "config": {"workload": "Llama-7B-shape decode FC set, Q4_1 group 128, M=1, 32 layers x (q,k,v,o 4096x4096; "
-                               "gate,up 11008x4096; down 4096x11008), distinct weights per layer",
-                   "fcs_per_step": n_fc, "bytes_per_step": step_bytes, "launch": "eager" if graph is None else "hip-graph"},
+        "config": {"workload": "Llama-7B-shape decode FC set, Q4_1 group 128, M=1: 32 layers x (q,k,v,o 4096x4096; gate,up "
+                               "11008x4096; down 4096x11008), distinct weights per layer, x~N(0,1), W~N(0,0.02)",
+                   "bytes_per_step": step_bytes, "launch": "hip-graph replay of llmops.fc_Q4A calls",
+                   "launches_per_layer": len(FUSED_PLAN),
+                   "plan": "q|k|v and gate|up packed tensors concatenated along N (one launch each), o and down separate"},
         "pct_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
+        "unfused_7_launches_per_layer": {"GB/s": round(step_bytes / (results["unfused"]["ms_per_step"] * 1e-3) / 1e9, 2),
+                                         "ms_per_step": round(results["unfused"]["ms_per_step"], 4)},
         "roofline": roof,
     }
     if not args.no_cpu:
@@ -141,52 +165,45 @@ def main():
     print(json.dumps(out))
 
 
-def measure_gemv(torch, llmops, weights, xs, stream, reps=5):
-    """Average duration of the dominant kernel over the whole FC set, from HIP events that bracket
-    runs of back-to-back launches on the launch stream."""
-    lib = llmops._lib.load()
-    import ctypes
-    total_bytes = 0
-    launches = 0
-    total_ms = 0.0
+def measure_shapes(torch, llmops, plan, dims, weights, xs, stream, reps=10):
+    """Per-shape average launch duration: one graph per shape over the 32 distinct weight sets."""
     per_shape = {}
-    with torch.cuda.stream(stream):
-        for name, N, K in LAYER_FCS:
-            x = xs[K]
-            xq, xd, gs = llmops.FC_dynamic_quantize_x(x, G)
-            y = torch.empty(1, 1, N, device=x.device)
-            Ng, Kg = -(-N // 32), K // G
-            ws = llmops._workspace(x.device, lib.llmops_fc_Q4A_workspace_bytes(1, K, Ng, Kg, G))
-            st = ctypes.c_void_p(stream.cuda_stream)
+    for i, ((name, _), (N, K)) in enumerate(zip(plan, dims)):
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=stream):
+            for layer in range(LAYERS):
+                llmops.fc_Q4A(xs[K], weights[layer][i], N)
+        g.replay()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        for _ in range(reps):
+            g.replay()
+        e1.record(stream)
+        torch.cuda.synchronize()
+        us = e0.elapsed_time(e1) * 1e3 / (reps * LAYERS)
+        b = fc_bytes(N, K)
+        per_shape[f"{name} {N}x{K}"] = {"us": round(us, 3), "GB/s": round(b / us / 1e3, 1), "bytes": b}
+        del g
+    return per_shape
 
-            def launch_all():
-                for layer in range(LAYERS):
-                    wq = weights[layer][[n for n, _, _ in LAYER_FCS].index(name)]
-                    llmops._lib.check(lib.llmops_fc_Q4A_prequantized(
-                        xq.data_ptr(), xd.data_ptr(), gs.data_ptr(), 1, wq.data_ptr(), Ng, Kg, G, N, y.data_ptr(),
-                        ws.data_ptr(), ws.numel(), st))
 
-            launch_all()
-            torch.cuda.synchronize()
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record(stream)
-            for _ in range(reps):
-                launch_all()
-            e1.record(stream)
-            torch.cuda.synchronize()
-            ms = e0.elapsed_time(e1)
-            n = reps * LAYERS
-            b = fc_bytes(N, K)
-            per_shape[name] = {"us": round(ms / n * 1e3, 3), "GB/s": round(b / (ms / n * 1e-3) / 1e9, 1)}
-            total_ms += ms
-            total_bytes += b * n
-            launches += n
-    achieved = total_bytes / (total_ms * 1e-3) / 1e9
-    return {"bound": "hbm", "kernel": "fc_gemv_kernel<128,1>", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
-            "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
-            "avg_launch_us": round(total_ms / launches * 1e3, 3),
-            "bytes_per_launch_avg": int(total_bytes / launches), "per_shape": per_shape,
-            "timing": "HIP events around back-to-back launches (includes inter-launch gaps)"}
+def dispatch_floor(torch, stream, n=64, reps=10):
+    """Average time per launch of a do-nothing kernel in a replayed graph: the gap between dependent launches."""
+    t = torch.zeros(64, device="cuda")
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g, stream=stream):
+        for _ in range(n):
+            t.add_(1.0)
+    g.replay()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record(stream)
+    for _ in range(reps):
+        g.replay()
+    e1.record(stream)
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e3 / (n * reps)
 
 
 def cpu_baseline(budget_s=12.0):

@@ -154,6 +154,19 @@ int llmops_embedding_q8c(float* out, const int64_t* ids, int64_t n, const int8_t
 /* embedding (ops/op_embedding.hpp:24-49): out[i,:] = w[ids[i],:]; ids int64 */
 int llmops_embedding(float* out, const int64_t* ids, int64_t n, const float* w, int64_t V, int64_t E, llmops_stream_t stream);
 
+/* ------------------------------------------------------------------------------------------
+ * Measurement helpers (no counterpart in the reference; used by bench.py and the profiles)
+ * ------------------------------------------------------------------------------------------ */
+
+/* read / copy `bytes` (multiple of 16) with `workgroups` workgroups of 256 threads streaming
+ * contiguous slabs: the machine's measured HBM ceiling and the calibration of traffic counters */
+int llmops_calib_read(const void* src, int64_t bytes, int workgroups, void* out4, llmops_stream_t stream);
+int llmops_calib_copy(const void* src, void* dst, int64_t bytes, int workgroups, llmops_stream_t stream);
+
+/* split-K planner knobs of the streaming FC kernel: number of workgroups to aim for and
+ * wavefronts per workgroup (4, 8, 16; 0 = default).  Values <= 0 / < 0 leave a knob unchanged. */
+void llmops_fc_set_tuning(int target_workgroups, int waves_per_workgroup);
+
 #ifdef __cplusplus
 }
 #endif

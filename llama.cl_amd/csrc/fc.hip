@@ -9,8 +9,8 @@ constexpr int kMaxGemvRows = 8;
 int launch_quant_x(const float* x, int64_t rows, int64_t K, int group_k, int8_t* xq, float* xd, float* gsum,
                    hipStream_t stream);
 size_t gemv_workspace_bytes(int64_t rows, int64_t Ng, int64_t Kg, int G);
-int launch_gemv(const uint8_t* w, const int8_t* xq, const float* xd, const float* gs, float* y, float* part,
-                unsigned* counters, int64_t rows, int64_t Ng, int64_t Kg, int G, int64_t N, hipStream_t st);
+int launch_gemv(const uint8_t* w, const float* x, const int8_t* xq, const float* xd, const float* gs, float* y,
+                float* part, unsigned* counters, int64_t rows, int64_t Ng, int64_t Kg, int G, int64_t N, hipStream_t st);
 int launch_gemv_partials(const uint8_t* w, const int8_t* xq, int32_t* acc, int64_t rows, int64_t Ng, int64_t Kg, int G,
                          hipStream_t st);
 size_t gemm_workspace_bytes(int64_t rows, int64_t Ng, int64_t Kg);
@@ -60,7 +60,7 @@ extern "C" int llmops_fc_Q4A(const float* x, int64_t rows, int64_t K, const int8
     LLMOPS_REQUIRE(N > (Ng - 1) * kGroupN && N <= Ng * kGroupN);
     LLMOPS_REQUIRE(Ng <= LLMOPS_FC_COUNTER_BYTES / 4);
     LLMOPS_REQUIRE(Ng * 64 < ((int64_t)1 << 31));
-    LLMOPS_REQUIRE(aligned(weiq, 16) && aligned(workspace, 256));
+    LLMOPS_REQUIRE(aligned(weiq, 16) && aligned(workspace, 256) && aligned(x, 8));
     const FcWorkspace lay = fc_layout(rows, Ng, Kg, group_k);
     if (workspace_bytes < lay.total)
         return fail(LLMOPS_EWORKSPACE, "fc_Q4A needs %zu workspace bytes, got %zu", lay.total, workspace_bytes);
@@ -71,10 +71,12 @@ extern "C" int llmops_fc_Q4A(const float* x, int64_t rows, int64_t K, const int8
     float* gs = reinterpret_cast<float*>(ws + lay.off_gs);
     float* part = reinterpret_cast<float*>(ws + lay.off_part);
     hipStream_t st = as_stream(stream);
+    const uint8_t* w = reinterpret_cast<const uint8_t*>(weiq);
+    // few rows: one launch, the streaming kernel quantizes the activations it needs on the fly
+    if (rows <= kMaxGemvRows)
+        return launch_gemv(w, x, nullptr, nullptr, nullptr, y, part, counters, rows, Ng, Kg, group_k, N, st);
     int rc = launch_quant_x(x, rows, K, group_k, xq, xd, gs, st);
     if (rc) return rc;
-    const uint8_t* w = reinterpret_cast<const uint8_t*>(weiq);
-    if (rows <= kMaxGemvRows) return launch_gemv(w, xq, xd, gs, y, part, counters, rows, Ng, Kg, group_k, N, st);
     return launch_gemm(w, xq, xd, gs, y, part, rows, Ng, Kg, group_k, N, st);
 }
 
@@ -96,7 +98,7 @@ extern "C" int llmops_fc_Q4A_prequantized(const int8_t* xq, const float* xd, con
     const uint8_t* w = reinterpret_cast<const uint8_t*>(weiq);
     hipStream_t st = as_stream(stream);
     if (rows <= kMaxGemvRows)
-        return launch_gemv(w, xq, xd, gsum, y, part, reinterpret_cast<unsigned*>(ws), rows, Ng, Kg, group_k, N, st);
+        return launch_gemv(w, nullptr, xq, xd, gsum, y, part, reinterpret_cast<unsigned*>(ws), rows, Ng, Kg, group_k, N, st);
     return launch_gemm(w, xq, xd, gsum, y, part, rows, Ng, Kg, group_k, N, st);
 }
 

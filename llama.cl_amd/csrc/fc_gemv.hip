@@ -3,8 +3,8 @@
 //
 // Data movement.  The packed tensor [Ng][Kg][block] is a set of Ng independent strips (32 output
 // columns each) whose blocks are contiguous in memory, so a strip is one linear stream.  Work is
-// cut into (strip, k-range) tiles: one 256-thread workgroup per tile, each of its 4 wavefronts
-// streaming a contiguous run of blocks with 16-byte loads per lane:
+// cut into (strip, k-range) tiles: one workgroup per tile, each of its NW wavefronts streaming a
+// contiguous run of blocks with 16-byte loads per lane:
 //
 //   lane = rs*8 + quad,  rs = 0..7 (k8-row slot), quad = 0..7 (4 adjacent columns)
 //   one wave-wide 16 B load = 8 k8-rows x 128 B = 64 k-values x 32 columns, perfectly coalesced
@@ -12,9 +12,17 @@
 //   high nibbles k 4..7), so (dw & 0x0F0F0F0F) and ((dw>>4) & 0x0F0F0F0F) feed two v_dot4
 //   against the lane's 8 activation codes with no shuffling.
 //
+// Activations.  The production kernel takes the raw fp32 row and quantizes, inside each
+// wavefront, exactly the k-groups that wavefront is about to stream (same operations as
+// FC_dynamic_quantize_x, hence the same int8 codes and scales; the raw group sum is a tree sum
+// instead of the left-to-right one).  The activation loads are issued ahead of the weight loads
+// and the quantization runs while the first weight blocks are still in flight; codes and scales
+// go through a wave-private LDS slot to the lanes that need them.  A second kernel variant takes
+// activations already quantized by llmops_FC_dynamic_quantize_x.
+//
 // Each lane keeps fp32 running sums for its 4 columns (x rows); per block it folds its int32
 // partial dot product in as (d*dx)*acc, and the lanes on a block's first k8-row add m*gsum.
-// The 8 row slots are summed at the end with xor-shuffles, the 4 waves through LDS, and the
+// The 8 row slots are summed at the end with lane exchanges, the NW waves through LDS, and the
 // k-splits of a strip through a scratch buffer: the workgroup that arrives last at the strip's
 // counter adds the splits in index order, so results do not depend on scheduling.
 //
@@ -25,13 +33,36 @@
 
 namespace llmops {
 
-int launch_quant_x(const float* x, int64_t rows, int64_t K, int group_k, int8_t* xq, float* xd, float* gsum,
-                   hipStream_t stream);
-
-constexpr int kMaxGemvRows = 8;
-
-__device__ __forceinline__ uint4 ldg16(const uint8_t* p) { return *reinterpret_cast<const uint4*>(p); }
+// weights are read exactly once: non-temporal loads keep them from displacing the activations,
+// scales and partial sums that are reused out of the caches
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ uint4 ldg16(const uint8_t* p) {
+    const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+    return make_uint4(v.x, v.y, v.z, v.w);
+}
 __device__ __forceinline__ uint2 ldg8(const uint8_t* p) { return *reinterpret_cast<const uint2*>(p); }
+
+// ---- lane exchanges on the VALU (DPP), no LDS round trips --------------------------------------
+template <int CTRL>
+__device__ __forceinline__ float dpp(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(v), __float_as_int(v), CTRL, 0xF, 0xF, false));
+}
+__device__ __forceinline__ float lane_bcast(float v, int lane) {
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), lane));
+}
+constexpr int kQuadXor1 = 0xB1, kQuadXor2 = 0x4E, kRowHalfMirror = 0x141, kRowMirror = 0x140, kRowRor8 = 0x128;
+
+// max and sum over each row of 16 lanes, result in every lane of the row
+__device__ __forceinline__ void row16_max_sum(float& mx, float& sm) {
+    mx = fmaxf(mx, dpp<kQuadXor1>(mx));
+    sm += dpp<kQuadXor1>(sm);
+    mx = fmaxf(mx, dpp<kQuadXor2>(mx));
+    sm += dpp<kQuadXor2>(sm);
+    mx = fmaxf(mx, dpp<kRowHalfMirror>(mx));
+    sm += dpp<kRowHalfMirror>(sm);
+    mx = fmaxf(mx, dpp<kRowMirror>(mx));
+    sm += dpp<kRowMirror>(sm);
+}
 
 // One "step" of a wavefront: G=128 -> one block (two 16 B loads per lane);
 //                            G=32  -> two adjacent blocks, one per half-wave (one load per lane).
@@ -39,6 +70,7 @@ template <int G>
 struct Step {
     static constexpr int kLoads = (G == 128) ? 2 : 1;
     static constexpr int kBlocksPerStep = (G == 128) ? 1 : 2;
+    static constexpr int kK = (G == 128) ? 128 : 64;  // k-values per step
     uint4 w[kLoads];
     uint2 dh, mh;  // 4 x fp16 d, 4 x fp16 m of the lane's columns
     bool valid;
@@ -70,16 +102,17 @@ __device__ __forceinline__ void load_step(Step<G>& st, const uint8_t* strip, int
     }
 }
 
-// int32 partial dot products of the lane's 4 columns over the lane's k8-rows of this step
+// int32 partial dot products of the lane's 4 columns over the lane's k8-rows of this step;
+// `codes` points at the step's activation codes (Step<G>::kK of them)
 template <int G>
-__device__ __forceinline__ void dot_step(const Step<G>& st, const int8_t* xq_row, int step, int lane, int acc[4]) {
+__device__ __forceinline__ void dot_step(const Step<G>& st, const int8_t* codes, int lane, int acc[4]) {
     const int rs = lane >> 3;
-    const int2 xa = *reinterpret_cast<const int2*>(xq_row + (int64_t)step * (G == 128 ? 128 : 64) + rs * 8);
+    const int2 xa = *reinterpret_cast<const int2*>(codes + rs * 8);
     const uint32_t* w0 = reinterpret_cast<const uint32_t*>(&st.w[0]);
 #pragma unroll
     for (int j = 0; j < 4; j++) acc[j] = dot8_q4(w0[j], xa.x, xa.y, 0);
     if (G == 128) {
-        const int2 xb = *reinterpret_cast<const int2*>(xq_row + (int64_t)step * 128 + 64 + rs * 8);
+        const int2 xb = *reinterpret_cast<const int2*>(codes + 64 + rs * 8);
         const uint32_t* w1 = reinterpret_cast<const uint32_t*>(&st.w[Step<G>::kLoads - 1]);
 #pragma unroll
         for (int j = 0; j < 4; j++) acc[j] = dot8_q4(w1[j], xb.x, xb.y, acc[j]);
@@ -93,67 +126,51 @@ __device__ __forceinline__ void unpack_h4(uint2 h, float out[4]) {
     out[3] = f16_bits_to_f32((uint16_t)(h.y >> 16));
 }
 
-template <int G, int MT>
-__global__ __launch_bounds__(256) void fc_gemv_kernel(const uint8_t* __restrict__ weiq, const int8_t* __restrict__ xq,
-                                                       const float* __restrict__ xd, const float* __restrict__ gs,
-                                                       float* __restrict__ y, float* part, unsigned* counters, int Kg,
-                                                       int64_t N, int rows, int S, int steps_per_split) {
-    constexpr int BPS = Step<G>::kBlocksPerStep;
-    __shared__ float red[4][MT][kGroupN];
-    __shared__ unsigned ticket_sh;
-
-    const int lane = threadIdx.x & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int nb = blockIdx.x / S, s = blockIdx.x % S;
-    const int quad = lane & 7, rs = lane >> 3;
-    const int T = (Kg + BPS - 1) / BPS;  // steps in a strip
-    const int t_lo = s * steps_per_split;
-    const int t_hi = min(T, t_lo + steps_per_split);
-    const int per_wave = (t_hi - t_lo + 3) >> 2;
-    const int t0 = min(t_hi, t_lo + wave * per_wave), t1 = min(t_hi, t0 + per_wave);
-    const uint8_t* strip = weiq + (int64_t)nb * Kg * block_bytes(G);
-    const int64_t Kp = (int64_t)Kg * G;  // padded K of the activation codes
-
-    float f[MT][4];
+// f[r][j] += (d*dx)*acc + m*gsum for the lane's 4 columns
+__device__ __forceinline__ void fold(float f[4], const int acc[4], uint2 dh, uint2 mh, float dx, float g) {
+    float d[4], m[4];
+    unpack_h4(dh, d);
+    unpack_h4(mh, m);
 #pragma unroll
-    for (int r = 0; r < MT; r++)
-#pragma unroll
-        for (int j = 0; j < 4; j++) f[r][j] = 0.0f;
-
-    Step<G> cur, nxt;
-    if (t0 < t1) load_step<G>(cur, strip, t0, Kg, lane);
-    for (int t = t0; t < t1; t++) {
-        if (t + 1 < t1) load_step<G>(nxt, strip, t + 1, Kg, lane);
-        // block index whose scales this lane applies
-        const int kb = (G == 128) ? t : t * 2 + (rs >> 2);
-        float d[4], m[4];
-        unpack_h4(cur.dh, d);
-        unpack_h4(cur.mh, m);
-        const bool first_row = (G == 128) ? (rs == 0) : ((rs & 3) == 0);
-#pragma unroll
-        for (int r = 0; r < MT; r++) {
-            if (r < rows && cur.valid) {
-                int acc[4];
-                dot_step<G>(cur, xq + r * Kp, t, lane, acc);
-                const float dx = xd[(int64_t)r * Kg + kb];
-                const float g = first_row ? gs[(int64_t)r * Kg + kb] : 0.0f;
-#pragma unroll
-                for (int j = 0; j < 4; j++) {
-                    f[r][j] = fmaf(d[j] * dx, (float)acc[j], f[r][j]);
-                    f[r][j] = fmaf(m[j], g, f[r][j]);
-                }
-            }
-        }
-        cur = nxt;
+    for (int j = 0; j < 4; j++) {
+        f[j] = fmaf(d[j] * dx, (float)acc[j], f[j]);
+        f[j] = fmaf(m[j], g, f[j]);
     }
+}
 
+struct TileRange {
+    int nb, s, t0, t1;
+};
+
+template <int G, int NW>
+__device__ __forceinline__ TileRange tile_range(int Kg, int S, int steps_per_split, int wave) {
+    constexpr int BPS = Step<G>::kBlocksPerStep;
+    TileRange r;
+    r.nb = blockIdx.x / S;
+    r.s = blockIdx.x % S;
+    const int T = (Kg + BPS - 1) / BPS;  // steps in a strip
+    const int t_lo = r.s * steps_per_split;
+    const int t_hi = min(T, t_lo + steps_per_split);
+    const int per_wave = (t_hi - t_lo + NW - 1) / NW;
+    r.t0 = min(t_hi, t_lo + wave * per_wave);
+    r.t1 = min(t_hi, r.t0 + per_wave);
+    return r;
+}
+
+// Sum the lanes' running sums over row slots, waves and k-splits and store the strip's outputs.
+template <int MT, int NW>
+__device__ __forceinline__ void finish_strip(float f[MT][4], float (*red)[MT][kGroupN], unsigned* ticket_sh, int nb, int s,
+                                             int S, int rows, int64_t N, float* __restrict__ y, float* part,
+                                             unsigned* counters) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int quad = lane & 7, rs = lane >> 3;
     // sum the 8 row slots (lane bits 3..5)
 #pragma unroll
     for (int r = 0; r < MT; r++)
 #pragma unroll
         for (int j = 0; j < 4; j++) {
             float v = f[r][j];
-            v += __shfl_xor(v, 8, 64);
+            v += dpp<kRowRor8>(v);
             v += __shfl_xor(v, 16, 64);
             v += __shfl_xor(v, 32, 64);
             f[r][j] = v;
@@ -167,28 +184,33 @@ __global__ __launch_bounds__(256) void fc_gemv_kernel(const uint8_t* __restrict_
     __syncthreads();
 
     const int tr = threadIdx.x >> 5, tn = threadIdx.x & 31;  // (row, column) this thread finalises
+    const bool mine = tr < MT && tr < rows;
+    if (S == 1 && !mine) return;
     const int64_t n = (int64_t)nb * kGroupN + tn;
     const int64_t Np = (int64_t)gridDim.x / S * kGroupN;
     float v = 0.0f;
-    if (tr < MT && tr < rows) v = ((red[0][tr][tn] + red[1][tr][tn]) + red[2][tr][tn]) + red[3][tr][tn];
+    if (mine) {
+#pragma unroll
+        for (int w = 0; w < NW; w++) v += red[w][tr][tn];
+    }
     if (S == 1) {
-        if (tr < MT && tr < rows && n < N) y[(int64_t)tr * N + n] = v;
+        if (n < N) y[(int64_t)tr * N + n] = v;
         return;
     }
     // Cross-workgroup hand-off without cache-wide fences: partial sums are written and read with
     // device-scope (write-through / cache-bypassing) accesses, and the arrival counter is a
-    // device-scope atomic.  __syncthreads() waits for this workgroup's stores to be acknowledged
-    // before thread 0 announces the arrival.  (A __threadfence() here makes every workgroup
-    // write back and invalidate its whole L2 slice, which costs far more than the kernel itself.)
-    if (tr < MT && tr < rows)
-        __hip_atomic_store(&part[((int64_t)s * rows + tr) * Np + n], v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the write-through stores above have been acknowledged
+    // device-scope atomic.  The explicit wait makes sure this workgroup's stores have been
+    // acknowledged before thread 0 announces the arrival.  (A __threadfence() here makes every
+    // workgroup write back and invalidate its whole L2 slice, which costs far more than the
+    // kernel itself.)
+    if (mine) __hip_atomic_store(&part[((int64_t)s * rows + tr) * Np + n], v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     if (threadIdx.x == 0)
-        ticket_sh = __hip_atomic_fetch_add(&counters[nb], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        *ticket_sh = __hip_atomic_fetch_add(&counters[nb], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __syncthreads();
-    if (ticket_sh != (unsigned)(S - 1)) return;
-    if (tr < MT && tr < rows && n < N) {
+    if (*ticket_sh != (unsigned)(S - 1)) return;
+    if (mine && n < N) {
         float acc = 0.0f;
         for (int i = 0; i < S; i++)
             acc += __hip_atomic_load(&part[((int64_t)i * rows + tr) * Np + n], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -197,8 +219,183 @@ __global__ __launch_bounds__(256) void fc_gemv_kernel(const uint8_t* __restrict_
     if (threadIdx.x == 0) __hip_atomic_store(&counters[nb], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // next launch
 }
 
+// ---- variant 1: activations already quantized (xq, xd, gs in global memory) -------------------
+template <int G, int MT, int NW>
+__global__ __launch_bounds__(NW * 64) void fc_gemv_kernel(const uint8_t* __restrict__ weiq, const int8_t* __restrict__ xq,
+                                                           const float* __restrict__ xd, const float* __restrict__ gs,
+                                                           float* __restrict__ y, float* part, unsigned* counters, int Kg,
+                                                           int64_t N, int rows, int S, int steps_per_split) {
+    __shared__ float red[NW][MT][kGroupN];
+    __shared__ unsigned ticket_sh;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int rs = lane >> 3;
+    const TileRange tr = tile_range<G, NW>(Kg, S, steps_per_split, wave);
+    const uint8_t* strip = weiq + (int64_t)tr.nb * Kg * block_bytes(G);
+    const int64_t Kp = (int64_t)Kg * G;  // padded K of the activation codes
+
+    float f[MT][4];
+#pragma unroll
+    for (int r = 0; r < MT; r++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) f[r][j] = 0.0f;
+
+    Step<G> cur, nxt;
+    if (tr.t0 < tr.t1) load_step<G>(cur, strip, tr.t0, Kg, lane);
+    for (int t = tr.t0; t < tr.t1; t++) {
+        if (t + 1 < tr.t1) load_step<G>(nxt, strip, t + 1, Kg, lane);
+        const int kb = (G == 128) ? t : t * 2 + (rs >> 2);  // block whose scales this lane applies
+        const bool first_row = (G == 128) ? (rs == 0) : ((rs & 3) == 0);
+        if (cur.valid) {
+#pragma unroll
+            for (int r = 0; r < MT; r++) {
+                if (r < rows) {
+                    int acc[4];
+                    dot_step<G>(cur, xq + r * Kp + (int64_t)t * Step<G>::kK, lane, acc);
+                    const float dx = xd[(int64_t)r * Kg + kb];
+                    const float g = first_row ? gs[(int64_t)r * Kg + kb] : 0.0f;
+                    fold(f[r], acc, cur.dh, cur.mh, dx, g);
+                }
+            }
+        }
+        cur = nxt;
+    }
+    finish_strip<MT, NW>(f, red, &ticket_sh, tr.nb, tr.s, S, rows, N, y, part, counters);
+}
+
+// ---- variant 2: raw fp32 activations, quantized by the wavefront that consumes them -----------
+template <int G>
+struct XRaw {
+    float v[(G == 128) ? 2 : 1];
+};
+
+template <int G>
+__device__ __forceinline__ void load_x(XRaw<G>& xr, const float* xrow, int step, int64_t K, int lane) {
+    if (G == 128) {
+        const float2 t = *reinterpret_cast<const float2*>(xrow + (int64_t)step * 128 + lane * 2);
+        xr.v[0] = t.x;
+        xr.v[(G == 128) ? 1 : 0] = t.y;
+    } else {
+        const int64_t k = (int64_t)step * 64 + lane;
+        xr.v[0] = k < K ? xrow[k] : 0.0f;
+    }
+}
+
+__device__ __forceinline__ int q8_code_rne(float v, float id) {
+    const float t = v * id;
+    if (t != t) return -128;  // what the reference's cvtps2dq + saturating packs give for NaN
+    return (int)fminf(127.0f, fmaxf(-128.0f, rintf(t)));
+}
+
+// Per-step record in LDS: the step's int8 codes followed by (dx, gsum) per block of the step
+template <int G>
+struct XSlot {
+    int8_t codes[Step<G>::kK];
+    float2 scale[Step<G>::kBlocksPerStep];
+};
+
+// FC_dynamic_quantize_x for one step (/root/reference/ops/op_fc.hpp:246-268): amax -> d = amax/127 ->
+// id = 1/d -> RNE codes; raw sum of the group
+template <int G>
+__device__ __forceinline__ void quantize_step(const XRaw<G>& xr, XSlot<G>* slot, int lane) {
+    if (G == 128) {
+        float amax = fmaxf(fabsf(xr.v[0]), fabsf(xr.v[(G == 128) ? 1 : 0]));
+        float sum = xr.v[0] + xr.v[(G == 128) ? 1 : 0];
+        row16_max_sum(amax, sum);
+        amax = fmaxf(fmaxf(lane_bcast(amax, 0), lane_bcast(amax, 16)), fmaxf(lane_bcast(amax, 32), lane_bcast(amax, 48)));
+        sum = (lane_bcast(sum, 0) + lane_bcast(sum, 16)) + (lane_bcast(sum, 32) + lane_bcast(sum, 48));
+        const float d = amax / 127.0f;
+        const float id = (d != 0.0f) ? (1.0f / d) : 0.0f;
+        const uint32_t c0 = (uint32_t)q8_code_rne(xr.v[0], id) & 0xFFu;
+        const uint32_t c1 = (uint32_t)q8_code_rne(xr.v[(G == 128) ? 1 : 0], id) & 0xFFu;
+        *reinterpret_cast<uint16_t*>(&slot->codes[lane * 2]) = (uint16_t)(c0 | (c1 << 8));
+        if (lane == 0) slot->scale[0] = make_float2(d, sum);
+    } else {
+        float amax = fabsf(xr.v[0]);
+        float sum = xr.v[0];
+        row16_max_sum(amax, sum);
+        // the two half-waves hold two different groups
+        const float a_lo = fmaxf(lane_bcast(amax, 0), lane_bcast(amax, 16)), a_hi = fmaxf(lane_bcast(amax, 32), lane_bcast(amax, 48));
+        const float s_lo = lane_bcast(sum, 0) + lane_bcast(sum, 16), s_hi = lane_bcast(sum, 32) + lane_bcast(sum, 48);
+        const bool hi = lane >= 32;
+        const float d = (hi ? a_hi : a_lo) / 127.0f;
+        const float id = (d != 0.0f) ? (1.0f / d) : 0.0f;
+        slot->codes[lane] = (int8_t)q8_code_rne(xr.v[0], id);
+        if ((lane & 31) == 0) slot->scale[(G == 128) ? 0 : (lane >> 5)] = make_float2(d, hi ? s_hi : s_lo);
+    }
+}
+
+// D = weight blocks kept in flight ahead of the one being consumed (per wave)
+template <int G, int MT, int NW, int D>
+__global__ __launch_bounds__(NW * 64) void fc_gemv_fused_kernel(const uint8_t* __restrict__ weiq, const float* __restrict__ x,
+                                                                 float* __restrict__ y, float* part, unsigned* counters,
+                                                                 int Kg, int64_t K, int64_t N, int rows, int S,
+                                                                 int steps_per_split) {
+    __shared__ float red[NW][MT][kGroupN];
+    __shared__ __align__(16) XSlot<G> xs[NW][MT];
+    __shared__ unsigned ticket_sh;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int rs = lane >> 3;
+    const TileRange tr = tile_range<G, NW>(Kg, S, steps_per_split, wave);
+    const uint8_t* strip = weiq + (int64_t)tr.nb * Kg * block_bytes(G);
+    const bool first_row = (G == 128) ? (rs == 0) : ((rs & 3) == 0);
+
+    float f[MT][4];
+#pragma unroll
+    for (int r = 0; r < MT; r++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) f[r][j] = 0.0f;
+
+    // ring of D+1 block buffers; the activation row of a step is fetched one step ahead
+    Step<G> buf[D + 1];
+    XRaw<G> xcur[MT], xnxt[MT];
+    if (tr.t0 < tr.t1) {
+#pragma unroll
+        for (int r = 0; r < MT; r++)
+            if (r < rows) load_x<G>(xcur[r], x + (int64_t)r * K, tr.t0, K, lane);
+    }
+#pragma unroll
+    for (int u = 0; u < D; u++)
+        if (tr.t0 + u < tr.t1) load_step<G>(buf[u], strip, tr.t0 + u, Kg, lane);
+
+    for (int tb = tr.t0; tb < tr.t1; tb += D + 1) {
+#pragma unroll
+        for (int u = 0; u < D + 1; u++) {
+            const int t = tb + u;
+            if (t < tr.t1) {
+                if (t + D < tr.t1) load_step<G>(buf[(u + D) % (D + 1)], strip, t + D, Kg, lane);
+                if (t + 1 < tr.t1) {
+#pragma unroll
+                    for (int r = 0; r < MT; r++)
+                        if (r < rows) load_x<G>(xnxt[r], x + (int64_t)r * K, t + 1, K, lane);
+                }
+                const Step<G>& cur = buf[u];
+#pragma unroll
+                for (int r = 0; r < MT; r++) {
+                    if (r < rows) {
+                        XSlot<G>* slot = &xs[wave][r];
+                        quantize_step<G>(xcur[r], slot, lane);
+                        __builtin_amdgcn_wave_barrier();  // LDS writes stay ahead of the reads below
+                        if (cur.valid) {
+                            int acc[4];
+                            dot_step<G>(cur, slot->codes, lane, acc);
+                            const float2 sc = slot->scale[(G == 128) ? 0 : (rs >> 2)];
+                            fold(f[r], acc, cur.dh, cur.mh, sc.x, first_row ? sc.y : 0.0f);
+                        }
+                        __builtin_amdgcn_wave_barrier();  // reads stay ahead of the next step's writes
+                    }
+                }
+#pragma unroll
+                for (int r = 0; r < MT; r++) xcur[r] = xnxt[r];
+            }
+        }
+    }
+    finish_strip<MT, NW>(f, red, &ticket_sh, tr.nb, tr.s, S, rows, N, y, part, counters);
+}
+
 // Integer core only: acc[r][n][kb] (int32).  One wavefront per step, same loads and same dot
-// code as fc_gemv_kernel; the row slots of a block are summed with xor-shuffles.
+// code as the streaming kernels; the row slots of a block are summed with xor-shuffles.
 template <int G>
 __global__ __launch_bounds__(64) void fc_gemv_partials_kernel(const uint8_t* __restrict__ weiq,
                                                                const int8_t* __restrict__ xq, int32_t* __restrict__ out,
@@ -215,7 +412,7 @@ __global__ __launch_bounds__(64) void fc_gemv_partials_kernel(const uint8_t* __r
     load_step<G>(st, strip, t, Kg, lane);
     for (int r = 0; r < rows; r++) {
         int acc[4] = {0, 0, 0, 0};
-        if (st.valid) dot_step<G>(st, xq + r * Kp, t, lane, acc);
+        if (st.valid) dot_step<G>(st, xq + r * Kp + (int64_t)t * Step<G>::kK, lane, acc);
 #pragma unroll
         for (int j = 0; j < 4; j++) {
             int v = acc[j];
@@ -233,40 +430,74 @@ __global__ __launch_bounds__(64) void fc_gemv_partials_kernel(const uint8_t* __r
     }
 }
 
-static int g_target_workgroups = 1024;
+static int g_target_workgroups = 256;  // split-K planner aims for this many workgroups
+static int g_waves_per_workgroup = 0;  // 0 = choose per shape
+static int g_prefetch_depth = 1;       // weight blocks in flight ahead of the current one
 
 struct GemvPlan {
-    int S, steps_per_split;
+    int S, steps_per_split, NW;
 };
 
-static GemvPlan plan_gemv(int64_t Ng, int64_t Kg, int G) {
+static GemvPlan plan_gemv(int64_t rows, int64_t Ng, int64_t Kg, int G) {
     const int bps = (G == 128) ? 1 : 2;
     const int T = (int)((Kg + bps - 1) / bps);
+    int NW = g_waves_per_workgroup;
+    if (NW == 0) NW = 16;
+    if (rows > 4 && NW > 8) NW = 8;  // one (row, column) finaliser thread per output of the strip
     int S = (int)((g_target_workgroups + Ng - 1) / Ng);
-    const int max_s = (T + 3) / 4;  // at least one step per wave
+    const int max_s = (T + NW - 1) / NW;  // at least one step per wave
     if (S > max_s) S = max_s;
     if (S < 1) S = 1;
     int sps = (T + S - 1) / S;
     S = (T + sps - 1) / sps;  // drop empty splits
-    return {S, sps};
+    return {S, sps, NW};
 }
 
 size_t gemv_workspace_bytes(int64_t rows, int64_t Ng, int64_t Kg, int G) {
-    const GemvPlan p = plan_gemv(Ng, Kg, G);
-    return (size_t)p.S * rows * Ng * kGroupN * sizeof(float);
+    // upper bound over every plan the tuning knobs can produce: S never exceeds the step count
+    const int bps = (G == 128) ? 1 : 2;
+    const int64_t T = (Kg + bps - 1) / bps;
+    int64_t S = (4096 + Ng - 1) / Ng;
+    if (S > T) S = T;
+    return (size_t)S * rows * Ng * kGroupN * sizeof(float);
+}
+
+template <int G, int MT, int NW>
+static void launch_gemv_t(const uint8_t* w, const float* x, const int8_t* xq, const float* xd, const float* gs, float* y,
+                          float* part, unsigned* counters, int64_t Ng, int64_t Kg, int64_t N, int rows, GemvPlan p,
+                          hipStream_t st) {
+    const unsigned grid = (unsigned)(Ng * p.S);
+    if (x == nullptr) {
+        fc_gemv_kernel<G, MT, NW><<<grid, NW * 64, 0, st>>>(w, xq, xd, gs, y, part, counters, (int)Kg, N, rows, p.S,
+                                                            p.steps_per_split);
+        return;
+    }
+#define LLMOPS_FUSED(DD)                                                                                             \
+    fc_gemv_fused_kernel<G, MT, NW, DD><<<grid, NW * 64, 0, st>>>(w, x, y, part, counters, (int)Kg, Kg * G, N, rows, p.S, \
+                                                                  p.steps_per_split)
+    if (MT == 1 && g_prefetch_depth >= 3) LLMOPS_FUSED((MT == 1 ? 3 : 1));
+    else if (MT == 1 && g_prefetch_depth == 2) LLMOPS_FUSED((MT == 1 ? 2 : 1));
+    else LLMOPS_FUSED(1);
+#undef LLMOPS_FUSED
 }
 
 template <int G, int MT>
-static void launch_gemv_t(const uint8_t* w, const int8_t* xq, const float* xd, const float* gs, float* y, float* part,
-                          unsigned* counters, int64_t Ng, int64_t Kg, int64_t N, int rows, GemvPlan p, hipStream_t st) {
-    fc_gemv_kernel<G, MT><<<(unsigned)(Ng * p.S), 256, 0, st>>>(w, xq, xd, gs, y, part, counters, (int)Kg, N, rows, p.S,
-                                                                p.steps_per_split);
+static void launch_gemv_nw(const uint8_t* w, const float* x, const int8_t* xq, const float* xd, const float* gs, float* y,
+                           float* part, unsigned* counters, int64_t Ng, int64_t Kg, int64_t N, int rows, GemvPlan p,
+                           hipStream_t st) {
+    if (p.NW >= 16 && MT <= 4)
+        launch_gemv_t<G, MT, (MT <= 4 ? 16 : 8)>(w, x, xq, xd, gs, y, part, counters, Ng, Kg, N, rows, p, st);
+    else if (p.NW >= 8)
+        launch_gemv_t<G, MT, 8>(w, x, xq, xd, gs, y, part, counters, Ng, Kg, N, rows, p, st);
+    else
+        launch_gemv_t<G, MT, 4>(w, x, xq, xd, gs, y, part, counters, Ng, Kg, N, rows, p, st);
 }
 
-int launch_gemv(const uint8_t* w, const int8_t* xq, const float* xd, const float* gs, float* y, float* part,
-                unsigned* counters, int64_t rows, int64_t Ng, int64_t Kg, int G, int64_t N, hipStream_t st) {
-    const GemvPlan p = plan_gemv(Ng, Kg, G);
-#define LLMOPS_GEMV_CASE(GG, MT) launch_gemv_t<GG, MT>(w, xq, xd, gs, y, part, counters, Ng, Kg, N, (int)rows, p, st)
+// x != nullptr: raw fp32 activations, quantized inside the kernel; else xq/xd/gs are used.
+int launch_gemv(const uint8_t* w, const float* x, const int8_t* xq, const float* xd, const float* gs, float* y,
+                float* part, unsigned* counters, int64_t rows, int64_t Ng, int64_t Kg, int G, int64_t N, hipStream_t st) {
+    const GemvPlan p = plan_gemv(rows, Ng, Kg, G);
+#define LLMOPS_GEMV_CASE(GG, MT) launch_gemv_nw<GG, MT>(w, x, xq, xd, gs, y, part, counters, Ng, Kg, N, (int)rows, p, st)
     if (G == 128) {
         if (rows == 1) LLMOPS_GEMV_CASE(128, 1);
         else if (rows == 2) LLMOPS_GEMV_CASE(128, 2);
@@ -297,7 +528,10 @@ int launch_gemv_partials(const uint8_t* w, const int8_t* xq, int32_t* acc, int64
 
 }  // namespace llmops
 
-// Development knob: number of workgroups the split-K planner aims for (default 1024).
-extern "C" void llmops_fc_set_target_workgroups(int n) {
-    if (n > 0) llmops::g_target_workgroups = n;
+extern "C" void llmops_fc_set_tuning(int target_workgroups, int waves_per_workgroup) {
+    if (target_workgroups > 0) llmops::g_target_workgroups = target_workgroups > 4096 ? 4096 : target_workgroups;
+    if (waves_per_workgroup >= 0) llmops::g_waves_per_workgroup = waves_per_workgroup;
+}
+extern "C" void llmops_fc_set_prefetch(int depth) {
+    if (depth >= 1) llmops::g_prefetch_depth = depth;
 }

@@ -36,6 +36,9 @@ SIGNATURES = {
     "llmops_embedding_q8c_quant_w": (c_int, [c_ptr, c_i64, c_i64, c_ptr, c_ptr, c_ptr]),
     "llmops_embedding_q8c": (c_int, [c_ptr, c_ptr, c_i64, c_ptr, c_ptr, c_i64, c_i64, c_ptr]),
     "llmops_embedding": (c_int, [c_ptr, c_ptr, c_i64, c_ptr, c_i64, c_i64, c_ptr]),
+    "llmops_calib_read": (c_int, [c_ptr, c_i64, c_int, c_ptr, c_ptr]),
+    "llmops_calib_copy": (c_int, [c_ptr, c_ptr, c_i64, c_int, c_ptr]),
+    "llmops_fc_set_tuning": (None, [c_int, c_int]),
 }
 
 _lib = None
