@@ -445,6 +445,7 @@ static GemvPlan plan_gemv(int64_t rows, int64_t Ng, int64_t Kg, int G) {
     if (NW == 0) NW = 16;
     if (rows > 4 && NW > 8) NW = 8;  // one (row, column) finaliser thread per output of the strip
     int S = (int)((g_target_workgroups + Ng - 1) / Ng);
+    if ((T + NW - 1) / NW <= 2) S = 1;    // a wave already has only 1-2 blocks: splitting buys nothing
     const int max_s = (T + NW - 1) / NW;  // at least one step per wave
     if (S > max_s) S = max_s;
     if (S < 1) S = 1;
