@@ -55,6 +55,7 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-decode", action="store_true", help="skip the full decode-step timing (BASELINE config 5)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU (the path is data-parallel per GPU; multi-GPU sharding is design "
@@ -159,6 +160,8 @@ def main():
                                          "ms_per_step": round(results["unfused"]["ms_per_step"], 4)},
         "roofline": roof,
     }
+    if not args.no_decode:
+        out["decode_step"] = decode_step(torch, stream)
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline()
     out["setup_s"] = round(setup_s, 1)
@@ -204,6 +207,36 @@ def dispatch_floor(torch, stream, n=64, reps=10):
     e1.record(stream)
     torch.cuda.synchronize()
     return e0.elapsed_time(e1) * 1e3 / (n * reps)
+
+
+def decode_step(torch, stream, kv_len=2048, reps=20):
+    """BASELINE config 5: one token through a random-init Llama-2-7B-shape model (32 layers, hidden 4096, FFN 11008,
+    32 heads, vocab 55296 lm_head, all FC Q4_1 group 128), fp32 KV cache filled to kv_len-1, batch 1; the step is
+    captured once as a HIP graph and replayed."""
+    from llmops.decode import LlamaDecoder, LLAMA_7B
+    from llmops.opset import KVCache
+
+    out = {}
+    model = LlamaDecoder(group_k=G, seed=5, embed_rows=1024)
+    for name, dtype in (("fp32_kv", torch.float32), ("fp16_kv", torch.float16)):
+        kv = KVCache(LLAMA_7B, 1, kv_len, dtype=dtype)
+        kv.cache.normal_()
+        dg = model.capture_decode(kv.cache, kv_len - 1, kv_len - 1, stream=stream)
+        with torch.cuda.stream(stream):
+            dg.replay()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(reps):
+                dg.replay()
+            torch.cuda.synchronize()
+            ms = (time.perf_counter() - t0) / reps * 1e3
+        kv_bytes = 2 * LLAMA_7B["layer_num"] * LLAMA_7B["head_num"] * kv_len * LLAMA_7B["head_size"] * kv.cache.element_size()
+        fc = model.fc_weight_size()
+        out[name] = {"ms_per_token": round(ms, 4), "GB_per_token": round((fc + kv_bytes) / 1e9, 3),
+                     "GB/s": round((fc + kv_bytes) / ms / 1e6, 1)}
+        del dg, kv
+    out["config"] = "Llama-2-7B shape, 32 layers, Q4_1(128) FCs incl. 55296x4096 lm_head, kv-len 2048, batch 1, HIP graph"
+    return out
 
 
 def cpu_baseline(budget_s=12.0):

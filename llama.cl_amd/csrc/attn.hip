@@ -67,9 +67,15 @@ __global__ void attn_prep_kernel(float* __restrict__ q, float* __restrict__ k, c
     const int64_t h = blockIdx.x % H, l = (blockIdx.x / H) % qL, b = blockIdx.x / (H * qL);
     const int64_t base = ((b * qL + l) * H + h) * S;
     const int slot = slots[l];
-    T* kdst = kc + ((b * H + h) * maxlen + slot) * S;
-    T* vdst = vc + ((b * H + h) * maxlen + slot) * S;
-    if (blockIdx.x < qL && threadIdx.x == 0) row_token[slots[blockIdx.x]] = (int32_t)blockIdx.x;
+    // slots live in device memory and cannot be validated on the host: a slot outside the cache is
+    // dropped (q and k are still rotated) rather than written through
+    const bool slot_ok = slot >= 0 && slot < maxlen;
+    T* kdst = kc + ((b * H + h) * maxlen + (slot_ok ? slot : 0)) * S;
+    T* vdst = vc + ((b * H + h) * maxlen + (slot_ok ? slot : 0)) * S;
+    if (blockIdx.x < qL && threadIdx.x == 0) {
+        const int s0 = slots[blockIdx.x];
+        if (s0 >= 0 && s0 < maxlen) row_token[s0] = (int32_t)blockIdx.x;
+    }
     for (int64_t i = threadIdx.x; i < S; i += blockDim.x) {
         if (i < half) {
             float q0 = q[base + i], q1 = q[base + i + half];
@@ -81,12 +87,14 @@ __global__ void attn_prep_kernel(float* __restrict__ q, float* __restrict__ k, c
             q[base + i + half] = q1;
             k[base + i] = k0;
             k[base + i + half] = k1;
-            store_cache(kdst + i, k0);
-            store_cache(kdst + i + half, k1);
-        } else if (i >= 2 * half) {
+            if (slot_ok) {
+                store_cache(kdst + i, k0);
+                store_cache(kdst + i + half, k1);
+            }
+        } else if (i >= 2 * half && slot_ok) {
             store_cache(kdst + i, k[base + i]);
         }
-        store_cache(vdst + i, v[base + i]);
+        if (slot_ok) store_cache(vdst + i, v[base + i]);
     }
 }
 

@@ -62,7 +62,7 @@ def _dev(t, dtype, rank=None, name="tensor"):
 def _workspace(device, nbytes):
     """Persistent per-device scratch.  Its first bytes hold the split-K arrival counters, which
     must start at zero and which the kernels leave at zero."""
-    key = (device.type, device.index)
+    key = (device.type, device.index if device.index is not None else torch.cuda.current_device())
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
         size = max(int(nbytes), 16 << 20)

@@ -1,0 +1,140 @@
+"""One Llama-shaped forward step built from ``llmops`` calls in the reference's op order
+(``Model.forward``, /root/reference/chatllama/main.py:331-380), on random-initialised weights.
+
+This is the caller of the hot path, kept as thin as the reference's: every arithmetic step is an
+``llmops`` op.  Two launch plans are offered:
+
+* ``plan="reference"``: the reference's sequence verbatim -- clone, rmsnorm, q/k/v projections as three
+  FCs, attention_rope2, o projection, iadd, clone, rmsnorm, gate, silu, up, imul, down, iadd.
+* ``plan="fused"`` (default): the same arithmetic with fewer launches -- q|k|v and gate|up packed
+  tensors concatenated along N so each pair/triple is one FC launch.
+
+A decode step (one token, batch 1) has fixed shapes and no host-side decisions, so it can be
+captured once as a HIP graph and replayed (``capture_decode``).
+"""
+import torch
+
+import llmops
+from llmops.opset import KVCache, llmop_embedding_q8c, llmop_fc_q4a, llmop_rmsnorm
+
+LLAMA_7B = dict(layer_num=32, head_num=32, head_size=128, hidden_size=4096, intermediate_size=11008,
+                vocab_size=55296, rms_norm_eps=1e-5, rope_base=10000.0)
+
+
+class LlamaDecoder:
+    def __init__(self, configs=None, group_k=128, seed=5, device="cuda", plan="fused", embed_rows=None):
+        cfg = dict(LLAMA_7B)
+        cfg.update(configs or {})
+        self.configs = cfg
+        self.plan = plan
+        self.device = torch.device(device)
+        gen = torch.Generator(device="cpu").manual_seed(seed)
+        H, F, V = cfg["hidden_size"], cfg["intermediate_size"], cfg["vocab_size"]
+
+        def fc(N, K, parts=1):
+            # parts > 1: several projections sharing one input, packed and concatenated along N
+            packed = []
+            for _ in range(parts):
+                w = (torch.randn(N, K, generator=gen) * 0.02).to(self.device)
+                packed.append(llmops.offline_FC_quant_Q4A(w, group_k))
+                del w
+            t = torch.cat(packed, dim=0) if parts > 1 else packed[0]
+            return llmop_fc_q4a(packed=t, N=N * parts)
+
+        self.layers = []
+        for _ in range(cfg["layer_num"]):
+            layer = {
+                "input_layernorm": llmop_rmsnorm(torch.ones(H, device=self.device), cfg["rms_norm_eps"]),
+                "post_attention_layernorm": llmop_rmsnorm(torch.ones(H, device=self.device), cfg["rms_norm_eps"]),
+                "o_proj": fc(H, H),
+                "down_proj": fc(H, F),
+            }
+            if plan == "fused":
+                layer["qkv_proj"] = fc(H, H, parts=3)
+                layer["gate_up_proj"] = fc(F, H, parts=2)
+            else:
+                layer["q_proj"], layer["k_proj"], layer["v_proj"] = fc(H, H), fc(H, H), fc(H, H)
+                layer["gate_proj"], layer["up_proj"] = fc(F, H), fc(F, H)
+            self.layers.append(layer)
+        self.norm = llmop_rmsnorm(torch.ones(H, device=self.device), cfg["rms_norm_eps"])
+        self.lm_head = fc(V, H)
+        # the embedding table is only gathered from (one row per token); a small table suffices for timing
+        rows = V if embed_rows is None else embed_rows
+        self.embed_tokens = llmop_embedding_q8c((torch.randn(rows, H, generator=gen)).to(self.device))
+        rd = cfg["head_size"]
+        inv_freq = 1.0 / (cfg["rope_base"] ** (torch.arange(0, rd, 2).float() / rd))  # chatllama/main.py:294-296
+        self.inv_freq = inv_freq.to(self.device)
+
+    def fc_weight_size(self):
+        n = 0
+        for layer in self.layers:
+            n += sum(op.weight_size() for op in layer.values() if isinstance(op, llmop_fc_q4a))
+        return n
+
+    def forward(self, input_ids, kv_cache, kv_cache_slots, position_id):
+        """input_ids int64 [B, qL]; returns logits fp32 [B, qL, vocab]."""
+        llmops.tensor_pool().clear()
+        H = self.configs["hidden_size"]
+        F = self.configs["intermediate_size"]
+        hidden_states = self.embed_tokens(input_ids)
+        for i, ops in enumerate(self.layers):
+            input_layernorm = llmops.clone(hidden_states)
+            ops["input_layernorm"](input_layernorm)
+            if self.plan == "fused":
+                qkv = ops["qkv_proj"](input_layernorm)
+                q, k, v = qkv[..., :H], qkv[..., H:2 * H], qkv[..., 2 * H:]
+                if not q.is_contiguous():  # more than one token: the op needs dense [B,qL,H*S] tensors
+                    q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+            else:
+                q = ops["q_proj"](input_layernorm)
+                k = ops["k_proj"](input_layernorm)
+                v = ops["v_proj"](input_layernorm)
+            llmops.attention_rope2(q, k, v, self.inv_freq, kv_cache, kv_cache_slots, position_id, i)
+            attn_output = ops["o_proj"](q)
+            llmops.iadd(attn_output, hidden_states)
+            post_attention_layernorm = llmops.clone(attn_output)
+            ops["post_attention_layernorm"](post_attention_layernorm)
+            if self.plan == "fused":
+                gate_up = ops["gate_up_proj"](post_attention_layernorm)
+                gate, up = gate_up[..., :F], gate_up[..., F:]
+                if not gate.is_contiguous():
+                    gate, up = gate.contiguous(), up.contiguous()
+            else:
+                gate = ops["gate_proj"](post_attention_layernorm)
+                up = ops["up_proj"](post_attention_layernorm)
+            llmops.itrans(gate, "silu")
+            llmops.imul(up, gate)
+            hidden_states = ops["down_proj"](up)
+            llmops.iadd(hidden_states, attn_output)
+        self.norm(hidden_states)
+        return self.lm_head(hidden_states)
+
+    def capture_decode(self, kv_cache, slot, position_id, stream=None):
+        """Capture one decode step (batch 1, one token, fixed slot/position) as a HIP graph.
+        Returns a DecodeGraph: write the token into ``.input_ids``, call ``.replay()``, read ``.logits``."""
+        stream = stream or torch.cuda.Stream()
+        input_ids = torch.zeros(1, 1, dtype=torch.int64, device=self.device)
+        slots = torch.tensor([slot], dtype=torch.int32, device=self.device)
+        with torch.cuda.stream(stream):
+            stream.wait_stream(torch.cuda.default_stream(self.device))
+            self.forward(input_ids, kv_cache, slots, position_id)  # warm-up: code objects, workspace size
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=stream):
+                logits = self.forward(input_ids, kv_cache, slots, position_id)
+        # the per-device workspace is captured by address too; pin the one in use
+        workspace = llmops._workspaces.get((self.device.type, self.device.index if self.device.index is not None
+                                            else torch.cuda.current_device()))
+        return DecodeGraph(graph, input_ids, slots, kv_cache, logits, stream, workspace)
+
+
+class DecodeGraph:
+    """A captured decode step together with every tensor whose address the graph has recorded.
+    The graph replays raw device pointers, so these tensors must live as long as the graph does."""
+
+    def __init__(self, graph, input_ids, slots, kv_cache, logits, stream, workspace):
+        self.graph, self.input_ids, self.slots, self.kv_cache, self.logits, self.stream, self.workspace = \
+            graph, input_ids, slots, kv_cache, logits, stream, workspace
+
+    def replay(self):
+        self.graph.replay()
