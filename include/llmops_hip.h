@@ -95,6 +95,13 @@ int llmops_fc_Q4A(const float* x, int64_t rows, int64_t K, const int8_t* weiq, i
                   int group_k, int64_t N, float* y, void* workspace, size_t workspace_bytes,
                   llmops_stream_t stream);
 
+/* fc_Q4A followed by iadd(y, residual) (ops/op_misc.hpp:55-79) in one launch for rows <= 8:
+ * y = fc_Q4A(x) + residual, residual fp32 [rows,N].  The decode step uses it for the o and down
+ * projections (chatllama/main.py:355-357,372-375). */
+int llmops_fc_Q4A_residual(const float* x, int64_t rows, int64_t K, const int8_t* weiq, int64_t Ng, int64_t Kg,
+                           int group_k, int64_t N, const float* residual, float* y, void* workspace,
+                           size_t workspace_bytes, llmops_stream_t stream);
+
 /* The second half of fc_Q4A on its own (ops/op_fc.hpp:318-423): the product for activations that
  * llmops_FC_dynamic_quantize_x has already quantized (xq int8 [rows,Kg*G], xd and gsum fp32
  * [rows,Kg]).  llmops_fc_Q4A == llmops_FC_dynamic_quantize_x into the workspace + this. */
@@ -117,7 +124,11 @@ int llmops_fc_Q4A_partials(const int8_t* xq, int64_t rows, const int8_t* weiq, i
 int llmops_rope_embed(float* x, int64_t B, int64_t H, int64_t L, int64_t S, const float* inv_freq,
                       int64_t half, int position_id, llmops_stream_t stream);
 
-/* workspace bytes for llmops_attention_rope (split-KV partial results) */
+/* workspace bytes for llmops_attention_rope (arrival counters, slot map, split-KV partial results).
+ * The first LLMOPS_ATTN_COUNTER_BYTES bytes must be zero when the library first sees the workspace;
+ * the library leaves them zero after every call.  One workspace must not be shared by calls that
+ * can overlap on the device. */
+#define LLMOPS_ATTN_COUNTER_BYTES 65536
 size_t llmops_attention_workspace_bytes(int64_t B, int64_t qL, int64_t H, int64_t S, int64_t maxlen);
 
 /* attention_rope2 / attention_rope (ops/op_attn.hpp:721-1029 and :518-718; ops/main.cpp:154-155;
@@ -141,6 +152,12 @@ int llmops_softmax(float* x, int64_t rows, int64_t K, llmops_stream_t stream);
 
 /* rmsnorm (ops/op_misc.hpp:142-181): x[r,:] *= rsqrt(mean(x[r,:]^2)+eps) * w, in place */
 int llmops_rmsnorm(float* x, int64_t rows, int64_t hidden, const float* w, float eps, llmops_stream_t stream);
+/* clone + rmsnorm (chatllama/main.py:345-346) in one launch: out = rmsnorm(x), x untouched */
+int llmops_rmsnorm_out(const float* x, float* out, int64_t rows, int64_t hidden, const float* w, float eps,
+                       llmops_stream_t stream);
+/* itrans(gate,"silu") + imul(up,gate) (chatllama/main.py:363-367) on a row that holds gate and up
+ * side by side: out[r,i] = silu(gate_up[r,i]) * gate_up[r,F+i] */
+int llmops_silu_mul(const float* gate_up, float* out, int64_t rows, int64_t F, llmops_stream_t stream);
 /* iadd / imul (ops/op_misc.hpp:55-107): a (+|*)= b; b is [rows,inner] or, if b_is_row, [inner] */
 int llmops_iadd(float* a, const float* b, int64_t rows, int64_t inner, int b_is_row, llmops_stream_t stream);
 int llmops_imul(float* a, const float* b, int64_t rows, int64_t inner, int b_is_row, llmops_stream_t stream);

@@ -197,25 +197,217 @@ __global__ __launch_bounds__(256) void attn_split_kernel(const float* __restrict
     }
 }
 
-// out[b,pq,h,:] = sum_c exp(m_c - M) * o_c / sum_c exp(m_c - M) * s_c ; 128 threads per query
+// Merge of the chunk records of one query: out = sum_c exp(m_c - M) o_c / sum_c exp(m_c - M) s_c.
+// LOAD fetches one float of a record (plain load after a kernel boundary, device-scope load
+// inside the single-launch decode kernel).  Chunk statistics go through LDS so that every
+// thread's loads are independent of each other.
+template <typename LOAD>
+__device__ __forceinline__ float merge_chunks(const float* rec, int nchunks, int tid, int nthreads, float* stat_sh,
+                                              LOAD load) {
+    constexpr int S = 128;
+    // stat_sh[c] = max, stat_sh[nchunks + c] = sum
+    for (int i = tid; i < 2 * nchunks; i += nthreads) {
+        const int c = i % nchunks, which = i / nchunks;
+        stat_sh[i] = load(rec + (int64_t)c * (S + 2) + which);
+    }
+    __syncthreads();
+    float M = -FLT_MAX;
+    for (int c = 0; c < nchunks; c++) M = fmaxf(M, stat_sh[c]);
+    float den = 0.0f, num = 0.0f;
+    if (tid < S) {
+        for (int c0 = 0; c0 < nchunks; c0 += 8) {
+            float o[8];
+#pragma unroll
+            for (int u = 0; u < 8; u++) o[u] = (c0 + u < nchunks) ? load(rec + (int64_t)(c0 + u) * (S + 2) + 2 + tid) : 0.0f;
+#pragma unroll
+            for (int u = 0; u < 8; u++) {
+                if (c0 + u < nchunks) {
+                    const float sum = stat_sh[nchunks + c0 + u];
+                    const float sc = (sum == 0.0f) ? 0.0f : expf(stat_sh[c0 + u] - M);
+                    den = fmaf(sc, sum, den);
+                    num = fmaf(sc, o[u], num);
+                }
+            }
+        }
+    }
+    return num * (1.0f / den);
+}
+
+constexpr int kMaxChunks = 2048;
+
 __global__ __launch_bounds__(128) void attn_merge_kernel(float* __restrict__ q, const float* __restrict__ part, int64_t qL,
                                                           int64_t H, int nchunks) {
     constexpr int S = 128;
+    __shared__ float stat_sh[2 * kMaxChunks];
     const int64_t bhq = blockIdx.x;
     const int64_t pq = bhq % qL, h = (bhq / qL) % H, b = bhq / (qL * H);
     const float* rec = part + (int64_t)bhq * nchunks * (S + 2);
-    float M = -FLT_MAX;
-    for (int c = 0; c < nchunks; c++) M = fmaxf(M, rec[(int64_t)c * (S + 2)]);
-    float den = 0.0f, num = 0.0f;
-    for (int c = 0; c < nchunks; c++) {
-        const float* r = rec + (int64_t)c * (S + 2);
-        const float sum = r[1];
-        if (sum == 0.0f) continue;
-        const float sc = expf(r[0] - M);
-        den = fmaf(sc, sum, den);
-        num = fmaf(sc, r[2 + threadIdx.x], num);
+    const float r = merge_chunks(rec, nchunks, threadIdx.x, 128, stat_sh, [](const float* p) { return *p; });
+    q[((b * qL + pq) * H + h) * S + threadIdx.x] = r;
+}
+
+// ---- single-launch decode attention (one query token) ------------------------------------------
+// Everything attention_rope2 does for qL == 1 in one kernel: every workgroup rotates q itself
+// (128 values), the workgroup whose chunk holds the new token's cache row rotates k, writes the
+// rotated k back in place and k, v into the cache, and attends to the new row from registers;
+// chunk records are handed to the last-arriving workgroup of the head (device-scope stores and
+// loads, one atomic ticket per head, no cache-wide fence), which merges them into q.
+template <typename T>
+__device__ __forceinline__ float cache_round(float v);
+template <>
+__device__ __forceinline__ float cache_round<float>(float v) {
+    return v;
+}
+template <>
+__device__ __forceinline__ float cache_round<__half>(float v) {
+    return __half2float(__float2half_rn(v));
+}
+template <typename T>
+__device__ __forceinline__ void store4(T* dst, float4 v);
+template <>
+__device__ __forceinline__ void store4<float>(float* dst, float4 v) {
+    *reinterpret_cast<float4*>(dst) = v;
+}
+template <>
+__device__ __forceinline__ void store4<__half>(__half* dst, float4 v) {
+    const __half2 a = __floats2half2_rn(v.x, v.y), b = __floats2half2_rn(v.z, v.w);
+    uint2 u;
+    u.x = *reinterpret_cast<const uint32_t*>(&a);
+    u.y = *reinterpret_cast<const uint32_t*>(&b);
+    *reinterpret_cast<uint2*>(dst) = u;
+}
+
+// rotate the lane's 4 elements (index e4 = first element) of a 128-wide head vector at `base`
+__device__ __forceinline__ float4 rope4(const float* base, int e4, const float* __restrict__ inv_freq, int half, int pos) {
+    const float4 own = *reinterpret_cast<const float4*>(base + e4);
+    if (e4 >= 2 * half) return own;
+    const bool low = e4 < half;
+    const float4 other = *reinterpret_cast<const float4*>(base + (low ? e4 + half : e4 - half));
+    const int f0 = low ? e4 : e4 - half;
+    float o[4] = {own.x, own.y, own.z, own.w}, p[4] = {other.x, other.y, other.z, other.w}, r[4];
+#pragma unroll
+    for (int c = 0; c < 4; c++) {
+        const float xita = inv_freq[f0 + c] * (float)pos;
+        const float cs = cosf(xita), sn = sinf(xita);
+        // pair (x0 = element i, x1 = element i+half): y0 = c*x0 - s*x1, y1 = s*x0 + c*x1
+        r[c] = low ? cs * o[c] - sn * p[c] : sn * p[c] + cs * o[c];
     }
-    q[((b * qL + pq) * H + h) * S + threadIdx.x] = num * (1.0f / den);
+    return make_float4(r[0], r[1], r[2], r[3]);
+}
+
+template <typename T, int PW>
+__global__ __launch_bounds__(256) void attn_decode_kernel(float* q, float* k, const float* __restrict__ v,
+                                                           const float* __restrict__ inv_freq, int half, T* kc, T* vc,
+                                                           int64_t H, int64_t maxlen, int64_t kvLen,
+                                                           const int32_t* __restrict__ slots, int position_id, float* part,
+                                                           unsigned* counters, int nchunks) {
+    constexpr int S = 128, C = 4 * PW, NL = PW / 2;
+    __shared__ float sc[C];
+    __shared__ float osh[4][2][S];
+    __shared__ float stat[2];
+    __shared__ unsigned ticket_sh;
+    __shared__ float stat_sh[2 * kMaxChunks];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int hf = lane >> 5, e = lane & 31;
+    const int chunk = blockIdx.x % nchunks;
+    const int64_t bh = blockIdx.x / nchunks;
+    const int64_t p0 = (int64_t)chunk * C;
+    T* kbase = kc + bh * maxlen * S;
+    T* vbase = vc + bh * maxlen * S;
+
+    float4 kv[NL], vv[NL];
+#pragma unroll
+    for (int i = 0; i < NL; i++) {
+        const int64_t p = p0 + wave * PW + i * 2 + hf;
+        const int64_t pc = p < kvLen ? p : kvLen - 1;
+        kv[i] = load4(kbase + pc * S + e * 4);
+        vv[i] = load4(vbase + pc * S + e * 4);
+    }
+    const int slot = slots[0];
+    const bool slot_ok = slot >= 0 && slot < maxlen;
+    const float4 qv = rope4(q + bh * S, e * 4, inv_freq, half, position_id);
+    // the workgroup that owns the new token's row (or the last chunk, if the row lies beyond kvLen)
+    const int owner = (slot_ok && slot / C < nchunks) ? slot / C : nchunks - 1;
+    if (chunk == owner) {
+        float4 kn = rope4(k + bh * S, e * 4, inv_freq, half, position_id);
+        float4 vn = *reinterpret_cast<const float4*>(v + bh * S + e * 4);
+        __syncthreads();  // every wave has read the raw k before it is overwritten
+        if (wave == 0 && hf == 0) {
+            *reinterpret_cast<float4*>(k + bh * S + e * 4) = kn;
+            if (slot_ok) {
+                store4<T>(kbase + (int64_t)slot * S + e * 4, kn);
+                store4<T>(vbase + (int64_t)slot * S + e * 4, vn);
+            }
+        }
+        kn = make_float4(cache_round<T>(kn.x), cache_round<T>(kn.y), cache_round<T>(kn.z), cache_round<T>(kn.w));
+        vn = make_float4(cache_round<T>(vn.x), cache_round<T>(vn.y), cache_round<T>(vn.z), cache_round<T>(vn.w));
+#pragma unroll
+        for (int i = 0; i < NL; i++) {
+            if (p0 + wave * PW + i * 2 + hf == slot) {
+                kv[i] = kn;
+                vv[i] = vn;
+            }
+        }
+    }
+    const float d_scale = 1.0f / sqrtf((float)S);
+#pragma unroll
+    for (int i = 0; i < NL; i++) {
+        float s = qv.x * kv[i].x;
+        s = fmaf(qv.y, kv[i].y, s);
+        s = fmaf(qv.z, kv[i].z, s);
+        s = fmaf(qv.w, kv[i].w, s);
+#pragma unroll
+        for (int o = 16; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
+        const int r = wave * PW + i * 2 + hf;
+        if (e == 0) sc[r] = (p0 + r < kvLen) ? s * d_scale : -FLT_MAX;
+    }
+    __syncthreads();
+    if (wave == 0) {
+        const float x = lane < C ? sc[lane] : -FLT_MAX;
+        const float mx = wave_max(x);
+        const float ex = (lane < C && x != -FLT_MAX) ? expf(x - mx) : 0.0f;
+        if (lane < C) sc[lane] = ex;
+        const float sum = wave_sum(ex);
+        if (lane == 0) {
+            stat[0] = mx;
+            stat[1] = sum;
+        }
+    }
+    __syncthreads();
+    float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+    for (int i = 0; i < NL; i++) {
+        const float w = sc[wave * PW + i * 2 + hf];
+        o.x = fmaf(w, vv[i].x, o.x);
+        o.y = fmaf(w, vv[i].y, o.y);
+        o.z = fmaf(w, vv[i].z, o.z);
+        o.w = fmaf(w, vv[i].w, o.w);
+    }
+    *reinterpret_cast<float4*>(&osh[wave][hf][e * 4]) = o;
+    __syncthreads();
+    float* rec0 = part + bh * nchunks * (S + 2);
+    float* rec = rec0 + (int64_t)chunk * (S + 2);
+    if (threadIdx.x < S) {
+        float a = 0.0f;
+#pragma unroll
+        for (int w = 0; w < 4; w++) a += osh[w][0][threadIdx.x] + osh[w][1][threadIdx.x];
+        __hip_atomic_store(&rec[2 + threadIdx.x], a, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    if (threadIdx.x == 0) {
+        __hip_atomic_store(&rec[0], stat[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(&rec[1], stat[1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the write-through stores above have been acknowledged
+    __syncthreads();
+    if (threadIdx.x == 0)
+        ticket_sh = __hip_atomic_fetch_add(&counters[bh], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    if (ticket_sh != (unsigned)(nchunks - 1)) return;
+    const float r = merge_chunks(rec0, nchunks, threadIdx.x, 256, stat_sh, [](const float* p) {
+        return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    });
+    if (threadIdx.x < S) q[bh * S + threadIdx.x] = r;
+    if (threadIdx.x == 0) __hip_atomic_store(&counters[bh], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // next launch
 }
 
 // ---- softmax op (ops/op_misc.hpp:183-194): one workgroup per row ------------------------------
@@ -275,7 +467,8 @@ extern "C" size_t llmops_attention_workspace_bytes(int64_t B, int64_t qL, int64_
     const int64_t bhq = B * H * qL;
     int64_t records = bhq * ((maxlen + 63) / 64);
     if (records < 2048) records = 2048;
-    return align_up((size_t)maxlen * sizeof(int32_t), 256) + (size_t)records * (S + 2) * sizeof(float);
+    return LLMOPS_ATTN_COUNTER_BYTES + align_up((size_t)maxlen * sizeof(int32_t), 256) +
+           (size_t)records * (S + 2) * sizeof(float);
 }
 
 template <typename T>
@@ -284,8 +477,31 @@ static int attention_impl(float* q, float* k, const float* v, int64_t B, int64_t
                           int position_id, int layer_id, void* workspace, hipStream_t st) {
     T* kc = cache + (int64_t)(2 * layer_id + 0) * B * H * maxlen * S;
     T* vc = cache + (int64_t)(2 * layer_id + 1) * B * H * maxlen * S;
-    int32_t* row_token = reinterpret_cast<int32_t*>(workspace);
-    float* part = reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(workspace) + align_up((size_t)maxlen * 4, 256));
+    uint8_t* wsb = reinterpret_cast<uint8_t*>(workspace);
+    unsigned* counters = reinterpret_cast<unsigned*>(wsb);
+    int32_t* row_token = reinterpret_cast<int32_t*>(wsb + LLMOPS_ATTN_COUNTER_BYTES);
+    float* part = reinterpret_cast<float*>(wsb + LLMOPS_ATTN_COUNTER_BYTES + align_up((size_t)maxlen * 4, 256));
+    int64_t kvLen = (int64_t)position_id + qL;
+    if (kvLen > maxlen) kvLen = maxlen;
+    const int64_t bhq = B * H * qL;
+    const int pw = pick_pw(bhq, kvLen);
+    const int nchunks = (int)((kvLen + 4 * pw - 1) / (4 * pw));
+    const unsigned grid = (unsigned)(bhq * nchunks);
+    if (qL == 1 && (half % 4) == 0 && nchunks <= kMaxChunks && B * H <= LLMOPS_ATTN_COUNTER_BYTES / 4) {
+        // decode: one launch
+        if (pw == 16)
+            attn_decode_kernel<T, 16><<<grid, 256, 0, st>>>(q, k, v, inv_freq, (int)half, kc, vc, H, maxlen, kvLen, slots,
+                                                          position_id, part, counters, nchunks);
+        else if (pw == 8)
+            attn_decode_kernel<T, 8><<<grid, 256, 0, st>>>(q, k, v, inv_freq, (int)half, kc, vc, H, maxlen, kvLen, slots,
+                                                         position_id, part, counters, nchunks);
+        else
+            attn_decode_kernel<T, 4><<<grid, 256, 0, st>>>(q, k, v, inv_freq, (int)half, kc, vc, H, maxlen, kvLen, slots,
+                                                         position_id, part, counters, nchunks);
+        LLMOPS_LAUNCH_CHECK();
+        return LLMOPS_OK;
+    }
+    LLMOPS_REQUIRE(nchunks <= kMaxChunks);
     if (qL > 1) {
         fill_i32_kernel<<<(unsigned)((maxlen + 255) / 256), 256, 0, st>>>(row_token, maxlen, -1);
         LLMOPS_LAUNCH_CHECK();
@@ -293,12 +509,6 @@ static int attention_impl(float* q, float* k, const float* v, int64_t B, int64_t
     attn_prep_kernel<T><<<(unsigned)(B * qL * H), 64, 0, st>>>(q, k, v, qL, H, S, inv_freq, half, kc, vc, maxlen, slots,
                                                               position_id, row_token);
     LLMOPS_LAUNCH_CHECK();
-    int64_t kvLen = (int64_t)position_id + qL;
-    if (kvLen > maxlen) kvLen = maxlen;
-    const int64_t bhq = B * H * qL;
-    const int pw = pick_pw(bhq, kvLen);
-    const int nchunks = (int)((kvLen + 4 * pw - 1) / (4 * pw));
-    const unsigned grid = (unsigned)(bhq * nchunks);
     if (pw == 16)
         attn_split_kernel<T, 16><<<grid, 256, 0, st>>>(q, kc, vc, qL, H, maxlen, kvLen, row_token, part, nchunks);
     else if (pw == 8)

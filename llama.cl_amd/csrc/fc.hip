@@ -10,7 +10,9 @@ int launch_quant_x(const float* x, int64_t rows, int64_t K, int group_k, int8_t*
                    hipStream_t stream);
 size_t gemv_workspace_bytes(int64_t rows, int64_t Ng, int64_t Kg, int G);
 int launch_gemv(const uint8_t* w, const float* x, const int8_t* xq, const float* xd, const float* gs, float* y,
-                float* part, unsigned* counters, int64_t rows, int64_t Ng, int64_t Kg, int G, int64_t N, hipStream_t st);
+                float* part, unsigned* counters, int64_t rows, int64_t Ng, int64_t Kg, int G, int64_t N,
+                const float* residual, hipStream_t st);
+int launch_add(float* a, const float* b, int64_t total, hipStream_t st);
 int launch_gemv_partials(const uint8_t* w, const int8_t* xq, int32_t* acc, int64_t rows, int64_t Ng, int64_t Kg, int G,
                          hipStream_t st);
 size_t gemm_workspace_bytes(int64_t rows, int64_t Ng, int64_t Kg);
@@ -50,9 +52,9 @@ extern "C" size_t llmops_fc_Q4A_workspace_bytes(int64_t rows, int64_t K, int64_t
     return fc_layout(rows, Ng, Kg, group_k).total;
 }
 
-extern "C" int llmops_fc_Q4A(const float* x, int64_t rows, int64_t K, const int8_t* weiq, int64_t Ng, int64_t Kg,
-                             int group_k, int64_t N, float* y, void* workspace, size_t workspace_bytes,
-                             llmops_stream_t stream) {
+static int fc_impl(const float* x, int64_t rows, int64_t K, const int8_t* weiq, int64_t Ng, int64_t Kg, int group_k,
+                   int64_t N, const float* residual, float* y, void* workspace, size_t workspace_bytes,
+                   llmops_stream_t stream) {
     LLMOPS_REQUIRE(valid_group(group_k));
     LLMOPS_REQUIRE(x != nullptr && weiq != nullptr && y != nullptr && workspace != nullptr);
     LLMOPS_REQUIRE(rows > 0 && K > 0 && Ng > 0 && Kg > 0);
@@ -74,10 +76,25 @@ extern "C" int llmops_fc_Q4A(const float* x, int64_t rows, int64_t K, const int8
     const uint8_t* w = reinterpret_cast<const uint8_t*>(weiq);
     // few rows: one launch, the streaming kernel quantizes the activations it needs on the fly
     if (rows <= kMaxGemvRows)
-        return launch_gemv(w, x, nullptr, nullptr, nullptr, y, part, counters, rows, Ng, Kg, group_k, N, st);
+        return launch_gemv(w, x, nullptr, nullptr, nullptr, y, part, counters, rows, Ng, Kg, group_k, N, residual, st);
     int rc = launch_quant_x(x, rows, K, group_k, xq, xd, gs, st);
     if (rc) return rc;
-    return launch_gemm(w, xq, xd, gs, y, part, rows, Ng, Kg, group_k, N, st);
+    rc = launch_gemm(w, xq, xd, gs, y, part, rows, Ng, Kg, group_k, N, st);
+    if (rc || residual == nullptr) return rc;
+    return launch_add(y, residual, rows * N, st);
+}
+
+extern "C" int llmops_fc_Q4A(const float* x, int64_t rows, int64_t K, const int8_t* weiq, int64_t Ng, int64_t Kg,
+                             int group_k, int64_t N, float* y, void* workspace, size_t workspace_bytes,
+                             llmops_stream_t stream) {
+    return fc_impl(x, rows, K, weiq, Ng, Kg, group_k, N, nullptr, y, workspace, workspace_bytes, stream);
+}
+
+extern "C" int llmops_fc_Q4A_residual(const float* x, int64_t rows, int64_t K, const int8_t* weiq, int64_t Ng,
+                                      int64_t Kg, int group_k, int64_t N, const float* residual, float* y,
+                                      void* workspace, size_t workspace_bytes, llmops_stream_t stream) {
+    LLMOPS_REQUIRE(residual != nullptr);
+    return fc_impl(x, rows, K, weiq, Ng, Kg, group_k, N, residual, y, workspace, workspace_bytes, stream);
 }
 
 extern "C" int llmops_fc_Q4A_prequantized(const int8_t* xq, const float* xd, const float* gsum, int64_t rows,
@@ -98,7 +115,8 @@ extern "C" int llmops_fc_Q4A_prequantized(const int8_t* xq, const float* xd, con
     const uint8_t* w = reinterpret_cast<const uint8_t*>(weiq);
     hipStream_t st = as_stream(stream);
     if (rows <= kMaxGemvRows)
-        return launch_gemv(w, nullptr, xq, xd, gsum, y, part, reinterpret_cast<unsigned*>(ws), rows, Ng, Kg, group_k, N, st);
+        return launch_gemv(w, nullptr, xq, xd, gsum, y, part, reinterpret_cast<unsigned*>(ws), rows, Ng, Kg, group_k, N,
+                           nullptr, st);
     return launch_gemm(w, xq, xd, gsum, y, part, rows, Ng, Kg, group_k, N, st);
 }
 

@@ -161,7 +161,7 @@ __device__ __forceinline__ TileRange tile_range(int Kg, int S, int steps_per_spl
 template <int MT, int NW>
 __device__ __forceinline__ void finish_strip(float f[MT][4], float (*red)[MT][kGroupN], unsigned* ticket_sh, int nb, int s,
                                              int S, int rows, int64_t N, float* __restrict__ y, float* part,
-                                             unsigned* counters) {
+                                             unsigned* counters, const float* __restrict__ residual) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int quad = lane & 7, rs = lane >> 3;
     // sum the 8 row slots (lane bits 3..5)
@@ -194,7 +194,7 @@ __device__ __forceinline__ void finish_strip(float f[MT][4], float (*red)[MT][kG
         for (int w = 0; w < NW; w++) v += red[w][tr][tn];
     }
     if (S == 1) {
-        if (n < N) y[(int64_t)tr * N + n] = v;
+        if (n < N) y[(int64_t)tr * N + n] = residual ? v + residual[(int64_t)tr * N + n] : v;
         return;
     }
     // Cross-workgroup hand-off without cache-wide fences: partial sums are written and read with
@@ -214,7 +214,7 @@ __device__ __forceinline__ void finish_strip(float f[MT][4], float (*red)[MT][kG
         float acc = 0.0f;
         for (int i = 0; i < S; i++)
             acc += __hip_atomic_load(&part[((int64_t)i * rows + tr) * Np + n], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        y[(int64_t)tr * N + n] = acc;
+        y[(int64_t)tr * N + n] = residual ? acc + residual[(int64_t)tr * N + n] : acc;
     }
     if (threadIdx.x == 0) __hip_atomic_store(&counters[nb], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // next launch
 }
@@ -224,7 +224,8 @@ template <int G, int MT, int NW>
 __global__ __launch_bounds__(NW * 64) void fc_gemv_kernel(const uint8_t* __restrict__ weiq, const int8_t* __restrict__ xq,
                                                            const float* __restrict__ xd, const float* __restrict__ gs,
                                                            float* __restrict__ y, float* part, unsigned* counters, int Kg,
-                                                           int64_t N, int rows, int S, int steps_per_split) {
+                                                           int64_t N, int rows, int S, int steps_per_split,
+                                                           const float* __restrict__ residual) {
     __shared__ float red[NW][MT][kGroupN];
     __shared__ unsigned ticket_sh;
     const int lane = threadIdx.x & 63;
@@ -260,7 +261,7 @@ __global__ __launch_bounds__(NW * 64) void fc_gemv_kernel(const uint8_t* __restr
         }
         cur = nxt;
     }
-    finish_strip<MT, NW>(f, red, &ticket_sh, tr.nb, tr.s, S, rows, N, y, part, counters);
+    finish_strip<MT, NW>(f, red, &ticket_sh, tr.nb, tr.s, S, rows, N, y, part, counters, residual);
 }
 
 // ---- variant 2: raw fp32 activations, quantized by the wavefront that consumes them -----------
@@ -330,7 +331,7 @@ template <int G, int MT, int NW, int D>
 __global__ __launch_bounds__(NW * 64) void fc_gemv_fused_kernel(const uint8_t* __restrict__ weiq, const float* __restrict__ x,
                                                                  float* __restrict__ y, float* part, unsigned* counters,
                                                                  int Kg, int64_t K, int64_t N, int rows, int S,
-                                                                 int steps_per_split) {
+                                                                 int steps_per_split, const float* __restrict__ residual) {
     __shared__ float red[NW][MT][kGroupN];
     __shared__ __align__(16) XSlot<G> xs[NW][MT];
     __shared__ unsigned ticket_sh;
@@ -391,7 +392,7 @@ __global__ __launch_bounds__(NW * 64) void fc_gemv_fused_kernel(const uint8_t* _
             }
         }
     }
-    finish_strip<MT, NW>(f, red, &ticket_sh, tr.nb, tr.s, S, rows, N, y, part, counters);
+    finish_strip<MT, NW>(f, red, &ticket_sh, tr.nb, tr.s, S, rows, N, y, part, counters, residual);
 }
 
 // Integer core only: acc[r][n][kb] (int32).  One wavefront per step, same loads and same dot
@@ -466,16 +467,16 @@ size_t gemv_workspace_bytes(int64_t rows, int64_t Ng, int64_t Kg, int G) {
 template <int G, int MT, int NW>
 static void launch_gemv_t(const uint8_t* w, const float* x, const int8_t* xq, const float* xd, const float* gs, float* y,
                           float* part, unsigned* counters, int64_t Ng, int64_t Kg, int64_t N, int rows, GemvPlan p,
-                          hipStream_t st) {
+                          const float* residual, hipStream_t st) {
     const unsigned grid = (unsigned)(Ng * p.S);
     if (x == nullptr) {
         fc_gemv_kernel<G, MT, NW><<<grid, NW * 64, 0, st>>>(w, xq, xd, gs, y, part, counters, (int)Kg, N, rows, p.S,
-                                                            p.steps_per_split);
+                                                            p.steps_per_split, residual);
         return;
     }
 #define LLMOPS_FUSED(DD)                                                                                             \
     fc_gemv_fused_kernel<G, MT, NW, DD><<<grid, NW * 64, 0, st>>>(w, x, y, part, counters, (int)Kg, Kg * G, N, rows, p.S, \
-                                                                  p.steps_per_split)
+                                                                  p.steps_per_split, residual)
     if (MT == 1 && g_prefetch_depth >= 3) LLMOPS_FUSED((MT == 1 ? 3 : 1));
     else if (MT == 1 && g_prefetch_depth == 2) LLMOPS_FUSED((MT == 1 ? 2 : 1));
     else LLMOPS_FUSED(1);
@@ -485,20 +486,22 @@ static void launch_gemv_t(const uint8_t* w, const float* x, const int8_t* xq, co
 template <int G, int MT>
 static void launch_gemv_nw(const uint8_t* w, const float* x, const int8_t* xq, const float* xd, const float* gs, float* y,
                            float* part, unsigned* counters, int64_t Ng, int64_t Kg, int64_t N, int rows, GemvPlan p,
-                           hipStream_t st) {
+                           const float* residual, hipStream_t st) {
     if (p.NW >= 16 && MT <= 4)
-        launch_gemv_t<G, MT, (MT <= 4 ? 16 : 8)>(w, x, xq, xd, gs, y, part, counters, Ng, Kg, N, rows, p, st);
+        launch_gemv_t<G, MT, (MT <= 4 ? 16 : 8)>(w, x, xq, xd, gs, y, part, counters, Ng, Kg, N, rows, p, residual, st);
     else if (p.NW >= 8)
-        launch_gemv_t<G, MT, 8>(w, x, xq, xd, gs, y, part, counters, Ng, Kg, N, rows, p, st);
+        launch_gemv_t<G, MT, 8>(w, x, xq, xd, gs, y, part, counters, Ng, Kg, N, rows, p, residual, st);
     else
-        launch_gemv_t<G, MT, 4>(w, x, xq, xd, gs, y, part, counters, Ng, Kg, N, rows, p, st);
+        launch_gemv_t<G, MT, 4>(w, x, xq, xd, gs, y, part, counters, Ng, Kg, N, rows, p, residual, st);
 }
 
 // x != nullptr: raw fp32 activations, quantized inside the kernel; else xq/xd/gs are used.
 int launch_gemv(const uint8_t* w, const float* x, const int8_t* xq, const float* xd, const float* gs, float* y,
-                float* part, unsigned* counters, int64_t rows, int64_t Ng, int64_t Kg, int G, int64_t N, hipStream_t st) {
+                float* part, unsigned* counters, int64_t rows, int64_t Ng, int64_t Kg, int G, int64_t N,
+                const float* residual, hipStream_t st) {
     const GemvPlan p = plan_gemv(rows, Ng, Kg, G);
-#define LLMOPS_GEMV_CASE(GG, MT) launch_gemv_nw<GG, MT>(w, x, xq, xd, gs, y, part, counters, Ng, Kg, N, (int)rows, p, st)
+#define LLMOPS_GEMV_CASE(GG, MT) \
+    launch_gemv_nw<GG, MT>(w, x, xq, xd, gs, y, part, counters, Ng, Kg, N, (int)rows, p, residual, st)
     if (G == 128) {
         if (rows == 1) LLMOPS_GEMV_CASE(128, 1);
         else if (rows == 2) LLMOPS_GEMV_CASE(128, 2);

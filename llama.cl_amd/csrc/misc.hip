@@ -5,11 +5,50 @@
 
 namespace llmops {
 
-// rmsnorm (ops/op_misc.hpp:142-181): one workgroup per row
-__global__ __launch_bounds__(256) void rmsnorm_kernel(float* __restrict__ x, int64_t hidden, const float* __restrict__ w,
-                                                       float eps) {
+// rmsnorm (ops/op_misc.hpp:142-181): one workgroup of 1024 threads per row; the row is read once
+// with 16-byte loads and kept in registers (hidden <= 4*1024*VPT), `out` may alias `x`
+template <int VPT>
+__global__ __launch_bounds__(1024) void rmsnorm_kernel(const float* __restrict__ x, float* out, int64_t hidden,
+                                                        const float* __restrict__ w, float eps) {
+    __shared__ float red[16];
+    const float* row = x + (int64_t)blockIdx.x * hidden;
+    float* orow = out + (int64_t)blockIdx.x * hidden;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    float4 v[VPT];
+    float ss = 0.0f;
+#pragma unroll
+    for (int i = 0; i < VPT; i++) {
+        const int64_t e = ((int64_t)i * 1024 + threadIdx.x) * 4;
+        v[i] = e < hidden ? *reinterpret_cast<const float4*>(row + e) : make_float4(0.f, 0.f, 0.f, 0.f);
+        ss = fmaf(v[i].x, v[i].x, ss);
+        ss = fmaf(v[i].y, v[i].y, ss);
+        ss = fmaf(v[i].z, v[i].z, ss);
+        ss = fmaf(v[i].w, v[i].w, ss);
+    }
+    ss = wave_sum(ss);
+    if (lane == 0) red[wave] = ss;
+    __syncthreads();
+    float tot = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 16; i++) tot += red[i];
+    const float rs = 1.0f / sqrtf(tot / (float)hidden + eps);
+#pragma unroll
+    for (int i = 0; i < VPT; i++) {
+        const int64_t e = ((int64_t)i * 1024 + threadIdx.x) * 4;
+        if (e < hidden) {
+            const float4 ww = *reinterpret_cast<const float4*>(w + e);
+            *reinterpret_cast<float4*>(orow + e) =
+                make_float4(v[i].x * rs * ww.x, v[i].y * rs * ww.y, v[i].z * rs * ww.z, v[i].w * rs * ww.w);
+        }
+    }
+}
+
+// general fallback (any hidden size, any alignment)
+__global__ __launch_bounds__(256) void rmsnorm_generic_kernel(const float* __restrict__ x, float* out, int64_t hidden,
+                                                               const float* __restrict__ w, float eps) {
     __shared__ float red[4];
-    float* row = x + (int64_t)blockIdx.x * hidden;
+    const float* row = x + (int64_t)blockIdx.x * hidden;
+    float* orow = out + (int64_t)blockIdx.x * hidden;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     float ss = 0.0f;
     for (int64_t i = threadIdx.x; i < hidden; i += 256) ss = fmaf(row[i], row[i], ss);
@@ -18,7 +57,18 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(float* __restrict__ x, int
     __syncthreads();
     const float rms = (((red[0] + red[1]) + red[2]) + red[3]) / (float)hidden;
     const float rs = 1.0f / sqrtf(rms + eps);
-    for (int64_t i = threadIdx.x; i < hidden; i += 256) row[i] = row[i] * rs * w[i];
+    __syncthreads();
+    for (int64_t i = threadIdx.x; i < hidden; i += 256) orow[i] = row[i] * rs * w[i];
+}
+
+// out[r, i] = silu(gu[r, i]) * gu[r, F + i]   (itrans "silu" followed by imul, ops/op_misc.hpp:83-138,
+// on a row that holds the gate and the up projection side by side)
+__global__ void silu_mul_kernel(const float* __restrict__ gu, float* __restrict__ out, int64_t rows, int64_t F) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= rows * F) return;
+    const int64_t r = i / F, c = i % F;
+    const float g = gu[r * 2 * F + c], u = gu[r * 2 * F + F + c];
+    out[i] = u * (g * (1.0f / (1.0f + expf(-g))));
 }
 
 template <bool MUL>
@@ -80,12 +130,48 @@ __global__ void emb_kernel(float* __restrict__ out, const int64_t* __restrict__ 
 
 using namespace llmops;
 
-extern "C" int llmops_rmsnorm(float* x, int64_t rows, int64_t hidden, const float* w, float eps, llmops_stream_t stream) {
-    LLMOPS_REQUIRE(x != nullptr && w != nullptr && rows > 0 && hidden > 0 && rows < ((int64_t)1 << 31));
-    rmsnorm_kernel<<<(unsigned)rows, 256, 0, as_stream(stream)>>>(x, hidden, w, eps);
+static int rmsnorm_launch(const float* x, float* out, int64_t rows, int64_t hidden, const float* w, float eps,
+                          llmops_stream_t stream) {
+    LLMOPS_REQUIRE(x != nullptr && out != nullptr && w != nullptr && rows > 0 && hidden > 0 && rows < ((int64_t)1 << 31));
+    hipStream_t st = as_stream(stream);
+    const bool vec = (hidden % 4) == 0 && aligned(x, 16) && aligned(out, 16) && aligned(w, 16);
+    if (vec && hidden <= 4096)
+        rmsnorm_kernel<1><<<(unsigned)rows, 1024, 0, st>>>(x, out, hidden, w, eps);
+    else if (vec && hidden <= 8192)
+        rmsnorm_kernel<2><<<(unsigned)rows, 1024, 0, st>>>(x, out, hidden, w, eps);
+    else if (vec && hidden <= 16384)
+        rmsnorm_kernel<4><<<(unsigned)rows, 1024, 0, st>>>(x, out, hidden, w, eps);
+    else
+        rmsnorm_generic_kernel<<<(unsigned)rows, 256, 0, st>>>(x, out, hidden, w, eps);
     LLMOPS_LAUNCH_CHECK();
     return LLMOPS_OK;
 }
+
+extern "C" int llmops_rmsnorm(float* x, int64_t rows, int64_t hidden, const float* w, float eps, llmops_stream_t stream) {
+    return rmsnorm_launch(x, x, rows, hidden, w, eps, stream);
+}
+
+extern "C" int llmops_rmsnorm_out(const float* x, float* out, int64_t rows, int64_t hidden, const float* w, float eps,
+                                  llmops_stream_t stream) {
+    return rmsnorm_launch(x, out, rows, hidden, w, eps, stream);
+}
+
+extern "C" int llmops_silu_mul(const float* gate_up, float* out, int64_t rows, int64_t F, llmops_stream_t stream) {
+    LLMOPS_REQUIRE(gate_up != nullptr && out != nullptr && rows > 0 && F > 0);
+    const int64_t total = rows * F;
+    LLMOPS_REQUIRE((total + 255) / 256 < ((int64_t)1 << 31));
+    silu_mul_kernel<<<(unsigned)((total + 255) / 256), 256, 0, as_stream(stream)>>>(gate_up, out, rows, F);
+    LLMOPS_LAUNCH_CHECK();
+    return LLMOPS_OK;
+}
+
+namespace llmops {
+int launch_add(float* a, const float* b, int64_t total, hipStream_t st) {
+    ibinary_kernel<false><<<(unsigned)((total + 255) / 256), 256, 0, st>>>(a, b, total, total, 0);
+    LLMOPS_LAUNCH_CHECK();
+    return LLMOPS_OK;
+}
+}  // namespace llmops
 
 static int ibinary(bool mul, float* a, const float* b, int64_t rows, int64_t inner, int b_is_row, llmops_stream_t stream) {
     LLMOPS_REQUIRE(a != nullptr && b != nullptr && rows > 0 && inner > 0);

@@ -23,7 +23,7 @@ from . import _lib
 __all__ = [
     "offline_FC_quant_Q4A", "offline_FC_dequant_Q4A", "fc_Q4A", "FC_dynamic_quantize_x", "fc_Q4A_partials",
     "attention_rope", "attention_rope2", "rope_embed", "softmax", "rmsnorm", "iadd", "imul", "itrans", "clone",
-    "empty", "ones", "embedding", "embedding_q8c_quant_w", "embedding_q8c", "tensor_pool", "set_default_group_k",
+    "rmsnorm_out", "silu_mul", "empty", "ones", "embedding", "embedding_q8c_quant_w", "embedding_q8c", "tensor_pool", "set_default_group_k",
     "group_k_of",
 ]
 
@@ -59,10 +59,10 @@ def _dev(t, dtype, rank=None, name="tensor"):
     _require(t.is_contiguous(), f"{name}.is_dense()")
 
 
-def _workspace(device, nbytes):
-    """Persistent per-device scratch.  Its first bytes hold the split-K arrival counters, which
-    must start at zero and which the kernels leave at zero."""
-    key = (device.type, device.index if device.index is not None else torch.cuda.current_device())
+def _workspace(device, nbytes, kind="fc"):
+    """Persistent per-device scratch, one per op family.  Its first bytes hold arrival counters,
+    which must start at zero and which the kernels leave at zero."""
+    key = (kind, device.type, device.index if device.index is not None else torch.cuda.current_device())
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
         size = max(int(nbytes), 16 << 20)
@@ -120,8 +120,9 @@ def FC_dynamic_quantize_x(input, group_k):
     return xq, xd, gs
 
 
-def fc_Q4A(input, weiq, N):
-    """fp32 [B,M,K] x packed [Ng,Kg,blk] -> fp32 [B,M,N] (ops/op_fc.hpp:286-426)."""
+def fc_Q4A(input, weiq, N, residual=None):
+    """fp32 [B,M,K] x packed [Ng,Kg,blk] -> fp32 [B,M,N] (ops/op_fc.hpp:286-426).
+    ``residual`` (extension, fp32 [B,M,N]): returns fc_Q4A(input) + residual in the same launch."""
     _dev(input, torch.float32, 3, "input")
     _dev(weiq, torch.int8, 3, "wei_quantized")
     g = group_k_of(weiq)
@@ -132,8 +133,14 @@ def fc_Q4A(input, weiq, N):
     need = lib.llmops_fc_Q4A_workspace_bytes(rows, K, Ng, Kg, g)
     ws = _workspace(input.device, need)
     out = torch.empty((B, M, int(N)), dtype=torch.float32, device=input.device)
-    _lib.check(lib.llmops_fc_Q4A(_ptr(input), rows, K, _ptr(weiq), Ng, Kg, g, int(N), _ptr(out), _ptr(ws), ws.numel(),
-                                 _stream(input)))
+    if residual is None:
+        _lib.check(lib.llmops_fc_Q4A(_ptr(input), rows, K, _ptr(weiq), Ng, Kg, g, int(N), _ptr(out), _ptr(ws), ws.numel(),
+                                     _stream(input)))
+    else:
+        _dev(residual, torch.float32, 3, "residual")
+        _require(tuple(residual.shape) == (B, M, int(N)), "residual.is({B, M, N})")
+        _lib.check(lib.llmops_fc_Q4A_residual(_ptr(input), rows, K, _ptr(weiq), Ng, Kg, g, int(N), _ptr(residual), _ptr(out),
+                                              _ptr(ws), ws.numel(), _stream(input)))
     return out
 
 
@@ -181,20 +188,15 @@ def attention_rope2(q, k, v, inv_freq, kv_cache, kvc_slots, position_id, layer_i
     _require(tuple(kvc_slots.shape) == (qL,), "kvc_slots.is({qL})")
     lib = _lib.load()
     need = lib.llmops_attention_workspace_bytes(B, qL, H, S, maxlen)
-    ws = _workspace(q.device, _lib_fc_counter_bytes() + need)
-    wptr = ctypes.c_void_p(ws.data_ptr() + _lib_fc_counter_bytes())
+    ws = _workspace(q.device, need, kind="attn")
     dt = 0 if kv_cache.dtype == torch.float32 else 1
     _lib.check(lib.llmops_attention_rope(_ptr(q), _ptr(k), _ptr(v), B, qL, H, S, _ptr(inv_freq), inv_freq.shape[0],
                                          _ptr(kv_cache), dt, planes, maxlen, _ptr(kvc_slots), int(position_id),
-                                         int(layer_id), wptr, ws.numel() - _lib_fc_counter_bytes(), _stream(q)))
+                                         int(layer_id), _ptr(ws), ws.numel(), _stream(q)))
 
 
 # the reference exports two kernels with one contract (ops/main.cpp:154-155)
 attention_rope = attention_rope2
-
-
-def _lib_fc_counter_bytes():
-    return 65536  # LLMOPS_FC_COUNTER_BYTES: keep other ops off the FC arrival counters
 
 
 def softmax(x):
@@ -212,6 +214,28 @@ def rmsnorm(input, weight, variance_epsilon):
     _require(input.shape[-1] == hidden, "input.size(-1) == hidden_states")
     _lib.check(_lib.load().llmops_rmsnorm(_ptr(input), input.numel() // hidden, hidden, _ptr(weight),
                                          float(variance_epsilon), _stream(input)))
+
+
+def rmsnorm_out(input, weight, variance_epsilon):
+    """Extension: clone + rmsnorm in one launch; returns the normalised copy, ``input`` is untouched."""
+    _dev(input, torch.float32, 3, "input")
+    _dev(weight, torch.float32, 1, "weight")
+    hidden = weight.shape[0]
+    _require(input.shape[-1] == hidden, "input.size(-1) == hidden_states")
+    out = torch.empty_like(input)
+    _lib.check(_lib.load().llmops_rmsnorm_out(_ptr(input), _ptr(out), input.numel() // hidden, hidden, _ptr(weight),
+                                             float(variance_epsilon), _stream(input)))
+    return out
+
+
+def silu_mul(gate_up):
+    """Extension: itrans(gate, "silu") + imul(up, gate) on fp32 [..., 2F] holding gate|up side by side -> [..., F]."""
+    _dev(gate_up, torch.float32, None, "gate_up")
+    _require(gate_up.shape[-1] % 2 == 0, "gate_up.size(-1) % 2 == 0")
+    F = gate_up.shape[-1] // 2
+    out = torch.empty(tuple(gate_up.shape[:-1]) + (F,), dtype=torch.float32, device=gate_up.device)
+    _lib.check(_lib.load().llmops_silu_mul(_ptr(gate_up), _ptr(out), gate_up.numel() // (2 * F), F, _stream(gate_up)))
+    return out
 
 
 def _ibinary(fn, a, b):

@@ -21,6 +21,8 @@ SIGNATURES = {
     "llmops_FC_dynamic_quantize_x": (c_int, [c_ptr, c_i64, c_i64, c_int, c_ptr, c_ptr, c_ptr, c_ptr]),
     "llmops_fc_Q4A_workspace_bytes": (c_size, [c_i64, c_i64, c_i64, c_i64, c_int]),
     "llmops_fc_Q4A": (c_int, [c_ptr, c_i64, c_i64, c_ptr, c_i64, c_i64, c_int, c_i64, c_ptr, c_ptr, c_size, c_ptr]),
+    "llmops_fc_Q4A_residual": (c_int, [c_ptr, c_i64, c_i64, c_ptr, c_i64, c_i64, c_int, c_i64, c_ptr, c_ptr, c_ptr, c_size,
+                                       c_ptr]),
     "llmops_fc_Q4A_prequantized": (c_int, [c_ptr, c_ptr, c_ptr, c_i64, c_ptr, c_i64, c_i64, c_int, c_i64, c_ptr, c_ptr,
                                            c_size, c_ptr]),
     "llmops_fc_Q4A_partials": (c_int, [c_ptr, c_i64, c_ptr, c_i64, c_i64, c_int, c_ptr, c_int, c_ptr]),
@@ -30,6 +32,8 @@ SIGNATURES = {
                                       c_i64, c_i64, c_ptr, c_int, c_int, c_ptr, c_size, c_ptr]),
     "llmops_softmax": (c_int, [c_ptr, c_i64, c_i64, c_ptr]),
     "llmops_rmsnorm": (c_int, [c_ptr, c_i64, c_i64, c_ptr, c_f32, c_ptr]),
+    "llmops_rmsnorm_out": (c_int, [c_ptr, c_ptr, c_i64, c_i64, c_ptr, c_f32, c_ptr]),
+    "llmops_silu_mul": (c_int, [c_ptr, c_ptr, c_i64, c_i64, c_ptr]),
     "llmops_iadd": (c_int, [c_ptr, c_ptr, c_i64, c_i64, c_int, c_ptr]),
     "llmops_imul": (c_int, [c_ptr, c_ptr, c_i64, c_i64, c_int, c_ptr]),
     "llmops_itrans_silu": (c_int, [c_ptr, c_i64, c_ptr]),

@@ -7,7 +7,8 @@ This is the caller of the hot path, kept as thin as the reference's: every arith
 * ``plan="reference"``: the reference's sequence verbatim -- clone, rmsnorm, q/k/v projections as three
   FCs, attention_rope2, o projection, iadd, clone, rmsnorm, gate, silu, up, imul, down, iadd.
 * ``plan="fused"`` (default): the same arithmetic with fewer launches -- q|k|v and gate|up packed
-  tensors concatenated along N so each pair/triple is one FC launch.
+  tensors concatenated along N so each pair/triple is one FC launch, clone+rmsnorm and silu+mul as
+  one op each, residual adds folded into the o and down projections.
 
 A decode step (one token, batch 1) has fixed shapes and no host-side decisions, so it can be
 captured once as a HIP graph and replayed (``capture_decode``).
@@ -77,37 +78,46 @@ class LlamaDecoder:
         H = self.configs["hidden_size"]
         F = self.configs["intermediate_size"]
         hidden_states = self.embed_tokens(input_ids)
+        step = self._layer_fused if self.plan == "fused" else self._layer_reference
         for i, ops in enumerate(self.layers):
-            input_layernorm = llmops.clone(hidden_states)
-            ops["input_layernorm"](input_layernorm)
-            if self.plan == "fused":
-                qkv = ops["qkv_proj"](input_layernorm)
-                q, k, v = qkv[..., :H], qkv[..., H:2 * H], qkv[..., 2 * H:]
-                if not q.is_contiguous():  # more than one token: the op needs dense [B,qL,H*S] tensors
-                    q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
-            else:
-                q = ops["q_proj"](input_layernorm)
-                k = ops["k_proj"](input_layernorm)
-                v = ops["v_proj"](input_layernorm)
-            llmops.attention_rope2(q, k, v, self.inv_freq, kv_cache, kv_cache_slots, position_id, i)
-            attn_output = ops["o_proj"](q)
-            llmops.iadd(attn_output, hidden_states)
-            post_attention_layernorm = llmops.clone(attn_output)
-            ops["post_attention_layernorm"](post_attention_layernorm)
-            if self.plan == "fused":
-                gate_up = ops["gate_up_proj"](post_attention_layernorm)
-                gate, up = gate_up[..., :F], gate_up[..., F:]
-                if not gate.is_contiguous():
-                    gate, up = gate.contiguous(), up.contiguous()
-            else:
-                gate = ops["gate_proj"](post_attention_layernorm)
-                up = ops["up_proj"](post_attention_layernorm)
-            llmops.itrans(gate, "silu")
-            llmops.imul(up, gate)
-            hidden_states = ops["down_proj"](up)
-            llmops.iadd(hidden_states, attn_output)
+            hidden_states = step(i, ops, hidden_states, kv_cache, kv_cache_slots, position_id)
         self.norm(hidden_states)
         return self.lm_head(hidden_states)
+
+    def _layer_reference(self, i, ops, hidden_states, kv_cache, kv_cache_slots, position_id):
+        """chatllama/main.py:344-375 verbatim."""
+        input_layernorm = llmops.clone(hidden_states)
+        ops["input_layernorm"](input_layernorm)
+        q = ops["q_proj"](input_layernorm)
+        k = ops["k_proj"](input_layernorm)
+        v = ops["v_proj"](input_layernorm)
+        llmops.attention_rope2(q, k, v, self.inv_freq, kv_cache, kv_cache_slots, position_id, i)
+        attn_output = ops["o_proj"](q)
+        llmops.iadd(attn_output, hidden_states)
+        post_attention_layernorm = llmops.clone(attn_output)
+        ops["post_attention_layernorm"](post_attention_layernorm)
+        gate = ops["gate_proj"](post_attention_layernorm)
+        llmops.itrans(gate, "silu")
+        up = ops["up_proj"](post_attention_layernorm)
+        llmops.imul(up, gate)
+        hidden_states = ops["down_proj"](up)
+        llmops.iadd(hidden_states, attn_output)
+        return hidden_states
+
+    def _layer_fused(self, i, ops, hidden_states, kv_cache, kv_cache_slots, position_id):
+        """Same arithmetic, 10 launches instead of 18: clone+rmsnorm, q|k|v and gate|up as one FC each,
+        silu+mul as one op, the two residual adds inside the o and down projections."""
+        H = self.configs["hidden_size"]
+        x = ops["input_layernorm"].out_of_place(hidden_states)
+        qkv = ops["qkv_proj"](x)
+        q, k, v = qkv[..., :H], qkv[..., H:2 * H], qkv[..., 2 * H:]
+        if not q.is_contiguous():  # more than one token: the op needs dense [B,qL,H*S] tensors
+            q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+        llmops.attention_rope2(q, k, v, self.inv_freq, kv_cache, kv_cache_slots, position_id, i)
+        attn_output = ops["o_proj"](q, residual=hidden_states)
+        x = ops["post_attention_layernorm"].out_of_place(attn_output)
+        act = llmops.silu_mul(ops["gate_up_proj"](x))
+        return ops["down_proj"](act, residual=attn_output)
 
     def capture_decode(self, kv_cache, slot, position_id, stream=None):
         """Capture one decode step (batch 1, one token, fixed slot/position) as a HIP graph.
@@ -122,9 +132,8 @@ class LlamaDecoder:
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph, stream=stream):
                 logits = self.forward(input_ids, kv_cache, slots, position_id)
-        # the per-device workspace is captured by address too; pin the one in use
-        workspace = llmops._workspaces.get((self.device.type, self.device.index if self.device.index is not None
-                                            else torch.cuda.current_device()))
+        # the per-device workspaces are captured by address too; pin the ones in use
+        workspace = [w for key, w in llmops._workspaces.items() if key[1] == self.device.type]
         return DecodeGraph(graph, input_ids, slots, kv_cache, logits, stream, workspace)
 
 

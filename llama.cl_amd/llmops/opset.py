@@ -77,8 +77,8 @@ class llmop_fc_q4a:
             self.N = weight.shape[0]
         self.bias = bias.detach() if bias is not None else None
 
-    def __call__(self, input):
-        out = llmops.fc_Q4A(input, self.weight, self.N)
+    def __call__(self, input, residual=None):
+        out = llmops.fc_Q4A(input, self.weight, self.N, residual=residual)
         if self.bias is not None:
             llmops.iadd(out, self.bias)
         return out
@@ -102,6 +102,9 @@ class llmop_rmsnorm:
 
     def __call__(self, input):
         llmops.rmsnorm(input, self.weight, self.eps)
+
+    def out_of_place(self, input):
+        return llmops.rmsnorm_out(input, self.weight, self.eps)
 
     def __repr__(self):
         return f"llmop_rmsnorm(weight: {list(self.weight.shape)}, eps: {self.eps})"

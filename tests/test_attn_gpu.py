@@ -182,3 +182,29 @@ def test_neighbours_golden(ops):
     assert np.array_equal(host(out), g["emb"][g["ids"]])
     with pytest.raises(RuntimeError):
         ops.itrans(x, "gelu")
+
+
+def test_fused_neighbours_vs_oracle(ops, orc):
+    """Extensions used by the decode step: rmsnorm_out == clone+rmsnorm, silu_mul == silu then imul,
+    fc_Q4A(residual=) == fc_Q4A then iadd."""
+    rng = np.random.default_rng(9)
+    for rows, hidden in ((1, 4096), (5, 4096), (2, 11008), (3, 1000)):
+        x = rng.standard_normal((1, rows, hidden)).astype(np.float32)
+        w = rng.standard_normal(hidden).astype(np.float32)
+        dx = dev(x)
+        out = ops.rmsnorm_out(dx, dev(w), 1e-5)
+        assert np.array_equal(host(dx), x)
+        assert np.allclose(host(out), orc.rmsnorm(x, w, 1e-5), rtol=1e-5, atol=1e-6)
+        ops.rmsnorm(dx, dev(w), 1e-5)
+        assert np.array_equal(host(dx), host(out))
+    gu = rng.standard_normal((1, 3, 2 * 11008)).astype(np.float32)
+    want = orc.imul(gu[..., 11008:].copy(), orc.silu(gu[..., :11008].copy()))
+    assert np.allclose(host(ops.silu_mul(dev(gu))), want, rtol=1e-6, atol=1e-7)
+    for rows, N, K in ((1, 4096, 4096), (1, 4096, 11008), (3, 96, 1024), (20, 96, 1024)):
+        w = (rng.standard_normal((N, K)) * 0.02).astype(np.float32)
+        x = rng.standard_normal((1, rows, K)).astype(np.float32)
+        res = rng.standard_normal((1, rows, N)).astype(np.float32)
+        wq = orc.quant_w(w, 128)
+        got = host(ops.fc_Q4A(dev(x), dev(wq), N, residual=dev(res)))
+        want = orc.iadd(orc.fc(x, wq, N), res)
+        assert max_rel_err(got, want) <= 1e-5
