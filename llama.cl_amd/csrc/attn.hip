@@ -215,12 +215,12 @@ __device__ __forceinline__ float merge_chunks(const float* rec, int nchunks, int
     for (int c = 0; c < nchunks; c++) M = fmaxf(M, stat_sh[c]);
     float den = 0.0f, num = 0.0f;
     if (tid < S) {
-        for (int c0 = 0; c0 < nchunks; c0 += 8) {
-            float o[8];
+        for (int c0 = 0; c0 < nchunks; c0 += 32) {
+            float o[32];
 #pragma unroll
-            for (int u = 0; u < 8; u++) o[u] = (c0 + u < nchunks) ? load(rec + (int64_t)(c0 + u) * (S + 2) + 2 + tid) : 0.0f;
+            for (int u = 0; u < 32; u++) o[u] = (c0 + u < nchunks) ? load(rec + (int64_t)(c0 + u) * (S + 2) + 2 + tid) : 0.0f;
 #pragma unroll
-            for (int u = 0; u < 8; u++) {
+            for (int u = 0; u < 32; u++) {
                 if (c0 + u < nchunks) {
                     const float sum = stat_sh[nchunks + c0 + u];
                     const float sc = (sum == 0.0f) ? 0.0f : expf(stat_sh[c0 + u] - M);
@@ -247,11 +247,12 @@ __global__ __launch_bounds__(128) void attn_merge_kernel(float* __restrict__ q, 
 }
 
 // ---- single-launch decode attention (one query token) ------------------------------------------
-// Everything attention_rope2 does for qL == 1 in one kernel: every workgroup rotates q itself
-// (128 values), the workgroup whose chunk holds the new token's cache row rotates k, writes the
-// rotated k back in place and k, v into the cache, and attends to the new row from registers;
-// chunk records are handed to the last-arriving workgroup of the head (device-scope stores and
-// loads, one atomic ticket per head, no cache-wide fence), which merges them into q.
+// attention_rope2 for qL == 1 in two launches instead of three: every workgroup rotates q itself
+// (cos/sin of the position computed once per workgroup, one angle per lane), the workgroup whose
+// chunk holds the new token's cache row rotates k, writes the rotated k back in place and k, v
+// into the cache, and attends to the new row from registers; attn_merge_kernel then combines the
+// chunk records into q.  (Merging inside this kernel through an arrival ticket was measured
+// slower: the last workgroup's device-scope loads of 32 chunk records cost more than a launch.)
 template <typename T>
 __device__ __forceinline__ float cache_round(float v);
 template <>
@@ -277,8 +278,9 @@ __device__ __forceinline__ void store4<__half>(__half* dst, float4 v) {
     *reinterpret_cast<uint2*>(dst) = u;
 }
 
-// rotate the lane's 4 elements (index e4 = first element) of a 128-wide head vector at `base`
-__device__ __forceinline__ float4 rope4(const float* base, int e4, const float* __restrict__ inv_freq, int half, int pos) {
+// rotate the lane's 4 elements (index e4 = first element) of a 128-wide head vector at `base`;
+// cs = cos table [half], sn = sin table [half] of the current position (LDS)
+__device__ __forceinline__ float4 rope4(const float* base, int e4, const float* cs, const float* sn, int half) {
     const float4 own = *reinterpret_cast<const float4*>(base + e4);
     if (e4 >= 2 * half) return own;
     const bool low = e4 < half;
@@ -287,10 +289,8 @@ __device__ __forceinline__ float4 rope4(const float* base, int e4, const float* 
     float o[4] = {own.x, own.y, own.z, own.w}, p[4] = {other.x, other.y, other.z, other.w}, r[4];
 #pragma unroll
     for (int c = 0; c < 4; c++) {
-        const float xita = inv_freq[f0 + c] * (float)pos;
-        const float cs = cosf(xita), sn = sinf(xita);
         // pair (x0 = element i, x1 = element i+half): y0 = c*x0 - s*x1, y1 = s*x0 + c*x1
-        r[c] = low ? cs * o[c] - sn * p[c] : sn * p[c] + cs * o[c];
+        r[c] = low ? cs[f0 + c] * o[c] - sn[f0 + c] * p[c] : sn[f0 + c] * p[c] + cs[f0 + c] * o[c];
     }
     return make_float4(r[0], r[1], r[2], r[3]);
 }
@@ -300,13 +300,12 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(float* q, float* k, co
                                                            const float* __restrict__ inv_freq, int half, T* kc, T* vc,
                                                            int64_t H, int64_t maxlen, int64_t kvLen,
                                                            const int32_t* __restrict__ slots, int position_id, float* part,
-                                                           unsigned* counters, int nchunks) {
+                                                           int nchunks) {
     constexpr int S = 128, C = 4 * PW, NL = PW / 2;
     __shared__ float sc[C];
     __shared__ float osh[4][2][S];
     __shared__ float stat[2];
-    __shared__ unsigned ticket_sh;
-    __shared__ float stat_sh[2 * kMaxChunks];
+    __shared__ float cs_sh[64], sn_sh[64];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int hf = lane >> 5, e = lane & 31;
     const int chunk = blockIdx.x % nchunks;
@@ -325,11 +324,17 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(float* q, float* k, co
     }
     const int slot = slots[0];
     const bool slot_ok = slot >= 0 && slot < maxlen;
-    const float4 qv = rope4(q + bh * S, e * 4, inv_freq, half, position_id);
+    if (threadIdx.x < half) {
+        const float xita = inv_freq[threadIdx.x] * (float)position_id;
+        cs_sh[threadIdx.x] = cosf(xita);
+        sn_sh[threadIdx.x] = sinf(xita);
+    }
+    __syncthreads();
+    const float4 qv = rope4(q + bh * S, e * 4, cs_sh, sn_sh, half);
     // the workgroup that owns the new token's row (or the last chunk, if the row lies beyond kvLen)
     const int owner = (slot_ok && slot / C < nchunks) ? slot / C : nchunks - 1;
     if (chunk == owner) {
-        float4 kn = rope4(k + bh * S, e * 4, inv_freq, half, position_id);
+        float4 kn = rope4(k + bh * S, e * 4, cs_sh, sn_sh, half);
         float4 vn = *reinterpret_cast<const float4*>(v + bh * S + e * 4);
         __syncthreads();  // every wave has read the raw k before it is overwritten
         if (wave == 0 && hf == 0) {
@@ -391,23 +396,12 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(float* q, float* k, co
         float a = 0.0f;
 #pragma unroll
         for (int w = 0; w < 4; w++) a += osh[w][0][threadIdx.x] + osh[w][1][threadIdx.x];
-        __hip_atomic_store(&rec[2 + threadIdx.x], a, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        rec[2 + threadIdx.x] = a;
     }
     if (threadIdx.x == 0) {
-        __hip_atomic_store(&rec[0], stat[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __hip_atomic_store(&rec[1], stat[1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        rec[0] = stat[0];
+        rec[1] = stat[1];
     }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the write-through stores above have been acknowledged
-    __syncthreads();
-    if (threadIdx.x == 0)
-        ticket_sh = __hip_atomic_fetch_add(&counters[bh], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __syncthreads();
-    if (ticket_sh != (unsigned)(nchunks - 1)) return;
-    const float r = merge_chunks(rec0, nchunks, threadIdx.x, 256, stat_sh, [](const float* p) {
-        return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    });
-    if (threadIdx.x < S) q[bh * S + threadIdx.x] = r;
-    if (threadIdx.x == 0) __hip_atomic_store(&counters[bh], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // next launch
 }
 
 // ---- softmax op (ops/op_misc.hpp:183-194): one workgroup per row ------------------------------
@@ -478,7 +472,6 @@ static int attention_impl(float* q, float* k, const float* v, int64_t B, int64_t
     T* kc = cache + (int64_t)(2 * layer_id + 0) * B * H * maxlen * S;
     T* vc = cache + (int64_t)(2 * layer_id + 1) * B * H * maxlen * S;
     uint8_t* wsb = reinterpret_cast<uint8_t*>(workspace);
-    unsigned* counters = reinterpret_cast<unsigned*>(wsb);
     int32_t* row_token = reinterpret_cast<int32_t*>(wsb + LLMOPS_ATTN_COUNTER_BYTES);
     float* part = reinterpret_cast<float*>(wsb + LLMOPS_ATTN_COUNTER_BYTES + align_up((size_t)maxlen * 4, 256));
     int64_t kvLen = (int64_t)position_id + qL;
@@ -487,21 +480,23 @@ static int attention_impl(float* q, float* k, const float* v, int64_t B, int64_t
     const int pw = pick_pw(bhq, kvLen);
     const int nchunks = (int)((kvLen + 4 * pw - 1) / (4 * pw));
     const unsigned grid = (unsigned)(bhq * nchunks);
-    if (qL == 1 && (half % 4) == 0 && nchunks <= kMaxChunks && B * H <= LLMOPS_ATTN_COUNTER_BYTES / 4) {
-        // decode: one launch
+    LLMOPS_REQUIRE(nchunks <= kMaxChunks);
+    if (qL == 1 && (half % 4) == 0) {
+        // decode: rope, cache update and split-KV attention in one launch, then the merge
         if (pw == 16)
             attn_decode_kernel<T, 16><<<grid, 256, 0, st>>>(q, k, v, inv_freq, (int)half, kc, vc, H, maxlen, kvLen, slots,
-                                                          position_id, part, counters, nchunks);
+                                                          position_id, part, nchunks);
         else if (pw == 8)
             attn_decode_kernel<T, 8><<<grid, 256, 0, st>>>(q, k, v, inv_freq, (int)half, kc, vc, H, maxlen, kvLen, slots,
-                                                         position_id, part, counters, nchunks);
+                                                         position_id, part, nchunks);
         else
             attn_decode_kernel<T, 4><<<grid, 256, 0, st>>>(q, k, v, inv_freq, (int)half, kc, vc, H, maxlen, kvLen, slots,
-                                                         position_id, part, counters, nchunks);
+                                                         position_id, part, nchunks);
+        LLMOPS_LAUNCH_CHECK();
+        attn_merge_kernel<<<(unsigned)bhq, 128, 0, st>>>(q, part, qL, H, nchunks);
         LLMOPS_LAUNCH_CHECK();
         return LLMOPS_OK;
     }
-    LLMOPS_REQUIRE(nchunks <= kMaxChunks);
     if (qL > 1) {
         fill_i32_kernel<<<(unsigned)((maxlen + 255) / 256), 256, 0, st>>>(row_token, maxlen, -1);
         LLMOPS_LAUNCH_CHECK();
