@@ -102,6 +102,17 @@ int llmops_fc_Q4A_residual(const float* x, int64_t rows, int64_t K, const int8_t
                            int group_k, int64_t N, const float* residual, float* y, void* workspace,
                            size_t workspace_bytes, llmops_stream_t stream);
 
+/* Decode-step form of fc_Q4A (rows <= 8) with the neighbouring ops of chatllama/main.py:344-375
+ * folded into the one launch.  Each option may be left out (NULL / 0):
+ *   norm_w, eps : x is rmsnorm'ed first (clone + rmsnorm, ops/op_misc.hpp:142-181); needs K % 4 == 0
+ *   residual    : y += residual (iadd, ops/op_misc.hpp:55-79), fp32 [rows,N_out]
+ *   glu         : weiq holds gate and up strips interleaved (strip 2i = gate strip i, 2i+1 = up strip i,
+ *                 Ng even) and y[r,n] = silu(gate[r,n]) * up[r,n] (itrans "silu" + imul), N_out = F
+ * N_out is the number of output columns (Ng*32-ish without glu, Ng/2*32-ish with it). */
+int llmops_fc_Q4A_decode(const float* x, int64_t rows, int64_t K, const int8_t* weiq, int64_t Ng, int64_t Kg,
+                         int group_k, int64_t N_out, const float* norm_w, float eps, const float* residual, int glu,
+                         float* y, void* workspace, size_t workspace_bytes, llmops_stream_t stream);
+
 /* The second half of fc_Q4A on its own (ops/op_fc.hpp:318-423): the product for activations that
  * llmops_FC_dynamic_quantize_x has already quantized (xq int8 [rows,Kg*G], xd and gsum fp32
  * [rows,Kg]).  llmops_fc_Q4A == llmops_FC_dynamic_quantize_x into the workspace + this. */

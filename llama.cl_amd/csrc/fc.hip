@@ -9,9 +9,11 @@ constexpr int kMaxGemvRows = 8;
 int launch_quant_x(const float* x, int64_t rows, int64_t K, int group_k, int8_t* xq, float* xd, float* gsum,
                    hipStream_t stream);
 size_t gemv_workspace_bytes(int64_t rows, int64_t Ng, int64_t Kg, int G);
-int launch_gemv(const uint8_t* w, const float* x, const int8_t* xq, const float* xd, const float* gs, float* y,
-                float* part, unsigned* counters, int64_t rows, int64_t Ng, int64_t Kg, int G, int64_t N,
-                const float* residual, hipStream_t st);
+int launch_gemv(const uint8_t* w, const int8_t* xq, const float* xd, const float* gs, float* y, float* part,
+                unsigned* counters, int64_t rows, int64_t Ng, int64_t Kg, int G, int64_t N, hipStream_t st);
+int launch_gemv_fused(const uint8_t* w, const float* x, float* y, float* part, unsigned* counters, int64_t rows, int64_t Ng,
+                      int64_t Kg, int G, int64_t N, const float* residual, const float* norm_w, float eps, bool glu,
+                      hipStream_t st);
 int launch_add(float* a, const float* b, int64_t total, hipStream_t st);
 int launch_gemv_partials(const uint8_t* w, const int8_t* xq, int32_t* acc, int64_t rows, int64_t Ng, int64_t Kg, int G,
                          hipStream_t st);
@@ -76,7 +78,7 @@ static int fc_impl(const float* x, int64_t rows, int64_t K, const int8_t* weiq, 
     const uint8_t* w = reinterpret_cast<const uint8_t*>(weiq);
     // few rows: one launch, the streaming kernel quantizes the activations it needs on the fly
     if (rows <= kMaxGemvRows)
-        return launch_gemv(w, x, nullptr, nullptr, nullptr, y, part, counters, rows, Ng, Kg, group_k, N, residual, st);
+        return launch_gemv_fused(w, x, y, part, counters, rows, Ng, Kg, group_k, N, residual, nullptr, 0.0f, false, st);
     int rc = launch_quant_x(x, rows, K, group_k, xq, xd, gs, st);
     if (rc) return rc;
     rc = launch_gemm(w, xq, xd, gs, y, part, rows, Ng, Kg, group_k, N, st);
@@ -97,6 +99,31 @@ extern "C" int llmops_fc_Q4A_residual(const float* x, int64_t rows, int64_t K, c
     return fc_impl(x, rows, K, weiq, Ng, Kg, group_k, N, residual, y, workspace, workspace_bytes, stream);
 }
 
+extern "C" int llmops_fc_Q4A_decode(const float* x, int64_t rows, int64_t K, const int8_t* weiq, int64_t Ng, int64_t Kg,
+                                    int group_k, int64_t N_out, const float* norm_w, float eps, const float* residual,
+                                    int glu, float* y, void* workspace, size_t workspace_bytes, llmops_stream_t stream) {
+    LLMOPS_REQUIRE(valid_group(group_k));
+    LLMOPS_REQUIRE(x != nullptr && weiq != nullptr && y != nullptr && workspace != nullptr);
+    LLMOPS_REQUIRE(rows > 0 && rows <= kMaxGemvRows);
+    LLMOPS_REQUIRE(K > 0 && Ng > 0 && Kg > 0 && K == Kg * group_k);
+    LLMOPS_REQUIRE(Ng <= LLMOPS_FC_COUNTER_BYTES / 4 && Ng * 64 < ((int64_t)1 << 31));
+    LLMOPS_REQUIRE(aligned(weiq, 16) && aligned(workspace, 256) && aligned(x, 8));
+    if (glu) {
+        LLMOPS_REQUIRE((Ng % 2) == 0 && residual == nullptr);
+        LLMOPS_REQUIRE(N_out > (Ng / 2 - 1) * kGroupN && N_out <= Ng / 2 * kGroupN);
+    } else {
+        LLMOPS_REQUIRE(N_out > (Ng - 1) * kGroupN && N_out <= Ng * kGroupN);
+    }
+    if (norm_w != nullptr) LLMOPS_REQUIRE((K % 4) == 0 && aligned(x, 16) && aligned(norm_w, 8));
+    const FcWorkspace lay = fc_layout(rows, Ng, Kg, group_k);
+    if (workspace_bytes < lay.total)
+        return fail(LLMOPS_EWORKSPACE, "fc_Q4A needs %zu workspace bytes, got %zu", lay.total, workspace_bytes);
+    uint8_t* ws = reinterpret_cast<uint8_t*>(workspace);
+    return launch_gemv_fused(reinterpret_cast<const uint8_t*>(weiq), x, y, reinterpret_cast<float*>(ws + lay.off_part),
+                             reinterpret_cast<unsigned*>(ws), rows, Ng, Kg, group_k, N_out, residual, norm_w, eps, glu != 0,
+                             as_stream(stream));
+}
+
 extern "C" int llmops_fc_Q4A_prequantized(const int8_t* xq, const float* xd, const float* gsum, int64_t rows,
                                           const int8_t* weiq, int64_t Ng, int64_t Kg, int group_k, int64_t N, float* y,
                                           void* workspace, size_t workspace_bytes, llmops_stream_t stream) {
@@ -115,8 +142,7 @@ extern "C" int llmops_fc_Q4A_prequantized(const int8_t* xq, const float* xd, con
     const uint8_t* w = reinterpret_cast<const uint8_t*>(weiq);
     hipStream_t st = as_stream(stream);
     if (rows <= kMaxGemvRows)
-        return launch_gemv(w, nullptr, xq, xd, gsum, y, part, reinterpret_cast<unsigned*>(ws), rows, Ng, Kg, group_k, N,
-                           nullptr, st);
+        return launch_gemv(w, xq, xd, gsum, y, part, reinterpret_cast<unsigned*>(ws), rows, Ng, Kg, group_k, N, st);
     return launch_gemm(w, xq, xd, gsum, y, part, rows, Ng, Kg, group_k, N, st);
 }
 

@@ -326,19 +326,48 @@ __device__ __forceinline__ void quantize_step(const XRaw<G>& xr, XSlot<G>* slot,
     }
 }
 
-// D = weight blocks kept in flight ahead of the one being consumed (per wave)
-template <int G, int MT, int NW, int D>
+__device__ __forceinline__ float wave_sum_dpp(float v) {
+    float dummy = 0.0f;
+    row16_max_sum(dummy, v);
+    return (lane_bcast(v, 0) + lane_bcast(v, 16)) + (lane_bcast(v, 32) + lane_bcast(v, 48));
+}
+
+// Optional work folded into the decode kernel (MODE bits):
+//   kNorm: the activation row is rmsnorm'ed first (ops/op_misc.hpp:142-181): every workgroup reads
+//          the whole row once (L2 resident), reduces the sum of squares and scales the groups it
+//          quantizes by rsqrt(mean+eps)*w.  Replaces clone + rmsnorm launches in front of the FC.
+//   kGlu : the packed tensor holds gate and up strips interleaved (strip 2i = gate strip i, strip
+//          2i+1 = up strip i); a workgroup computes both and stores silu(gate)*up
+//          (itrans "silu" + imul, ops/op_misc.hpp:83-138).  Replaces two launches behind the FC.
+constexpr int kNorm = 1, kGlu = 2;
+
+template <int G, int MT, int NW, int MODE>
 __global__ __launch_bounds__(NW * 64) void fc_gemv_fused_kernel(const uint8_t* __restrict__ weiq, const float* __restrict__ x,
                                                                  float* __restrict__ y, float* part, unsigned* counters,
                                                                  int Kg, int64_t K, int64_t N, int rows, int S,
-                                                                 int steps_per_split, const float* __restrict__ residual) {
+                                                                 int steps_per_split, const float* __restrict__ residual,
+                                                                 const float* __restrict__ norm_w, float eps) {
+    constexpr bool NORM = (MODE & kNorm) != 0, GLU = (MODE & kGlu) != 0;
+    constexpr int NWS = GLU ? NW / 2 : NW;  // waves per strip
     __shared__ float red[NW][MT][kGroupN];
     __shared__ __align__(16) XSlot<G> xs[NW][MT];
+    __shared__ float nred[NORM ? NW : 1][MT];
     __shared__ unsigned ticket_sh;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int rs = lane >> 3;
-    const TileRange tr = tile_range<G, NW>(Kg, S, steps_per_split, wave);
+    TileRange tr;
+    if (GLU) {  // S == 1: blockIdx.x is the strip pair, each half of the workgroup owns one strip
+        constexpr int BPS = Step<G>::kBlocksPerStep;
+        const int T = (Kg + BPS - 1) / BPS;
+        const int per_wave = (T + NWS - 1) / NWS;
+        tr.nb = blockIdx.x * 2 + wave / NWS;
+        tr.s = 0;
+        tr.t0 = min(T, (wave % NWS) * per_wave);
+        tr.t1 = min(T, tr.t0 + per_wave);
+    } else {
+        tr = tile_range<G, NW>(Kg, S, steps_per_split, wave);
+    }
     const uint8_t* strip = weiq + (int64_t)tr.nb * Kg * block_bytes(G);
     const bool first_row = (G == 128) ? (rs == 0) : ((rs & 3) == 0);
 
@@ -348,51 +377,112 @@ __global__ __launch_bounds__(NW * 64) void fc_gemv_fused_kernel(const uint8_t* _
 #pragma unroll
         for (int j = 0; j < 4; j++) f[r][j] = 0.0f;
 
-    // ring of D+1 block buffers; the activation row of a step is fetched one step ahead
-    Step<G> buf[D + 1];
-    XRaw<G> xcur[MT], xnxt[MT];
+    // double-buffered weight blocks; the activation row of a step is fetched one step ahead
+    Step<G> cur, nxt;
+    XRaw<G> xcur[MT], xnxt[MT], wcur, wnxt;
     if (tr.t0 < tr.t1) {
 #pragma unroll
         for (int r = 0; r < MT; r++)
             if (r < rows) load_x<G>(xcur[r], x + (int64_t)r * K, tr.t0, K, lane);
+        if (NORM) load_x<G>(wcur, norm_w, tr.t0, K, lane);
+        load_step<G>(cur, strip, tr.t0, Kg, lane);
     }
-#pragma unroll
-    for (int u = 0; u < D; u++)
-        if (tr.t0 + u < tr.t1) load_step<G>(buf[u], strip, tr.t0 + u, Kg, lane);
 
-    for (int tb = tr.t0; tb < tr.t1; tb += D + 1) {
+    float rsn[MT];
+    if (NORM) {
+        // sum of squares of every row, while the first weight block is in flight
 #pragma unroll
-        for (int u = 0; u < D + 1; u++) {
-            const int t = tb + u;
-            if (t < tr.t1) {
-                if (t + D < tr.t1) load_step<G>(buf[(u + D) % (D + 1)], strip, t + D, Kg, lane);
-                if (t + 1 < tr.t1) {
-#pragma unroll
-                    for (int r = 0; r < MT; r++)
-                        if (r < rows) load_x<G>(xnxt[r], x + (int64_t)r * K, t + 1, K, lane);
+        for (int r = 0; r < MT; r++) {
+            float ss = 0.0f;
+            if (r < rows) {
+                for (int64_t e = (int64_t)threadIdx.x * 4; e < K; e += NW * 64 * 4) {
+                    const float4 v = *reinterpret_cast<const float4*>(x + (int64_t)r * K + e);
+                    ss = fmaf(v.x, v.x, ss);
+                    ss = fmaf(v.y, v.y, ss);
+                    ss = fmaf(v.z, v.z, ss);
+                    ss = fmaf(v.w, v.w, ss);
                 }
-                const Step<G>& cur = buf[u];
-#pragma unroll
-                for (int r = 0; r < MT; r++) {
-                    if (r < rows) {
-                        XSlot<G>* slot = &xs[wave][r];
-                        quantize_step<G>(xcur[r], slot, lane);
-                        __builtin_amdgcn_wave_barrier();  // LDS writes stay ahead of the reads below
-                        if (cur.valid) {
-                            int acc[4];
-                            dot_step<G>(cur, slot->codes, lane, acc);
-                            const float2 sc = slot->scale[(G == 128) ? 0 : (rs >> 2)];
-                            fold(f[r], acc, cur.dh, cur.mh, sc.x, first_row ? sc.y : 0.0f);
-                        }
-                        __builtin_amdgcn_wave_barrier();  // reads stay ahead of the next step's writes
-                    }
-                }
-#pragma unroll
-                for (int r = 0; r < MT; r++) xcur[r] = xnxt[r];
             }
+            ss = wave_sum_dpp(ss);
+            if (lane == 0) nred[NORM ? wave : 0][r] = ss;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int r = 0; r < MT; r++) {
+            float tot = 0.0f;
+#pragma unroll
+            for (int w = 0; w < NW; w++) tot += nred[NORM ? w : 0][r];
+            rsn[r] = 1.0f / sqrtf(tot / (float)K + eps);
         }
     }
-    finish_strip<MT, NW>(f, red, &ticket_sh, tr.nb, tr.s, S, rows, N, y, part, counters, residual);
+
+    for (int t = tr.t0; t < tr.t1; t++) {
+        if (t + 1 < tr.t1) {
+            load_step<G>(nxt, strip, t + 1, Kg, lane);
+#pragma unroll
+            for (int r = 0; r < MT; r++)
+                if (r < rows) load_x<G>(xnxt[r], x + (int64_t)r * K, t + 1, K, lane);
+            if (NORM) load_x<G>(wnxt, norm_w, t + 1, K, lane);
+        }
+#pragma unroll
+        for (int r = 0; r < MT; r++) {
+            if (r < rows) {
+                if (NORM) {
+#pragma unroll
+                    for (int i = 0; i < (G == 128 ? 2 : 1); i++) xcur[r].v[i] = xcur[r].v[i] * rsn[r] * wcur.v[i];
+                }
+                XSlot<G>* slot = &xs[wave][r];
+                quantize_step<G>(xcur[r], slot, lane);
+                __builtin_amdgcn_wave_barrier();  // LDS writes stay ahead of the reads below
+                if (cur.valid) {
+                    int acc[4];
+                    dot_step<G>(cur, slot->codes, lane, acc);
+                    const float2 sc = slot->scale[(G == 128) ? 0 : (rs >> 2)];
+                    fold(f[r], acc, cur.dh, cur.mh, sc.x, first_row ? sc.y : 0.0f);
+                }
+                __builtin_amdgcn_wave_barrier();  // reads stay ahead of the next step's writes
+            }
+        }
+        cur = nxt;
+#pragma unroll
+        for (int r = 0; r < MT; r++) xcur[r] = xnxt[r];
+        if (NORM) wcur = wnxt;
+    }
+
+    if (!GLU) {
+        finish_strip<MT, NW>(f, red, &ticket_sh, tr.nb, tr.s, S, rows, N, y, part, counters, residual);
+        return;
+    }
+    // gate/up epilogue: sum row slots, then the two halves of the workgroup, then silu(gate)*up
+    const int quad = lane & 7;
+#pragma unroll
+    for (int r = 0; r < MT; r++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            float v = f[r][j];
+            v += dpp<kRowRor8>(v);
+            v += __shfl_xor(v, 16, 64);
+            v += __shfl_xor(v, 32, 64);
+            f[r][j] = v;
+        }
+    if (rs == 0) {
+#pragma unroll
+        for (int r = 0; r < MT; r++)
+#pragma unroll
+            for (int j = 0; j < 4; j++) red[wave][r][quad * 4 + j] = f[r][j];
+    }
+    __syncthreads();
+    const int trow = threadIdx.x >> 5, tn = threadIdx.x & 31;
+    if (trow < MT && trow < rows) {
+        float g = 0.0f, u = 0.0f;
+#pragma unroll
+        for (int w = 0; w < NWS; w++) {
+            g += red[w][trow][tn];
+            u += red[GLU ? w + NWS : w][trow][tn];
+        }
+        const int64_t n = (int64_t)blockIdx.x * kGroupN + tn;  // N = number of output columns (F)
+        if (n < N) y[(int64_t)trow * N + n] = u * (g * (1.0f / (1.0f + expf(-g))));
+    }
 }
 
 // Integer core only: acc[r][n][kb] (int32).  One wavefront per step, same loads and same dot
@@ -432,17 +522,16 @@ __global__ __launch_bounds__(64) void fc_gemv_partials_kernel(const uint8_t* __r
 }
 
 static int g_target_workgroups = 256;  // split-K planner aims for this many workgroups
-static int g_waves_per_workgroup = 0;  // 0 = choose per shape
-static int g_prefetch_depth = 1;       // weight blocks in flight ahead of the current one
+static int g_waves_per_workgroup = 0;  // 0 = choose per shape (pre-quantized variant only)
 
 struct GemvPlan {
     int S, steps_per_split, NW;
 };
 
-static GemvPlan plan_gemv(int64_t rows, int64_t Ng, int64_t Kg, int G) {
+static GemvPlan plan_gemv(int64_t rows, int64_t Ng, int64_t Kg, int G, bool fused) {
     const int bps = (G == 128) ? 1 : 2;
     const int T = (int)((Kg + bps - 1) / bps);
-    int NW = g_waves_per_workgroup;
+    int NW = fused ? 0 : g_waves_per_workgroup;
     if (NW == 0) NW = 16;
     if (rows > 4 && NW > 8) NW = 8;  // one (row, column) finaliser thread per output of the strip
     int S = (int)((g_target_workgroups + Ng - 1) / Ng);
@@ -464,44 +553,78 @@ size_t gemv_workspace_bytes(int64_t rows, int64_t Ng, int64_t Kg, int G) {
     return (size_t)S * rows * Ng * kGroupN * sizeof(float);
 }
 
+struct FusedOps {
+    const float* residual;  // y += residual
+    const float* norm_w;    // x = rmsnorm(x, norm_w, eps) first
+    float eps;
+    bool glu;               // interleaved gate/up strips, y = silu(gate)*up
+};
+
 template <int G, int MT, int NW>
-static void launch_gemv_t(const uint8_t* w, const float* x, const int8_t* xq, const float* xd, const float* gs, float* y,
-                          float* part, unsigned* counters, int64_t Ng, int64_t Kg, int64_t N, int rows, GemvPlan p,
-                          const float* residual, hipStream_t st) {
-    const unsigned grid = (unsigned)(Ng * p.S);
-    if (x == nullptr) {
-        fc_gemv_kernel<G, MT, NW><<<grid, NW * 64, 0, st>>>(w, xq, xd, gs, y, part, counters, (int)Kg, N, rows, p.S,
-                                                            p.steps_per_split, residual);
-        return;
+static void launch_fused_t(const uint8_t* w, const float* x, float* y, float* part, unsigned* counters, int64_t Ng,
+                           int64_t Kg, int64_t N, int rows, GemvPlan p, const FusedOps& o, hipStream_t st) {
+    const int64_t K = Kg * G;
+#define LLMOPS_FUSED(MODE, GRID)                                                                                      \
+    fc_gemv_fused_kernel<G, MT, NW, MODE><<<(unsigned)(GRID), NW * 64, 0, st>>>(w, x, y, part, counters, (int)Kg, K, N, rows, \
+                                                                                p.S, p.steps_per_split, o.residual,  \
+                                                                                o.norm_w, o.eps)
+    if (o.glu) {
+        if (o.norm_w) LLMOPS_FUSED(kNorm | kGlu, Ng / 2);
+        else LLMOPS_FUSED(kGlu, Ng / 2);
+    } else {
+        if (o.norm_w) LLMOPS_FUSED(kNorm, Ng * p.S);
+        else LLMOPS_FUSED(0, Ng * p.S);
     }
-#define LLMOPS_FUSED(DD)                                                                                             \
-    fc_gemv_fused_kernel<G, MT, NW, DD><<<grid, NW * 64, 0, st>>>(w, x, y, part, counters, (int)Kg, Kg * G, N, rows, p.S, \
-                                                                  p.steps_per_split, residual)
-    if (MT == 1 && g_prefetch_depth >= 3) LLMOPS_FUSED((MT == 1 ? 3 : 1));
-    else if (MT == 1 && g_prefetch_depth == 2) LLMOPS_FUSED((MT == 1 ? 2 : 1));
-    else LLMOPS_FUSED(1);
 #undef LLMOPS_FUSED
 }
 
-template <int G, int MT>
-static void launch_gemv_nw(const uint8_t* w, const float* x, const int8_t* xq, const float* xd, const float* gs, float* y,
-                           float* part, unsigned* counters, int64_t Ng, int64_t Kg, int64_t N, int rows, GemvPlan p,
-                           const float* residual, hipStream_t st) {
-    if (p.NW >= 16 && MT <= 4)
-        launch_gemv_t<G, MT, (MT <= 4 ? 16 : 8)>(w, x, xq, xd, gs, y, part, counters, Ng, Kg, N, rows, p, residual, st);
-    else if (p.NW >= 8)
-        launch_gemv_t<G, MT, 8>(w, x, xq, xd, gs, y, part, counters, Ng, Kg, N, rows, p, residual, st);
-    else
-        launch_gemv_t<G, MT, 4>(w, x, xq, xd, gs, y, part, counters, Ng, Kg, N, rows, p, residual, st);
+// raw fp32 activations, quantized inside the kernel (+ optional rmsnorm / residual / gate-up epilogue)
+int launch_gemv_fused(const uint8_t* w, const float* x, float* y, float* part, unsigned* counters, int64_t rows, int64_t Ng,
+                      int64_t Kg, int G, int64_t N, const float* residual, const float* norm_w, float eps, bool glu,
+                      hipStream_t st) {
+    GemvPlan p = plan_gemv(rows, Ng, Kg, G, true);
+    if (glu) p.S = 1;
+    const FusedOps o{residual, norm_w, eps, glu};
+#define LLMOPS_CASE(GG, MT, NWW) launch_fused_t<GG, MT, NWW>(w, x, y, part, counters, Ng, Kg, N, (int)rows, p, o, st)
+    if (G == 128) {
+        if (rows == 1) LLMOPS_CASE(128, 1, 16);
+        else if (rows == 2) LLMOPS_CASE(128, 2, 16);
+        else if (rows <= 4) LLMOPS_CASE(128, 4, 16);
+        else LLMOPS_CASE(128, 8, 8);
+    } else {
+        if (rows == 1) LLMOPS_CASE(32, 1, 16);
+        else if (rows == 2) LLMOPS_CASE(32, 2, 16);
+        else if (rows <= 4) LLMOPS_CASE(32, 4, 16);
+        else LLMOPS_CASE(32, 8, 8);
+    }
+#undef LLMOPS_CASE
+    LLMOPS_LAUNCH_CHECK();
+    return LLMOPS_OK;
 }
 
-// x != nullptr: raw fp32 activations, quantized inside the kernel; else xq/xd/gs are used.
-int launch_gemv(const uint8_t* w, const float* x, const int8_t* xq, const float* xd, const float* gs, float* y,
-                float* part, unsigned* counters, int64_t rows, int64_t Ng, int64_t Kg, int G, int64_t N,
-                const float* residual, hipStream_t st) {
-    const GemvPlan p = plan_gemv(rows, Ng, Kg, G);
-#define LLMOPS_GEMV_CASE(GG, MT) \
-    launch_gemv_nw<GG, MT>(w, x, xq, xd, gs, y, part, counters, Ng, Kg, N, (int)rows, p, residual, st)
+template <int G, int MT, int NW>
+static void launch_gemv_t(const uint8_t* w, const int8_t* xq, const float* xd, const float* gs, float* y, float* part,
+                          unsigned* counters, int64_t Ng, int64_t Kg, int64_t N, int rows, GemvPlan p, hipStream_t st) {
+    fc_gemv_kernel<G, MT, NW><<<(unsigned)(Ng * p.S), NW * 64, 0, st>>>(w, xq, xd, gs, y, part, counters, (int)Kg, N, rows,
+                                                                      p.S, p.steps_per_split, nullptr);
+}
+
+template <int G, int MT>
+static void launch_gemv_nw(const uint8_t* w, const int8_t* xq, const float* xd, const float* gs, float* y, float* part,
+                           unsigned* counters, int64_t Ng, int64_t Kg, int64_t N, int rows, GemvPlan p, hipStream_t st) {
+    if (p.NW >= 16 && MT <= 4)
+        launch_gemv_t<G, MT, (MT <= 4 ? 16 : 8)>(w, xq, xd, gs, y, part, counters, Ng, Kg, N, rows, p, st);
+    else if (p.NW >= 8)
+        launch_gemv_t<G, MT, 8>(w, xq, xd, gs, y, part, counters, Ng, Kg, N, rows, p, st);
+    else
+        launch_gemv_t<G, MT, 4>(w, xq, xd, gs, y, part, counters, Ng, Kg, N, rows, p, st);
+}
+
+// activations already quantized by llmops_FC_dynamic_quantize_x
+int launch_gemv(const uint8_t* w, const int8_t* xq, const float* xd, const float* gs, float* y, float* part,
+                unsigned* counters, int64_t rows, int64_t Ng, int64_t Kg, int G, int64_t N, hipStream_t st) {
+    const GemvPlan p = plan_gemv(rows, Ng, Kg, G, false);
+#define LLMOPS_GEMV_CASE(GG, MT) launch_gemv_nw<GG, MT>(w, xq, xd, gs, y, part, counters, Ng, Kg, N, (int)rows, p, st)
     if (G == 128) {
         if (rows == 1) LLMOPS_GEMV_CASE(128, 1);
         else if (rows == 2) LLMOPS_GEMV_CASE(128, 2);
@@ -536,6 +659,4 @@ extern "C" void llmops_fc_set_tuning(int target_workgroups, int waves_per_workgr
     if (target_workgroups > 0) llmops::g_target_workgroups = target_workgroups > 4096 ? 4096 : target_workgroups;
     if (waves_per_workgroup >= 0) llmops::g_waves_per_workgroup = waves_per_workgroup;
 }
-extern "C" void llmops_fc_set_prefetch(int depth) {
-    if (depth >= 1) llmops::g_prefetch_depth = depth;
-}
+

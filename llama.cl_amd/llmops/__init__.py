@@ -21,7 +21,7 @@ import torch
 from . import _lib
 
 __all__ = [
-    "offline_FC_quant_Q4A", "offline_FC_dequant_Q4A", "fc_Q4A", "FC_dynamic_quantize_x", "fc_Q4A_partials",
+    "offline_FC_quant_Q4A", "offline_FC_dequant_Q4A", "fc_Q4A", "fc_Q4A_decode", "interleave_gate_up", "FC_dynamic_quantize_x", "fc_Q4A_partials",
     "attention_rope", "attention_rope2", "rope_embed", "softmax", "rmsnorm", "iadd", "imul", "itrans", "clone",
     "rmsnorm_out", "silu_mul", "empty", "ones", "embedding", "embedding_q8c_quant_w", "embedding_q8c", "tensor_pool", "set_default_group_k",
     "group_k_of",
@@ -141,6 +141,51 @@ def fc_Q4A(input, weiq, N, residual=None):
         _require(tuple(residual.shape) == (B, M, int(N)), "residual.is({B, M, N})")
         _lib.check(lib.llmops_fc_Q4A_residual(_ptr(input), rows, K, _ptr(weiq), Ng, Kg, g, int(N), _ptr(residual), _ptr(out),
                                               _ptr(ws), ws.numel(), _stream(input)))
+    return out
+
+
+def interleave_gate_up(gate_packed, up_packed):
+    """Packed gate and up tensors [Ng,Kg,blk] -> one tensor [2*Ng,Kg,blk] with strips alternating
+    gate, up, gate, up ... : the layout ``fc_Q4A_decode(..., glu=True)`` consumes."""
+    _require(gate_packed.shape == up_packed.shape, "gate.shape() == up.shape()")
+    return torch.stack((gate_packed, up_packed), dim=1).reshape(-1, *gate_packed.shape[1:]).contiguous()
+
+
+def fc_Q4A_decode(input, weiq, N_out, norm=None, residual=None, glu=False):
+    """Extension: fc_Q4A with its neighbours of the decode step folded in (one launch for B*M <= 8).
+
+    norm=(weight, eps): input is rmsnorm'ed first;  residual: added to the result;
+    glu=True: ``weiq`` holds interleaved gate/up strips (``interleave_gate_up``) and the result is
+    silu(gate)*up with N_out = F columns.  With more than 8 rows the same arithmetic is composed
+    from the separate ops."""
+    _dev(input, torch.float32, 3, "input")
+    _dev(weiq, torch.int8, 3, "wei_quantized")
+    g = group_k_of(weiq)
+    B, M, K = input.shape
+    Ng, Kg, _ = weiq.shape
+    rows = B * M
+    N_out = int(N_out)
+    if norm is not None:
+        _dev(norm[0], torch.float32, 1, "norm weight")
+        _require(norm[0].shape[0] == K, "weight.size(0) == K")
+    if residual is not None:
+        _dev(residual, torch.float32, 3, "residual")
+        _require(tuple(residual.shape) == (B, M, N_out), "residual.is({B, M, N})")
+    if rows > 8:
+        x = input if norm is None else rmsnorm_out(input, norm[0], norm[1])
+        if glu:
+            _require(N_out % 32 == 0, "F % 32 == 0")
+            y = fc_Q4A(x, weiq, 2 * N_out).view(B, M, N_out // 32, 2, 32)
+            gu = torch.cat((y[..., 0, :].reshape(B, M, N_out), y[..., 1, :].reshape(B, M, N_out)), dim=-1)
+            return silu_mul(gu)
+        return fc_Q4A(x, weiq, N_out, residual=residual)
+    lib = _lib.load()
+    ws = _workspace(input.device, lib.llmops_fc_Q4A_workspace_bytes(rows, K, Ng, Kg, g))
+    out = torch.empty((B, M, N_out), dtype=torch.float32, device=input.device)
+    _lib.check(lib.llmops_fc_Q4A_decode(_ptr(input), rows, K, _ptr(weiq), Ng, Kg, g, N_out,
+                                        _ptr(norm[0]) if norm is not None else None, float(norm[1]) if norm is not None else 0.0,
+                                        _ptr(residual) if residual is not None else None, int(bool(glu)), _ptr(out), _ptr(ws),
+                                        ws.numel(), _stream(input)))
     return out
 
 

@@ -7,8 +7,8 @@ This is the caller of the hot path, kept as thin as the reference's: every arith
 * ``plan="reference"``: the reference's sequence verbatim -- clone, rmsnorm, q/k/v projections as three
   FCs, attention_rope2, o projection, iadd, clone, rmsnorm, gate, silu, up, imul, down, iadd.
 * ``plan="fused"`` (default): the same arithmetic with fewer launches -- q|k|v and gate|up packed
-  tensors concatenated along N so each pair/triple is one FC launch, clone+rmsnorm and silu+mul as
-  one op each, residual adds folded into the o and down projections.
+  tensors fused into one FC launch each, rmsnorm folded into the FC that consumes it, silu*up into
+  the gate|up epilogue, residual adds into the o and down projections (``llmops.fc_Q4A_decode``).
 
 A decode step (one token, batch 1) has fixed shapes and no host-side decisions, so it can be
 captured once as a HIP graph and replayed (``capture_decode``).
@@ -52,7 +52,8 @@ class LlamaDecoder:
             }
             if plan == "fused":
                 layer["qkv_proj"] = fc(H, H, parts=3)
-                layer["gate_up_proj"] = fc(F, H, parts=2)
+                gate, up = fc(F, H), fc(F, H)
+                layer["gate_up_proj"] = llmop_fc_q4a(packed=llmops.interleave_gate_up(gate.weight, up.weight), N=2 * F)
             else:
                 layer["q_proj"], layer["k_proj"], layer["v_proj"] = fc(H, H), fc(H, H), fc(H, H)
                 layer["gate_proj"], layer["up_proj"] = fc(F, H), fc(F, H)
@@ -105,19 +106,19 @@ class LlamaDecoder:
         return hidden_states
 
     def _layer_fused(self, i, ops, hidden_states, kv_cache, kv_cache_slots, position_id):
-        """Same arithmetic, 10 launches instead of 18: clone+rmsnorm, q|k|v and gate|up as one FC each,
-        silu+mul as one op, the two residual adds inside the o and down projections."""
-        H = self.configs["hidden_size"]
-        x = ops["input_layernorm"].out_of_place(hidden_states)
-        qkv = ops["qkv_proj"](x)
+        """Same arithmetic, 6 launches per decode layer instead of 18: rmsnorm inside the q|k|v and
+        gate|up FCs, silu*up in the gate|up epilogue (interleaved strips), residual adds inside the o
+        and down projections, rope + cache update inside the attention kernel."""
+        H, F = self.configs["hidden_size"], self.configs["intermediate_size"]
+        n1, n2 = ops["input_layernorm"], ops["post_attention_layernorm"]
+        qkv = llmops.fc_Q4A_decode(hidden_states, ops["qkv_proj"].weight, 3 * H, norm=(n1.weight, n1.eps))
         q, k, v = qkv[..., :H], qkv[..., H:2 * H], qkv[..., 2 * H:]
         if not q.is_contiguous():  # more than one token: the op needs dense [B,qL,H*S] tensors
             q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
         llmops.attention_rope2(q, k, v, self.inv_freq, kv_cache, kv_cache_slots, position_id, i)
-        attn_output = ops["o_proj"](q, residual=hidden_states)
-        x = ops["post_attention_layernorm"].out_of_place(attn_output)
-        act = llmops.silu_mul(ops["gate_up_proj"](x))
-        return ops["down_proj"](act, residual=attn_output)
+        attn_output = llmops.fc_Q4A_decode(q, ops["o_proj"].weight, H, residual=hidden_states)
+        act = llmops.fc_Q4A_decode(attn_output, ops["gate_up_proj"].weight, F, norm=(n2.weight, n2.eps), glu=True)
+        return llmops.fc_Q4A_decode(act, ops["down_proj"].weight, H, residual=attn_output)
 
     def capture_decode(self, kv_cache, slot, position_id, stream=None):
         """Capture one decode step (batch 1, one token, fixed slot/position) as a HIP graph.

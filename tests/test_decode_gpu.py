@@ -35,9 +35,10 @@ def oracle_forward(orc, model, ids, cache, slots, pos):
         q, _, cache = orc.attention(q, k, v, inv, cache, slots, pos, i)
         attn = orc.iadd(fc(ops["o_proj"], q), hidden)
         x = orc.rmsnorm(attn, ops["post_attention_layernorm"].weight.cpu().numpy(), CFG["rms_norm_eps"])
-        if "gate_up_proj" in ops:
-            gu = fc(ops["gate_up_proj"], x)
-            gate, up = gu[..., :F].copy(), gu[..., F:].copy()
+        if "gate_up_proj" in ops:  # strips alternate gate, up, gate, up ...
+            gu = fc(ops["gate_up_proj"], x).reshape(x.shape[:-1] + (F // 32, 2, 32))
+            gate = gu[..., 0, :].reshape(x.shape[:-1] + (F,)).copy()
+            up = gu[..., 1, :].reshape(x.shape[:-1] + (F,)).copy()
         else:
             gate, up = fc(ops["gate_proj"], x), fc(ops["up_proj"], x)
         hidden = orc.iadd(fc(ops["down_proj"], orc.imul(up, orc.silu(gate))), attn)
@@ -96,6 +97,7 @@ def test_layer_ops_teacher_forced(orc):
         close(x, orc.rmsnorm(h(hidden), h(ops["input_layernorm"].weight), eps), 1e-5)
         qkv = ops["qkv_proj"](x)
         close(qkv, orc.fc(h(x), h(ops["qkv_proj"].weight), 3 * H), 1e-5)
+        qkv_saved = h(qkv)  # q and k are updated in place by the attention below
         q, k, v = (t.contiguous() for t in (qkv[..., :H], qkv[..., H:2 * H], qkv[..., 2 * H:]))
         q0, k0, v0, c0 = h(q), h(k), h(v), h(kv.cache)
         llmops.attention_rope2(q, k, v, model.inv_freq, kv.cache, slots, pos, 0)
@@ -112,8 +114,10 @@ def test_layer_ops_teacher_forced(orc):
         ops["post_attention_layernorm"](x)
         close(x, orc.rmsnorm(h(attn), h(ops["post_attention_layernorm"].weight), eps), 1e-5)
         gu = ops["gate_up_proj"](x)
-        close(gu, orc.fc(h(x), h(ops["gate_up_proj"].weight), 2 * F), 1e-5)
-        gate, up = gu[..., :F].contiguous(), gu[..., F:].contiguous()
+        want_gu = orc.fc(h(x), h(ops["gate_up_proj"].weight), 2 * F)
+        close(gu, want_gu, 1e-5)
+        gu5 = gu.view(1, qL, F // 32, 2, 32)
+        gate, up = gu5[..., 0, :].reshape(1, qL, F).contiguous(), gu5[..., 1, :].reshape(1, qL, F).contiguous()
         g0, u0 = h(gate), h(up)
         llmops.itrans(gate, "silu")
         close(gate, orc.silu(g0), 1e-5)
@@ -121,6 +125,11 @@ def test_layer_ops_teacher_forced(orc):
         assert np.array_equal(h(up), orc.imul(u0, h(gate)))
         down = ops["down_proj"](up)
         close(down, orc.fc(h(up), h(ops["down_proj"].weight), H), 1e-5)
+        # the folded forms give the same results as the separate ops above
+        n1, n2 = ops["input_layernorm"], ops["post_attention_layernorm"]
+        close(llmops.fc_Q4A_decode(hidden, ops["qkv_proj"].weight, 3 * H, norm=(n1.weight, n1.eps)), qkv_saved, 1e-4)
+        close(llmops.fc_Q4A_decode(attn, ops["gate_up_proj"].weight, F, norm=(n2.weight, n2.eps), glu=True), h(up), 1e-4)
+        close(llmops.fc_Q4A_decode(up, ops["down_proj"].weight, H, residual=attn), orc.iadd(h(down), h(attn)), 1e-5)
 
 
 def test_decode_graph_replay_matches_eager():

@@ -205,3 +205,32 @@ def test_fc_argument_errors(ops):
         ops.fc_Q4A(x, torch.zeros(1, 2, 1000, dtype=torch.int8, device="cuda"), 32)  # not a block size
     with pytest.raises(RuntimeError):
         ops.offline_FC_quant_Q4A(torch.zeros(4, 4, 4, device="cuda"))               # rank 3 weight (ops/op_fc.hpp:152)
+
+
+@pytest.mark.parametrize("G", [32, 128])
+@pytest.mark.parametrize("rows", [1, 2, 3, 8, 20])
+def test_fc_decode_folded_ops_vs_oracle(ops, orc, G, rows):
+    """fc_Q4A_decode: rmsnorm prologue, residual epilogue and the interleaved gate/up epilogue, each
+    against the oracle's separate ops.  A folded rmsnorm may differ from the separate one by an ulp,
+    which can flip an int8 code on a rounding boundary, hence 1e-4 instead of 1e-5 there."""
+    rng = np.random.default_rng(rows + G)
+    K, F = 1024, 352
+    x = rng.standard_normal((1, rows, K)).astype(np.float32)
+    nw = (1.0 + 0.1 * rng.standard_normal(K)).astype(np.float32)
+    wg = (rng.standard_normal((F, K)) * 0.02).astype(np.float32)
+    wu = (rng.standard_normal((F, K)) * 0.02).astype(np.float32)
+    res = rng.standard_normal((1, rows, F)).astype(np.float32)
+    pg, pu = orc.quant_w(wg, G), orc.quant_w(wu, G)
+    xn = orc.rmsnorm(x, nw, 1e-5)
+    # norm only, norm + residual
+    got = host(ops.fc_Q4A_decode(dev(x), dev(pg), F, norm=(dev(nw), 1e-5)))
+    assert max_rel_err(got, orc.fc(xn, pg, F)) <= 1e-4
+    got = host(ops.fc_Q4A_decode(dev(x), dev(pg), F, norm=(dev(nw), 1e-5), residual=dev(res)))
+    assert max_rel_err(got, orc.iadd(orc.fc(xn, pg, F), res)) <= 1e-4
+    # gate/up epilogue with and without the norm
+    il = ops.interleave_gate_up(dev(pg), dev(pu))
+    assert np.array_equal(host(il)[0::2], pg) and np.array_equal(host(il)[1::2], pu)
+    want = orc.imul(orc.fc(x, pu, F), orc.silu(orc.fc(x, pg, F)))
+    assert max_rel_err(host(ops.fc_Q4A_decode(dev(x), il, F, glu=True)), want) <= 1e-5
+    want = orc.imul(orc.fc(xn, pu, F), orc.silu(orc.fc(xn, pg, F)))
+    assert max_rel_err(host(ops.fc_Q4A_decode(dev(x), il, F, norm=(dev(nw), 1e-5), glu=True)), want) <= 1e-4
