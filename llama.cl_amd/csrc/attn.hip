@@ -198,55 +198,51 @@ __global__ __launch_bounds__(256) void attn_split_kernel(const float* __restrict
 }
 
 // Merge of the chunk records of one query: out = sum_c exp(m_c - M) o_c / sum_c exp(m_c - M) s_c.
-// LOAD fetches one float of a record (plain load after a kernel boundary, device-scope load
-// inside the single-launch decode kernel).  Chunk statistics go through LDS so that every
-// thread's loads are independent of each other.
+// LOAD fetches one float of a record.
 template <typename LOAD>
-__device__ __forceinline__ float merge_chunks(const float* rec, int nchunks, int tid, int nthreads, float* stat_sh,
-                                              LOAD load) {
-    constexpr int S = 128;
-    // stat_sh[c] = max, stat_sh[nchunks + c] = sum
-    for (int i = tid; i < 2 * nchunks; i += nthreads) {
-        const int c = i % nchunks, which = i / nchunks;
-        stat_sh[i] = load(rec + (int64_t)c * (S + 2) + which);
-    }
-    __syncthreads();
-    float M = -FLT_MAX;
-    for (int c = 0; c < nchunks; c++) M = fmaxf(M, stat_sh[c]);
-    float den = 0.0f, num = 0.0f;
-    if (tid < S) {
-        for (int c0 = 0; c0 < nchunks; c0 += 32) {
-            float o[32];
+__device__ __forceinline__ float merge_chunks(const float* rec, int nchunks, int tid, LOAD load) {
+    constexpr int S = 128, CB = 32;
+    float M = -FLT_MAX, den = 0.0f, num = 0.0f;
+    // every thread reads the (few) chunk statistics itself, so all loads of a batch of chunks are
+    // independent and in flight together; batches are folded in with the running-max rescaling
+    for (int c0 = 0; c0 < nchunks; c0 += CB) {
+        float m[CB], sm[CB], o[CB];
 #pragma unroll
-            for (int u = 0; u < 32; u++) o[u] = (c0 + u < nchunks) ? load(rec + (int64_t)(c0 + u) * (S + 2) + 2 + tid) : 0.0f;
-#pragma unroll
-            for (int u = 0; u < 32; u++) {
-                if (c0 + u < nchunks) {
-                    const float sum = stat_sh[nchunks + c0 + u];
-                    const float sc = (sum == 0.0f) ? 0.0f : expf(stat_sh[c0 + u] - M);
-                    den = fmaf(sc, sum, den);
-                    num = fmaf(sc, o[u], num);
-                }
-            }
+        for (int u = 0; u < CB; u++) {
+            const bool ok = c0 + u < nchunks;
+            const float* r = rec + (int64_t)(ok ? c0 + u : c0) * (S + 2);
+            m[u] = ok ? load(r) : -FLT_MAX;
+            sm[u] = ok ? load(r + 1) : 0.0f;
+            o[u] = ok ? load(r + 2 + tid) : 0.0f;
         }
+        float Mb = M;
+#pragma unroll
+        for (int u = 0; u < CB; u++) Mb = fmaxf(Mb, m[u]);
+        const float rescale = (den == 0.0f) ? 0.0f : expf(M - Mb);
+        den *= rescale;
+        num *= rescale;
+#pragma unroll
+        for (int u = 0; u < CB; u++) {
+            const float sc = (sm[u] == 0.0f) ? 0.0f : expf(m[u] - Mb);
+            den = fmaf(sc, sm[u], den);
+            num = fmaf(sc, o[u], num);
+        }
+        M = Mb;
     }
     return num * (1.0f / den);
 }
 
-constexpr int kMaxChunks = 2048;
-
 __global__ __launch_bounds__(128) void attn_merge_kernel(float* __restrict__ q, const float* __restrict__ part, int64_t qL,
                                                           int64_t H, int nchunks) {
     constexpr int S = 128;
-    __shared__ float stat_sh[2 * kMaxChunks];
     const int64_t bhq = blockIdx.x;
     const int64_t pq = bhq % qL, h = (bhq / qL) % H, b = bhq / (qL * H);
     const float* rec = part + (int64_t)bhq * nchunks * (S + 2);
-    const float r = merge_chunks(rec, nchunks, threadIdx.x, 128, stat_sh, [](const float* p) { return *p; });
+    const float r = merge_chunks(rec, nchunks, threadIdx.x, [](const float* p) { return *p; });
     q[((b * qL + pq) * H + h) * S + threadIdx.x] = r;
 }
 
-// ---- single-launch decode attention (one query token) ------------------------------------------
+// ---- decode attention (one query token) ------------------------------------------------------
 // attention_rope2 for qL == 1 in two launches instead of three: every workgroup rotates q itself
 // (cos/sin of the position computed once per workgroup, one angle per lane), the workgroup whose
 // chunk holds the new token's cache row rotates k, writes the rotated k back in place and k, v
@@ -480,7 +476,6 @@ static int attention_impl(float* q, float* k, const float* v, int64_t B, int64_t
     const int pw = pick_pw(bhq, kvLen);
     const int nchunks = (int)((kvLen + 4 * pw - 1) / (4 * pw));
     const unsigned grid = (unsigned)(bhq * nchunks);
-    LLMOPS_REQUIRE(nchunks <= kMaxChunks);
     if (qL == 1 && (half % 4) == 0) {
         // decode: rope, cache update and split-KV attention in one launch, then the merge
         if (pw == 16)

@@ -377,6 +377,20 @@ __global__ __launch_bounds__(NW * 64) void fc_gemv_fused_kernel(const uint8_t* _
 #pragma unroll
         for (int j = 0; j < 4; j++) f[r][j] = 0.0f;
 
+    // The loads return in issue order, so everything the rmsnorm statistic needs is requested
+    // before the first weight block: the statistic is then computed while that block is in flight.
+    constexpr int NV = 4;  // float4 per thread held for the statistic (covers K <= NV*4*threads)
+    float4 nv[NORM ? MT : 1][NV];
+    if (NORM) {
+#pragma unroll
+        for (int r = 0; r < MT; r++)
+#pragma unroll
+            for (int i = 0; i < NV; i++) {
+                const int64_t e = ((int64_t)i * NW * 64 + threadIdx.x) * 4;
+                nv[NORM ? r : 0][i] = (r < rows && e < K) ? *reinterpret_cast<const float4*>(x + (int64_t)r * K + e)
+                                                         : make_float4(0.f, 0.f, 0.f, 0.f);
+            }
+    }
     // double-buffered weight blocks; the activation row of a step is fetched one step ahead
     Step<G> cur, nxt;
     XRaw<G> xcur[MT], xnxt[MT], wcur, wnxt;
@@ -390,12 +404,19 @@ __global__ __launch_bounds__(NW * 64) void fc_gemv_fused_kernel(const uint8_t* _
 
     float rsn[MT];
     if (NORM) {
-        // sum of squares of every row, while the first weight block is in flight
 #pragma unroll
         for (int r = 0; r < MT; r++) {
             float ss = 0.0f;
-            if (r < rows) {
-                for (int64_t e = (int64_t)threadIdx.x * 4; e < K; e += NW * 64 * 4) {
+#pragma unroll
+            for (int i = 0; i < NV; i++) {
+                const float4 v = nv[NORM ? r : 0][i];
+                ss = fmaf(v.x, v.x, ss);
+                ss = fmaf(v.y, v.y, ss);
+                ss = fmaf(v.z, v.z, ss);
+                ss = fmaf(v.w, v.w, ss);
+            }
+            if (r < rows) {  // rows longer than the preloaded part
+                for (int64_t e = ((int64_t)NV * NW * 64 + threadIdx.x) * 4; e < K; e += NW * 64 * 4) {
                     const float4 v = *reinterpret_cast<const float4*>(x + (int64_t)r * K + e);
                     ss = fmaf(v.x, v.x, ss);
                     ss = fmaf(v.y, v.y, ss);
