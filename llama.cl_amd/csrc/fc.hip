@@ -6,8 +6,8 @@ namespace llmops {
 
 constexpr int kMaxGemvRows = 8;
 
-int launch_quant_x(const float* x, int64_t rows, int64_t K, int group_k, int8_t* xq, float* xd, float* gsum,
-                   hipStream_t stream);
+int launch_quant_x(const float* x, int64_t rows, int64_t K, int group_k, int8_t* xq, float* xd, float* gsum, float2* xsT,
+                   bool exact_sum, hipStream_t stream);
 size_t gemv_workspace_bytes(int64_t rows, int64_t Ng, int64_t Kg, int G);
 int launch_gemv(const uint8_t* w, const int8_t* xq, const float* xd, const float* gs, float* y, float* part,
                 unsigned* counters, int64_t rows, int64_t Ng, int64_t Kg, int G, int64_t N, hipStream_t st);
@@ -17,16 +17,16 @@ int launch_gemv_fused(const uint8_t* w, const float* x, float* y, float* part, u
 int launch_add(float* a, const float* b, int64_t total, hipStream_t st);
 int launch_gemv_partials(const uint8_t* w, const int8_t* xq, int32_t* acc, int64_t rows, int64_t Ng, int64_t Kg, int G,
                          hipStream_t st);
-size_t gemm_workspace_bytes(int64_t rows, int64_t Ng, int64_t Kg);
-int launch_gemm(const uint8_t* w, const int8_t* xq, const float* xd, const float* gs, float* y, float* part,
-                int64_t rows, int64_t Ng, int64_t Kg, int G, int64_t N, hipStream_t st);
+size_t gemm_workspace_bytes(int64_t rows, int64_t Ng, int64_t Kg, int G);
+int launch_gemm(const uint8_t* w, const int8_t* xq, const float* xd, const float* gs, const float2* xsT, float* y,
+                float* part, int64_t rows, int64_t Ng, int64_t Kg, int G, int64_t N, hipStream_t st);
 int launch_gemm_partials(const uint8_t* w, const int8_t* xq, int32_t* acc, int64_t rows, int64_t Ng, int64_t Kg, int G,
                          hipStream_t st);
 
 static inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
 struct FcWorkspace {
-    size_t off_xq, off_xd, off_gs, off_part, total;
+    size_t off_xq, off_xd, off_gs, off_xst, off_part, total;
 };
 
 static FcWorkspace fc_layout(int64_t rows, int64_t Ng, int64_t Kg, int G) {
@@ -38,8 +38,10 @@ static FcWorkspace fc_layout(int64_t rows, int64_t Ng, int64_t Kg, int G) {
     o = align_up(o + (size_t)rows * Kg * sizeof(float), 256);
     w.off_gs = o;
     o = align_up(o + (size_t)rows * Kg * sizeof(float), 256);
+    w.off_xst = o;
+    o = align_up(o + (size_t)rows * Kg * 2 * sizeof(float), 256);
     w.off_part = o;
-    o = align_up(o + (rows <= kMaxGemvRows ? gemv_workspace_bytes(rows, Ng, Kg, G) : gemm_workspace_bytes(rows, Ng, Kg)), 256);
+    o = align_up(o + (rows <= kMaxGemvRows ? gemv_workspace_bytes(rows, Ng, Kg, G) : gemm_workspace_bytes(rows, Ng, Kg, G)), 256);
     w.total = o;
     return w;
 }
@@ -79,9 +81,10 @@ static int fc_impl(const float* x, int64_t rows, int64_t K, const int8_t* weiq, 
     // few rows: one launch, the streaming kernel quantizes the activations it needs on the fly
     if (rows <= kMaxGemvRows)
         return launch_gemv_fused(w, x, y, part, counters, rows, Ng, Kg, group_k, N, residual, nullptr, 0.0f, false, st);
-    int rc = launch_quant_x(x, rows, K, group_k, xq, xd, gs, st);
+    float2* xst = reinterpret_cast<float2*>(ws + lay.off_xst);
+    int rc = launch_quant_x(x, rows, K, group_k, xq, xd, gs, xst, false, st);
     if (rc) return rc;
-    rc = launch_gemm(w, xq, xd, gs, y, part, rows, Ng, Kg, group_k, N, st);
+    rc = launch_gemm(w, xq, xd, gs, xst, y, part, rows, Ng, Kg, group_k, N, st);
     if (rc || residual == nullptr) return rc;
     return launch_add(y, residual, rows * N, st);
 }
@@ -143,7 +146,7 @@ extern "C" int llmops_fc_Q4A_prequantized(const int8_t* xq, const float* xd, con
     hipStream_t st = as_stream(stream);
     if (rows <= kMaxGemvRows)
         return launch_gemv(w, xq, xd, gsum, y, part, reinterpret_cast<unsigned*>(ws), rows, Ng, Kg, group_k, N, st);
-    return launch_gemm(w, xq, xd, gsum, y, part, rows, Ng, Kg, group_k, N, st);
+    return launch_gemm(w, xq, xd, gsum, nullptr, y, part, rows, Ng, Kg, group_k, N, st);
 }
 
 extern "C" int llmops_fc_Q4A_partials(const int8_t* xq, int64_t rows, const int8_t* weiq, int64_t Ng, int64_t Kg,

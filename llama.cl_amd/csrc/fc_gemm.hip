@@ -20,6 +20,8 @@
 namespace llmops {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
+typedef unsigned int v4u __attribute__((ext_vector_type(4)));
+typedef float v2f __attribute__((ext_vector_type(2)));
 
 __device__ __forceinline__ uint32_t lo4(uint32_t w) { return w & 0x0F0F0F0Fu; }
 __device__ __forceinline__ uint32_t hi4(uint32_t w) { return (w >> 4) & 0x0F0F0F0Fu; }
@@ -160,6 +162,209 @@ __global__ __launch_bounds__(256) void fc_gemm_kernel(const uint8_t* __restrict_
         }
 }
 
+// ---- LDS-tiled kernel for group 128 ---------------------------------------------------------------
+// Workgroup = 4 wavefronts (2 x 2), tile = BM rows x 128 columns (4 strips), one k-group per
+// iteration.  Per iteration the workgroup stages into LDS, through registers and double buffered:
+//   A : BM rows x 128 activation codes (row stride 144 B so that the 16 rows a ds_read_b128 wave
+//       access touches fall into different banks)
+//   B : the 4 packed blocks as they are in memory (nibbles + fp16 d + fp16 m, 2176 B each)
+//   XS: (dx, gsum) of the BM rows for this k-group
+// The global loads of iteration kb+1 are issued before the MFMAs of iteration kb and written to the
+// other LDS buffer after them; one barrier per iteration.  Each wave owns 64 rows x 64 columns
+// (RT = BM/32 row tiles x 4 column sets); operand mapping as in mma_group above, but from LDS.
+constexpr int kAStride = 144;
+constexpr int kBlk128 = 2176;
+
+template <int RT>
+struct GemmSmem {
+    static constexpr int BM = RT * 32;
+    uint8_t a[2][BM * kAStride];
+    uint8_t b[2][4 * kBlk128];
+    float2 xs[2][BM];
+};
+
+template <int RT, bool PARTIALS>
+__global__ __launch_bounds__(256) void fc_gemm_lds_kernel(const uint8_t* __restrict__ weiq, const int8_t* __restrict__ xq,
+                                                           const float* __restrict__ xd, const float* __restrict__ gs,
+                                                           const float2* __restrict__ xsT, float* __restrict__ out,
+                                                           int32_t* __restrict__ out_i, int Ng, int Kg, int64_t ldo,
+                                                           int64_t N, int rows, int kb_per_split, int64_t split_stride) {
+    constexpr int BM = RT * 32;
+    constexpr int A_CHUNKS = BM * 8;                     // 16-byte chunks of the A tile
+    constexpr int A_PER_THREAD = A_CHUNKS / 256;         // RT
+    constexpr int B_CHUNKS = 4 * (kBlk128 / 16);         // 544
+    constexpr int B_PER_THREAD = (B_CHUNKS + 255) / 256; // 3
+    extern __shared__ __align__(16) uint8_t smem_raw[];
+    GemmSmem<RT>& sm = *reinterpret_cast<GemmSmem<RT>*>(smem_raw);
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wr = wave >> 1, wc = wave & 1;  // wave's row half / column half
+    const int g = lane >> 4, jj = lane & 15, q = jj & 7, sp = jj >> 3;
+    const int strip0 = blockIdx.x * 4;
+    const int row0 = blockIdx.y * BM;
+    const int kb0 = blockIdx.z * kb_per_split, kb1 = min(Kg, kb0 + kb_per_split);
+    const int64_t Kp = (int64_t)Kg * 128;
+
+    // ---- global -> register staging of one k-group (macros: the arrays must stay in registers) ----
+    v4u ra[A_PER_THREAD], rb[B_PER_THREAD];  // native vector types: these must live in registers
+    v2f rxs = {0.f, 0.f};
+    // per-thread source addresses that do not depend on kb
+    const int8_t* asrc[A_PER_THREAD];
+    int adst[A_PER_THREAD];
+#pragma unroll
+    for (int i = 0; i < A_PER_THREAD; i++) {
+        const int c = tid + i * 256, r = c >> 3, part = c & 7;
+        asrc[i] = xq + (int64_t)min(rows - 1, row0 + r) * Kp + part * 16;
+        adst[i] = r * kAStride + part * 16;
+    }
+    const uint8_t* bsrc[B_PER_THREAD];
+#pragma unroll
+    for (int i = 0; i < B_PER_THREAD; i++) {
+        const int c = min(B_CHUNKS - 1, tid + i * 256);
+        const int st = c / (kBlk128 / 16), off = c % (kBlk128 / 16);
+        bsrc[i] = weiq + (int64_t)min(Ng - 1, strip0 + st) * Kg * kBlk128 + off * 16;
+    }
+    const int64_t xrow = min(rows - 1, row0 + (tid < BM ? tid : 0));
+#define LLMOPS_FETCH(KB)                                                                                              \
+    do {                                                                                                              \
+        _Pragma("unroll") for (int i = 0; i < A_PER_THREAD; i++)                                                      \
+            ra[i] = *reinterpret_cast<const v4u*>(asrc[i] + (int64_t)(KB) * 128);                                     \
+        _Pragma("unroll") for (int i = 0; i < B_PER_THREAD; i++)                                                      \
+            rb[i] = *reinterpret_cast<const v4u*>(bsrc[i] + (int64_t)(KB) * kBlk128); /* clamped address */            \
+        if (!PARTIALS)                                                                                                \
+            rxs = xsT ? *reinterpret_cast<const v2f*>(&xsT[(int64_t)(KB) * rows + xrow])                             \
+                      : v2f{xd[xrow * Kg + (KB)], gs[xrow * Kg + (KB)]};                                            \
+    } while (0)
+#define LLMOPS_STASH(BUF)                                                                                  \
+    do {                                                                                                   \
+        _Pragma("unroll") for (int i = 0; i < A_PER_THREAD; i++)                                           \
+            *reinterpret_cast<v4u*>(&sm.a[BUF][adst[i]]) = ra[i];                                          \
+        _Pragma("unroll") for (int i = 0; i < B_PER_THREAD; i++)                                           \
+            if (tid + i * 256 < B_CHUNKS) *reinterpret_cast<v4u*>(&sm.b[BUF][(tid + i * 256) * 16]) = rb[i]; \
+        if (tid < BM) *reinterpret_cast<v2f*>(&sm.xs[BUF][tid]) = rxs;                                                            \
+    } while (0)
+
+    float f[RT][4][4];
+#pragma unroll
+    for (int t = 0; t < RT; t++)
+#pragma unroll
+        for (int c = 0; c < 4; c++)
+#pragma unroll
+            for (int v = 0; v < 4; v++) f[t][c][v] = 0.0f;
+
+    if (kb0 < kb1) {
+        LLMOPS_FETCH(kb0);
+        LLMOPS_STASH(0);
+    }
+    __syncthreads();
+
+    const int strip_l = wc * 2 + sp;  // strip (0..3) of the tile this lane's B operands come from
+    for (int kb = kb0; kb < kb1; kb++) {
+        const int buf = (kb - kb0) & 1;
+        if (kb + 1 < kb1) LLMOPS_FETCH(kb + 1);
+
+        const uint8_t* bblk = &sm.b[buf][strip_l * kBlk128];
+        const uint8_t* abase = &sm.a[buf][(wr * (BM / 2) + jj) * kAStride + g * 16];
+        v4i acc[RT][4];
+#pragma unroll
+        for (int t = 0; t < RT; t++)
+#pragma unroll
+            for (int c = 0; c < 4; c++) acc[t][c] = v4i{0, 0, 0, 0};
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            const uint4 wa = *reinterpret_cast<const uint4*>(bblk + h * 1024 + (2 * g) * kRowBytes + q * 16);
+            const uint4 wb = *reinterpret_cast<const uint4*>(bblk + h * 1024 + (2 * g + 1) * kRowBytes + q * 16);
+            const uint32_t* pa = reinterpret_cast<const uint32_t*>(&wa);
+            const uint32_t* pb = reinterpret_cast<const uint32_t*>(&wb);
+            v4i b[4];
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+                b[c][0] = (int)lo4(pa[c]);
+                b[c][1] = (int)hi4(pa[c]);
+                b[c][2] = (int)lo4(pb[c]);
+                b[c][3] = (int)hi4(pb[c]);
+            }
+#pragma unroll
+            for (int t = 0; t < RT; t++) {
+                const v4i a = *reinterpret_cast<const v4i*>(abase + t * 16 * kAStride + h * 64);
+#pragma unroll
+                for (int c = 0; c < 4; c++) acc[t][c] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b[c], acc[t][c], 0, 0, 0);
+            }
+        }
+
+        if (PARTIALS) {
+            const int strip = strip0 + strip_l;
+            if (strip < Ng) {
+#pragma unroll
+                for (int t = 0; t < RT; t++)
+#pragma unroll
+                    for (int v = 0; v < 4; v++) {
+                        const int row = row0 + wr * (BM / 2) + t * 16 + g * 4 + v;
+                        if (row < rows) {
+#pragma unroll
+                            for (int c = 0; c < 4; c++)
+                                out_i[((int64_t)row * ((int64_t)Ng * kGroupN) + strip * kGroupN + q * 4 + c) * Kg + kb] =
+                                    acc[t][c][v];
+                        }
+                    }
+            }
+        } else {
+            const uint2 dh = *reinterpret_cast<const uint2*>(bblk + 2048 + q * 8);
+            const uint2 mh = *reinterpret_cast<const uint2*>(bblk + 2048 + 64 + q * 8);
+            float d[4], m[4];
+            d[0] = f16_bits_to_f32((uint16_t)(dh.x & 0xFFFFu));
+            d[1] = f16_bits_to_f32((uint16_t)(dh.x >> 16));
+            d[2] = f16_bits_to_f32((uint16_t)(dh.y & 0xFFFFu));
+            d[3] = f16_bits_to_f32((uint16_t)(dh.y >> 16));
+            m[0] = f16_bits_to_f32((uint16_t)(mh.x & 0xFFFFu));
+            m[1] = f16_bits_to_f32((uint16_t)(mh.x >> 16));
+            m[2] = f16_bits_to_f32((uint16_t)(mh.y & 0xFFFFu));
+            m[3] = f16_bits_to_f32((uint16_t)(mh.y >> 16));
+#pragma unroll
+            for (int t = 0; t < RT; t++) {
+                // (dx, gsum) of the 4 rows this lane holds results for: rows wr*BM/2 + t*16 + 4g + v
+                const float4* xp = reinterpret_cast<const float4*>(&sm.xs[buf][wr * (BM / 2) + t * 16 + g * 4]);
+                const float4 x01 = xp[0], x23 = xp[1];
+                const float dxv[4] = {x01.x, x01.z, x23.x, x23.z};
+                const float gsv[4] = {x01.y, x01.w, x23.y, x23.w};
+#pragma unroll
+                for (int v = 0; v < 4; v++)
+#pragma unroll
+                    for (int c = 0; c < 4; c++) {
+                        f[t][c][v] = fmaf(d[c] * dxv[v], (float)acc[t][c][v], f[t][c][v]);
+                        f[t][c][v] = fmaf(m[c], gsv[v], f[t][c][v]);
+                    }
+            }
+        }
+
+        if (kb + 1 < kb1) LLMOPS_STASH(buf ^ 1);
+        __syncthreads();
+    }
+#undef LLMOPS_FETCH
+#undef LLMOPS_STASH
+
+    if (PARTIALS) return;
+    const int strip = strip0 + strip_l;
+    if (strip >= Ng) return;
+    float* o = out + (int64_t)blockIdx.z * split_stride;
+    const int64_t n0 = (int64_t)strip * kGroupN + q * 4;
+#pragma unroll
+    for (int t = 0; t < RT; t++)
+#pragma unroll
+        for (int v = 0; v < 4; v++) {
+            const int row = row0 + wr * (BM / 2) + t * 16 + g * 4 + v;
+            if (row >= rows) continue;
+            float* dst = o + (int64_t)row * ldo + n0;
+            if (n0 + 3 < N && (ldo & 3) == 0) {
+                *reinterpret_cast<float4*>(dst) = make_float4(f[t][0][v], f[t][1][v], f[t][2][v], f[t][3][v]);
+            } else {
+#pragma unroll
+                for (int c = 0; c < 4; c++)
+                    if (n0 + c < N) dst[c] = f[t][c][v];
+            }
+        }
+}
+
 // y[row][n] = sum over splits (index order) of part[s][row][n]
 __global__ void gemm_reduce_kernel(const float* __restrict__ part, float* __restrict__ y, int64_t rows, int64_t N,
                                    int64_t ldp, int64_t split_stride, int S) {
@@ -205,14 +410,21 @@ __global__ __launch_bounds__(256) void fc_gemm_partials_kernel(const uint8_t* __
 
 struct GemmPlan {
     int RT, S, kb_per_split;
+    bool lds;
 };
 
-static GemmPlan plan_gemm(int64_t rows, int64_t Ng, int64_t Kg) {
+static GemmPlan plan_gemm(int64_t rows, int64_t Ng, int64_t Kg, int G) {
     GemmPlan p;
-    p.RT = rows > 32 ? 4 : (rows > 16 ? 2 : 1);
-    const int64_t row_blocks = (rows + p.RT * 16 - 1) / (p.RT * 16);
-    const int64_t waves = ((Ng + 1) / 2) * row_blocks;
-    int S = (int)((2048 + waves - 1) / waves);  // aim for >= 2048 wavefronts
+    p.lds = (G == 128);
+    int64_t tiles;
+    if (p.lds) {
+        p.RT = rows > 64 ? 4 : (rows > 32 ? 2 : 1);            // BM = 32 * RT rows per workgroup
+        tiles = ((Ng + 3) / 4) * ((rows + p.RT * 32 - 1) / (p.RT * 32));
+    } else {
+        p.RT = rows > 32 ? 4 : (rows > 16 ? 2 : 1);            // RT*16 rows per wave
+        tiles = (((Ng + 1) / 2 + 3) / 4) * ((rows + p.RT * 16 - 1) / (p.RT * 16));
+    }
+    int S = (int)((512 + tiles - 1) / tiles);  // aim for >= 512 workgroups (2 per CU)
     if (S > Kg) S = (int)Kg;
     if (S < 1) S = 1;
     p.kb_per_split = (int)((Kg + S - 1) / S);
@@ -220,8 +432,8 @@ static GemmPlan plan_gemm(int64_t rows, int64_t Ng, int64_t Kg) {
     return p;
 }
 
-size_t gemm_workspace_bytes(int64_t rows, int64_t Ng, int64_t Kg) {
-    const GemmPlan p = plan_gemm(rows, Ng, Kg);
+size_t gemm_workspace_bytes(int64_t rows, int64_t Ng, int64_t Kg, int G) {
+    const GemmPlan p = plan_gemm(rows, Ng, Kg, G);
     return p.S > 1 ? (size_t)p.S * rows * Ng * kGroupN * sizeof(float) : 0;
 }
 
@@ -234,24 +446,41 @@ static void launch_gemm_t(const uint8_t* w, const int8_t* xq, const float* xd, c
                                                 split_stride);
 }
 
-int launch_gemm(const uint8_t* w, const int8_t* xq, const float* xd, const float* gs, float* y, float* part,
-                int64_t rows, int64_t Ng, int64_t Kg, int G, int64_t N, hipStream_t st) {
-    const GemmPlan p = plan_gemm(rows, Ng, Kg);
+template <int RT>
+static int launch_gemm_lds_t(const uint8_t* w, const int8_t* xq, const float* xd, const float* gs, const float2* xsT,
+                             float* out, int64_t Ng, int64_t Kg, int64_t ldo, int64_t N, int64_t rows, const GemmPlan& p,
+                             int64_t split_stride, hipStream_t st) {
+    static bool configured = false;  // opt in to more than 64 KiB of dynamic LDS once per kernel
+    if (!configured) {
+        LLMOPS_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&fc_gemm_lds_kernel<RT, false>),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(GemmSmem<RT>)));
+        configured = true;
+    }
+    dim3 grid((unsigned)((Ng + 3) / 4), (unsigned)((rows + RT * 32 - 1) / (RT * 32)), (unsigned)p.S);
+    fc_gemm_lds_kernel<RT, false><<<grid, 256, sizeof(GemmSmem<RT>), st>>>(w, xq, xd, gs, xsT, out, nullptr, (int)Ng, (int)Kg,
+                                                                          ldo, N, (int)rows, p.kb_per_split, split_stride);
+    return LLMOPS_OK;
+}
+
+int launch_gemm(const uint8_t* w, const int8_t* xq, const float* xd, const float* gs, const float2* xsT, float* y,
+                float* part, int64_t rows, int64_t Ng, int64_t Kg, int G, int64_t N, hipStream_t st) {
+    const GemmPlan p = plan_gemm(rows, Ng, Kg, G);
     const int64_t Np = Ng * kGroupN;
     float* out = p.S > 1 ? part : y;
     const int64_t ldo = p.S > 1 ? Np : N;
+    const int64_t Nw = p.S > 1 ? Np : N;
     const int64_t ss = rows * Np;
-#define LLMOPS_GEMM_CASE(GG, RR) launch_gemm_t<GG, RR>(w, xq, xd, gs, out, Ng, Kg, ldo, p.S > 1 ? Np : N, rows, p, ss, st)
-    if (G == 128) {
-        if (p.RT == 4) LLMOPS_GEMM_CASE(128, 4);
-        else if (p.RT == 2) LLMOPS_GEMM_CASE(128, 2);
-        else LLMOPS_GEMM_CASE(128, 1);
+    if (p.lds) {
+        int rc;
+        if (p.RT == 4) rc = launch_gemm_lds_t<4>(w, xq, xd, gs, xsT, out, Ng, Kg, ldo, Nw, rows, p, ss, st);
+        else if (p.RT == 2) rc = launch_gemm_lds_t<2>(w, xq, xd, gs, xsT, out, Ng, Kg, ldo, Nw, rows, p, ss, st);
+        else rc = launch_gemm_lds_t<1>(w, xq, xd, gs, xsT, out, Ng, Kg, ldo, Nw, rows, p, ss, st);
+        if (rc) return rc;
     } else {
-        if (p.RT == 4) LLMOPS_GEMM_CASE(32, 4);
-        else if (p.RT == 2) LLMOPS_GEMM_CASE(32, 2);
-        else LLMOPS_GEMM_CASE(32, 1);
+        if (p.RT == 4) launch_gemm_t<32, 4>(w, xq, xd, gs, out, Ng, Kg, ldo, Nw, rows, p, ss, st);
+        else if (p.RT == 2) launch_gemm_t<32, 2>(w, xq, xd, gs, out, Ng, Kg, ldo, Nw, rows, p, ss, st);
+        else launch_gemm_t<32, 1>(w, xq, xd, gs, out, Ng, Kg, ldo, Nw, rows, p, ss, st);
     }
-#undef LLMOPS_GEMM_CASE
     LLMOPS_LAUNCH_CHECK();
     if (p.S > 1) {
         const int64_t total = rows * N;
@@ -263,11 +492,20 @@ int launch_gemm(const uint8_t* w, const int8_t* xq, const float* xd, const float
 
 int launch_gemm_partials(const uint8_t* w, const int8_t* xq, int32_t* acc, int64_t rows, int64_t Ng, int64_t Kg, int G,
                          hipStream_t st) {
-    dim3 grid((unsigned)(((Ng + 1) / 2 + 3) / 4), (unsigned)((rows + 15) / 16), (unsigned)Kg);
-    if (G == 128)
-        fc_gemm_partials_kernel<128><<<grid, 256, 0, st>>>(w, xq, acc, (int)Ng, (int)Kg, (int)rows);
-    else
+    if (G == 128) {  // the production LDS-tiled loop, writing its int32 tiles instead of folding them
+        static bool configured = false;
+        if (!configured) {
+            LLMOPS_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&fc_gemm_lds_kernel<2, true>),
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(GemmSmem<2>)));
+            configured = true;
+        }
+        dim3 grid((unsigned)((Ng + 3) / 4), (unsigned)((rows + 63) / 64), 1);
+        fc_gemm_lds_kernel<2, true><<<grid, 256, sizeof(GemmSmem<2>), st>>>(w, xq, nullptr, nullptr, nullptr, nullptr, acc,
+                                                                          (int)Ng, (int)Kg, 0, 0, (int)rows, (int)Kg, 0);
+    } else {
+        dim3 grid((unsigned)(((Ng + 1) / 2 + 3) / 4), (unsigned)((rows + 15) / 16), (unsigned)Kg);
         fc_gemm_partials_kernel<32><<<grid, 256, 0, st>>>(w, xq, acc, (int)Ng, (int)Kg, (int)rows);
+    }
     LLMOPS_LAUNCH_CHECK();
     return LLMOPS_OK;
 }

@@ -20,10 +20,13 @@ __device__ __forceinline__ int q8_code(float v, float id) {
     return (int)fminf(127.0f, fmaxf(-128.0f, rintf(t)));
 }
 
-template <int G>
+// EXACT_SUM: raw group sum accumulated left to right (bit-equal to the reference); otherwise a
+// tree sum, which is what the prefill FC uses (the sum only feeds its fp32 output).
+// xsT (optional): the same scale and sum again as float2 [Kg][rows] for the GEMM's tile loads.
+template <int G, bool EXACT_SUM>
 __global__ __launch_bounds__(256) void quant_x_kernel(const float* __restrict__ x, int64_t rows, int64_t K, int64_t Kg,
                                                        int8_t* __restrict__ xq, float* __restrict__ xd,
-                                                       float* __restrict__ gsum) {
+                                                       float* __restrict__ gsum, float2* __restrict__ xsT) {
     constexpr int E = (G >= 64) ? G / 64 : 1;  // elements per lane
     constexpr int LANES = G / E;               // lanes that hold data
     const int lane = threadIdx.x & 63;
@@ -60,15 +63,22 @@ __global__ __launch_bounds__(256) void quant_x_kernel(const float* __restrict__ 
         }
     }
 
-    // left-to-right fp32 sum of the raw group, computed redundantly by every lane
     float s = 0.0f;
+    if (EXACT_SUM) {
+        // left-to-right fp32 sum of the raw group, computed redundantly by every lane
 #pragma unroll
-    for (int i = 0; i < G; i++) {
-        if (i < len) s += lane_value(v[i % E], i / E);
+        for (int i = 0; i < G; i++) {
+            if (i < len) s += lane_value(v[i % E], i / E);
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < E; j++) s += v[j];
+        s = wave_sum(s);
     }
     if (lane == 0) {
         xd[r * Kg + kb] = d;
         gsum[r * Kg + kb] = s;
+        if (xsT != nullptr) xsT[kb * rows + r] = make_float2(d, s);
     }
 }
 
@@ -78,15 +88,18 @@ using namespace llmops;
 
 namespace llmops {
 // shared with fc.hip
-int launch_quant_x(const float* x, int64_t rows, int64_t K, int group_k, int8_t* xq, float* xd, float* gsum,
-                   hipStream_t stream) {
+int launch_quant_x(const float* x, int64_t rows, int64_t K, int group_k, int8_t* xq, float* xd, float* gsum, float2* xsT,
+                   bool exact_sum, hipStream_t stream) {
     const int64_t Kg = (K + group_k - 1) / group_k;
     const int64_t items = rows * Kg;
     const unsigned grid = (unsigned)((items + 3) / 4);
-    if (group_k == 32)
-        quant_x_kernel<32><<<grid, 256, 0, stream>>>(x, rows, K, Kg, xq, xd, gsum);
-    else
-        quant_x_kernel<128><<<grid, 256, 0, stream>>>(x, rows, K, Kg, xq, xd, gsum);
+    if (group_k == 32) {
+        if (exact_sum) quant_x_kernel<32, true><<<grid, 256, 0, stream>>>(x, rows, K, Kg, xq, xd, gsum, xsT);
+        else quant_x_kernel<32, false><<<grid, 256, 0, stream>>>(x, rows, K, Kg, xq, xd, gsum, xsT);
+    } else {
+        if (exact_sum) quant_x_kernel<128, true><<<grid, 256, 0, stream>>>(x, rows, K, Kg, xq, xd, gsum, xsT);
+        else quant_x_kernel<128, false><<<grid, 256, 0, stream>>>(x, rows, K, Kg, xq, xd, gsum, xsT);
+    }
     LLMOPS_LAUNCH_CHECK();
     return LLMOPS_OK;
 }
@@ -100,5 +113,5 @@ extern "C" int llmops_FC_dynamic_quantize_x(const float* x, int64_t rows, int64_
     LLMOPS_REQUIRE(aligned(xq, 2));
     const int64_t Kg = (K + group_k - 1) / group_k;
     LLMOPS_REQUIRE(rows * Kg < ((int64_t)1 << 33));
-    return launch_quant_x(x, rows, K, group_k, xq, xd, gsum, as_stream(stream));
+    return launch_quant_x(x, rows, K, group_k, xq, xd, gsum, nullptr, true, as_stream(stream));
 }
