@@ -22,6 +22,7 @@ namespace llmops {
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef unsigned int v4u __attribute__((ext_vector_type(4)));
 typedef float v2f __attribute__((ext_vector_type(2)));
+typedef float v4f __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ uint32_t lo4(uint32_t w) { return w & 0x0F0F0F0Fu; }
 __device__ __forceinline__ uint32_t hi4(uint32_t w) { return (w >> 4) & 0x0F0F0F0Fu; }
@@ -184,7 +185,7 @@ struct GemmSmem {
 };
 
 template <int RT, bool PARTIALS>
-__global__ __launch_bounds__(256) void fc_gemm_lds_kernel(const uint8_t* __restrict__ weiq, const int8_t* __restrict__ xq,
+__global__ __launch_bounds__(256, 2) void fc_gemm_lds_kernel(const uint8_t* __restrict__ weiq, const int8_t* __restrict__ xq,
                                                            const float* __restrict__ xd, const float* __restrict__ gs,
                                                            const float2* __restrict__ xsT, float* __restrict__ out,
                                                            int32_t* __restrict__ out_i, int Ng, int Kg, int64_t ldo,
@@ -244,13 +245,20 @@ __global__ __launch_bounds__(256) void fc_gemm_lds_kernel(const uint8_t* __restr
         if (tid < BM) *reinterpret_cast<v2f*>(&sm.xs[BUF][tid]) = rxs;                                                            \
     } while (0)
 
-    float f[RT][4][4];
+    v4f f[RT][4];
 #pragma unroll
     for (int t = 0; t < RT; t++)
 #pragma unroll
-        for (int c = 0; c < 4; c++)
+        for (int c = 0; c < 4; c++) f[t][c] = v4f{0.f, 0.f, 0.f, 0.f};
+    // Min term sum_kb m[n,kb]*gsum[row,kb]: a rank-Kg product, done four k-groups at a time by
+    // v_mfma_f32_16x16x4_f32 straight into the fp32 accumulators (same tile layout as the int8
+    // MFMAs).  Lane (jj, g) keeps gsum of row jj and m of its columns for the group with index g
+    // of the current four.
+    float gk[RT], mk[4];
 #pragma unroll
-            for (int v = 0; v < 4; v++) f[t][c][v] = 0.0f;
+    for (int t = 0; t < RT; t++) gk[t] = 0.0f;
+#pragma unroll
+    for (int c = 0; c < 4; c++) mk[c] = 0.0f;
 
     if (kb0 < kb1) {
         LLMOPS_FETCH(kb0);
@@ -320,20 +328,32 @@ __global__ __launch_bounds__(256) void fc_gemm_lds_kernel(const uint8_t* __restr
             m[1] = f16_bits_to_f32((uint16_t)(mh.x >> 16));
             m[2] = f16_bits_to_f32((uint16_t)(mh.y & 0xFFFFu));
             m[3] = f16_bits_to_f32((uint16_t)(mh.y >> 16));
+            const int slot4 = (kb - kb0) & 3;
+            const bool mine4 = slot4 == g;
+#pragma unroll
+            for (int c = 0; c < 4; c++) mk[c] = mine4 ? m[c] : mk[c];
 #pragma unroll
             for (int t = 0; t < RT; t++) {
-                // (dx, gsum) of the 4 rows this lane holds results for: rows wr*BM/2 + t*16 + 4g + v
+                const float gsr = sm.xs[buf][wr * (BM / 2) + t * 16 + jj].y;
+                gk[t] = mine4 ? gsr : gk[t];
+                // dx of the 4 rows this lane holds results for: rows wr*BM/2 + t*16 + 4g + v
                 const float4* xp = reinterpret_cast<const float4*>(&sm.xs[buf][wr * (BM / 2) + t * 16 + g * 4]);
                 const float4 x01 = xp[0], x23 = xp[1];
                 const float dxv[4] = {x01.x, x01.z, x23.x, x23.z};
-                const float gsv[4] = {x01.y, x01.w, x23.y, x23.w};
 #pragma unroll
                 for (int v = 0; v < 4; v++)
 #pragma unroll
-                    for (int c = 0; c < 4; c++) {
-                        f[t][c][v] = fmaf(d[c] * dxv[v], (float)acc[t][c][v], f[t][c][v]);
-                        f[t][c][v] = fmaf(m[c], gsv[v], f[t][c][v]);
-                    }
+                    for (int c = 0; c < 4; c++) f[t][c][v] = fmaf(d[c] * dxv[v], (float)acc[t][c][v], f[t][c][v]);
+            }
+            if (slot4 == 3 || kb + 1 == kb1) {
+#pragma unroll
+                for (int t = 0; t < RT; t++) {
+#pragma unroll
+                    for (int c = 0; c < 4; c++) f[t][c] = __builtin_amdgcn_mfma_f32_16x16x4f32(gk[t], mk[c], f[t][c], 0, 0, 0);
+                    gk[t] = 0.0f;
+                }
+#pragma unroll
+                for (int c = 0; c < 4; c++) mk[c] = 0.0f;
             }
         }
 
