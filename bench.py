@@ -56,7 +56,13 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-decode", action="store_true", help="skip the full decode-step timing (BASELINE config 5)")
+    ap.add_argument("--no-extra", action="store_true", help="skip the prefill GEMM (config 3) and attention (config 4) legs")
+    ap.add_argument("--calib", action="store_true",
+                    help="only run the plain copy/read kernels over 1 GiB (reference points for traffic counters and "
+                         "for the attainable HBM rate) and print their rates")
     args = ap.parse_args()
+    if args.calib:
+        return calib()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU (the path is data-parallel per GPU; multi-GPU sharding is design "
               "only, see DESIGN.md). Re-run with --gpus 1.", file=sys.stderr)
@@ -162,8 +168,20 @@ def main():
     }
     if not args.no_decode:
         out["decode_step"] = decode_step(torch, stream)
+    if not args.no_extra:
+        out["prefill_gemm"] = prefill_gemm(torch, llmops, stream)
+        out["decode_attention"] = decode_attention(torch, llmops, stream)
     if not args.no_cpu:
-        out["cpu_baseline"] = cpu_baseline()
+        # the reference's allocator announces itself on stdout (ops/tensor.hpp:88-91); keep stdout for the JSON line
+        sys.stdout.flush()
+        saved = os.dup(1)
+        os.dup2(2, 1)
+        try:
+            out["cpu_baseline"] = cpu_baseline()
+        finally:
+            sys.stdout.flush()
+            os.dup2(saved, 1)
+            os.close(saved)
     out["setup_s"] = round(setup_s, 1)
     print(json.dumps(out))
 
@@ -239,6 +257,105 @@ def decode_step(torch, stream, kv_len=2048, reps=20):
     return out
 
 
+def calib(nbytes=1 << 30, reps=5):
+    """Plain copy (reads nbytes, writes nbytes per launch) and plain read (reads nbytes) with 16-byte accesses."""
+    import ctypes
+    import torch
+    import llmops
+    lib = llmops._lib.load()
+    src = torch.randint(0, 255, (nbytes,), dtype=torch.uint8, device="cuda")
+    dst = torch.empty_like(src)
+    out4 = torch.zeros(4, dtype=torch.int32, device="cuda")
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    res = {"bytes": nbytes}
+    for name, fn in (("copy", lambda: lib.llmops_calib_copy(src.data_ptr(), dst.data_ptr(), nbytes, 4096, st)),
+                     ("read", lambda: lib.llmops_calib_read(src.data_ptr(), nbytes, 8192, out4.data_ptr(), st))):
+        fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            llmops._lib.check(fn())
+        e1.record()
+        torch.cuda.synchronize()
+        us = e0.elapsed_time(e1) * 1e3 / reps
+        res[name] = {"us": round(us, 1), "GB/s_read": round(nbytes / us / 1e3, 1)}
+    print(json.dumps({"calib": res}))
+
+
+INT8_MFMA_PEAK_TOPS = 5033.0  # MI355X published dense int8 rate
+
+
+def _time_graph(torch, stream, fn, reps=5):
+    """Average milliseconds of one fn() call inside a replayed HIP graph (HIP events on the launch stream)."""
+    fn()
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g, stream=stream):
+        fn()
+    g.replay()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record(stream)
+    for _ in range(reps):
+        g.replay()
+    e1.record(stream)
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / reps
+
+
+def prefill_gemm(torch, llmops, stream):
+    """BASELINE config 3: Q4_1(128) prefill FC, x fp32 [1,M,K], M in {16,128,512,2048}, 4096->11008 and
+    11008->4096.  Time covers activation quantization + int8 MFMA GEMM (+ split-K reduce), cycling 8 distinct
+    weight copies.  Q8 activation groups are 128 wide, like the weights (the reference has one group size)."""
+    out = {}
+    gen = torch.Generator(device="cpu").manual_seed(3)
+    with torch.cuda.stream(stream):
+        for N, K in ((11008, 4096), (4096, 11008)):
+            w0 = llmops.offline_FC_quant_Q4A((torch.randn(N, K, generator=gen) * 0.02).cuda(), G)
+            ws = [torch.roll(w0, i + 1, 0).contiguous() for i in range(8)]
+            for M in (16, 128, 512, 2048):
+                x = torch.randn(1, M, K, generator=gen).cuda()
+
+                def run():
+                    for w in ws:
+                        llmops.fc_Q4A(x, w, N)
+
+                us = _time_graph(torch, stream, run) * 1e3 / len(ws)
+                ops = 2.0 * M * N * K
+                out[f"{K}->{N} M={M}"] = {"us": round(us, 2), "TOPS": round(ops / us / 1e6, 1),
+                                          "pct_int8_mfma_peak": round(ops / us / 1e6 / INT8_MFMA_PEAK_TOPS * 100, 2),
+                                          "GB/s": round(fc_bytes(N, K, M) / us / 1e3, 1)}
+            del ws, w0
+    return out
+
+
+def decode_attention(torch, llmops, stream):
+    """BASELINE config 4: decode attention with rotary over the KV cache: 32 heads x 128, one query token,
+    kv-len 256 / 2048, fp32 and fp16 cache, cycling the 32 layers' planes of one cache."""
+    out = {}
+    H, S, layers = 32, 128, 32
+    gen = torch.Generator(device="cpu").manual_seed(4)
+    inv_freq = (1.0 / (10000.0 ** (torch.arange(0, S, 2).float() / S))).cuda()
+    with torch.cuda.stream(stream):
+        for kv in (256, 2048):
+            for name, dt, e in (("fp32", torch.float32, 4), ("fp16", torch.float16, 2)):
+                cache = torch.randn(2 * layers, 1, H, kv, S, generator=gen).to(dt).cuda()
+                q, k, v = (torch.randn(1, 1, H * S, generator=gen).cuda() for _ in range(3))
+                slots = torch.tensor([kv - 1], dtype=torch.int32).cuda()
+
+                def run():
+                    for layer in range(layers):
+                        llmops.attention_rope2(q, k, v, inv_freq, cache, slots, kv - 1, layer)
+
+                us = _time_graph(torch, stream, run) * 1e3 / layers
+                byts = 2 * H * kv * S * e + 16 * H * S
+                out[f"kv={kv} {name}"] = {"us": round(us, 2), "GB/s": round(byts / us / 1e3, 1),
+                                          "pct_hbm_peak": round(byts / us / 1e3 / HBM_PEAK_GBS * 100, 2), "bytes": byts}
+                del cache
+    return out
+
+
 def cpu_baseline(budget_s=12.0):
     """The CPU path timed on this machine's host cores: a bounded sample (whole layers of the same FC
     set, cycling distinct weight copies as ops/perf_ops.py:234-241 does) for about `budget_s` seconds."""
@@ -267,11 +384,62 @@ def cpu_baseline(budget_s=12.0):
         done += 1
     dt = time.perf_counter() - t0
     layer_bytes = sum(fc_bytes(N, K) for _, N, K in LAYER_FCS)
-    return {"value": round(done * layer_bytes / dt / 1e9, 2), "unit": "GB/s", "cores": eng.max_threads(), "kind": kind,
-            "isa": eng.isa,
-            "sample": f"{done} passes over one layer's 7 decode FCs (Q4_1 g128, M=1), cycling {copies} distinct "
-                      f"layer weight sets, {dt:.1f} s", "ms_per_layer": round(dt / done * 1e3, 3),
-            "ms_per_32_layers": round(dt / done * 32e3, 2)}
+    res = {"value": round(done * layer_bytes / dt / 1e9, 2), "unit": "GB/s", "cores": eng.max_threads(), "kind": kind,
+           "isa": eng.isa,
+           "sample": f"{done} passes over one layer's 7 decode FCs (Q4_1 g128, M=1), cycling {copies} distinct "
+                     f"layer weight sets, {dt:.1f} s", "ms_per_layer": round(dt / done * 1e3, 3),
+           "ms_per_32_layers": round(dt / done * 32e3, 2)}
+    # the other two pieces of a decode step on the same host cores: attention over a 2048-row fp32 cache
+    # (4 layers' planes cycled) and the 55296x4096 lm_head, a few seconds each
+    H, S, kv, nl = 32, 128, 2048, 4
+    cache = rng.standard_normal((2 * nl, 1, H, kv, S)).astype(np.float32)
+    q, k, v = (rng.standard_normal((1, 1, H * S)).astype(np.float32) for _ in range(3))
+    inv_freq = (1.0 / (10000.0 ** (np.arange(0, S, 2, dtype=np.float32) / np.float32(S)))).astype(np.float32)
+    slots = np.array([kv - 1], np.int32)
+    att = _CpuAttention(eng, q, k, v, inv_freq, cache, slots, kv - 1)
+    att.run(0)
+    n, t0 = 0, time.perf_counter()
+    while time.perf_counter() - t0 < 4.0:
+        att.run(n % nl)
+        n += 1
+    attn_ms = (time.perf_counter() - t0) / n * 1e3
+    wl = O.quant_w((rng.standard_normal((55296, 4096)) * 0.02).astype(np.float32), G)
+    eng.fc(xs[4096], wl, 55296)
+    n, t0 = 0, time.perf_counter()
+    while time.perf_counter() - t0 < 3.0:
+        eng.fc(xs[4096], wl, 55296)
+        n += 1
+    head_ms = (time.perf_counter() - t0) / n * 1e3
+    res["decode_step_cpu"] = {"attention_ms_per_layer_kv2048_fp32": round(attn_ms, 3), "lm_head_ms": round(head_ms, 3),
+                              "ms_per_token_fc_attention_lm_head": round(32 * (dt / done * 1e3 + attn_ms) + head_ms, 2),
+                              "note": "32 x (7 FCs + attention_rope2 at kv-len 2048) + lm_head; norms and element-wise ops "
+                                      "not included"}
+    return res
+
+
+class _CpuAttention:
+    """attention_rope2 on the host through the raw C entry point (no array copies inside the timed call)."""
+
+    def __init__(self, eng, q, k, v, inv_freq, cache, slots, pos):
+        import ctypes
+        self.eng, self.arrs, self.pos = eng, (q, k, v, inv_freq, cache, slots), pos
+        self.c = ctypes
+
+    def run(self, layer):
+        c = self.c
+        q, k, v, f, cache, slots = self.arrs
+        P = lambda a: c.c_void_p(a.ctypes.data)
+        i64 = c.c_int64
+        planes, B, H, maxlen, S = cache.shape
+        if self.eng.kind == "reference":
+            self.eng._warm_rope_table(f)
+            rc = self.eng.lib.ref_attention_rope(c.c_int(2), P(q), P(k), P(v), i64(B), i64(1), i64(H), i64(S), P(f),
+                                                 i64(f.shape[0]), P(cache), i64(planes), i64(maxlen), P(slots),
+                                                 c.c_int(self.pos), c.c_int(layer))
+            assert rc == 0
+        else:
+            self.eng.lib.orc_attention(P(q), P(k), P(v), i64(B), i64(1), i64(H), i64(S), P(f), i64(f.shape[0]), P(cache),
+                                       i64(planes), i64(maxlen), P(slots), c.c_int(self.pos), c.c_int(layer))
 
 
 if __name__ == "__main__":
