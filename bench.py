@@ -10,7 +10,7 @@ one pass over all 224 FCs through the C ABI (`llmops_fc_Q4A`), replayed as a HIP
 weights are resident in HBM before the timed region.
 
 Prints one JSON line: whole-job GB/s over the algorithmic bytes (packed weights + fp32 x + fp32 y),
-the roofline record of the dominant kernel (`fc_gemv_kernel`), and the CPU baseline (the
+the roofline record of the dominant kernel (`fc_gemv_fused_kernel`), and the CPU baseline (the
 reference's own AVX kernels from oracle/_ref when present, else this repo's C restatement) timed
 on this machine's host cores over a bounded sample of the same workload.
 """
@@ -25,6 +25,12 @@ sys.path.insert(0, ROOT)
 sys.path.insert(0, os.path.join(ROOT, "llama.cl_amd"))
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
+# HBM bytes per launch of the dominant kernel over the fused plan, from hardware counters: FETCH_SIZE and WRITE_SIZE
+# of two `rocprofv3 --pmc` runs of this file, each scaled by what the same counter reads for the plain 1 GiB copy
+# of `--calib` (one FETCH_SIZE count = 2.000 KiB, one WRITE_SIZE count = 1.000 KiB on this part); the summary with
+# the per-shape figures is profiles/fc_gemv_fused_kernel__hbm_traffic_pmc.md.  Counters cannot be read from inside
+# this process, so the figure is the recorded one and only holds for the fused plan at group 128, M=1.
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 27158024
 G = 128
 LAYERS = 32
 # (name, N, K) of one layer's FCs, in the order the model calls them (chatllama/main.py:344-375)
@@ -136,8 +142,9 @@ def main():
     value = step_bytes / (main_r["ms_per_step"] * 1e-3) / 1e9
     avg_us = main_r["event_ms_per_step"] * 1e3 / main_r["launches"]
     achieved = step_bytes / (main_r["event_ms_per_step"] * 1e-3) / 1e9
-    roof = {"bound": "hbm", "kernel": "fc_gemv_fused_kernel<128,1,16,1>", "achieved": round(achieved, 1),
-            "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+    roof = {"bound": "hbm", "kernel": "fc_gemv_fused_kernel<128,1,16,0>", "achieved": round(achieved, 1),
+            "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH,
+            "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a 1 GiB copy kernel (recorded run)",
             "avg_launch_us": round(avg_us, 3), "launches_per_step": main_r["launches"],
             "bytes_per_launch_avg": int(step_bytes / main_r["launches"]), "per_shape": per_shape,
             "dispatch_floor_us": round(floor_us, 3),
