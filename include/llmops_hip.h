@@ -183,6 +183,53 @@ int llmops_embedding_q8c(float* out, const int64_t* ids, int64_t n, const int8_t
 int llmops_embedding(float* out, const int64_t* ids, int64_t n, const float* w, int64_t V, int64_t E, llmops_stream_t stream);
 
 /* ------------------------------------------------------------------------------------------
+ * A chain of dependent single-row FCs in one persistent launch
+ * ------------------------------------------------------------------------------------------
+ * What a decoder layer does between two attention calls (chatllama/main.py:344-375): rmsnorm ->
+ * fc_Q4A (q|k|v) ... fc_Q4A (o) -> iadd -> rmsnorm -> fc_Q4A (gate, up) -> itrans("silu"), imul ->
+ * fc_Q4A (down) -> iadd.  Each op is llmops_fc_Q4A_decode with rows = 1; op i+1 may take op i's
+ * output as its input (x = NULL).  One resident grid runs all ops, keeps the next op's weights
+ * streaming while an op's result crosses the chip, and separates consecutive ops by one grid-wide
+ * barrier (also when op i+1 reads an external x).  Outputs equal llmops_fc_Q4A_decode's within
+ * fp32 summation order (the int32 dot products are the same).
+ *
+ * Rules: K = Kg*group_k <= 16384; group 32 needs an even Kg; glu excludes residual; an external x
+ * must not be the y of an earlier op of the chain (use x = NULL for the previous op's output);
+ * residual must not be the y of the immediately preceding op (it may be any other y, and it may
+ * be the op's own y: in-place h += fc(...)).  */
+typedef struct llmops_chain_op {
+    const int8_t* weiq;    /* packed [Ng][Kg][block]; glu: gate/up strips interleaved */
+    int64_t Ng, Kg;
+    int64_t N_out;         /* outputs (glu: of silu(gate)*up) */
+    const float* x;        /* fp32 [K], or NULL = output of the previous op */
+    const float* norm_w;   /* optional fp32 [K]: rmsnorm(x)*norm_w first */
+    const float* residual; /* optional fp32 [N_out], added to the output */
+    float* y;              /* fp32 [N_out], always written */
+    float eps;
+    int32_t glu;
+} llmops_chain_op;
+
+/* bytes of device memory for the plan (op table) of n_ops ops */
+size_t llmops_fc_chain_plan_bytes(int n_ops);
+/* workspace bytes (sync words + one partial-sum region per op) for this chain on the current device */
+int llmops_fc_chain_workspace_bytes(const llmops_chain_op* ops, int n_ops, int group_k, size_t* bytes);
+/* Validates the chain, cuts every op over the device's compute units and writes the op table to
+ * `plan` (device memory) with a synchronous copy: call it outside stream capture.  The first 256
+ * bytes of `workspace` must be zero when the library first sees it and are left zero by every
+ * launch that ends with status 0.  `ops` itself is not referenced after the call. */
+int llmops_fc_chain_build(const llmops_chain_op* ops, int n_ops, int group_k, void* plan, size_t plan_bytes,
+                          void* workspace, size_t workspace_bytes);
+/* Enqueues the chain (one kernel; capturable).  Two launches that share a workspace must not overlap. */
+int llmops_fc_chain_run(const void* plan, int n_ops, int group_k, void* workspace, llmops_stream_t stream);
+/* Synchronous read of the chain's status word: 0 = ok, 1 = a barrier wait ran out (the grid was
+ * not co-resident or a launch overlapped another), 2 = plan built for another grid.  After a
+ * non-zero status the outputs are invalid and the first 256 workspace bytes must be zeroed again. */
+int llmops_fc_chain_status(const void* workspace, int32_t* status);
+/* knobs: LDS ring depth in steps per wavefront (2..4, 0 = default), workgroups (0 = one per CU),
+ * barrier wait limit in 100 MHz ticks (<= 0 keeps it) */
+void llmops_fc_chain_set_tuning(int ring_depth, int grid, long long spin_limit_ticks);
+
+/* ------------------------------------------------------------------------------------------
  * Measurement helpers (no counterpart in the reference; used by bench.py and the profiles)
  * ------------------------------------------------------------------------------------------ */
 

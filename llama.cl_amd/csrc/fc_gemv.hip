@@ -30,113 +30,9 @@
 // sums are exact, the fp32 accumulation order differs from the reference's kb-sequential chain
 // (bounded well inside the 1e-3 contract).
 #include "common.h"
+#include "gemv_device.h"
 
 namespace llmops {
-
-// weights are read exactly once: non-temporal loads keep them from displacing the activations,
-// scales and partial sums that are reused out of the caches
-typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
-__device__ __forceinline__ uint4 ldg16(const uint8_t* p) {
-    const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
-    return make_uint4(v.x, v.y, v.z, v.w);
-}
-__device__ __forceinline__ uint2 ldg8(const uint8_t* p) { return *reinterpret_cast<const uint2*>(p); }
-
-// ---- lane exchanges on the VALU (DPP), no LDS round trips --------------------------------------
-template <int CTRL>
-__device__ __forceinline__ float dpp(float v) {
-    return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(v), __float_as_int(v), CTRL, 0xF, 0xF, false));
-}
-__device__ __forceinline__ float lane_bcast(float v, int lane) {
-    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), lane));
-}
-constexpr int kQuadXor1 = 0xB1, kQuadXor2 = 0x4E, kRowHalfMirror = 0x141, kRowMirror = 0x140, kRowRor8 = 0x128;
-
-// max and sum over each row of 16 lanes, result in every lane of the row
-__device__ __forceinline__ void row16_max_sum(float& mx, float& sm) {
-    mx = fmaxf(mx, dpp<kQuadXor1>(mx));
-    sm += dpp<kQuadXor1>(sm);
-    mx = fmaxf(mx, dpp<kQuadXor2>(mx));
-    sm += dpp<kQuadXor2>(sm);
-    mx = fmaxf(mx, dpp<kRowHalfMirror>(mx));
-    sm += dpp<kRowHalfMirror>(sm);
-    mx = fmaxf(mx, dpp<kRowMirror>(mx));
-    sm += dpp<kRowMirror>(sm);
-}
-
-// One "step" of a wavefront: G=128 -> one block (two 16 B loads per lane);
-//                            G=32  -> two adjacent blocks, one per half-wave (one load per lane).
-template <int G>
-struct Step {
-    static constexpr int kLoads = (G == 128) ? 2 : 1;
-    static constexpr int kBlocksPerStep = (G == 128) ? 1 : 2;
-    static constexpr int kK = (G == 128) ? 128 : 64;  // k-values per step
-    uint4 w[kLoads];
-    uint2 dh, mh;  // 4 x fp16 d, 4 x fp16 m of the lane's columns
-    bool valid;
-};
-
-template <int G>
-__device__ __forceinline__ void load_step(Step<G>& st, const uint8_t* strip, int step, int kb_end, int lane) {
-    const int quad = lane & 7, rs = lane >> 3;
-    if (G == 128) {
-        const uint8_t* blk = strip + (int64_t)step * block_bytes(128);
-        st.valid = true;
-        st.w[0] = ldg16(blk + lane * 16);
-        st.w[Step<G>::kLoads - 1] = ldg16(blk + 1024 + lane * 16);
-        st.dh = ldg8(blk + 2048 + quad * 8);
-        st.mh = ldg8(blk + 2048 + 64 + quad * 8);
-    } else {
-        const int kb = step * 2 + (rs >> 2);
-        st.valid = kb < kb_end;
-        const uint8_t* blk = strip + (int64_t)kb * block_bytes(32);
-        if (st.valid) {
-            st.w[0] = ldg16(blk + (rs & 3) * kRowBytes + quad * 16);
-            st.dh = ldg8(blk + 512 + quad * 8);
-            st.mh = ldg8(blk + 512 + 64 + quad * 8);
-        } else {
-            st.w[0] = make_uint4(0, 0, 0, 0);
-            st.dh = make_uint2(0, 0);
-            st.mh = make_uint2(0, 0);
-        }
-    }
-}
-
-// int32 partial dot products of the lane's 4 columns over the lane's k8-rows of this step;
-// `codes` points at the step's activation codes (Step<G>::kK of them)
-template <int G>
-__device__ __forceinline__ void dot_step(const Step<G>& st, const int8_t* codes, int lane, int acc[4]) {
-    const int rs = lane >> 3;
-    const int2 xa = *reinterpret_cast<const int2*>(codes + rs * 8);
-    const uint32_t* w0 = reinterpret_cast<const uint32_t*>(&st.w[0]);
-#pragma unroll
-    for (int j = 0; j < 4; j++) acc[j] = dot8_q4(w0[j], xa.x, xa.y, 0);
-    if (G == 128) {
-        const int2 xb = *reinterpret_cast<const int2*>(codes + 64 + rs * 8);
-        const uint32_t* w1 = reinterpret_cast<const uint32_t*>(&st.w[Step<G>::kLoads - 1]);
-#pragma unroll
-        for (int j = 0; j < 4; j++) acc[j] = dot8_q4(w1[j], xb.x, xb.y, acc[j]);
-    }
-}
-
-__device__ __forceinline__ void unpack_h4(uint2 h, float out[4]) {
-    out[0] = f16_bits_to_f32((uint16_t)(h.x & 0xFFFFu));
-    out[1] = f16_bits_to_f32((uint16_t)(h.x >> 16));
-    out[2] = f16_bits_to_f32((uint16_t)(h.y & 0xFFFFu));
-    out[3] = f16_bits_to_f32((uint16_t)(h.y >> 16));
-}
-
-// f[r][j] += (d*dx)*acc + m*gsum for the lane's 4 columns
-__device__ __forceinline__ void fold(float f[4], const int acc[4], uint2 dh, uint2 mh, float dx, float g) {
-    float d[4], m[4];
-    unpack_h4(dh, d);
-    unpack_h4(mh, m);
-#pragma unroll
-    for (int j = 0; j < 4; j++) {
-        f[j] = fmaf(d[j] * dx, (float)acc[j], f[j]);
-        f[j] = fmaf(m[j], g, f[j]);
-    }
-}
 
 struct TileRange {
     int nb, s, t0, t1;
@@ -265,73 +161,6 @@ __global__ __launch_bounds__(NW * 64) void fc_gemv_kernel(const uint8_t* __restr
 }
 
 // ---- variant 2: raw fp32 activations, quantized by the wavefront that consumes them -----------
-template <int G>
-struct XRaw {
-    float v[(G == 128) ? 2 : 1];
-};
-
-template <int G>
-__device__ __forceinline__ void load_x(XRaw<G>& xr, const float* xrow, int step, int64_t K, int lane) {
-    if (G == 128) {
-        const float2 t = *reinterpret_cast<const float2*>(xrow + (int64_t)step * 128 + lane * 2);
-        xr.v[0] = t.x;
-        xr.v[(G == 128) ? 1 : 0] = t.y;
-    } else {
-        const int64_t k = (int64_t)step * 64 + lane;
-        xr.v[0] = k < K ? xrow[k] : 0.0f;
-    }
-}
-
-__device__ __forceinline__ int q8_code_rne(float v, float id) {
-    const float t = v * id;
-    if (t != t) return -128;  // what the reference's cvtps2dq + saturating packs give for NaN
-    return (int)fminf(127.0f, fmaxf(-128.0f, rintf(t)));
-}
-
-// Per-step record in LDS: the step's int8 codes followed by (dx, gsum) per block of the step
-template <int G>
-struct XSlot {
-    int8_t codes[Step<G>::kK];
-    float2 scale[Step<G>::kBlocksPerStep];
-};
-
-// FC_dynamic_quantize_x for one step (/root/reference/ops/op_fc.hpp:246-268): amax -> d = amax/127 ->
-// id = 1/d -> RNE codes; raw sum of the group
-template <int G>
-__device__ __forceinline__ void quantize_step(const XRaw<G>& xr, XSlot<G>* slot, int lane) {
-    if (G == 128) {
-        float amax = fmaxf(fabsf(xr.v[0]), fabsf(xr.v[(G == 128) ? 1 : 0]));
-        float sum = xr.v[0] + xr.v[(G == 128) ? 1 : 0];
-        row16_max_sum(amax, sum);
-        amax = fmaxf(fmaxf(lane_bcast(amax, 0), lane_bcast(amax, 16)), fmaxf(lane_bcast(amax, 32), lane_bcast(amax, 48)));
-        sum = (lane_bcast(sum, 0) + lane_bcast(sum, 16)) + (lane_bcast(sum, 32) + lane_bcast(sum, 48));
-        const float d = amax / 127.0f;
-        const float id = (d != 0.0f) ? (1.0f / d) : 0.0f;
-        const uint32_t c0 = (uint32_t)q8_code_rne(xr.v[0], id) & 0xFFu;
-        const uint32_t c1 = (uint32_t)q8_code_rne(xr.v[(G == 128) ? 1 : 0], id) & 0xFFu;
-        *reinterpret_cast<uint16_t*>(&slot->codes[lane * 2]) = (uint16_t)(c0 | (c1 << 8));
-        if (lane == 0) slot->scale[0] = make_float2(d, sum);
-    } else {
-        float amax = fabsf(xr.v[0]);
-        float sum = xr.v[0];
-        row16_max_sum(amax, sum);
-        // the two half-waves hold two different groups
-        const float a_lo = fmaxf(lane_bcast(amax, 0), lane_bcast(amax, 16)), a_hi = fmaxf(lane_bcast(amax, 32), lane_bcast(amax, 48));
-        const float s_lo = lane_bcast(sum, 0) + lane_bcast(sum, 16), s_hi = lane_bcast(sum, 32) + lane_bcast(sum, 48);
-        const bool hi = lane >= 32;
-        const float d = (hi ? a_hi : a_lo) / 127.0f;
-        const float id = (d != 0.0f) ? (1.0f / d) : 0.0f;
-        slot->codes[lane] = (int8_t)q8_code_rne(xr.v[0], id);
-        if ((lane & 31) == 0) slot->scale[(G == 128) ? 0 : (lane >> 5)] = make_float2(d, hi ? s_hi : s_lo);
-    }
-}
-
-__device__ __forceinline__ float wave_sum_dpp(float v) {
-    float dummy = 0.0f;
-    row16_max_sum(dummy, v);
-    return (lane_bcast(v, 0) + lane_bcast(v, 16)) + (lane_bcast(v, 32) + lane_bcast(v, 48));
-}
-
 // Optional work folded into the decode kernel (MODE bits):
 //   kNorm: the activation row is rmsnorm'ed first (ops/op_misc.hpp:142-181): every workgroup reads
 //          the whole row once (L2 resident), reduces the sum of squares and scales the groups it
