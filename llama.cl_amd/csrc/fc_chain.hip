@@ -193,7 +193,8 @@ __device__ __forceinline__ void chain_materialize(const ChainOpDev& p, int wg, i
 
 template <int G, int R>
 __global__ __launch_bounds__(kChainThreads) void fc_chain_kernel(const ChainOpDev* __restrict__ ops, int n_ops,
-                                                                 unsigned* sync, long long spin_limit) {
+                                                                 unsigned* sync, long long spin_limit,
+                                                                 long long* trace) {
     using Cfg = ChainCfg<G>;
     constexpr int SB = Cfg::kStepBytes, KK = Step<G>::kK, UPW = Cfg::kUnitsPerWave, EPL = Cfg::kElemsPerLane;
     __shared__ __align__(16) uint8_t ring[kChainWaves][R][SB];
@@ -232,6 +233,7 @@ __global__ __launch_bounds__(kChainThreads) void fc_chain_kernel(const ChainOpDe
         const int ga = chain_wg_begin(op.geom, wg), gb = chain_wg_end(op.geom, wg);
         const int T = op.geom.T;
 
+        if (trace != nullptr && threadIdx.x == 0) trace[((int64_t)wg * n_ops + i) * 4 + 0] = wall_clock64();
         if (ga < gb) {  // uniform over the workgroup
             // ---- input row: resolve, optional rmsnorm, quantize once into LDS ---------------------
             XRaw<G> xv[UPW];
@@ -279,6 +281,7 @@ __global__ __launch_bounds__(kChainThreads) void fc_chain_kernel(const ChainOpDe
                 if (unit < op.Tin) quantize_step<G>(xv[j], &xrow[unit], lane);
             }
             __syncthreads();
+            if (trace != nullptr && threadIdx.x == 0) trace[((int64_t)wg * n_ops + i) * 4 + 1] = wall_clock64();
 
             // ---- stream this wave's steps out of its ring -----------------------------------------
             float f[4] = {0.0f, 0.0f, 0.0f, 0.0f};
@@ -327,6 +330,7 @@ __global__ __launch_bounds__(kChainThreads) void fc_chain_kernel(const ChainOpDe
         if (ga < gb) {
             // ---- sum the waves per strip (fixed order) and store this workgroup's partial sums ------
             __syncthreads();
+            if (trace != nullptr && threadIdx.x == 0) trace[((int64_t)wg * n_ops + i) * 4 + 2] = wall_clock64();
             const int s_lo = ga / T, s_hi = (gb - 1) / T;
             const int s = s_lo + (threadIdx.x >> 5), col = threadIdx.x & 31;
             if (s <= s_hi) {
@@ -354,6 +358,7 @@ __global__ __launch_bounds__(kChainThreads) void fc_chain_kernel(const ChainOpDe
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
         if (threadIdx.x == 0) __hip_atomic_fetch_add(&sync[kSyncBar], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (trace != nullptr && threadIdx.x == 0) trace[((int64_t)wg * n_ops + i) * 4 + 3] = wall_clock64();
         a = b = issued = 0;
         if (i + 1 < n_ops) {
             const ChainGeom ng = ops[i + 1].geom;
@@ -408,6 +413,7 @@ __global__ __launch_bounds__(kChainThreads) void fc_chain_kernel(const ChainOpDe
 static int g_chain_ring = 0;  // 0 = default depth
 static int g_chain_grid = 0;  // 0 = one workgroup per CU
 static long long g_chain_spin_limit = 100000000LL;  // 1 s of the 100 MHz wall clock
+static long long* g_chain_trace = nullptr;          // optional per-workgroup phase timestamps
 
 static int chain_grid(int* out) {
     int dev = 0, cus = 0;
@@ -460,7 +466,7 @@ static int chain_check_op(const llmops_chain_op* ops, int i, int G, int P, Chain
 
 template <int G, int R>
 static void chain_launch(const ChainOpDev* plan, int n_ops, unsigned* sync, int grid, hipStream_t st) {
-    fc_chain_kernel<G, R><<<(unsigned)grid, kChainThreads, 0, st>>>(plan, n_ops, sync, g_chain_spin_limit);
+    fc_chain_kernel<G, R><<<(unsigned)grid, kChainThreads, 0, st>>>(plan, n_ops, sync, g_chain_spin_limit, g_chain_trace);
 }
 
 }  // namespace llmops
@@ -559,6 +565,8 @@ extern "C" int llmops_fc_chain_status(const void* workspace, int32_t* status) {
     *status = (int32_t)words[kSyncStatus];
     return LLMOPS_OK;
 }
+
+extern "C" void llmops_fc_chain_set_trace(void* buffer) { llmops::g_chain_trace = reinterpret_cast<long long*>(buffer); }
 
 extern "C" void llmops_fc_chain_set_tuning(int ring_depth, int grid, long long spin_limit_ticks) {
     if (ring_depth >= 0) llmops::g_chain_ring = ring_depth;

@@ -54,6 +54,7 @@ SIGNATURES = {
     "llmops_fc_chain_run": (c_int, [c_ptr, c_int, c_int, c_ptr, c_ptr]),
     "llmops_fc_chain_status": (c_int, [c_ptr, c_ptr]),
     "llmops_fc_chain_set_tuning": (None, [c_int, c_int, ctypes.c_longlong]),
+    "llmops_fc_chain_set_trace": (None, [c_ptr]),
     "llmops_calib_read": (c_int, [c_ptr, c_i64, c_int, c_ptr, c_ptr]),
     "llmops_calib_copy": (c_int, [c_ptr, c_ptr, c_i64, c_int, c_ptr]),
     "llmops_fc_set_tuning": (None, [c_int, c_int]),
