@@ -187,16 +187,16 @@ int llmops_embedding(float* out, const int64_t* ids, int64_t n, const float* w, 
  * ------------------------------------------------------------------------------------------
  * What a decoder layer does between two attention calls (chatllama/main.py:344-375): rmsnorm ->
  * fc_Q4A (q|k|v) ... fc_Q4A (o) -> iadd -> rmsnorm -> fc_Q4A (gate, up) -> itrans("silu"), imul ->
- * fc_Q4A (down) -> iadd.  Each op is llmops_fc_Q4A_decode with rows = 1; op i+1 may take op i's
- * output as its input (x = NULL).  One resident grid runs all ops, keeps the next op's weights
- * streaming while an op's result crosses the chip, and separates consecutive ops by one grid-wide
- * barrier (also when op i+1 reads an external x).  Outputs equal llmops_fc_Q4A_decode's within
- * fp32 summation order (the int32 dot products are the same).
+ * fc_Q4A (down) -> iadd.  Each op is llmops_fc_Q4A_decode with rows = 1.  An op's x and residual
+ * may be buffers written before the launch or the y of an earlier op of the chain (x = NULL is
+ * short for the previous op's y); the kernel then waits for exactly the values it needs.  One
+ * resident grid runs all ops and keeps weights streaming across op boundaries.  Outputs equal
+ * llmops_fc_Q4A_decode's within fp32 summation order (the int32 dot products are the same).
  *
- * Rules: K = Kg*group_k <= 16384; group 32 needs an even Kg; glu excludes residual; an external x
- * must not be the y of an earlier op of the chain (use x = NULL for the previous op's output);
- * residual must not be the y of the immediately preceding op (it may be any other y, and it may
- * be the op's own y: in-place h += fc(...)).  */
+ * Rules: K = Kg*group_k <= 16384; Ng <= 8 * (compute units) (4 * with glu); group 32 needs an even
+ * Kg; glu excludes residual; every op has its own y; a buffer that is read as written before the
+ * launch (x or residual that is no earlier op's y) must not be the y of that op or a later one,
+ * except that a residual may be the op's own y (in place).  */
 typedef struct llmops_chain_op {
     const int8_t* weiq;    /* packed [Ng][Kg][block]; glu: gate/up strips interleaved */
     int64_t Ng, Kg;

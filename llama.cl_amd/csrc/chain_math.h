@@ -1,12 +1,14 @@
 // Integer bookkeeping of the persistent decode chain, shared by the host planner and the kernel
 // (and by the CPU-side exhaustive check of the decomposition in the tests).
 //
-// An FC with Ng strips of T steps each is one linear stream of Ttot = Ng*T steps (a step is what a
+// An FC with Ng strips of T steps each is one linear stream of Ng*T steps (a step is what a
 // wavefront loads at once: one group-128 block or two group-32 blocks; strips are contiguous in the
-// packed tensor, so the stream is contiguous memory).  The stream is cut into equal runs of W steps,
-// one per workgroup, and every run into 16 nearly equal wave runs.  A strip whose steps fall into
-// several workgroups gets one partial sum per workgroup ("contributor"), stored side by side; whoever
-// needs the FC's output adds the contributors in workgroup order.
+// packed tensor, so the stream is contiguous memory).  Strips are dealt out in whole "units" (one
+// strip, or a gate/up strip pair when the op ends in silu(gate)*up): every active workgroup gets m
+// consecutive units, so every output column is finished inside one workgroup.  Consecutive ops
+// start at different workgroups (rot), so the workgroups that idle in one op are the ones that
+// stream the next op's weights ahead.  Inside a workgroup the steps are cut into nearly equal
+// contiguous runs, one per streaming wavefront; a run never covers more than two strips.
 #pragma once
 #include <stdint.h>
 
@@ -19,54 +21,54 @@
 
 namespace llmops {
 
-constexpr int kChainWaves = 16;          // wavefronts per workgroup
-constexpr int kChainMaxStripsPerWg = 17;  // W <= 16*T  =>  a workgroup touches at most 17 strips
-constexpr int kChainMaxContrib = 5;       // W >= ceil(T/4) => a strip has at most 5 contributors
+constexpr int kChainWaves = 16;       // wavefronts per workgroup
+constexpr int kChainStreamWaves = 8;  // of which stream weights; the others handle activations
+constexpr int kChainServiceWaves = kChainWaves - kChainStreamWaves;
 
 struct ChainGeom {
-    int T;     // steps per strip
-    int Ttot;  // steps of the whole FC
-    int W;     // steps per workgroup
+    int T;       // steps per strip
+    int us;      // strips per unit (1, or 2 for gate/up pairs)
+    int units;   // units of the op
+    int m;       // units per active workgroup
+    int active;  // workgroups that get work
+    int rot;     // first active workgroup
 };
 
-LLMOPS_HD int chain_wg_begin(const ChainGeom& g, int wg) {
-    const int64_t v = (int64_t)wg * g.W;
-    return v < g.Ttot ? (int)v : g.Ttot;
-}
-LLMOPS_HD int chain_wg_end(const ChainGeom& g, int wg) { return chain_wg_begin(g, wg + 1); }
-
-// steps [a, b) of wave `w` inside the workgroup run [ga, gb)
-LLMOPS_HD void chain_wave_range(int ga, int gb, int w, int& a, int& b) {
-    const int len = gb - ga;
-    a = ga + (w * len) / kChainWaves;
-    b = ga + ((w + 1) * len) / kChainWaves;
-}
-
-// (strip+1)*T <= Ttot < 2^30, so 32-bit arithmetic is exact
-LLMOPS_HD int chain_first_wg(const ChainGeom& g, int strip) { return (int)(((uint32_t)strip * (uint32_t)g.T) / (uint32_t)g.W); }
-LLMOPS_HD int chain_last_wg(const ChainGeom& g, int strip) {
-    return (int)((((uint32_t)strip + 1u) * (uint32_t)g.T - 1u) / (uint32_t)g.W);
-}
-
-// Host-side choice of W for a grid of P workgroups; returns false when the FC does not fit the
-// kernel's fixed bounds (then the caller must split it along N).
-inline bool chain_plan_geom(int Ng, int T, int P, ChainGeom& g, int& active_wgs, int& contributors) {
-    const int64_t Ttot = (int64_t)Ng * T;
-    if (Ng <= 0 || T <= 0 || P <= 0 || Ttot >= ((int64_t)1 << 30)) return false;
-    int64_t W = (Ttot + P - 1) / P;
-    const int64_t Wmin = (T + 3) / 4;
-    if (W < Wmin) W = Wmin;
-    if (W > (int64_t)kChainWaves * T) return false;
-    g.T = T;
-    g.Ttot = (int)Ttot;
-    g.W = (int)W;
-    active_wgs = (int)((Ttot + W - 1) / W);
-    contributors = 1;
-    for (int s = 0; s < Ng; s++) {
-        const int c = chain_last_wg(g, s) - chain_first_wg(g, s) + 1;
-        if (c > contributors) contributors = c;
+// the units [u0, u1) of workgroup `wg` in a grid of P (empty when the workgroup idles in this op)
+LLMOPS_HD void chain_wg_units(const ChainGeom& g, int wg, int P, int& u0, int& u1) {
+    int local = wg - g.rot;
+    if (local < 0) local += P;
+    if (local >= g.active) {
+        u0 = u1 = 0;
+        return;
     }
-    return contributors <= kChainMaxContrib;
+    u0 = local * g.m;
+    u1 = u0 + g.m;
+    if (u1 > g.units) u1 = g.units;
+}
+
+// steps [a, b) (in the op's linear stream) of streaming wave `w` of a workgroup that owns units [u0, u1)
+LLMOPS_HD void chain_wave_range(const ChainGeom& g, int u0, int u1, int w, int& a, int& b) {
+    const int tu = g.T * g.us;
+    const int ga = u0 * tu, len = (u1 - u0) * tu;
+    a = ga + (w * len) / kChainStreamWaves;
+    b = ga + ((w + 1) * len) / kChainStreamWaves;
+}
+
+// Host-side plan of one op for a grid of P workgroups; `rot` is where the previous op's active
+// workgroups ended.  Returns false when the op does not fit the kernel's fixed bounds.
+inline bool chain_plan_geom(int Ng, int T, int us, int P, int rot, ChainGeom& g) {
+    if (Ng <= 0 || T <= 0 || P <= 0 || (us != 1 && us != 2) || (Ng % us) != 0) return false;
+    if ((int64_t)Ng * T >= ((int64_t)1 << 30)) return false;
+    g.T = T;
+    g.us = us;
+    g.units = Ng / us;
+    g.m = (g.units + P - 1) / P;
+    // a wave's run must not span more than two strips: (m*us*T)/waves <= T
+    if (g.m * us > kChainStreamWaves) return false;
+    g.active = (g.units + g.m - 1) / g.m;
+    g.rot = rot % P;
+    return true;
 }
 
 }  // namespace llmops

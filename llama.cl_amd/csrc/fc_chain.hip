@@ -3,35 +3,36 @@
 // Why.  A decode step is a string of small dependent FCs (9-48 MB of weights each).  Launched one
 // by one, each pays the dispatch gap plus a load -> quantize -> dot -> reduce latency chain during
 // which HBM idles.  Weights do not depend on activations, so here one resident grid (one workgroup
-// of 16 wavefronts per CU) walks the whole chain and keeps the weight stream of the NEXT FC in
-// flight while the current one finishes and its result crosses the chip:
+// of 16 wavefronts per CU) walks the whole chain and never stops streaming weights:
 //
-//   * every wavefront owns a ring of R step slots in LDS (160 KB per CU) filled by direct
-//     global->LDS loads (global_load_lds_dwordx4: no registers held while the data is in flight);
-//   * an FC's steps are cut evenly over all workgroups (chain_math.h), so every CU streams the
-//     same number of bytes whatever the shape;
-//   * a strip that spans several workgroups is not finished by a ticket hand-off: each workgroup
-//     stores its partial sums (write-through) and the CONSUMER of the FC's output adds them while
-//     it loads its input row, so an FC boundary costs exactly one grid-wide barrier;
-//   * right after arriving at that barrier a wavefront refills its ring with the first steps of the
-//     next FC, and only then waits.
+//   * Wavefronts are specialised.  Streaming waves own a ring of R step slots in LDS (160 KB per CU)
+//     that they fill with direct global->LDS loads (global_load_lds_dwordx4: no registers are held
+//     while data is in flight) and they issue nothing else to memory, so the ring runs ahead across
+//     op boundaries: while an op's result travels across the chip, the next op's weights arrive.
+//     Service waves do everything that has memory latency on the critical path: they fetch and
+//     quantize the input row, sum the streaming waves' results and publish the outputs.  (Loads of
+//     one wave return in issue order, so a wave that keeps a deep weight ring in flight would see
+//     every activation load queue behind it; hence the split.)
+//   * Work is dealt out in whole output strips (chain_math.h): every output column is finished
+//     inside one workgroup, in a fixed order, so results do not depend on timing.
+//   * There is no grid barrier.  Outputs are published as 8-byte (value, launch epoch) pairs with
+//     write-through stores and consumers poll the pairs they need until the epoch matches: an op
+//     boundary costs one store->load trip through the memory side instead of store -> acknowledge ->
+//     counter -> poll -> load.  The epoch is a counter in the workspace that the last workgroup to
+//     leave advances, so stale pairs of earlier launches (also graph replays) never match.
 //
-// Per FC and workgroup: resolve the input row (sum the previous FC's partials, optional
-// silu(gate)*up, optional rmsnorm), quantize it once into LDS (same operations as
-// FC_dynamic_quantize_x, /root/reference/ops/op_fc.hpp:221-272), stream the workgroup's steps
-// (same dot4 inner product and fp32 fold as the single-FC kernel; arithmetic of fc_Q4A,
-// ops/op_fc.hpp:286-426), reduce over waves in a fixed order, store the partials, barrier.
-// Summation orders are fixed by the decomposition, so results do not depend on timing.
+// Per op and workgroup: service waves resolve the input row (plain or published pairs; optional
+// rmsnorm) and quantize it once into LDS (same operations as FC_dynamic_quantize_x,
+// /root/reference/ops/op_fc.hpp:221-272); streaming waves run the dot4 inner product and fp32 fold
+// of the single-FC kernel over their steps (arithmetic of fc_Q4A, ops/op_fc.hpp:286-426); service
+// waves add the waves per strip, apply residual or silu(gate)*up, and publish.
 //
-// Memory visibility across the 8 XCDs (each has its own L2): partial sums, materialized outputs
-// and the barrier counter are written with device-scope write-through stores / atomics; partial
-// sums are read back with ordinary cached loads, which is sound because every FC of a chain has
-// its own partial region and no line of it is touched before the barrier that completes it;
-// residual inputs, which may alias outputs written earlier in the same launch, are read with
-// device-scope loads.  No cache-wide fences.
+// Memory visibility across the 8 XCDs (each has its own L2): published pairs are written with
+// device-scope write-through stores and read with device-scope (L2-bypassing) loads; everything
+// else the kernel reads was written before the launch.  No cache-wide fences.
 //
-// Every wait is bounded: the barrier spin gives up after `spin_limit` ticks of the 100 MHz
-// wall clock, raises the status word and lets every workgroup leave.
+// Every wait is bounded: a poll that does not complete within `spin_limit` ticks of the 100 MHz
+// wall clock raises the status word and lets every workgroup leave.
 #include "chain_math.h"
 #include "common.h"
 #include "gemv_device.h"
@@ -45,24 +46,24 @@ constexpr int kChainMaxK = 16384;  // input row length the LDS staging is sized 
 constexpr int kChainSyncBytes = 256;
 
 // sync words at the start of the workspace
-enum { kSyncBar = 0, kSyncDone = 1, kSyncStatus = 2 };
+enum { kSyncEpoch = 0, kSyncDone = 1, kSyncStatus = 2 };
 
 struct ChainOpDev {
-    const uint8_t* w;       // packed weights [Ng][Kg][block]
-    const float* x;         // input row, or nullptr: the previous op's output
-    const float* norm_w;    // optional rmsnorm weight
-    const float* residual;  // optional, added to the output
-    float* y;               // materialized output (may be nullptr for an inner op)
-    float* part;            // partial sums [contributors][Np]
-    ChainGeom geom;         // T, Ttot, W
-    int32_t contrib;  // partial-sum slots per strip
-    int32_t Np;       // Ng*32
-    int32_t N_out;  // valid outputs (GLU: Np/2 at most)
+    const uint8_t* w;          // packed weights [Ng][Kg][block]
+    const float* x_plain;      // input row written before the launch, or
+    const uint64_t* x_pairs;   //   (value, epoch) pairs published by an earlier op of this launch
+    const float* norm_w;       // optional rmsnorm weight
+    const float* res_plain;    // optional residual, plain or
+    const uint64_t* res_pairs;  //   published by an earlier op
+    float* y;                  // plain output for the caller
+    uint64_t* y_pairs;         // published output for later ops of this launch
+    ChainGeom geom;
+    int32_t N_out;  // valid outputs
     int32_t K;
     int32_t Tin;  // input steps: K / Step::kK
-    int32_t glu;
     int32_t grid;  // workgroups the plan was made for
     float eps;
+    int32_t pad_;
 };
 
 template <int G>
@@ -70,7 +71,7 @@ struct ChainCfg {
     static constexpr int kStepBytes = Step<G>::kBlocksPerStep * (int)block_bytes(G);  // 2176 / 1280
     static constexpr int kLoads = (kStepBytes + 1023) / 1024;                         // wave-wide 16 B loads per step
     static constexpr int kXSteps = kChainMaxK / Step<G>::kK;
-    static constexpr int kUnitsPerWave = kXSteps / kChainWaves;
+    static constexpr int kUnitsPerWave = kXSteps / kChainServiceWaves;
     static constexpr int kElemsPerLane = Step<G>::kK / 64;
 };
 
@@ -127,16 +128,15 @@ __device__ __forceinline__ void ring_read(Step<G>& st, const uint8_t* slot, int 
 }
 
 // wait until at most `loads` of this wave's vector-memory operations are outstanding
-template <int MAXV>
 __device__ __forceinline__ void wait_vm(int loads) {
-    static_assert(MAXV <= 15, "ring too deep for the wait table");
     switch (loads) {
 #define LLMOPS_W(n) \
     case n:         \
         asm volatile("s_waitcnt vmcnt(" #n ")" ::: "memory"); \
         break;
         LLMOPS_W(1) LLMOPS_W(2) LLMOPS_W(3) LLMOPS_W(4) LLMOPS_W(5) LLMOPS_W(6) LLMOPS_W(7) LLMOPS_W(8)
-        LLMOPS_W(9) LLMOPS_W(10) LLMOPS_W(11) LLMOPS_W(12) LLMOPS_W(13) LLMOPS_W(14) LLMOPS_W(15)
+        LLMOPS_W(9) LLMOPS_W(10) LLMOPS_W(11) LLMOPS_W(12) LLMOPS_W(13) LLMOPS_W(14) LLMOPS_W(15) LLMOPS_W(16)
+        LLMOPS_W(17) LLMOPS_W(18) LLMOPS_W(19) LLMOPS_W(20) LLMOPS_W(21) LLMOPS_W(22) LLMOPS_W(23) LLMOPS_W(24)
 #undef LLMOPS_W
         default:
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -147,48 +147,53 @@ __device__ __forceinline__ void wait_vm(int loads) {
 // The op table holds plain pointers, which the compiler would have to treat as generic ("flat")
 // addresses; every one of them is device global memory, and saying so gives global_load/_store.
 typedef __attribute__((address_space(1))) float gfloat;
+typedef __attribute__((address_space(1))) uint64_t gu64;
 __device__ __forceinline__ float ld_global(const float* p) { return *(const gfloat*)p; }
-__device__ __forceinline__ float ld_agent(const float* p) {
-    return __hip_atomic_load((const gfloat*)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+__device__ __forceinline__ uint64_t ld_pair(const uint64_t* p) {
+    return __hip_atomic_load((const gu64*)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
-__device__ __forceinline__ void st_agent(float* p, float v) {
-    __hip_atomic_store((gfloat*)p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-
-// sum of the contributor slots at flat column index idx, in workgroup order; every op stores all
-// `contrib` slots of every strip (unused ones as zeros), so no per-strip bookkeeping is needed here
-__device__ __forceinline__ float chain_sum(const ChainOpDev& p, int idx) {
-    // branch-free so that all loads are in flight together: a slot beyond `contrib` re-reads slot 0
-    float v[kChainMaxContrib];
-#pragma unroll
-    for (int c = 0; c < kChainMaxContrib; c++) v[c] = ld_global(p.part + (int64_t)(c < p.contrib ? c : 0) * p.Np + idx);
-    float s = v[0];
-#pragma unroll
-    for (int c = 1; c < kChainMaxContrib; c++) s += (c < p.contrib) ? v[c] : 0.0f;
-    return s;
+__device__ __forceinline__ void st_pair(uint64_t* p, float v, uint32_t epoch) {
+    __hip_atomic_store((gu64*)p, ((uint64_t)epoch << 32) | (uint64_t)__float_as_uint(v), __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// output element k of op p: contributors added up; gate/up pairs combined as silu(gate)*up
-// (itrans "silu" + imul, ops/op_misc.hpp:83-138)
-__device__ __forceinline__ float chain_resolve(const ChainOpDev& p, int k) {
-    if (!p.glu) return chain_sum(p, k);
-    const int u = k >> 5, col = k & 31;
-    const float g = chain_sum(p, (2 * u) * kGroupN + col);
-    const float up = chain_sum(p, (2 * u + 1) * kGroupN + col);
-    return up * (g * (1.0f / (1.0f + expf(-g))));
-}
-
-// the share of op p's output that this workgroup writes out (128 outputs per wave at a time)
-__device__ __forceinline__ void chain_materialize(const ChainOpDev& p, int wg, int grid, int wave, int lane) {
-    if (p.y == nullptr) return;
-    const int chunks = (p.N_out + 127) >> 7;
-    for (int u = wg + grid * wave; u < chunks; u += grid * kChainWaves) {
-#pragma unroll
-        for (int e = 0; e < 2; e++) {
-            const int k = u * 128 + lane * 2 + e;
-            if (k < p.N_out) st_agent(p.y + k, chain_resolve(p, k));
+// Bounded wait bookkeeping of a polling loop: returns true when the caller should give up.
+struct ChainClock {
+    long long t_begin, limit;
+    unsigned* sync;
+    int* pending;
+    __device__ __forceinline__ bool expired() const {
+        if (*reinterpret_cast<volatile int*>(pending) != 0) return true;
+        if (wall_clock64() - t_begin > limit) {
+            __hip_atomic_store(&sync[kSyncStatus], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            *reinterpret_cast<volatile int*>(pending) = 1;
+            return true;
         }
+        return false;
     }
+};
+
+// position of a streaming wave in the chain-long sequence of its steps
+struct ChainCursor {
+    int op, t, end;
+    const uint8_t* base;
+};
+
+template <int G>
+__device__ __forceinline__ bool cursor_next(ChainCursor& c, const ChainOpDev* __restrict__ ops, int n_ops, int wg,
+                                            int grid, int wave, const uint8_t*& src) {
+    while (c.t >= c.end) {
+        c.op++;
+        if (c.op >= n_ops) return false;
+        const ChainGeom g = ops[c.op].geom;
+        int u0, u1;
+        chain_wg_units(g, wg, grid, u0, u1);
+        chain_wave_range(g, u0, u1, wave, c.t, c.end);
+        c.base = ops[c.op].w;
+    }
+    src = c.base + (int64_t)c.t * ChainCfg<G>::kStepBytes;
+    c.t++;
+    return true;
 }
 
 template <int G, int R>
@@ -197,98 +202,58 @@ __global__ __launch_bounds__(kChainThreads) void fc_chain_kernel(const ChainOpDe
                                                                  long long* trace) {
     using Cfg = ChainCfg<G>;
     constexpr int SB = Cfg::kStepBytes, KK = Step<G>::kK, UPW = Cfg::kUnitsPerWave, EPL = Cfg::kElemsPerLane;
-    __shared__ __align__(16) uint8_t ring[kChainWaves][R][SB];
+    constexpr int NS = kChainStreamWaves, NV = kChainServiceWaves;
+    __shared__ __align__(16) uint8_t ring[NS][R][SB];
     __shared__ __align__(16) XSlot<G> xrow[Cfg::kXSteps];
-    __shared__ float red[kChainWaves][2][kGroupN];
-    __shared__ int winfo[kChainWaves][2];  // first strip of the wave, number of strips it flushed
-    __shared__ float nred[kChainWaves];
-    __shared__ int abort_sh;
+    __shared__ float red[NS][2][kGroupN];
+    __shared__ int winfo[NS][2];  // first strip of the wave's run, number of strips it flushed
+    __shared__ float nred[NV];
+    __shared__ int svc_count;  // service-wave rendezvous (the workgroup barrier also involves the streaming waves)
+    __shared__ int abort_sh;       // read by every wave right after S1; only written before S1
+    __shared__ int abort_pending;  // raised by whoever runs out of time, folded into abort_sh before the next S1
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int quad = lane & 7, rs = lane >> 3;
     const int wg = blockIdx.x, grid = gridDim.x;
-    const bool first_row = (G == 128) ? (rs == 0) : ((rs & 3) == 0);
-    uint8_t* myring = &ring[wave][0][0];
-    const long long t_begin = wall_clock64();
+    const bool streamer = wave < NS;
+    const uint32_t epoch = __hip_atomic_load(&sync[kSyncEpoch], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1u;
 
-    bool aborted = false;
-    if (ops[0].grid != grid) {  // the plan was cut for another grid: nothing below would line up
-        if (threadIdx.x == 0) __hip_atomic_store(&sync[kSyncStatus], 2u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        aborted = true;
+    if (threadIdx.x == 0) {
+        abort_sh = (ops[0].grid != grid) ? 1 : 0;  // a plan cut for another grid: nothing would line up
+        abort_pending = abort_sh;
+        svc_count = 0;
+        if (ops[0].grid != grid)
+            __hip_atomic_store(&sync[kSyncStatus], 2u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
+    __syncthreads();
 
-    // ring state of this wave for the op it is about to run: steps [a, b), `issued` of them requested
-    int a = 0, b = 0, issued = 0;
-    if (!aborted) {
-        chain_wave_range(chain_wg_begin(ops[0].geom, wg), chain_wg_end(ops[0].geom, wg), wave, a, b);
-        const uint8_t* wsrc = ops[0].w;
-        for (; issued < R && a + issued < b; issued++)
-            ring_issue<G>(wsrc + (int64_t)(a + issued) * SB, myring + issued * SB, lane);
-    }
-
-    for (int i = 0; i < n_ops && !aborted; i++) {
-        const ChainOpDev op = ops[i];                  // by value: the table entries live in scalar registers
-        const ChainOpDev prev = ops[i > 0 ? i - 1 : 0];
-        const int ga = chain_wg_begin(op.geom, wg), gb = chain_wg_end(op.geom, wg);
-        const int T = op.geom.T;
-
-        if (trace != nullptr && threadIdx.x == 0) trace[((int64_t)wg * n_ops + i) * 4 + 0] = wall_clock64();
-        if (ga < gb) {  // uniform over the workgroup
-            // ---- input row: resolve, optional rmsnorm, quantize once into LDS ---------------------
-            XRaw<G> xv[UPW];
-#pragma unroll
-            for (int j = 0; j < UPW; j++) {
-                const int unit = wave + kChainWaves * j;
-#pragma unroll
-                for (int e = 0; e < EPL; e++) {
-                    const int k = unit * KK + lane * EPL + e;
-                    float v = 0.0f;
-                    if (unit < op.Tin) v = (op.x != nullptr) ? ld_global(op.x + k) : chain_resolve(prev, k);
-                    xv[j].v[e] = v;
-                }
+    if (streamer) {
+        // ================= streaming waves: weights only =================
+        const bool first_row = (G == 128) ? (rs == 0) : ((rs & 3) == 0);
+        uint8_t* myring = &ring[wave][0][0];
+        ChainCursor cur{-1, 0, 0, nullptr};
+        int issued = 0, consumed = 0, fill = 0, slot = 0;
+        if (abort_sh == 0) {
+            const uint8_t* src;
+            while (issued < R && cursor_next<G>(cur, ops, n_ops, wg, grid, wave, src)) {
+                ring_issue<G>(src, myring + fill * SB, lane);
+                issued++;
+                fill = (fill + 1 == R) ? 0 : fill + 1;
             }
-            if (op.norm_w != nullptr) {  // rmsnorm (ops/op_misc.hpp:142-181): x * rsqrt(mean(x^2)+eps) * w
-                XRaw<G> nw[UPW];
-#pragma unroll
-                for (int j = 0; j < UPW; j++) {
-                    const int unit = wave + kChainWaves * j;
-#pragma unroll
-                    for (int e = 0; e < EPL; e++)
-                        nw[j].v[e] = (unit < op.Tin) ? ld_global(op.norm_w + unit * KK + lane * EPL + e) : 0.0f;
-                }
-                float ss = 0.0f;
-#pragma unroll
-                for (int j = 0; j < UPW; j++)
-#pragma unroll
-                    for (int e = 0; e < EPL; e++) ss = fmaf(xv[j].v[e], xv[j].v[e], ss);
-                ss = wave_sum_dpp(ss);
-                if (lane == 0) nred[wave] = ss;
-                __syncthreads();
-                float tot = 0.0f;
-#pragma unroll
-                for (int w = 0; w < kChainWaves; w++) tot += nred[w];
-                const float rsn = 1.0f / sqrtf(tot / (float)op.K + op.eps);
-#pragma unroll
-                for (int j = 0; j < UPW; j++)
-#pragma unroll
-                    for (int e = 0; e < EPL; e++)
-                        xv[j].v[e] = xv[j].v[e] * rsn * nw[j].v[e];
-            }
-#pragma unroll
-            for (int j = 0; j < UPW; j++) {
-                const int unit = wave + kChainWaves * j;
-                if (unit < op.Tin) quantize_step<G>(xv[j], &xrow[unit], lane);
-            }
-            __syncthreads();
-            if (trace != nullptr && threadIdx.x == 0) trace[((int64_t)wg * n_ops + i) * 4 + 1] = wall_clock64();
-
-            // ---- stream this wave's steps out of its ring -----------------------------------------
+        }
+        for (int i = 0; i < n_ops; i++) {
+            __syncthreads();  // S1: the input row of op i is quantized in LDS
+            if (abort_sh != 0) break;
+            const ChainGeom g = ops[i].geom;
+            int u0, u1, a, b;
+            chain_wg_units(g, wg, grid, u0, u1);
+            chain_wave_range(g, u0, u1, wave, a, b);
+            const int T = g.T;
             float f[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-            int ts = a % T, nseg = 0, slot = 0, fill = issued % R;
-            const uint8_t* wsrc = op.w;
+            int ts = a % T, nseg = 0;
             for (int c = 0; c < b - a; c++) {
-                wait_vm<(R - 1) * Cfg::kLoads>((issued - c - 1) * Cfg::kLoads);
+                wait_vm((issued - consumed - 1) * Cfg::kLoads);
                 Step<G> st;
                 ring_read<G>(st, myring + slot * SB, lane);
                 const XSlot<G>* xs = &xrow[ts];
@@ -296,15 +261,17 @@ __global__ __launch_bounds__(kChainThreads) void fc_chain_kernel(const ChainOpDe
                 dot_step<G>(st, xs->codes, lane, acc);
                 const float2 sc = xs->scale[(G == 128) ? 0 : (rs >> 2)];
                 fold(f, acc, st.dh, st.mh, sc.x, first_row ? sc.y : 0.0f);
-                // the slot is free once its reads have returned; refill it with this op's next step
+                // the slot is free once its reads have returned; refill it with the next step of the chain
                 asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-                if (a + issued < b) {
-                    ring_issue<G>(wsrc + (int64_t)(a + issued) * SB, myring + fill * SB, lane);
+                consumed++;
+                slot = (slot + 1 == R) ? 0 : slot + 1;
+                const uint8_t* src;
+                if (cursor_next<G>(cur, ops, n_ops, wg, grid, wave, src)) {
+                    ring_issue<G>(src, myring + fill * SB, lane);
                     issued++;
                     fill = (fill + 1 == R) ? 0 : fill + 1;
                 }
-                slot = (slot + 1 == R) ? 0 : slot + 1;
-                if (++ts == T || c + 1 == b - a) {  // end of a strip, or of the run: hand the sums to the workgroup
+                if (++ts == T || c + 1 == b - a) {  // end of a strip, or of the run: hand the sums over
 #pragma unroll
                     for (int j = 0; j < 4; j++) {
                         float v = f[j];
@@ -322,87 +289,162 @@ __global__ __launch_bounds__(kChainThreads) void fc_chain_kernel(const ChainOpDe
                 winfo[wave][0] = a / T;
                 winfo[wave][1] = nseg;
             }
+            __syncthreads();  // S2: this op's sums are in LDS
         }
-
-        // ---- outputs of the previous op that this workgroup writes out ----------------------------
-        if (i > 0) chain_materialize(prev, wg, grid, wave, lane);
-
-        if (ga < gb) {
-            // ---- sum the waves per strip (fixed order) and store this workgroup's partial sums ------
-            __syncthreads();
-            if (trace != nullptr && threadIdx.x == 0) trace[((int64_t)wg * n_ops + i) * 4 + 2] = wall_clock64();
-            const int s_lo = ga / T, s_hi = (gb - 1) / T;
-            const int s = s_lo + (threadIdx.x >> 5), col = threadIdx.x & 31;
-            if (s <= s_hi) {
-                float v = 0.0f;
-#pragma unroll
-                for (int w = 0; w < kChainWaves; w++) {
-                    const int fs = winfo[w][0], ns = winfo[w][1];
-                    if (ns > 0 && fs == s) v += red[w][0][col];
-                    if (ns > 1 && fs + 1 == s) v += red[w][1][col];
-                }
-                const int first = chain_first_wg(op.geom, s);
-                const int c = wg - first;
-                const int n = s * kGroupN + col;
-                if (c == 0) {
-                    if (op.residual != nullptr && n < op.N_out) v += ld_agent(op.residual + n);
-                    // slots that no workgroup owns for this strip read as zero
-                    for (int z = chain_last_wg(op.geom, s) - first + 1; z < op.contrib; z++)
-                        st_agent(op.part + (int64_t)z * op.Np + n, 0.0f);
-                }
-                st_agent(op.part + (int64_t)c * op.Np + n, v);
-            }
-        }
-
-        // ---- grid barrier: stores acknowledged, arrive, refill the ring for the next op, wait ------
+        // ring loads still in flight target this workgroup's LDS: drain before leaving
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads();
-        if (threadIdx.x == 0) __hip_atomic_fetch_add(&sync[kSyncBar], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        if (trace != nullptr && threadIdx.x == 0) trace[((int64_t)wg * n_ops + i) * 4 + 3] = wall_clock64();
-        a = b = issued = 0;
-        if (i + 1 < n_ops) {
-            const ChainGeom ng = ops[i + 1].geom;
-            chain_wave_range(chain_wg_begin(ng, wg), chain_wg_end(ng, wg), wave, a, b);
-            const uint8_t* wsrc = ops[i + 1].w;
-            for (; issued < R && a + issued < b; issued++)
-                ring_issue<G>(wsrc + (int64_t)(a + issued) * SB, myring + issued * SB, lane);
-        }
-        if (threadIdx.x == 0) {
-            const unsigned target = (unsigned)(i + 1) * (unsigned)grid;
-            int bad = 0;
-            unsigned spins = 0;
-            while (__hip_atomic_load(&sync[kSyncBar], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < target) {
-                __builtin_amdgcn_s_sleep(1);
-                if ((++spins & 31u) == 0u) {
-                    if (__hip_atomic_load(&sync[kSyncStatus], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) {
-                        bad = 1;
-                        break;
+    } else {
+        // ================= service waves: activations in, results out =================
+        const int sw = wave - NS;                     // 0..NV-1
+        const int stid = threadIdx.x - NS * 64;       // 0..NV*64-1
+        const ChainClock clk{wall_clock64(), spin_limit, sync, &abort_pending};
+        int rendezvous = 0;
+        for (int i = 0; i < n_ops; i++) {
+            const ChainOpDev op = ops[i];  // by value: the table entry lives in scalar registers
+            int u0, u1;
+            chain_wg_units(op.geom, wg, grid, u0, u1);
+            const bool active = u0 < u1;
+            if (trace != nullptr && stid == 0) trace[((int64_t)wg * n_ops + i) * 4 + 0] = wall_clock64();
+            if (*reinterpret_cast<volatile int*>(&abort_pending) != 0) abort_sh = 1;  // before S1, see above
+
+            if (active && *reinterpret_cast<volatile int*>(&abort_pending) == 0) {
+                // ---- input row: fetch, optional rmsnorm, quantize once into LDS ----------------------
+                XRaw<G> xv[UPW];
+                if (op.x_pairs != nullptr) {
+                    bool done = false;
+                    unsigned spins = 0;
+                    while (!done) {
+                        bool ok = true;
+#pragma unroll
+                        for (int j = 0; j < UPW; j++) {
+                            const int unit = sw + NV * j;
+#pragma unroll
+                            for (int e = 0; e < EPL; e++) {
+                                float v = 0.0f;
+                                if (unit < op.Tin) {
+                                    const uint64_t pr = ld_pair(op.x_pairs + unit * KK + lane * EPL + e);
+                                    ok = ok && ((uint32_t)(pr >> 32) == epoch);
+                                    v = __uint_as_float((uint32_t)pr);
+                                }
+                                xv[j].v[e] = v;
+                            }
+                        }
+                        done = __all(ok);
+                        if (!done) {
+                            __builtin_amdgcn_s_sleep(4);
+                            if ((++spins & 15u) == 0u && clk.expired()) break;
+                        }
                     }
-                    if (wall_clock64() - t_begin > spin_limit) {
-                        __hip_atomic_store(&sync[kSyncStatus], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                        bad = 1;
-                        break;
+                } else {
+#pragma unroll
+                    for (int j = 0; j < UPW; j++) {
+                        const int unit = sw + NV * j;
+#pragma unroll
+                        for (int e = 0; e < EPL; e++)
+                            xv[j].v[e] = (unit < op.Tin) ? ld_global(op.x_plain + unit * KK + lane * EPL + e) : 0.0f;
                     }
                 }
+                if (op.norm_w != nullptr) {  // rmsnorm (ops/op_misc.hpp:142-181): x * rsqrt(mean(x^2)+eps) * w
+                    XRaw<G> nw[UPW];
+#pragma unroll
+                    for (int j = 0; j < UPW; j++) {
+                        const int unit = sw + NV * j;
+#pragma unroll
+                        for (int e = 0; e < EPL; e++)
+                            nw[j].v[e] = (unit < op.Tin) ? ld_global(op.norm_w + unit * KK + lane * EPL + e) : 0.0f;
+                    }
+                    float ss = 0.0f;
+#pragma unroll
+                    for (int j = 0; j < UPW; j++)
+#pragma unroll
+                        for (int e = 0; e < EPL; e++) ss = fmaf(xv[j].v[e], xv[j].v[e], ss);
+                    ss = wave_sum_dpp(ss);
+                    // rendezvous of the service waves only (the streaming waves sit in the workgroup barrier)
+                    rendezvous += NV;
+                    if (lane == 0) {
+                        nred[sw] = ss;
+                        __hip_atomic_fetch_add(&svc_count, 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+                    }
+                    unsigned spins = 0;
+                    while (__hip_atomic_load(&svc_count, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP) < rendezvous) {
+                        __builtin_amdgcn_s_sleep(1);
+                        if ((++spins & 255u) == 0u && clk.expired()) break;
+                    }
+                    float tot = 0.0f;
+#pragma unroll
+                    for (int w = 0; w < NV; w++) tot += nred[w];
+                    const float rsn = 1.0f / sqrtf(tot / (float)op.K + op.eps);
+#pragma unroll
+                    for (int j = 0; j < UPW; j++)
+#pragma unroll
+                        for (int e = 0; e < EPL; e++) xv[j].v[e] = xv[j].v[e] * rsn * nw[j].v[e];
+                }
+#pragma unroll
+                for (int j = 0; j < UPW; j++) {
+                    const int unit = sw + NV * j;
+                    if (unit < op.Tin) quantize_step<G>(xv[j], &xrow[unit], lane);
+                }
             }
-            abort_sh = bad;
+            if (trace != nullptr && stid == 0) trace[((int64_t)wg * n_ops + i) * 4 + 1] = wall_clock64();
+            __syncthreads();  // S1
+            if (abort_sh != 0) break;
+
+            // ---- while the streaming waves work: fetch the residual of the columns this thread finishes ----
+            const int j = stid >> 5, col = stid & 31;
+            const int unit = u0 + j;
+            const bool mine = active && unit < u1;
+            const int n = unit * kGroupN + col;  // output column (glu: of silu(gate)*up)
+            float resv = 0.0f;
+            if (mine && n < op.N_out) {
+                if (op.res_pairs != nullptr) {
+                    unsigned spins = 0;
+                    for (;;) {
+                        const uint64_t pr = ld_pair(op.res_pairs + n);
+                        if ((uint32_t)(pr >> 32) == epoch) {
+                            resv = __uint_as_float((uint32_t)pr);
+                            break;
+                        }
+                        __builtin_amdgcn_s_sleep(4);
+                        if ((++spins & 15u) == 0u && clk.expired()) break;
+                    }
+                } else if (op.res_plain != nullptr) {
+                    resv = ld_global(op.res_plain + n);
+                }
+            }
+            __syncthreads();  // S2
+            if (trace != nullptr && stid == 0) trace[((int64_t)wg * n_ops + i) * 4 + 2] = wall_clock64();
+
+            // ---- add the waves per strip in a fixed order, finish and publish ---------------------
+            if (mine) {
+                const int us = op.geom.us;
+                float sum[2] = {0.0f, 0.0f};
+#pragma unroll
+                for (int h = 0; h < 2; h++) {
+                    const int s = unit * us + h;
+                    if (h < us) {
+#pragma unroll
+                        for (int w = 0; w < NS; w++) {
+                            const int fs = winfo[w][0], ns = winfo[w][1];
+                            if (ns > 0 && fs == s) sum[h] += red[w][0][col];
+                            if (ns > 1 && fs + 1 == s) sum[h] += red[w][1][col];
+                        }
+                    }
+                }
+                float v = sum[0];
+                if (us == 2) v = sum[1] * (v * (1.0f / (1.0f + expf(-v))));  // silu(gate)*up (ops/op_misc.hpp:83-138)
+                v += resv;
+                st_pair(op.y_pairs + n, v, epoch);
+                if (n < op.N_out) *(gfloat*)(op.y + n) = v;
+            }
+            if (trace != nullptr && stid == 0) trace[((int64_t)wg * n_ops + i) * 4 + 3] = wall_clock64();
         }
-        __syncthreads();
-        if (abort_sh) aborted = true;
     }
 
-    if (!aborted) {
-        const ChainOpDev last = ops[n_ops - 1];
-        chain_materialize(last, wg, grid, wave, lane);
-    }
-
-    // every ring load that is still in flight targets this workgroup's LDS: drain before leaving
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     if (threadIdx.x == 0) {
         const unsigned old = __hip_atomic_fetch_add(&sync[kSyncDone], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        if (old == (unsigned)grid - 1u) {  // last one out leaves the counters ready for the next launch
-            __hip_atomic_store(&sync[kSyncBar], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (old == (unsigned)grid - 1u) {  // last one out: the next launch gets a fresh epoch
+            __hip_atomic_store(&sync[kSyncEpoch], epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             __hip_atomic_store(&sync[kSyncDone], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
     }
@@ -426,13 +468,25 @@ static int chain_grid(int* out) {
 
 static inline size_t chain_align(size_t v) { return (v + 255) / 256 * 256; }
 
-struct ChainPlanHost {
-    ChainGeom geom;
-    int active, contrib;
-};
+// bytes of the published (value, epoch) pairs of one op
+static inline size_t chain_pairs_bytes(const llmops_chain_op& o) {
+    return chain_align((size_t)(o.Ng / (o.glu ? 2 : 1)) * kGroupN * sizeof(uint64_t));
+}
+
+// the latest op before `i` whose output buffer is `p` (-1: none), and whether `i` or a later op writes `p`
+static int chain_producer(const llmops_chain_op* ops, int i, const void* p) {
+    for (int j = i - 1; j >= 0; j--)
+        if (ops[j].y == p) return j;
+    return -1;
+}
+static bool chain_written_from(const llmops_chain_op* ops, int n_ops, int i, const void* p) {
+    for (int j = i; j < n_ops; j++)
+        if (ops[j].y == p) return true;
+    return false;
+}
 
 // checks one op of the chain and cuts it; on failure the thread's error text says why
-static int chain_check_op(const llmops_chain_op* ops, int i, int G, int P, ChainPlanHost& ph) {
+static int chain_check_op(const llmops_chain_op* ops, int n_ops, int i, int G, int P, int rot, ChainGeom& geom) {
     const llmops_chain_op& o = ops[i];
     const int bps = (G == 128) ? 1 : 2;
     LLMOPS_REQUIRE(o.weiq != nullptr && o.y != nullptr);
@@ -448,17 +502,27 @@ static int chain_check_op(const llmops_chain_op* ops, int i, int G, int P, Chain
         LLMOPS_REQUIRE(o.N_out > (o.Ng - 1) * kGroupN && o.N_out <= o.Ng * kGroupN);
     }
     if (o.x == nullptr) {
-        LLMOPS_REQUIRE(i > 0);                // "previous op's output" needs a previous op
+        LLMOPS_REQUIRE(i > 0);  // "previous op's output" needs a previous op
         LLMOPS_REQUIRE(ops[i - 1].N_out == K);
     } else {
         LLMOPS_REQUIRE(aligned(o.x, 4));
-        // a row that this launch also writes would be read through caches that may hold its old lines
-        for (int j = 0; j < i; j++) LLMOPS_REQUIRE(o.x != ops[j].y);
+        const int src = chain_producer(ops, i, o.x);
+        if (src >= 0) LLMOPS_REQUIRE(ops[src].N_out == K);
+        // a row that is read as it was before the launch must not be overwritten during the launch:
+        // without grid-wide barriers a fast workgroup may be ops ahead of a slow one
+        if (src < 0) LLMOPS_REQUIRE(!chain_written_from(ops, n_ops, i, o.x));
     }
-    // the residual is read before the barrier that ends this op; the previous op's output is only
-    // written out after that op's barrier by other workgroups, which may still be at it
-    if (o.residual != nullptr && i > 0) LLMOPS_REQUIRE(o.residual != ops[i - 1].y);
-    if (!chain_plan_geom((int)o.Ng, (int)(o.Kg / bps), P, ph.geom, ph.active, ph.contrib))
+    if (o.residual != nullptr) {
+        LLMOPS_REQUIRE(aligned(o.residual, 4));
+        const int src = chain_producer(ops, i, o.residual);
+        if (src >= 0) LLMOPS_REQUIRE(ops[src].N_out == o.N_out);
+        // plain residual: only this op itself may write the buffer (in place, column by column)
+        if (src < 0) LLMOPS_REQUIRE(!chain_written_from(ops, n_ops, i + 1, o.residual));
+    }
+    // an output buffer is written by one op only: plain stores of two ops to one address could reach
+    // memory in either order (different L2s)
+    LLMOPS_REQUIRE(chain_producer(ops, i, o.y) < 0);
+    if (!chain_plan_geom((int)o.Ng, (int)(o.Kg / bps), o.glu ? 2 : 1, P, rot, geom))
         return fail(LLMOPS_EINVAL, "chain op %d (Ng=%lld, Kg=%lld) does not fit the persistent kernel; split it along N", i,
                     (long long)o.Ng, (long long)o.Kg);
     return LLMOPS_OK;
@@ -484,11 +548,13 @@ extern "C" int llmops_fc_chain_workspace_bytes(const llmops_chain_op* ops, int n
     int rc = chain_grid(&P);
     if (rc) return rc;
     size_t total = kChainSyncBytes;
+    int rot = 0;
     for (int i = 0; i < n_ops; i++) {
-        ChainPlanHost ph;
-        rc = chain_check_op(ops, i, group_k, P, ph);
+        ChainGeom g;
+        rc = chain_check_op(ops, n_ops, i, group_k, P, rot, g);
         if (rc) return rc;
-        total += chain_align((size_t)ph.contrib * ops[i].Ng * kGroupN * sizeof(float));
+        rot = (g.rot + g.active) % P;
+        total += chain_pairs_bytes(ops[i]);
     }
     *bytes = total;
     return LLMOPS_OK;
@@ -506,28 +572,30 @@ extern "C" int llmops_fc_chain_build(const llmops_chain_op* ops, int n_ops, int 
     const int bps = (group_k == 128) ? 1 : 2;
     std::vector<ChainOpDev> dev((size_t)n_ops);
     size_t off = kChainSyncBytes;
+    int rot = 0;
     for (int i = 0; i < n_ops; i++) {
-        ChainPlanHost ph;
-        rc = chain_check_op(ops, i, group_k, P, ph);
-        if (rc) return rc;
         const llmops_chain_op& o = ops[i];
         ChainOpDev& d = dev[(size_t)i];
+        rc = chain_check_op(ops, n_ops, i, group_k, P, rot, d.geom);
+        if (rc) return rc;
+        rot = (d.geom.rot + d.geom.active) % P;
         d.w = reinterpret_cast<const uint8_t*>(o.weiq);
-        d.x = o.x;
+        const int xsrc = (o.x == nullptr) ? i - 1 : chain_producer(ops, i, o.x);
+        d.x_plain = (xsrc < 0) ? o.x : nullptr;
+        d.x_pairs = (xsrc >= 0) ? dev[(size_t)xsrc].y_pairs : nullptr;
         d.norm_w = o.norm_w;
-        d.residual = o.residual;
+        const int rsrc = (o.residual == nullptr) ? -1 : chain_producer(ops, i, o.residual);
+        d.res_plain = (o.residual != nullptr && rsrc < 0) ? o.residual : nullptr;
+        d.res_pairs = (rsrc >= 0) ? dev[(size_t)rsrc].y_pairs : nullptr;
         d.y = o.y;
-        d.part = reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(workspace) + off);
-        d.geom = ph.geom;
-        d.contrib = ph.contrib;
-        d.Np = (int32_t)(o.Ng * kGroupN);
+        d.y_pairs = reinterpret_cast<uint64_t*>(reinterpret_cast<uint8_t*>(workspace) + off);
         d.N_out = (int32_t)o.N_out;
         d.K = (int32_t)(o.Kg * group_k);
         d.Tin = (int32_t)(o.Kg / bps);
-        d.glu = o.glu ? 1 : 0;
         d.grid = P;
         d.eps = o.eps;
-        off += chain_align((size_t)ph.contrib * o.Ng * kGroupN * sizeof(float));
+        d.pad_ = 0;
+        off += chain_pairs_bytes(o);
     }
     if (workspace_bytes < off)
         return fail(LLMOPS_EWORKSPACE, "fc chain needs %zu workspace bytes, got %zu", off, workspace_bytes);
@@ -544,15 +612,15 @@ extern "C" int llmops_fc_chain_run(const void* plan, int n_ops, int group_k, voi
     const ChainOpDev* p = reinterpret_cast<const ChainOpDev*>(plan);
     unsigned* sync = reinterpret_cast<unsigned*>(workspace);
     hipStream_t st = as_stream(stream);
-    const int ring = g_chain_ring > 0 ? g_chain_ring : 4;
+    const int ring = g_chain_ring > 0 ? g_chain_ring : 6;
     if (group_k == 128) {
-        if (ring <= 2) chain_launch<128, 2>(p, n_ops, sync, P, st);
-        else if (ring == 3) chain_launch<128, 3>(p, n_ops, sync, P, st);
-        else chain_launch<128, 4>(p, n_ops, sync, P, st);
+        if (ring <= 4) chain_launch<128, 4>(p, n_ops, sync, P, st);
+        else if (ring <= 6) chain_launch<128, 6>(p, n_ops, sync, P, st);
+        else chain_launch<128, 8>(p, n_ops, sync, P, st);
     } else {
-        if (ring <= 2) chain_launch<32, 2>(p, n_ops, sync, P, st);
-        else if (ring == 3) chain_launch<32, 3>(p, n_ops, sync, P, st);
-        else chain_launch<32, 4>(p, n_ops, sync, P, st);
+        if (ring <= 4) chain_launch<32, 4>(p, n_ops, sync, P, st);
+        else if (ring <= 6) chain_launch<32, 6>(p, n_ops, sync, P, st);
+        else chain_launch<32, 8>(p, n_ops, sync, P, st);
     }
     LLMOPS_LAUNCH_CHECK();
     return LLMOPS_OK;
