@@ -228,9 +228,9 @@ int llmops_fc_chain_status(const void* workspace, int32_t* status);
 /* knobs: LDS ring depth in steps per wavefront (2..4, 0 = default), workgroups (0 = one per CU),
  * barrier wait limit in 100 MHz ticks (<= 0 keeps it) */
 void llmops_fc_chain_set_tuning(int ring_depth, int grid, long long spin_limit_ticks);
-/* diagnostics: when `buffer` (device, int64 [grid][n_ops][4]) is set, every workgroup records the
- * 100 MHz wall clock at four points of every op (start, input row quantized, stream done, arrived
- * at the barrier).  NULL switches it off. */
+/* diagnostics: when `buffer` (device, int64 [grid][n_ops][4]) is set, the first service wave of every
+ * workgroup records the 100 MHz wall clock at four points of every op (op start, input row
+ * quantized, all sums in LDS, outputs published).  NULL switches it off. */
 void llmops_fc_chain_set_trace(void* buffer);
 
 /* ------------------------------------------------------------------------------------------
