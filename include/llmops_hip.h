@@ -246,6 +246,10 @@ int llmops_calib_copy(const void* src, void* dst, int64_t bytes, int workgroups,
  * wavefronts per workgroup (4, 8, 16; 0 = default).  Values <= 0 / < 0 leave a knob unchanged. */
 void llmops_fc_set_tuning(int target_workgroups, int waves_per_workgroup);
 
+/* prefill GEMM planner knob: force the row-tile factor of the LDS-tiled MFMA kernel (1, 2 or 4:
+ * 32, 64 or 128 rows per workgroup); 0 = choose per shape */
+void llmops_gemm_set_tuning(int row_tile_factor);
+
 #ifdef __cplusplus
 }
 #endif

@@ -185,7 +185,7 @@ struct GemmSmem {
 };
 
 template <int RT, bool PARTIALS>
-__global__ __launch_bounds__(256, 2) void fc_gemm_lds_kernel(const uint8_t* __restrict__ weiq, const int8_t* __restrict__ xq,
+__global__ __launch_bounds__(256, (RT == 4 ? 2 : (RT == 2 ? 3 : 4))) void fc_gemm_lds_kernel(const uint8_t* __restrict__ weiq, const int8_t* __restrict__ xq,
                                                            const float* __restrict__ xd, const float* __restrict__ gs,
                                                            const float2* __restrict__ xsT, float* __restrict__ out,
                                                            int32_t* __restrict__ out_i, int Ng, int Kg, int64_t ldo,
@@ -433,22 +433,50 @@ struct GemmPlan {
     bool lds;
 };
 
-static GemmPlan plan_gemm(int64_t rows, int64_t Ng, int64_t Kg, int G) {
-    GemmPlan p;
-    p.lds = (G == 128);
-    int64_t tiles;
-    if (p.lds) {
-        p.RT = rows > 64 ? 4 : (rows > 32 ? 2 : 1);            // BM = 32 * RT rows per workgroup
-        tiles = ((Ng + 3) / 4) * ((rows + p.RT * 32 - 1) / (p.RT * 32));
-    } else {
-        p.RT = rows > 32 ? 4 : (rows > 16 ? 2 : 1);            // RT*16 rows per wave
-        tiles = (((Ng + 1) / 2 + 3) / 4) * ((rows + p.RT * 16 - 1) / (p.RT * 16));
-    }
-    int S = (int)((512 + tiles - 1) / tiles);  // aim for >= 512 workgroups (2 per CU)
+static int g_gemm_rt = 0;  // 0 = choose per shape
+
+// Split-K factor for `tiles` output tiles on a machine with `slots` resident workgroups.
+static void gemm_split(int64_t tiles, int64_t slots, int64_t Kg, GemmPlan& p) {
+    int S = (int)((slots + tiles - 1) / tiles);
     if (S > Kg) S = (int)Kg;
     if (S < 1) S = 1;
     p.kb_per_split = (int)((Kg + S - 1) / S);
     p.S = (int)((Kg + p.kb_per_split - 1) / p.kb_per_split);
+}
+
+static GemmPlan plan_gemm(int64_t rows, int64_t Ng, int64_t Kg, int G) {
+    GemmPlan p;
+    p.lds = (G == 128);
+    if (!p.lds) {
+        p.RT = rows > 32 ? 4 : (rows > 16 ? 2 : 1);  // RT*16 rows per wave
+        gemm_split((((Ng + 1) / 2 + 3) / 4) * ((rows + p.RT * 16 - 1) / (p.RT * 16)), 512, Kg, p);
+        return p;
+    }
+    // BM = 32*RT rows per workgroup.  Bigger tiles reuse the unpacked weights over more rows but need
+    // more registers: RT = 4 runs two workgroups per CU, RT = 2 three, RT = 1 four.  Measured rate per
+    // row at full occupancy (M = 2048): 1.0 : 0.98 : 0.77.  What decides between them at smaller M is
+    // how evenly the tiles fill the machine, so the plan takes the RT with the least estimated time:
+    // rounds of resident workgroups x (rows per tile x workgroups sharing a CU / efficiency) x share of
+    // K per split.
+    static const int kRT[3] = {4, 2, 1};
+    static const int kWgPerCu[3] = {2, 3, 4};
+    static const double kEff[3] = {1.0, 0.98, 0.77};
+    double best = 0.0;
+    for (int i = 0; i < 3; i++) {
+        if (g_gemm_rt > 0 && kRT[i] != g_gemm_rt) continue;
+        GemmPlan q = p;
+        q.RT = kRT[i];
+        const int64_t bm = 32 * q.RT, slots = 256 * kWgPerCu[i];
+        const int64_t tiles = ((Ng + 3) / 4) * ((rows + bm - 1) / bm);
+        gemm_split(tiles, slots, Kg, q);
+        const int64_t rounds = (tiles * q.S + slots - 1) / slots;
+        double cost = (double)rounds * (double)(bm * kWgPerCu[i]) / kEff[i] * (double)q.kb_per_split / (double)Kg;
+        if (q.S > 1) cost *= 1.1;  // the partial sums take a second launch
+        if (best == 0.0 || cost < best) {
+            best = cost;
+            p = q;
+        }
+    }
     return p;
 }
 
@@ -531,3 +559,5 @@ int launch_gemm_partials(const uint8_t* w, const int8_t* xq, int32_t* acc, int64
 }
 
 }  // namespace llmops
+
+extern "C" void llmops_gemm_set_tuning(int rows_per_wave_tile) { llmops::g_gemm_rt = rows_per_wave_tile; }
