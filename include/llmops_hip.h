@@ -108,10 +108,15 @@ int llmops_fc_Q4A_residual(const float* x, int64_t rows, int64_t K, const int8_t
  *   residual    : y += residual (iadd, ops/op_misc.hpp:55-79), fp32 [rows,N_out]
  *   glu         : weiq holds gate and up strips interleaved (strip 2i = gate strip i, 2i+1 = up strip i,
  *                 Ng even) and y[r,n] = silu(gate[r,n]) * up[r,n] (itrans "silu" + imul), N_out = F
+ *   sumsq_out   : fp32 [rows,Ng], receives the sum of squares of every strip's 32 outputs (after the
+ *                 residual add); not with glu
+ *   sumsq_in, sumsq_parts : with norm_w: fp32 [rows,sumsq_parts] whose row sums are sum(x^2) -- what the
+ *                 FC that produced x left in its sumsq_out -- so that the rmsnorm does not read the row again
  * N_out is the number of output columns (Ng*32-ish without glu, Ng/2*32-ish with it). */
 int llmops_fc_Q4A_decode(const float* x, int64_t rows, int64_t K, const int8_t* weiq, int64_t Ng, int64_t Kg,
                          int group_k, int64_t N_out, const float* norm_w, float eps, const float* residual, int glu,
-                         float* y, void* workspace, size_t workspace_bytes, llmops_stream_t stream);
+                         const float* sumsq_in, int64_t sumsq_parts, float* sumsq_out, float* y, void* workspace,
+                         size_t workspace_bytes, llmops_stream_t stream);
 
 /* The second half of fc_Q4A on its own (ops/op_fc.hpp:318-423): the product for activations that
  * llmops_FC_dynamic_quantize_x has already quantized (xq int8 [rows,Kg*G], xd and gsum fp32

@@ -13,7 +13,7 @@ int launch_gemv(const uint8_t* w, const int8_t* xq, const float* xd, const float
                 unsigned* counters, int64_t rows, int64_t Ng, int64_t Kg, int G, int64_t N, hipStream_t st);
 int launch_gemv_fused(const uint8_t* w, const float* x, float* y, float* part, unsigned* counters, int64_t rows, int64_t Ng,
                       int64_t Kg, int G, int64_t N, const float* residual, const float* norm_w, float eps, bool glu,
-                      hipStream_t st);
+                      const float* sumsq_in, int sumsq_parts, float* sumsq_out, hipStream_t st);
 int launch_add(float* a, const float* b, int64_t total, hipStream_t st);
 int launch_gemv_partials(const uint8_t* w, const int8_t* xq, int32_t* acc, int64_t rows, int64_t Ng, int64_t Kg, int G,
                          hipStream_t st);
@@ -80,7 +80,8 @@ static int fc_impl(const float* x, int64_t rows, int64_t K, const int8_t* weiq, 
     const uint8_t* w = reinterpret_cast<const uint8_t*>(weiq);
     // few rows: one launch, the streaming kernel quantizes the activations it needs on the fly
     if (rows <= kMaxGemvRows)
-        return launch_gemv_fused(w, x, y, part, counters, rows, Ng, Kg, group_k, N, residual, nullptr, 0.0f, false, st);
+        return launch_gemv_fused(w, x, y, part, counters, rows, Ng, Kg, group_k, N, residual, nullptr, 0.0f, false, nullptr, 0,
+                                 nullptr, st);
     float2* xst = reinterpret_cast<float2*>(ws + lay.off_xst);
     int rc = launch_quant_x(x, rows, K, group_k, xq, xd, gs, xst, false, st);
     if (rc) return rc;
@@ -104,7 +105,8 @@ extern "C" int llmops_fc_Q4A_residual(const float* x, int64_t rows, int64_t K, c
 
 extern "C" int llmops_fc_Q4A_decode(const float* x, int64_t rows, int64_t K, const int8_t* weiq, int64_t Ng, int64_t Kg,
                                     int group_k, int64_t N_out, const float* norm_w, float eps, const float* residual,
-                                    int glu, float* y, void* workspace, size_t workspace_bytes, llmops_stream_t stream) {
+                                    int glu, const float* sumsq_in, int64_t sumsq_parts, float* sumsq_out, float* y,
+                                    void* workspace, size_t workspace_bytes, llmops_stream_t stream) {
     LLMOPS_REQUIRE(valid_group(group_k));
     LLMOPS_REQUIRE(x != nullptr && weiq != nullptr && y != nullptr && workspace != nullptr);
     LLMOPS_REQUIRE(rows > 0 && rows <= kMaxGemvRows);
@@ -118,13 +120,15 @@ extern "C" int llmops_fc_Q4A_decode(const float* x, int64_t rows, int64_t K, con
         LLMOPS_REQUIRE(N_out > (Ng - 1) * kGroupN && N_out <= Ng * kGroupN);
     }
     if (norm_w != nullptr) LLMOPS_REQUIRE((K % 4) == 0 && aligned(x, 16) && aligned(norm_w, 8));
+    if (sumsq_in != nullptr) LLMOPS_REQUIRE(norm_w != nullptr && sumsq_parts > 0 && sumsq_parts <= 65536);
+    if (sumsq_out != nullptr) LLMOPS_REQUIRE(!glu);
     const FcWorkspace lay = fc_layout(rows, Ng, Kg, group_k);
     if (workspace_bytes < lay.total)
         return fail(LLMOPS_EWORKSPACE, "fc_Q4A needs %zu workspace bytes, got %zu", lay.total, workspace_bytes);
     uint8_t* ws = reinterpret_cast<uint8_t*>(workspace);
     return launch_gemv_fused(reinterpret_cast<const uint8_t*>(weiq), x, y, reinterpret_cast<float*>(ws + lay.off_part),
                              reinterpret_cast<unsigned*>(ws), rows, Ng, Kg, group_k, N_out, residual, norm_w, eps, glu != 0,
-                             as_stream(stream));
+                             sumsq_in, (int)sumsq_parts, sumsq_out, as_stream(stream));
 }
 
 extern "C" int llmops_fc_Q4A_prequantized(const int8_t* xq, const float* xd, const float* gsum, int64_t rows,

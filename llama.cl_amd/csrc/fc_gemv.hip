@@ -53,11 +53,21 @@ __device__ __forceinline__ TileRange tile_range(int Kg, int S, int steps_per_spl
     return r;
 }
 
+// Sum of squares of a strip's 32 outputs (threads tr*32 .. tr*32+31 hold them, zeros for padding):
+// the next FC's rmsnorm adds these per-strip sums instead of re-reading the whole row.
+__device__ __forceinline__ void strip_sumsq(float out, bool mine, int tr, int nb, int strips, float* __restrict__ sumsq_out) {
+    float sq = out * out;
+#pragma unroll
+    for (int o = 16; o > 0; o >>= 1) sq += __shfl_xor(sq, o, 64);
+    if (mine && (threadIdx.x & 31) == 0) sumsq_out[(int64_t)tr * strips + nb] = sq;
+}
+
 // Sum the lanes' running sums over row slots, waves and k-splits and store the strip's outputs.
 template <int MT, int NW>
 __device__ __forceinline__ void finish_strip(float f[MT][4], float (*red)[MT][kGroupN], unsigned* ticket_sh, int nb, int s,
                                              int S, int rows, int64_t N, float* __restrict__ y, float* part,
-                                             unsigned* counters, const float* __restrict__ residual) {
+                                             unsigned* counters, const float* __restrict__ residual,
+                                             float* __restrict__ sumsq_out = nullptr) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int quad = lane & 7, rs = lane >> 3;
     // sum the 8 row slots (lane bits 3..5)
@@ -81,7 +91,7 @@ __device__ __forceinline__ void finish_strip(float f[MT][4], float (*red)[MT][kG
 
     const int tr = threadIdx.x >> 5, tn = threadIdx.x & 31;  // (row, column) this thread finalises
     const bool mine = tr < MT && tr < rows;
-    if (S == 1 && !mine) return;
+    if (S == 1 && !mine && sumsq_out == nullptr) return;
     const int64_t n = (int64_t)nb * kGroupN + tn;
     const int64_t Np = (int64_t)gridDim.x / S * kGroupN;
     float v = 0.0f;
@@ -90,7 +100,9 @@ __device__ __forceinline__ void finish_strip(float f[MT][4], float (*red)[MT][kG
         for (int w = 0; w < NW; w++) v += red[w][tr][tn];
     }
     if (S == 1) {
-        if (n < N) y[(int64_t)tr * N + n] = residual ? v + residual[(int64_t)tr * N + n] : v;
+        const float out = (mine && n < N) ? (residual ? v + residual[(int64_t)tr * N + n] : v) : 0.0f;
+        if (mine && n < N) y[(int64_t)tr * N + n] = out;
+        if (sumsq_out != nullptr) strip_sumsq(out, mine, tr, nb, (int)(gridDim.x / S), sumsq_out);
         return;
     }
     // Cross-workgroup hand-off without cache-wide fences: partial sums are written and read with
@@ -106,12 +118,15 @@ __device__ __forceinline__ void finish_strip(float f[MT][4], float (*red)[MT][kG
         *ticket_sh = __hip_atomic_fetch_add(&counters[nb], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __syncthreads();
     if (*ticket_sh != (unsigned)(S - 1)) return;
+    float out = 0.0f;
     if (mine && n < N) {
         float acc = 0.0f;
         for (int i = 0; i < S; i++)
             acc += __hip_atomic_load(&part[((int64_t)i * rows + tr) * Np + n], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        y[(int64_t)tr * N + n] = residual ? acc + residual[(int64_t)tr * N + n] : acc;
+        out = residual ? acc + residual[(int64_t)tr * N + n] : acc;
+        y[(int64_t)tr * N + n] = out;
     }
+    if (sumsq_out != nullptr) strip_sumsq(out, mine, tr, nb, (int)(gridDim.x / S), sumsq_out);
     if (threadIdx.x == 0) __hip_atomic_store(&counters[nb], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // next launch
 }
 
@@ -168,15 +183,23 @@ __global__ __launch_bounds__(NW * 64) void fc_gemv_kernel(const uint8_t* __restr
 //   kGlu : the packed tensor holds gate and up strips interleaved (strip 2i = gate strip i, strip
 //          2i+1 = up strip i); a workgroup computes both and stores silu(gate)*up
 //          (itrans "silu" + imul, ops/op_misc.hpp:83-138).  Replaces two launches behind the FC.
-constexpr int kNorm = 1, kGlu = 2;
+//   kSums: with kNorm, the sum of squares of the row comes as per-strip partial sums left behind by
+//          the FC that produced the row; every wave adds them up by itself (no pass over the row, no
+//          workgroup barrier).
+constexpr int kNorm = 1, kGlu = 2, kSums = 4;
 
+// One activation row needs few registers; asking for eight waves per SIMD (two workgroups of 16 waves
+// per CU) keeps every variant at or below 64 registers, so that grids of 257..512 workgroups are
+// resident at once.  (The second launch-bound argument counts waves per SIMD.)
 template <int G, int MT, int NW, int MODE>
-__global__ __launch_bounds__(NW * 64) void fc_gemv_fused_kernel(const uint8_t* __restrict__ weiq, const float* __restrict__ x,
+__global__ __launch_bounds__(NW * 64, (MT == 1 ? NW / 2 : 1)) void fc_gemv_fused_kernel(const uint8_t* __restrict__ weiq, const float* __restrict__ x,
                                                                  float* __restrict__ y, float* part, unsigned* counters,
                                                                  int Kg, int64_t K, int64_t N, int rows, int S,
                                                                  int steps_per_split, const float* __restrict__ residual,
-                                                                 const float* __restrict__ norm_w, float eps) {
-    constexpr bool NORM = (MODE & kNorm) != 0, GLU = (MODE & kGlu) != 0;
+                                                                 const float* __restrict__ norm_w, float eps,
+                                                                 const float* __restrict__ sumsq_in, int sumsq_parts,
+                                                                 float* __restrict__ sumsq_out) {
+    constexpr bool NORM = (MODE & kNorm) != 0, GLU = (MODE & kGlu) != 0, SUMS = (MODE & kSums) != 0;
     constexpr int NWS = GLU ? NW / 2 : NW;  // waves per strip
     __shared__ float red[NW][MT][kGroupN];
     __shared__ __align__(16) XSlot<G> xs[NW][MT];
@@ -208,9 +231,20 @@ __global__ __launch_bounds__(NW * 64) void fc_gemv_fused_kernel(const uint8_t* _
 
     // The loads return in issue order, so everything the rmsnorm statistic needs is requested
     // before the first weight block: the statistic is then computed while that block is in flight.
-    constexpr int NV = 4;  // float4 per thread held for the statistic (covers K <= NV*4*threads)
+    constexpr int NV = (NORM && !SUMS) ? 4 : 1;  // float4 per thread held for the statistic (covers K <= NV*4*threads)
     float4 nv[NORM ? MT : 1][NV];
-    if (NORM) {
+    // SUMS: this lane's share of the handed-over partial sums: four loads per row in flight together.
+    // They are only added up after the first weight loads have been issued (below): using them here
+    // would make the wave wait for them before it asks for anything else.
+    float p4[(NORM && SUMS) ? MT : 1][4];
+    if (NORM && SUMS) {
+#pragma unroll
+        for (int r = 0; r < MT; r++)
+#pragma unroll
+            for (int u = 0; u < 4; u++)
+                p4[(NORM && SUMS) ? r : 0][u] =
+                    (r < rows && lane + 64 * u < sumsq_parts) ? sumsq_in[(int64_t)r * sumsq_parts + lane + 64 * u] : 0.0f;
+    } else if (NORM) {
 #pragma unroll
         for (int r = 0; r < MT; r++)
 #pragma unroll
@@ -232,7 +266,16 @@ __global__ __launch_bounds__(NW * 64) void fc_gemv_fused_kernel(const uint8_t* _
     }
 
     float rsn[MT];
-    if (NORM) {
+    if (NORM && SUMS) {
+#pragma unroll
+        for (int r = 0; r < MT; r++) {
+            const int rr = (NORM && SUMS) ? r : 0;
+            float a = (p4[rr][0] + p4[rr][1]) + (p4[rr][2] + p4[rr][3]);
+            if (r < rows)
+                for (int i = lane + 256; i < sumsq_parts; i += 64) a += sumsq_in[(int64_t)r * sumsq_parts + i];
+            rsn[r] = 1.0f / sqrtf(wave_sum_dpp(a) / (float)K + eps);
+        }
+    } else if (NORM) {
 #pragma unroll
         for (int r = 0; r < MT; r++) {
             float ss = 0.0f;
@@ -300,7 +343,7 @@ __global__ __launch_bounds__(NW * 64) void fc_gemv_fused_kernel(const uint8_t* _
     }
 
     if (!GLU) {
-        finish_strip<MT, NW>(f, red, &ticket_sh, tr.nb, tr.s, S, rows, N, y, part, counters, residual);
+        finish_strip<MT, NW>(f, red, &ticket_sh, tr.nb, tr.s, S, rows, N, y, part, counters, residual, sumsq_out);
         return;
     }
     // gate/up epilogue: sum row slots, then the two halves of the workgroup, then silu(gate)*up
@@ -408,6 +451,9 @@ struct FusedOps {
     const float* norm_w;    // x = rmsnorm(x, norm_w, eps) first
     float eps;
     bool glu;               // interleaved gate/up strips, y = silu(gate)*up
+    const float* sumsq_in;  // per-part sums of squares of x (instead of reading the row for the rmsnorm)
+    int sumsq_parts;
+    float* sumsq_out;       // per-strip sums of squares of y [rows, Ng]
 };
 
 template <int G, int MT, int NW>
@@ -417,12 +463,16 @@ static void launch_fused_t(const uint8_t* w, const float* x, float* y, float* pa
 #define LLMOPS_FUSED(MODE, GRID)                                                                                      \
     fc_gemv_fused_kernel<G, MT, NW, MODE><<<(unsigned)(GRID), NW * 64, 0, st>>>(w, x, y, part, counters, (int)Kg, K, N, rows, \
                                                                                 p.S, p.steps_per_split, o.residual,  \
-                                                                                o.norm_w, o.eps)
+                                                                                o.norm_w, o.eps, o.sumsq_in,         \
+                                                                                o.sumsq_parts, o.sumsq_out)
+    const bool sums = o.norm_w != nullptr && o.sumsq_in != nullptr;
     if (o.glu) {
-        if (o.norm_w) LLMOPS_FUSED(kNorm | kGlu, Ng / 2);
+        if (sums) LLMOPS_FUSED(kNorm | kGlu | kSums, Ng / 2);
+        else if (o.norm_w) LLMOPS_FUSED(kNorm | kGlu, Ng / 2);
         else LLMOPS_FUSED(kGlu, Ng / 2);
     } else {
-        if (o.norm_w) LLMOPS_FUSED(kNorm, Ng * p.S);
+        if (sums) LLMOPS_FUSED(kNorm | kSums, Ng * p.S);
+        else if (o.norm_w) LLMOPS_FUSED(kNorm, Ng * p.S);
         else LLMOPS_FUSED(0, Ng * p.S);
     }
 #undef LLMOPS_FUSED
@@ -431,10 +481,10 @@ static void launch_fused_t(const uint8_t* w, const float* x, float* y, float* pa
 // raw fp32 activations, quantized inside the kernel (+ optional rmsnorm / residual / gate-up epilogue)
 int launch_gemv_fused(const uint8_t* w, const float* x, float* y, float* part, unsigned* counters, int64_t rows, int64_t Ng,
                       int64_t Kg, int G, int64_t N, const float* residual, const float* norm_w, float eps, bool glu,
-                      hipStream_t st) {
+                      const float* sumsq_in, int sumsq_parts, float* sumsq_out, hipStream_t st) {
     GemvPlan p = plan_gemv(rows, Ng, Kg, G, true);
     if (glu) p.S = 1;
-    const FusedOps o{residual, norm_w, eps, glu};
+    const FusedOps o{residual, norm_w, eps, glu, sumsq_in, sumsq_parts, sumsq_out};
 #define LLMOPS_CASE(GG, MT, NWW) launch_fused_t<GG, MT, NWW>(w, x, y, part, counters, Ng, Kg, N, (int)rows, p, o, st)
     if (G == 128) {
         if (rows == 1) LLMOPS_CASE(128, 1, 16);

@@ -151,13 +151,15 @@ def interleave_gate_up(gate_packed, up_packed):
     return torch.stack((gate_packed, up_packed), dim=1).reshape(-1, *gate_packed.shape[1:]).contiguous()
 
 
-def fc_Q4A_decode(input, weiq, N_out, norm=None, residual=None, glu=False):
+def fc_Q4A_decode(input, weiq, N_out, norm=None, residual=None, glu=False, sumsq_in=None, want_sumsq=False):
     """Extension: fc_Q4A with its neighbours of the decode step folded in (one launch for B*M <= 8).
 
     norm=(weight, eps): input is rmsnorm'ed first;  residual: added to the result;
     glu=True: ``weiq`` holds interleaved gate/up strips (``interleave_gate_up``) and the result is
-    silu(gate)*up with N_out = F columns.  With more than 8 rows the same arithmetic is composed
-    from the separate ops."""
+    silu(gate)*up with N_out = F columns.  want_sumsq=True returns ``(out, sumsq)`` where ``sumsq``
+    [B*M, strips] holds the sum of squares of every 32 outputs; passed as ``sumsq_in`` to the FC that
+    rmsnorms ``out`` it saves that FC the pass over the row.  With more than 8 rows the same
+    arithmetic is composed from the separate ops."""
     _dev(input, torch.float32, 3, "input")
     _dev(weiq, torch.int8, 3, "wei_quantized")
     g = group_k_of(weiq)
@@ -171,6 +173,10 @@ def fc_Q4A_decode(input, weiq, N_out, norm=None, residual=None, glu=False):
     if residual is not None:
         _dev(residual, torch.float32, 3, "residual")
         _require(tuple(residual.shape) == (B, M, N_out), "residual.is({B, M, N})")
+    if sumsq_in is not None:
+        _dev(sumsq_in, torch.float32, 2, "sumsq_in")
+        _require(norm is not None and sumsq_in.shape[0] == rows, "sumsq_in.is({B*M, parts}) with norm")
+    _require(not (want_sumsq and glu), "no sumsq with glu")
     if rows > 8:
         x = input if norm is None else rmsnorm_out(input, norm[0], norm[1])
         if glu:
@@ -178,15 +184,23 @@ def fc_Q4A_decode(input, weiq, N_out, norm=None, residual=None, glu=False):
             y = fc_Q4A(x, weiq, 2 * N_out).view(B, M, N_out // 32, 2, 32)
             gu = torch.cat((y[..., 0, :].reshape(B, M, N_out), y[..., 1, :].reshape(B, M, N_out)), dim=-1)
             return silu_mul(gu)
-        return fc_Q4A(x, weiq, N_out, residual=residual)
+        out = fc_Q4A(x, weiq, N_out, residual=residual)
+        if want_sumsq:
+            pad = torch.nn.functional.pad(out.reshape(rows, N_out), (0, Ng * 32 - N_out))
+            return out, pad.view(rows, Ng, 32).square().sum(-1)
+        return out
     lib = _lib.load()
     ws = _workspace(input.device, lib.llmops_fc_Q4A_workspace_bytes(rows, K, Ng, Kg, g))
     out = torch.empty((B, M, N_out), dtype=torch.float32, device=input.device)
+    sumsq = torch.empty((rows, Ng), dtype=torch.float32, device=input.device) if want_sumsq else None
     _lib.check(lib.llmops_fc_Q4A_decode(_ptr(input), rows, K, _ptr(weiq), Ng, Kg, g, N_out,
                                         _ptr(norm[0]) if norm is not None else None, float(norm[1]) if norm is not None else 0.0,
-                                        _ptr(residual) if residual is not None else None, int(bool(glu)), _ptr(out), _ptr(ws),
+                                        _ptr(residual) if residual is not None else None, int(bool(glu)),
+                                        _ptr(sumsq_in) if sumsq_in is not None else None,
+                                        sumsq_in.shape[1] if sumsq_in is not None else 0,
+                                        _ptr(sumsq) if sumsq is not None else None, _ptr(out), _ptr(ws),
                                         ws.numel(), _stream(input)))
-    return out
+    return (out, sumsq) if want_sumsq else out
 
 
 class FcChain:

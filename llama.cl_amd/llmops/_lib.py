@@ -30,7 +30,7 @@ SIGNATURES = {
     "llmops_fc_Q4A_residual": (c_int, [c_ptr, c_i64, c_i64, c_ptr, c_i64, c_i64, c_int, c_i64, c_ptr, c_ptr, c_ptr, c_size,
                                        c_ptr]),
     "llmops_fc_Q4A_decode": (c_int, [c_ptr, c_i64, c_i64, c_ptr, c_i64, c_i64, c_int, c_i64, c_ptr, c_f32, c_ptr, c_int, c_ptr,
-                                     c_ptr, c_size, c_ptr]),
+                                     c_i64, c_ptr, c_ptr, c_ptr, c_size, c_ptr]),
     "llmops_fc_Q4A_prequantized": (c_int, [c_ptr, c_ptr, c_ptr, c_i64, c_ptr, c_i64, c_i64, c_int, c_i64, c_ptr, c_ptr,
                                            c_size, c_ptr]),
     "llmops_fc_Q4A_partials": (c_int, [c_ptr, c_i64, c_ptr, c_i64, c_i64, c_int, c_ptr, c_int, c_ptr]),

@@ -79,9 +79,14 @@ class LlamaDecoder:
         H = self.configs["hidden_size"]
         F = self.configs["intermediate_size"]
         hidden_states = self.embed_tokens(input_ids)
-        step = self._layer_fused if self.plan == "fused" else self._layer_reference
+        if self.plan == "fused":
+            sumsq = None  # per-strip sums of squares of hidden_states, handed from FC to FC for the rmsnorms
+            for i, ops in enumerate(self.layers):
+                hidden_states, sumsq = self._layer_fused(i, ops, hidden_states, sumsq, kv_cache, kv_cache_slots, position_id)
+            return llmops.fc_Q4A_decode(hidden_states, self.lm_head.weight, self.lm_head.N,
+                                        norm=(self.norm.weight, self.norm.eps), sumsq_in=sumsq)
         for i, ops in enumerate(self.layers):
-            hidden_states = step(i, ops, hidden_states, kv_cache, kv_cache_slots, position_id)
+            hidden_states = self._layer_reference(i, ops, hidden_states, kv_cache, kv_cache_slots, position_id)
         self.norm(hidden_states)
         return self.lm_head(hidden_states)
 
@@ -105,20 +110,22 @@ class LlamaDecoder:
         llmops.iadd(hidden_states, attn_output)
         return hidden_states
 
-    def _layer_fused(self, i, ops, hidden_states, kv_cache, kv_cache_slots, position_id):
+    def _layer_fused(self, i, ops, hidden_states, sumsq, kv_cache, kv_cache_slots, position_id):
         """Same arithmetic, 6 launches per decode layer instead of 18: rmsnorm inside the q|k|v and
-        gate|up FCs, silu*up in the gate|up epilogue (interleaved strips), residual adds inside the o
-        and down projections, rope + cache update inside the attention kernel."""
+        gate|up FCs (fed with the sums of squares that the FC producing their input leaves behind),
+        silu*up in the gate|up epilogue (interleaved strips), residual adds inside the o and down
+        projections, rope + cache update inside the attention kernel."""
         H, F = self.configs["hidden_size"], self.configs["intermediate_size"]
         n1, n2 = ops["input_layernorm"], ops["post_attention_layernorm"]
-        qkv = llmops.fc_Q4A_decode(hidden_states, ops["qkv_proj"].weight, 3 * H, norm=(n1.weight, n1.eps))
+        qkv = llmops.fc_Q4A_decode(hidden_states, ops["qkv_proj"].weight, 3 * H, norm=(n1.weight, n1.eps), sumsq_in=sumsq)
         q, k, v = qkv[..., :H], qkv[..., H:2 * H], qkv[..., 2 * H:]
         if not q.is_contiguous():  # more than one token: the op needs dense [B,qL,H*S] tensors
             q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
         llmops.attention_rope2(q, k, v, self.inv_freq, kv_cache, kv_cache_slots, position_id, i)
-        attn_output = llmops.fc_Q4A_decode(q, ops["o_proj"].weight, H, residual=hidden_states)
-        act = llmops.fc_Q4A_decode(attn_output, ops["gate_up_proj"].weight, F, norm=(n2.weight, n2.eps), glu=True)
-        return llmops.fc_Q4A_decode(act, ops["down_proj"].weight, H, residual=attn_output)
+        attn_output, ss = llmops.fc_Q4A_decode(q, ops["o_proj"].weight, H, residual=hidden_states, want_sumsq=True)
+        act = llmops.fc_Q4A_decode(attn_output, ops["gate_up_proj"].weight, F, norm=(n2.weight, n2.eps), glu=True,
+                                   sumsq_in=ss)
+        return llmops.fc_Q4A_decode(act, ops["down_proj"].weight, H, residual=attn_output, want_sumsq=True)
 
     def capture_decode(self, kv_cache, slot, position_id, stream=None):
         """Capture one decode step (batch 1, one token, fixed slot/position) as a HIP graph.

@@ -234,3 +234,36 @@ def test_fc_decode_folded_ops_vs_oracle(ops, orc, G, rows):
     assert max_rel_err(host(ops.fc_Q4A_decode(dev(x), il, F, glu=True)), want) <= 1e-5
     want = orc.imul(orc.fc(xn, pu, F), orc.silu(orc.fc(xn, pg, F)))
     assert max_rel_err(host(ops.fc_Q4A_decode(dev(x), il, F, norm=(dev(nw), 1e-5), glu=True)), want) <= 1e-4
+
+
+@pytest.mark.parametrize("G", [32, 128])
+@pytest.mark.parametrize("rows", [1, 3, 8, 20])
+@pytest.mark.parametrize("N,K", [(1000, 1024), (4096, 11008)])
+def test_fc_decode_sumsq_handover(ops, orc, G, rows, N, K):
+    """The per-strip sums of squares an FC leaves behind (also through the split-K hand-off: K = 11008),
+    and the rmsnorm of the next FC fed with them instead of reading its input row."""
+    rng = np.random.default_rng(rows + G + N)
+    x = rng.standard_normal((1, rows, K)).astype(np.float32)
+    w = (rng.standard_normal((N, K)) * 0.02).astype(np.float32)
+    res = rng.standard_normal((1, rows, N)).astype(np.float32)
+    pw = dev(orc.quant_w(w, G))
+    y, ss = ops.fc_Q4A_decode(dev(x), pw, N, residual=dev(res), want_sumsq=True)
+    yh = host(y).astype(np.float64).reshape(rows, N)
+    strips = -(-N // 32)
+    pad = np.zeros((rows, strips * 32))
+    pad[:, :N] = yh
+    want = (pad.reshape(rows, strips, 32) ** 2).sum(-1)
+    assert host(ss).shape == (rows, strips)
+    assert np.abs(host(ss) - want).max() <= 1e-5 * want.max()
+    # consumer: rmsnorm(y) @ W2 with and without the handed-over sums must agree to rounding
+    if N % G == 0:
+        F = 352
+        w2 = (rng.standard_normal((F, N)) * 0.02).astype(np.float32)
+        nw = (1.0 + 0.1 * rng.standard_normal(N)).astype(np.float32)
+        p2 = dev(orc.quant_w(w2, G))
+        a = host(ops.fc_Q4A_decode(y, p2, F, norm=(dev(nw), 1e-5)))
+        b = host(ops.fc_Q4A_decode(y, p2, F, norm=(dev(nw), 1e-5), sumsq_in=ss))
+        assert max_rel_err(b, a) <= 1e-4
+        # against the oracle the contract of fc_Q4A applies: the rmsnorm here and there differ by an ulp,
+        # which flips an int8 code now and then (K = 4096 values per output)
+        assert max_rel_err(b, orc.fc(orc.rmsnorm(host(y), nw, 1e-5), host(p2), F)) <= 1e-3
