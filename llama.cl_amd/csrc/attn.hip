@@ -18,6 +18,7 @@
 // every p' in (pq, qL).  Excluded rows get weight exactly 0, as the reference's exp() returns 0
 // for lowest()-max.
 #include <float.h>
+#include <limits.h>
 
 #include "common.h"
 
@@ -400,6 +401,146 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(float* q, float* k, co
     }
 }
 
+// ---- prefill: tiled attention with fp32 MFMA -------------------------------------------------
+// Many query tokens share the K and V rows they look at, so the split kernel above (one workgroup
+// per query and chunk) re-reads the cache qL times.  Here a workgroup owns 128 queries of one head
+// (4 waves x 32 queries, ONE QUERY PER LANE PAIR) and walks the cache in tiles of 32 rows that are
+// staged once in LDS:
+//
+//   S^T = K_tile * Q^T     v_mfma_f32_32x32x2_f32: A = K[kv = lane%32][k = lane/32 + 2i] from LDS,
+//                          B = the lane's own query row, kept in 64 registers.  The result puts
+//                          query lane%32 into the lane, 16 cache rows 8j + 4*(lane/32) + v each.
+//   mask, online softmax   per lane, plus one exchange with lane^32 (the other 16 rows of the tile)
+//   O^T += V_tile^T * P^T  B = the lane's 16 probabilities exactly as they sit in registers (the k
+//                          index of this product is just a summation index, so the cache rows are
+//                          taken in the order 8j + 4*(lane/32) + v), A = V[that row][column] from LDS.
+//
+// Everything a lane holds (running max, sum, 4 x 16 output values) belongs to its own query, so
+// the rescaling needs no cross-lane traffic, and no probability ever goes through LDS.  Tiles that
+// no query of a wave may see (in-chunk causal mask, ops/op_attn.hpp:1007-1011) are skipped.
+// K rows are padded to 130 floats and V rows to 136 so that both operand reads are free of bank
+// conflicts.  Arithmetic is fp32 throughout (fp16 caches are widened when a tile is staged).
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+template <typename T>
+__global__ __launch_bounds__(256, 2) void attn_prefill_kernel(float* q, const T* __restrict__ kc, const T* __restrict__ vc,
+                                                             int64_t qL, int64_t H, int64_t maxlen, int64_t kvLen,
+                                                             const int32_t* __restrict__ row_token, int qtiles) {
+    constexpr int S = 128, BQ = 128, BK = 32, KS = 130, VS = 136;
+    __shared__ __align__(16) float ksh[BK * KS];
+    __shared__ __align__(16) float vsh[BK * VS];
+    __shared__ __align__(16) int tok[BK];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int hf = lane >> 5, c32 = lane & 31;
+    const int qt = blockIdx.x % qtiles;
+    const int64_t bh = blockIdx.x / qtiles, b = bh / H, h = bh % H;
+    const int64_t q_lo_wave = (int64_t)qt * BQ + wave * 32;
+    const int64_t pq = q_lo_wave + c32;  // this lane's query token
+    const bool valid = pq < qL;
+    const int64_t q_hi_wave = (q_lo_wave + 31 < qL ? q_lo_wave + 31 : qL - 1);
+    float* qrow = q + ((b * qL + (valid ? pq : qL - 1)) * H + h) * S;
+    const T* kbase = kc + bh * maxlen * S;
+    const T* vbase = vc + bh * maxlen * S;
+
+    // the lane's query row, elements hf, hf+2, hf+4, ... (the k-values its MFMA operand slots cover)
+    float qreg[64];
+#pragma unroll
+    for (int i = 0; i < 32; i++) {
+        const float4 t = *reinterpret_cast<const float4*>(qrow + i * 4);
+        qreg[2 * i] = hf ? t.y : t.x;
+        qreg[2 * i + 1] = hf ? t.w : t.z;
+    }
+    const float d_scale = 1.0f / sqrtf((float)S);
+    float m_run = -FLT_MAX, l_run = 0.0f;
+    v16f o[4];
+#pragma unroll
+    for (int c = 0; c < 4; c++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) o[c][r] = 0.0f;
+
+    const int trow = threadIdx.x >> 3, tseg = threadIdx.x & 7;  // staging: row of the tile, 16-column segment
+    for (int64_t kv0 = 0; kv0 < kvLen; kv0 += BK) {
+        __syncthreads();  // the previous tile has been consumed
+        {
+            const int64_t r = kv0 + trow < kvLen ? kv0 + trow : kvLen - 1;
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const int col = tseg * 16 + u * 4;
+                const float4 kk = load4(kbase + r * S + col);
+                const float4 vv = load4(vbase + r * S + col);
+                float2* kd = reinterpret_cast<float2*>(&ksh[trow * KS + col]);  // 8-byte aligned (KS even)
+                kd[0] = make_float2(kk.x, kk.y);
+                kd[1] = make_float2(kk.z, kk.w);
+                *reinterpret_cast<float4*>(&vsh[trow * VS + col]) = vv;
+            }
+            if (threadIdx.x < BK) tok[threadIdx.x] = (kv0 + threadIdx.x < kvLen) ? row_token[kv0 + threadIdx.x] : INT_MAX;
+        }
+        __syncthreads();
+        // skip the tile if even the wave's last query may not see any of its rows
+        int tmin = tok[c32];
+#pragma unroll
+        for (int off = 16; off > 0; off >>= 1) tmin = min(tmin, __shfl_xor(tmin, off, 64));
+        if (q_lo_wave >= qL || (int64_t)tmin > q_hi_wave) continue;
+
+        v16f sacc;
+#pragma unroll
+        for (int r = 0; r < 16; r++) sacc[r] = 0.0f;
+        const float* kp = &ksh[c32 * KS + hf];
+#pragma unroll
+        for (int i = 0; i < 64; i++) sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(kp[2 * i], qreg[i], sacc, 0, 0, 0);
+
+        // scale, mask (rows written by later tokens of this call, rows beyond kvLen), running max
+        float mx = -FLT_MAX;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int4 t4 = *reinterpret_cast<const int4*>(&tok[8 * j + 4 * hf]);
+            const int tt[4] = {t4.x, t4.y, t4.z, t4.w};
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                const float sv = (valid && (int64_t)tt[v] <= pq) ? sacc[4 * j + v] * d_scale : -FLT_MAX;
+                sacc[4 * j + v] = sv;
+                mx = fmaxf(mx, sv);
+            }
+        }
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        const float m_new = fmaxf(m_run, mx);
+        const float alpha = expf(m_run - m_new);  // 0 on the first visible tile, 1 while nothing is visible
+        float psum = 0.0f;
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const float pv = (sacc[r] == -FLT_MAX) ? 0.0f : expf(sacc[r] - m_new);
+            sacc[r] = pv;
+            psum += pv;
+        }
+        psum += __shfl_xor(psum, 32, 64);
+        l_run = l_run * alpha + psum;
+        m_run = m_new;
+#pragma unroll
+        for (int c = 0; c < 4; c++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) o[c][r] *= alpha;
+
+        // O^T += V^T P^T; step i of the product takes cache row 8*(i/4) + 4*hf + i%4 of the tile
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            const float* vp = &vsh[(8 * (i / 4) + 4 * hf + (i % 4)) * VS + c32];
+#pragma unroll
+            for (int c = 0; c < 4; c++) o[c] = __builtin_amdgcn_mfma_f32_32x32x2f32(vp[32 * c], sacc[i], o[c], 0, 0, 0);
+        }
+    }
+
+    if (!valid) return;
+    const float inv = 1.0f / l_run;
+    // the lane holds columns 32c + 8j + 4*hf + v of its query's output row
+#pragma unroll
+    for (int c = 0; c < 4; c++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const float4 out = make_float4(o[c][4 * j] * inv, o[c][4 * j + 1] * inv, o[c][4 * j + 2] * inv, o[c][4 * j + 3] * inv);
+            *reinterpret_cast<float4*>(qrow + 32 * c + 8 * j + 4 * hf) = out;
+        }
+}
+
 // ---- softmax op (ops/op_misc.hpp:183-194): one workgroup per row ------------------------------
 __global__ __launch_bounds__(256) void softmax_kernel(float* __restrict__ x, int64_t K) {
     __shared__ float red[4];
@@ -426,6 +567,8 @@ __global__ __launch_bounds__(256) void softmax_kernel(float* __restrict__ x, int
 }
 
 static inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+static int g_prefill_min_tokens = 32;  // query tokens per call from which the tiled MFMA kernel is used
 
 static int pick_pw(int64_t bhq, int64_t kvLen) {
     // smallest chunk count that still gives ~1024 workgroups; chunk = 4*PW rows
@@ -499,6 +642,13 @@ static int attention_impl(float* q, float* k, const float* v, int64_t B, int64_t
     attn_prep_kernel<T><<<(unsigned)(B * qL * H), 64, 0, st>>>(q, k, v, qL, H, S, inv_freq, half, kc, vc, maxlen, slots,
                                                               position_id, row_token);
     LLMOPS_LAUNCH_CHECK();
+    if (qL >= g_prefill_min_tokens) {
+        // enough query tokens to share K/V tiles: the MFMA kernel reads the cache once per 128 queries
+        const int qtiles = (int)((qL + 127) / 128);
+        attn_prefill_kernel<T><<<(unsigned)(B * H * qtiles), 256, 0, st>>>(q, kc, vc, qL, H, maxlen, kvLen, row_token, qtiles);
+        LLMOPS_LAUNCH_CHECK();
+        return LLMOPS_OK;
+    }
     if (pw == 16)
         attn_split_kernel<T, 16><<<grid, 256, 0, st>>>(q, kc, vc, qL, H, maxlen, kvLen, row_token, part, nchunks);
     else if (pw == 8)

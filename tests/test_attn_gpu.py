@@ -139,6 +139,54 @@ def test_attention_prefill_chunks_vs_oracle(ops, orc):
         assert np.abs(cache_after - cache_ref).max() <= 1e-5
 
 
+@pytest.mark.parametrize("cache_dtype", [torch.float32, torch.float16])
+def test_attention_prefill_tiled_vs_oracle(ops, orc, cache_dtype):
+    """Chunks of 32 and more query tokens take the tiled MFMA kernel: several query tiles and waves,
+    tiles that are skipped by the in-chunk mask, a chunk that follows earlier context, a chunk that
+    wraps the ring buffer, and kv lengths that are not multiples of the 32-row tile."""
+    rng = np.random.default_rng(9)
+    B, H, S, maxlen = 2, 3, 128, 300
+    inv_freq = (1.0 / (10000.0 ** (np.arange(0, S, 2, dtype=np.float32) / np.float32(S)))).astype(np.float32)
+    cache = rng.standard_normal((2, B, H, maxlen, S)).astype(np.float32)
+    if cache_dtype == torch.float16:
+        cache = cache.astype(np.float16).astype(np.float32)
+    for past, qL in ((0, 32), (0, 200), (37, 131), (250, 90), (0, 300)):   # (250, 90) wraps the ring buffer
+        q, k, v = (rng.standard_normal((B, qL, H * S)).astype(np.float32) for _ in range(3))
+        slots = ((past + np.arange(qL)) % maxlen).astype(np.int32)
+        g = dict(q=q, k=k, v=v, cache=cache, inv_freq=inv_freq, slots=slots, position_id=past, layer_id=0)
+        out, k_rot, cache_after = run_attention(ops, g, cache_dtype=cache_dtype)
+        if cache_dtype == torch.float16:   # target: fp32 math on the fp16-rounded cache, new rows included
+            kr = orc.rope(k.reshape(B, qL, H, S).transpose(0, 2, 1, 3).copy(), inv_freq, past)
+            c16 = cache.copy()
+            for l, sl in enumerate(slots):
+                c16[0, :, :, sl] = kr[:, :, l].astype(np.float16).astype(np.float32)
+                c16[1, :, :, sl] = v[:, l].reshape(B, H, S).astype(np.float16).astype(np.float32)
+            want = _attend_cache(orc, q, inv_freq, c16, slots, past, maxlen)
+            assert max_rel_err(out, want) <= TOL, (past, qL)
+        else:
+            want, k_ref, cache_ref = orc.attention(q, k, v, inv_freq, cache, slots, past, 0)
+            assert max_rel_err(out, want) <= 1e-4, (past, qL)
+            assert np.abs(cache_after - cache_ref).max() <= 1e-5
+
+
+def _attend_cache(orc, q, inv_freq, cache, slots, past, maxlen):
+    """fp64 attention of the rotated queries over a finished cache with the reference's in-chunk mask."""
+    B, qL, HS = q.shape
+    H, S = cache.shape[2], cache.shape[4]
+    qr = orc.rope(q.reshape(B, qL, H, S).transpose(0, 2, 1, 3).copy(), inv_freq, past).astype(np.float64)
+    kv_len = min(past + qL, maxlen)
+    K, V = cache[0, :, :, :kv_len].astype(np.float64), cache[1, :, :, :kv_len].astype(np.float64)
+    w = np.einsum("bhqs,bhks->bhqk", qr, K) / np.sqrt(S)
+    for pq in range(qL):
+        for later in range(pq + 1, qL):
+            if slots[later] < kv_len:
+                w[:, :, pq, slots[later]] = -np.inf
+    w = np.exp(w - w.max(-1, keepdims=True))
+    w /= w.sum(-1, keepdims=True)
+    o = np.einsum("bhqk,bhks->bhqs", w, V)
+    return o.transpose(0, 2, 1, 3).reshape(B, qL, HS)
+
+
 def test_rope_and_softmax_golden(ops):
     g = load_golden("misc.npz")
     x = dev(g["rope_x"])
