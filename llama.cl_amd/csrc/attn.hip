@@ -432,8 +432,10 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(float* q, const T*
     __shared__ __align__(16) int tok[BK];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int hf = lane >> 5, c32 = lane & 31;
-    const int qt = blockIdx.x % qtiles;
-    const int64_t bh = blockIdx.x / qtiles, b = bh / H, h = bh % H;
+    // late query tiles see the most cache rows: they are dealt out first so that they do not form the tail
+    const int64_t bhs = gridDim.x / qtiles;
+    const int qt = qtiles - 1 - (int)(blockIdx.x / bhs);
+    const int64_t bh = blockIdx.x % bhs, b = bh / H, h = bh % H;
     const int64_t q_lo_wave = (int64_t)qt * BQ + wave * 32;
     const int64_t pq = q_lo_wave + c32;  // this lane's query token
     const bool valid = pq < qL;
@@ -458,24 +460,34 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(float* q, const T*
 #pragma unroll
         for (int r = 0; r < 16; r++) o[c][r] = 0.0f;
 
-    const int trow = threadIdx.x >> 3, tseg = threadIdx.x & 7;  // staging: row of the tile, 16-column segment
+    // staging: every thread moves 16 columns of one row of the K and of the V tile.  The next tile's
+    // global loads are issued before the current tile is computed on and land in registers meanwhile.
+    const int trow = threadIdx.x >> 3, tseg = threadIdx.x & 7;
+    float4 kst[4], vst[4];
+    int tst = INT_MAX;
+#define LLMOPS_STAGE_LOAD(KV0)                                                                          \
+    do {                                                                                                \
+        const int64_t r_ = (KV0) + trow < kvLen ? (KV0) + trow : kvLen - 1;                             \
+        _Pragma("unroll") for (int u = 0; u < 4; u++) {                                                 \
+            kst[u] = load4(kbase + r_ * S + tseg * 16 + u * 4);                                         \
+            vst[u] = load4(vbase + r_ * S + tseg * 16 + u * 4);                                         \
+        }                                                                                               \
+        if (threadIdx.x < BK) tst = ((KV0) + threadIdx.x < kvLen) ? row_token[(KV0) + threadIdx.x] : INT_MAX; \
+    } while (0)
+    LLMOPS_STAGE_LOAD(0);
     for (int64_t kv0 = 0; kv0 < kvLen; kv0 += BK) {
         __syncthreads();  // the previous tile has been consumed
-        {
-            const int64_t r = kv0 + trow < kvLen ? kv0 + trow : kvLen - 1;
 #pragma unroll
-            for (int u = 0; u < 4; u++) {
-                const int col = tseg * 16 + u * 4;
-                const float4 kk = load4(kbase + r * S + col);
-                const float4 vv = load4(vbase + r * S + col);
-                float2* kd = reinterpret_cast<float2*>(&ksh[trow * KS + col]);  // 8-byte aligned (KS even)
-                kd[0] = make_float2(kk.x, kk.y);
-                kd[1] = make_float2(kk.z, kk.w);
-                *reinterpret_cast<float4*>(&vsh[trow * VS + col]) = vv;
-            }
-            if (threadIdx.x < BK) tok[threadIdx.x] = (kv0 + threadIdx.x < kvLen) ? row_token[kv0 + threadIdx.x] : INT_MAX;
+        for (int u = 0; u < 4; u++) {
+            const int col = tseg * 16 + u * 4;
+            float2* kd = reinterpret_cast<float2*>(&ksh[trow * KS + col]);  // 8-byte aligned (KS even)
+            kd[0] = make_float2(kst[u].x, kst[u].y);
+            kd[1] = make_float2(kst[u].z, kst[u].w);
+            *reinterpret_cast<float4*>(&vsh[trow * VS + col]) = vst[u];
         }
+        if (threadIdx.x < BK) tok[threadIdx.x] = tst;
         __syncthreads();
+        if (kv0 + BK < kvLen) LLMOPS_STAGE_LOAD(kv0 + BK);
         // skip the tile if even the wave's last query may not see any of its rows
         int tmin = tok[c32];
 #pragma unroll
@@ -529,6 +541,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(float* q, const T*
         }
     }
 
+#undef LLMOPS_STAGE_LOAD
     if (!valid) return;
     const float inv = 1.0f / l_run;
     // the lane holds columns 32c + 8j + 4*hf + v of its query's output row
