@@ -178,6 +178,7 @@ def main():
     if not args.no_extra:
         out["prefill_gemm"] = prefill_gemm(torch, llmops, stream)
         out["decode_attention"] = decode_attention(torch, llmops, stream)
+        out["prefill_attention"] = prefill_attention(torch, llmops, stream)
     if not args.no_cpu:
         # the reference's allocator announces itself on stdout (ops/tensor.hpp:88-91); keep stdout for the JSON line
         sys.stdout.flush()
@@ -255,10 +256,21 @@ def decode_step(torch, stream, kv_len=2048, reps=20):
                 dg.replay()
             torch.cuda.synchronize()
             ms = (time.perf_counter() - t0) / reps * 1e3
+        # the same step launched op by op (no graph): what a caller that cannot capture graphs gets
+        with torch.cuda.stream(stream):
+            ids = torch.zeros(1, 1, dtype=torch.int64, device="cuda")
+            slots = torch.tensor([kv_len - 1], dtype=torch.int32, device="cuda")
+            model.forward(ids, kv.cache, slots, kv_len - 1)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(5):
+                model.forward(ids, kv.cache, slots, kv_len - 1)
+            torch.cuda.synchronize()
+            eager_ms = (time.perf_counter() - t0) / 5 * 1e3
         kv_bytes = 2 * LLAMA_7B["layer_num"] * LLAMA_7B["head_num"] * kv_len * LLAMA_7B["head_size"] * kv.cache.element_size()
         fc = model.fc_weight_size()
-        out[name] = {"ms_per_token": round(ms, 4), "GB_per_token": round((fc + kv_bytes) / 1e9, 3),
-                     "GB/s": round((fc + kv_bytes) / ms / 1e6, 1)}
+        out[name] = {"ms_per_token": round(ms, 4), "ms_per_token_eager": round(eager_ms, 3),
+                     "GB_per_token": round((fc + kv_bytes) / 1e9, 3), "GB/s": round((fc + kv_bytes) / ms / 1e6, 1)}
         del dg, kv
     out["config"] = "Llama-2-7B shape, 32 layers, Q4_1(128) FCs incl. 55296x4096 lm_head, kv-len 2048, batch 1, HIP graph"
     return out
@@ -360,6 +372,33 @@ def decode_attention(torch, llmops, stream):
                 out[f"kv={kv} {name}"] = {"us": round(us, 2), "GB/s": round(byts / us / 1e3, 1),
                                           "pct_hbm_peak": round(byts / us / 1e3 / HBM_PEAK_GBS * 100, 2), "bytes": byts}
                 del cache
+    return out
+
+
+def prefill_attention(torch, llmops, stream):
+    """Prompt attention (rope + cache update + causal attention over the chunk itself): 32 heads x 128, fp32
+    cache, qL tokens starting at position 0.  FLOPs counted for the causal half: 4 * H * S * qL^2 / 2."""
+    out = {}
+    H, S = 32, 128
+    gen = torch.Generator(device="cpu").manual_seed(6)
+    inv_freq = (1.0 / (10000.0 ** (torch.arange(0, S, 2).float() / S))).cuda()
+    with torch.cuda.stream(stream):
+        for qL in (128, 512, 2048):
+            cache = torch.zeros(2, 1, H, 2048, S).cuda()
+            q0, k0, v = (torch.randn(1, qL, H * S, generator=gen).cuda() for _ in range(3))
+            slots = torch.arange(qL, dtype=torch.int32).cuda()
+            qs = [q0.clone() for _ in range(4)]
+            ks = [k0.clone() for _ in range(4)]
+
+            def run():
+                for q, k in zip(qs, ks):
+                    llmops.attention_rope2(q, k, v, inv_freq, cache, slots, 0, 0)
+
+            ms = _time_graph(torch, stream, run, reps=3) / len(qs)
+            flops = 4.0 * H * S * qL * qL / 2
+            out[f"qL={qL}"] = {"ms": round(ms, 4), "TFLOP/s_causal": round(flops / ms / 1e9, 2),
+                               "pct_fp32_mfma_peak": round(flops / ms / 1e9 / 157.3 * 100, 2)}
+            del cache
     return out
 
 
