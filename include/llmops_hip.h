@@ -74,6 +74,11 @@ int llmops_offline_FC_dequant_Q4A(const int8_t* weiq, int64_t Ng, int64_t Kg, in
 int llmops_FC_dynamic_quantize_x(const float* x, int64_t rows, int64_t K, int group_k, int8_t* xq,
                                  float* xd, float* gsum, llmops_stream_t stream);
 
+/* The form of FC_dynamic_quantize_x that the prefill FC runs (many rows, K % group_k == 0): xq and
+ * xd bit-exact as above; gsum is summed as a tree (it only feeds the fp32 output, ops/op_fc.hpp:408). */
+int llmops_FC_dynamic_quantize_x_rows(const float* x, int64_t rows, int64_t K, int group_k, int8_t* xq,
+                                      float* xd, float* gsum, llmops_stream_t stream);
+
 /* ------------------------------------------------------------------------------------------
  * Q4_1 x Q8 fully connected
  * ------------------------------------------------------------------------------------------ */

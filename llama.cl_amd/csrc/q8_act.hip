@@ -82,6 +82,41 @@ __global__ __launch_bounds__(256) void quant_x_kernel(const float* __restrict__ 
     }
 }
 
+// Prefill variant (many rows): G/4 threads per group, each with one 16-byte load and one packed
+// 4-code store, so a workgroup quantizes 256/(G/4) groups with fully coalesced traffic.  Codes and
+// scales are the same bits as above; the raw group sum is a tree sum (it only feeds the fp32 output).
+template <int G>
+__global__ __launch_bounds__(256) void quant_x_rows_kernel(const float* __restrict__ x, int64_t items, int64_t K, int64_t Kg,
+                                                            int64_t rows, int8_t* __restrict__ xq, float* __restrict__ xd,
+                                                            float* __restrict__ gsum, float2* __restrict__ xsT) {
+    constexpr int TPG = G / 4;        // threads per group
+    constexpr int GPW = 256 / TPG;    // groups per workgroup
+    const int sub = threadIdx.x % TPG;
+    const int64_t item = (int64_t)blockIdx.x * GPW + threadIdx.x / TPG;
+    const bool live = item < items;   // a group's threads are all live or all idle: the shuffles below stay inside a group
+    const int64_t it = live ? item : items - 1;
+    const int64_t r = it / Kg, kb = it % Kg;
+    const float4 v = *reinterpret_cast<const float4*>(x + r * K + kb * G + sub * 4);
+    float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+    float s = (v.x + v.y) + (v.z + v.w);
+#pragma unroll
+    for (int o = TPG / 2; o > 0; o >>= 1) {
+        amax = fmaxf(amax, __shfl_xor(amax, o, 64));
+        s += __shfl_xor(s, o, 64);
+    }
+    const float d = amax / 127.0f;
+    const float id = (d != 0.0f) ? (1.0f / d) : 0.0f;
+    const uint32_t c = ((uint32_t)q8_code(v.x, id) & 0xFFu) | (((uint32_t)q8_code(v.y, id) & 0xFFu) << 8) |
+                       (((uint32_t)q8_code(v.z, id) & 0xFFu) << 16) | (((uint32_t)q8_code(v.w, id) & 0xFFu) << 24);
+    if (!live) return;
+    *reinterpret_cast<uint32_t*>(xq + (r * Kg + kb) * G + sub * 4) = c;
+    if (sub == 0) {
+        xd[r * Kg + kb] = d;
+        gsum[r * Kg + kb] = s;
+        if (xsT != nullptr) xsT[kb * rows + r] = make_float2(d, s);
+    }
+}
+
 }  // namespace llmops
 
 using namespace llmops;
@@ -92,6 +127,14 @@ int launch_quant_x(const float* x, int64_t rows, int64_t K, int group_k, int8_t*
                    bool exact_sum, hipStream_t stream) {
     const int64_t Kg = (K + group_k - 1) / group_k;
     const int64_t items = rows * Kg;
+    if (!exact_sum && K == Kg * group_k && aligned(x, 16) && aligned(xq, 4)) {  // whole groups only: vector loads
+        if (group_k == 32)
+            quant_x_rows_kernel<32><<<(unsigned)((items + 31) / 32), 256, 0, stream>>>(x, items, K, Kg, rows, xq, xd, gsum, xsT);
+        else
+            quant_x_rows_kernel<128><<<(unsigned)((items + 7) / 8), 256, 0, stream>>>(x, items, K, Kg, rows, xq, xd, gsum, xsT);
+        LLMOPS_LAUNCH_CHECK();
+        return LLMOPS_OK;
+    }
     const unsigned grid = (unsigned)((items + 3) / 4);
     if (group_k == 32) {
         if (exact_sum) quant_x_kernel<32, true><<<grid, 256, 0, stream>>>(x, rows, K, Kg, xq, xd, gsum, xsT);
@@ -114,4 +157,14 @@ extern "C" int llmops_FC_dynamic_quantize_x(const float* x, int64_t rows, int64_
     const int64_t Kg = (K + group_k - 1) / group_k;
     LLMOPS_REQUIRE(rows * Kg < ((int64_t)1 << 33));
     return launch_quant_x(x, rows, K, group_k, xq, xd, gsum, nullptr, true, as_stream(stream));
+}
+
+extern "C" int llmops_FC_dynamic_quantize_x_rows(const float* x, int64_t rows, int64_t K, int group_k, int8_t* xq,
+                                                 float* xd, float* gsum, llmops_stream_t stream) {
+    LLMOPS_REQUIRE(valid_group(group_k));
+    LLMOPS_REQUIRE(x != nullptr && xq != nullptr && xd != nullptr && gsum != nullptr);
+    LLMOPS_REQUIRE(rows > 0 && K > 0 && (K % group_k) == 0);
+    LLMOPS_REQUIRE(aligned(x, 16) && aligned(xq, 4));
+    LLMOPS_REQUIRE(rows * (K / group_k) < ((int64_t)1 << 33));
+    return launch_quant_x(x, rows, K, group_k, xq, xd, gsum, nullptr, false, as_stream(stream));
 }

@@ -104,8 +104,9 @@ def offline_FC_dequant_Q4A(weiq):
     return out
 
 
-def FC_dynamic_quantize_x(input, group_k):
-    """fp32 [..,K] -> (xq int8 [..,Kg*G], xd fp32 [..,Kg], gsum fp32 [..,Kg]) (ops/op_fc.hpp:221-272)."""
+def FC_dynamic_quantize_x(input, group_k, rows_variant=False):
+    """fp32 [..,K] -> (xq int8 [..,Kg*G], xd fp32 [..,Kg], gsum fp32 [..,Kg]) (ops/op_fc.hpp:221-272).
+    ``rows_variant=True`` runs the kernel the prefill FC uses (same codes and scales, tree-summed gsum)."""
     _dev(input, torch.float32, None, "input")
     _require(group_k in (32, 128), "group_k in (32, 128)")
     K = input.shape[-1]
@@ -115,8 +116,9 @@ def FC_dynamic_quantize_x(input, group_k):
     xq = torch.empty(lead + (Kg * group_k,), dtype=torch.int8, device=input.device)
     xd = torch.empty(lead + (Kg,), dtype=torch.float32, device=input.device)
     gs = torch.empty(lead + (Kg,), dtype=torch.float32, device=input.device)
-    _lib.check(_lib.load().llmops_FC_dynamic_quantize_x(_ptr(input), rows, K, group_k, _ptr(xq), _ptr(xd), _ptr(gs),
-                                                       _stream(input)))
+    lib = _lib.load()
+    fn = lib.llmops_FC_dynamic_quantize_x_rows if rows_variant else lib.llmops_FC_dynamic_quantize_x
+    _lib.check(fn(_ptr(input), rows, K, group_k, _ptr(xq), _ptr(xd), _ptr(gs), _stream(input)))
     return xq, xd, gs
 
 

@@ -84,6 +84,23 @@ def test_quant_x_random_vs_oracle(ops, orc, G, rows, K):
     assert list(host(xq)[0, :8]) == [127, 2, 4, -2, -4, 0, 2, 0]
 
 
+@pytest.mark.parametrize("G", [32, 128])
+@pytest.mark.parametrize("rows,K", [(1, 4096), (17, 11008), (2048, 4096), (3, 128)])
+def test_quant_x_rows_variant_vs_oracle(ops, orc, G, rows, K):
+    """The quantizer of the prefill FC: codes and scales bit-exact, group sum within fp32 rounding."""
+    rng = np.random.default_rng(rows + K + 1)
+    x = rng.standard_normal((rows, K)).astype(np.float32)
+    x[0, :8] = [127, 2.5, 3.5, -2.5, -3.5, 0.5, 1.5, -0.5]
+    x[0, 8:G] = 0
+    x[-1, -G:] = 0
+    xq, xd, gs = ops.FC_dynamic_quantize_x(dev(x), G, rows_variant=True)
+    wq, wd, wg = orc.quant_x(x, G)
+    assert np.array_equal(host(xq), wq)
+    assert np.array_equal(host(xd).view(np.uint32), wd.view(np.uint32))
+    assert np.abs(host(gs) - wg).max() <= 1e-5 * max(1.0, np.abs(x).max() * G)
+    assert list(host(xq)[0, :8]) == [127, 2, 4, -2, -4, 0, 2, 0]
+
+
 # ---- int32 partial sums -------------------------------------------------------------------------
 @pytest.mark.parametrize("G", [32, 128])
 @pytest.mark.parametrize("mfma", [False, True])
