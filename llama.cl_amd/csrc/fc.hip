@@ -22,6 +22,9 @@ int launch_gemm(const uint8_t* w, const int8_t* xq, const float* xd, const float
                 float* part, int64_t rows, int64_t Ng, int64_t Kg, int G, int64_t N, hipStream_t st);
 int launch_gemm_partials(const uint8_t* w, const int8_t* xq, int32_t* acc, int64_t rows, int64_t Ng, int64_t Kg, int G,
                          hipStream_t st);
+int launch_fc_rows(const uint8_t* w, const int8_t* xq, const float2* xsT, float* y, int64_t rows, int64_t Ng, int64_t Kg,
+                   int64_t N, const float* residual, hipStream_t st);
+bool gemm_rows_kernel_enabled();
 
 static inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
@@ -85,6 +88,11 @@ static int fc_impl(const float* x, int64_t rows, int64_t K, const int8_t* weiq, 
     float2* xst = reinterpret_cast<float2*>(ws + lay.off_xst);
     int rc = launch_quant_x(x, rows, K, group_k, xq, xd, gs, xst, false, st);
     if (rc) return rc;
+    // up to 16 rows are still bound by the weight stream: one strip per workgroup, MFMA inner product
+    // (measured against the tiled kernel: 15 vs 18 us at 16 rows, 11008x4096; with two row tiles per
+    // wave, 17..32 rows, the streaming kernel runs out of registers and loses, 32 vs 20 us)
+    if (group_k == 128 && rows <= 16 && Ng >= 64 && gemm_rows_kernel_enabled())
+        return launch_fc_rows(w, xq, xst, y, rows, Ng, Kg, N, residual, st);
     rc = launch_gemm(w, xq, xd, gs, xst, y, part, rows, Ng, Kg, group_k, N, st);
     if (rc || residual == nullptr) return rc;
     return launch_add(y, residual, rows * N, st);

@@ -433,7 +433,8 @@ struct GemmPlan {
     bool lds;
 };
 
-static int g_gemm_rt = 0;  // 0 = choose per shape
+static int g_gemm_rt = 0;  // 0 = choose per shape; -1 = also keep 9..32 rows on the tiled kernel
+bool gemm_rows_kernel_enabled() { return g_gemm_rt >= 0; }
 
 // Split-K factor for `tiles` output tiles on a machine with `slots` resident workgroups.
 static void gemm_split(int64_t tiles, int64_t slots, int64_t Kg, GemmPlan& p) {

@@ -284,3 +284,18 @@ def test_fc_decode_sumsq_handover(ops, orc, G, rows, N, K):
         # against the oracle the contract of fc_Q4A applies: the rmsnorm here and there differ by an ulp,
         # which flips an int8 code now and then (K = 4096 values per output)
         assert max_rel_err(b, orc.fc(orc.rmsnorm(host(y), nw, 1e-5), host(p2), F)) <= 1e-3
+
+
+@pytest.mark.parametrize("rows", [9, 12, 16])
+@pytest.mark.parametrize("N,K", [(2070, 1024), (4096, 4096)])
+def test_fc_rows_9_to_16_streaming_mfma(ops, orc, rows, N, K):
+    """9..16 rows at group 128 with at least 64 strips take the weight-streaming MFMA kernel
+    (one strip per workgroup): output and residual epilogue against the oracle, N not a multiple of 32."""
+    rng = np.random.default_rng(rows + N)
+    x = rng.standard_normal((1, rows, K)).astype(np.float32)
+    w = (rng.standard_normal((N, K)) * 0.02).astype(np.float32)
+    res = rng.standard_normal((1, rows, N)).astype(np.float32)
+    pw = orc.quant_w(w, 128)
+    want = orc.fc(x, pw, N)
+    assert max_rel_err(host(ops.fc_Q4A(dev(x), dev(pw), N)), want) <= 1e-5
+    assert max_rel_err(host(ops.fc_Q4A(dev(x), dev(pw), N, residual=dev(res))), want + res) <= 1e-5
