@@ -111,13 +111,16 @@ int llmops_fc_Q4A_residual(const float* x, int64_t rows, int64_t K, const int8_t
  * folded into the one launch.  Each option may be left out (NULL / 0):
  *   norm_w, eps : x is rmsnorm'ed first (clone + rmsnorm, ops/op_misc.hpp:142-181); needs K % 4 == 0
  *   residual    : y += residual (iadd, ops/op_misc.hpp:55-79), fp32 [rows,N_out]
- *   glu         : weiq holds gate and up strips interleaved (strip 2i = gate strip i, 2i+1 = up strip i,
+ *   glu == 1    : weiq holds gate and up strips interleaved (strip 2i = gate strip i, 2i+1 = up strip i,
  *                 Ng even) and y[r,n] = silu(gate[r,n]) * up[r,n] (itrans "silu" + imul), N_out = F
+ *   glu == 2    : the same two ops on the input side: x is fp32 [rows,2K], a gate|up row (gate in columns
+ *                 [0,K), up in [K,2K)), and the FC's input is silu(gate)*up; not with norm_w.  The FC in front
+ *                 then runs without glu on the gate and up weights stacked along N.
  *   sumsq_out   : fp32 [rows,Ng], receives the sum of squares of every strip's 32 outputs (after the
- *                 residual add); not with glu
+ *                 residual add); not with glu == 1
  *   sumsq_in, sumsq_parts : with norm_w: fp32 [rows,sumsq_parts] whose row sums are sum(x^2) -- what the
  *                 FC that produced x left in its sumsq_out -- so that the rmsnorm does not read the row again
- * N_out is the number of output columns (Ng*32-ish without glu, Ng/2*32-ish with it). */
+ * N_out is the number of output columns (Ng*32-ish; Ng/2*32-ish with glu == 1). */
 int llmops_fc_Q4A_decode(const float* x, int64_t rows, int64_t K, const int8_t* weiq, int64_t Ng, int64_t Kg,
                          int group_k, int64_t N_out, const float* norm_w, float eps, const float* residual, int glu,
                          const float* sumsq_in, int64_t sumsq_parts, float* sumsq_out, float* y, void* workspace,

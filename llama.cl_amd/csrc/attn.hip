@@ -352,16 +352,42 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(float* q, float* k, co
         }
     }
     const float d_scale = 1.0f / sqrtf((float)S);
+    // NL partial dot products per lane, each to be summed over the 32 lanes of a half-wave.  Summing
+    // them one by one takes 5 lane exchanges each; instead the lanes split the rows between them while
+    // they add: at every exchange a lane keeps one half of its rows and hands the other half to its
+    // partner, so NL rows cost NL/2 + NL/4 + .. + 1 exchanges plus one per remaining lane bit.
+    float sp[NL];
 #pragma unroll
     for (int i = 0; i < NL; i++) {
         float s = qv.x * kv[i].x;
         s = fmaf(qv.y, kv[i].y, s);
         s = fmaf(qv.z, kv[i].z, s);
-        s = fmaf(qv.w, kv[i].w, s);
+        sp[i] = fmaf(qv.w, kv[i].w, s);
+    }
+    int row_of_lane = 0;  // which of the NL rows this lane ends up holding
+    {
+        int n = NL, off = 16;
 #pragma unroll
-        for (int o = 16; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
-        const int r = wave * PW + i * 2 + hf;
-        if (e == 0) sc[r] = (p0 + r < kvLen) ? s * d_scale : -FLT_MAX;
+        for (; n > 1; n >>= 1, off >>= 1) {
+            const bool up = (e & off) != 0;
+#pragma unroll
+            for (int j = 0; j < NL / 2; j++) {
+                if (j < n / 2) {
+                    const float keep = up ? sp[j + n / 2] : sp[j];
+                    const float send = up ? sp[j] : sp[j + n / 2];
+                    sp[j] = keep + __shfl_xor(send, off, 64);
+                }
+            }
+            row_of_lane = row_of_lane * 2 + (up ? 1 : 0);
+        }
+#pragma unroll
+        for (; off > 0; off >>= 1) sp[0] += __shfl_xor(sp[0], off, 64);
+    }
+    {
+        // lanes whose remaining (low) bits are zero write the row they hold
+        constexpr int kLowMask = (NL >= 8) ? 3 : (NL == 4 ? 7 : 15);
+        const int r = wave * PW + row_of_lane * 2 + hf;
+        if ((e & kLowMask) == 0) sc[r] = (p0 + r < kvLen) ? sp[0] * d_scale : -FLT_MAX;
     }
     __syncthreads();
     if (wave == 0) {

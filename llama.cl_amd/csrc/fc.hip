@@ -12,7 +12,7 @@ size_t gemv_workspace_bytes(int64_t rows, int64_t Ng, int64_t Kg, int G);
 int launch_gemv(const uint8_t* w, const int8_t* xq, const float* xd, const float* gs, float* y, float* part,
                 unsigned* counters, int64_t rows, int64_t Ng, int64_t Kg, int G, int64_t N, hipStream_t st);
 int launch_gemv_fused(const uint8_t* w, const float* x, float* y, float* part, unsigned* counters, int64_t rows, int64_t Ng,
-                      int64_t Kg, int G, int64_t N, const float* residual, const float* norm_w, float eps, bool glu,
+                      int64_t Kg, int G, int64_t N, const float* residual, const float* norm_w, float eps, int glu,
                       const float* sumsq_in, int sumsq_parts, float* sumsq_out, hipStream_t st);
 int launch_add(float* a, const float* b, int64_t total, hipStream_t st);
 int launch_gemv_partials(const uint8_t* w, const int8_t* xq, int32_t* acc, int64_t rows, int64_t Ng, int64_t Kg, int G,
@@ -83,7 +83,7 @@ static int fc_impl(const float* x, int64_t rows, int64_t K, const int8_t* weiq, 
     const uint8_t* w = reinterpret_cast<const uint8_t*>(weiq);
     // few rows: one launch, the streaming kernel quantizes the activations it needs on the fly
     if (rows <= kMaxGemvRows)
-        return launch_gemv_fused(w, x, y, part, counters, rows, Ng, Kg, group_k, N, residual, nullptr, 0.0f, false, nullptr, 0,
+        return launch_gemv_fused(w, x, y, part, counters, rows, Ng, Kg, group_k, N, residual, nullptr, 0.0f, 0, nullptr, 0,
                                  nullptr, st);
     float2* xst = reinterpret_cast<float2*>(ws + lay.off_xst);
     int rc = launch_quant_x(x, rows, K, group_k, xq, xd, gs, xst, false, st);
@@ -121,7 +121,8 @@ extern "C" int llmops_fc_Q4A_decode(const float* x, int64_t rows, int64_t K, con
     LLMOPS_REQUIRE(K > 0 && Ng > 0 && Kg > 0 && K == Kg * group_k);
     LLMOPS_REQUIRE(Ng <= LLMOPS_FC_COUNTER_BYTES / 4 && Ng * 64 < ((int64_t)1 << 31));
     LLMOPS_REQUIRE(aligned(weiq, 16) && aligned(workspace, 256) && aligned(x, 8));
-    if (glu) {
+    LLMOPS_REQUIRE(glu >= 0 && glu <= 2);
+    if (glu == 1) {
         LLMOPS_REQUIRE((Ng % 2) == 0 && residual == nullptr);
         LLMOPS_REQUIRE(N_out > (Ng / 2 - 1) * kGroupN && N_out <= Ng / 2 * kGroupN);
     } else {
@@ -129,13 +130,14 @@ extern "C" int llmops_fc_Q4A_decode(const float* x, int64_t rows, int64_t K, con
     }
     if (norm_w != nullptr) LLMOPS_REQUIRE((K % 4) == 0 && aligned(x, 16) && aligned(norm_w, 8));
     if (sumsq_in != nullptr) LLMOPS_REQUIRE(norm_w != nullptr && sumsq_parts > 0 && sumsq_parts <= 65536);
-    if (sumsq_out != nullptr) LLMOPS_REQUIRE(!glu);
+    if (sumsq_out != nullptr) LLMOPS_REQUIRE(glu != 1);
+    if (glu == 2) LLMOPS_REQUIRE(norm_w == nullptr && sumsq_in == nullptr);
     const FcWorkspace lay = fc_layout(rows, Ng, Kg, group_k);
     if (workspace_bytes < lay.total)
         return fail(LLMOPS_EWORKSPACE, "fc_Q4A needs %zu workspace bytes, got %zu", lay.total, workspace_bytes);
     uint8_t* ws = reinterpret_cast<uint8_t*>(workspace);
     return launch_gemv_fused(reinterpret_cast<const uint8_t*>(weiq), x, y, reinterpret_cast<float*>(ws + lay.off_part),
-                             reinterpret_cast<unsigned*>(ws), rows, Ng, Kg, group_k, N_out, residual, norm_w, eps, glu != 0,
+                             reinterpret_cast<unsigned*>(ws), rows, Ng, Kg, group_k, N_out, residual, norm_w, eps, glu,
                              sumsq_in, (int)sumsq_parts, sumsq_out, as_stream(stream));
 }
 

@@ -186,7 +186,11 @@ __global__ __launch_bounds__(NW * 64) void fc_gemv_kernel(const uint8_t* __restr
 //   kSums: with kNorm, the sum of squares of the row comes as per-strip partial sums left behind by
 //          the FC that produced the row; every wave adds them up by itself (no pass over the row, no
 //          workgroup barrier).
-constexpr int kNorm = 1, kGlu = 2, kSums = 4;
+//   kGluIn: the activation row is a gate|up row of 2K floats (gate in [0,K), up in [K,2K)) and the
+//          FC's input is silu(gate)*up, formed as the two halves are loaded.  The FC that produces
+//          the row then keeps one strip per workgroup (no pairing of gate and up strips), which
+//          spreads its strips more evenly over the compute units.
+constexpr int kNorm = 1, kGlu = 2, kSums = 4, kGluIn = 8;
 
 // One activation row needs few registers; asking for eight waves per SIMD (two workgroups of 16 waves
 // per CU) keeps every variant at or below 64 registers, so that grids of 257..512 workgroups are
@@ -200,6 +204,9 @@ __global__ __launch_bounds__(NW * 64, (MT == 1 ? NW / 2 : 1)) void fc_gemv_fused
                                                                  const float* __restrict__ sumsq_in, int sumsq_parts,
                                                                  float* __restrict__ sumsq_out) {
     constexpr bool NORM = (MODE & kNorm) != 0, GLU = (MODE & kGlu) != 0, SUMS = (MODE & kSums) != 0;
+    constexpr bool GLUIN = (MODE & kGluIn) != 0;
+    static_assert(!(GLUIN && NORM), "the gate|up input has no rmsnorm");
+    const int64_t xstride = GLUIN ? 2 * K : K;  // floats between activation rows
     constexpr int NWS = GLU ? NW / 2 : NW;  // waves per strip
     __shared__ float red[NW][MT][kGroupN];
     __shared__ __align__(16) XSlot<G> xs[NW][MT];
@@ -257,10 +264,14 @@ __global__ __launch_bounds__(NW * 64, (MT == 1 ? NW / 2 : 1)) void fc_gemv_fused
     // double-buffered weight blocks; the activation row of a step is fetched one step ahead
     Step<G> cur, nxt;
     XRaw<G> xcur[MT], xnxt[MT], wcur, wnxt;
+    XRaw<G> ucur[GLUIN ? MT : 1], unxt[GLUIN ? MT : 1];  // the up half of a gate|up row
     if (tr.t0 < tr.t1) {
 #pragma unroll
         for (int r = 0; r < MT; r++)
-            if (r < rows) load_x<G>(xcur[r], x + (int64_t)r * K, tr.t0, K, lane);
+            if (r < rows) {
+                load_x<G>(xcur[r], x + (int64_t)r * xstride, tr.t0, K, lane);
+                if (GLUIN) load_x<G>(ucur[GLUIN ? r : 0], x + (int64_t)r * xstride + K, tr.t0, K, lane);
+            }
         if (NORM) load_x<G>(wcur, norm_w, tr.t0, K, lane);
         load_step<G>(cur, strip, tr.t0, Kg, lane);
     }
@@ -314,7 +325,10 @@ __global__ __launch_bounds__(NW * 64, (MT == 1 ? NW / 2 : 1)) void fc_gemv_fused
             load_step<G>(nxt, strip, t + 1, Kg, lane);
 #pragma unroll
             for (int r = 0; r < MT; r++)
-                if (r < rows) load_x<G>(xnxt[r], x + (int64_t)r * K, t + 1, K, lane);
+                if (r < rows) {
+                    load_x<G>(xnxt[r], x + (int64_t)r * xstride, t + 1, K, lane);
+                    if (GLUIN) load_x<G>(unxt[GLUIN ? r : 0], x + (int64_t)r * xstride + K, t + 1, K, lane);
+                }
             if (NORM) load_x<G>(wnxt, norm_w, t + 1, K, lane);
         }
 #pragma unroll
@@ -323,6 +337,13 @@ __global__ __launch_bounds__(NW * 64, (MT == 1 ? NW / 2 : 1)) void fc_gemv_fused
                 if (NORM) {
 #pragma unroll
                     for (int i = 0; i < (G == 128 ? 2 : 1); i++) xcur[r].v[i] = xcur[r].v[i] * rsn[r] * wcur.v[i];
+                }
+                if (GLUIN) {  // silu(gate)*up, the arithmetic of silu_mul_kernel
+#pragma unroll
+                    for (int i = 0; i < (G == 128 ? 2 : 1); i++) {
+                        const float g = xcur[r].v[i];
+                        xcur[r].v[i] = ucur[GLUIN ? r : 0].v[i] * (g * (1.0f / (1.0f + expf(-g))));
+                    }
                 }
                 XSlot<G>* slot = &xs[wave][r];
                 quantize_step<G>(xcur[r], slot, lane);
@@ -339,6 +360,10 @@ __global__ __launch_bounds__(NW * 64, (MT == 1 ? NW / 2 : 1)) void fc_gemv_fused
         cur = nxt;
 #pragma unroll
         for (int r = 0; r < MT; r++) xcur[r] = xnxt[r];
+        if (GLUIN) {
+#pragma unroll
+            for (int r = 0; r < MT; r++) ucur[GLUIN ? r : 0] = unxt[GLUIN ? r : 0];
+        }
         if (NORM) wcur = wnxt;
     }
 
@@ -451,6 +476,7 @@ struct FusedOps {
     const float* norm_w;    // x = rmsnorm(x, norm_w, eps) first
     float eps;
     bool glu;               // interleaved gate/up strips, y = silu(gate)*up
+    bool glu_in;            // x is a gate|up row of 2K floats, the input is silu(gate)*up
     const float* sumsq_in;  // per-part sums of squares of x (instead of reading the row for the rmsnorm)
     int sumsq_parts;
     float* sumsq_out;       // per-strip sums of squares of y [rows, Ng]
@@ -466,7 +492,9 @@ static void launch_fused_t(const uint8_t* w, const float* x, float* y, float* pa
                                                                                 o.norm_w, o.eps, o.sumsq_in,         \
                                                                                 o.sumsq_parts, o.sumsq_out)
     const bool sums = o.norm_w != nullptr && o.sumsq_in != nullptr;
-    if (o.glu) {
+    if (o.glu_in) {
+        LLMOPS_FUSED(kGluIn, Ng * p.S);
+    } else if (o.glu) {
         if (sums) LLMOPS_FUSED(kNorm | kGlu | kSums, Ng / 2);
         else if (o.norm_w) LLMOPS_FUSED(kNorm | kGlu, Ng / 2);
         else LLMOPS_FUSED(kGlu, Ng / 2);
@@ -480,11 +508,11 @@ static void launch_fused_t(const uint8_t* w, const float* x, float* y, float* pa
 
 // raw fp32 activations, quantized inside the kernel (+ optional rmsnorm / residual / gate-up epilogue)
 int launch_gemv_fused(const uint8_t* w, const float* x, float* y, float* part, unsigned* counters, int64_t rows, int64_t Ng,
-                      int64_t Kg, int G, int64_t N, const float* residual, const float* norm_w, float eps, bool glu,
+                      int64_t Kg, int G, int64_t N, const float* residual, const float* norm_w, float eps, int glu,
                       const float* sumsq_in, int sumsq_parts, float* sumsq_out, hipStream_t st) {
     GemvPlan p = plan_gemv(rows, Ng, Kg, G, true);
-    if (glu) p.S = 1;
-    const FusedOps o{residual, norm_w, eps, glu, sumsq_in, sumsq_parts, sumsq_out};
+    if (glu == 1) p.S = 1;
+    const FusedOps o{residual, norm_w, eps, glu == 1, glu == 2, sumsq_in, sumsq_parts, sumsq_out};
 #define LLMOPS_CASE(GG, MT, NWW) launch_fused_t<GG, MT, NWW>(w, x, y, part, counters, Ng, Kg, N, (int)rows, p, o, st)
     if (G == 128) {
         if (rows == 1) LLMOPS_CASE(128, 1, 16);

@@ -153,12 +153,15 @@ def interleave_gate_up(gate_packed, up_packed):
     return torch.stack((gate_packed, up_packed), dim=1).reshape(-1, *gate_packed.shape[1:]).contiguous()
 
 
-def fc_Q4A_decode(input, weiq, N_out, norm=None, residual=None, glu=False, sumsq_in=None, want_sumsq=False):
+def fc_Q4A_decode(input, weiq, N_out, norm=None, residual=None, glu=False, sumsq_in=None, want_sumsq=False,
+                  glu_in=False):
     """Extension: fc_Q4A with its neighbours of the decode step folded in (one launch for B*M <= 8).
 
     norm=(weight, eps): input is rmsnorm'ed first;  residual: added to the result;
     glu=True: ``weiq`` holds interleaved gate/up strips (``interleave_gate_up``) and the result is
-    silu(gate)*up with N_out = F columns.  want_sumsq=True returns ``(out, sumsq)`` where ``sumsq``
+    silu(gate)*up with N_out = F columns.  glu_in=True: ``input`` is a gate|up row [B, M, 2K] (what an FC
+    over the gate and up weights stacked along N leaves behind) and the FC runs on silu(gate)*up.
+    want_sumsq=True returns ``(out, sumsq)`` where ``sumsq``
     [B*M, strips] holds the sum of squares of every 32 outputs; passed as ``sumsq_in`` to the FC that
     rmsnorms ``out`` it saves that FC the pass over the row.  With more than 8 rows the same
     arithmetic is composed from the separate ops."""
@@ -169,6 +172,9 @@ def fc_Q4A_decode(input, weiq, N_out, norm=None, residual=None, glu=False, sumsq
     Ng, Kg, _ = weiq.shape
     rows = B * M
     N_out = int(N_out)
+    if glu_in:
+        _require(K % 2 == 0 and norm is None and not glu, "glu_in: input.size(2) % 2 == 0, no norm, no glu")
+        K //= 2
     if norm is not None:
         _dev(norm[0], torch.float32, 1, "norm weight")
         _require(norm[0].shape[0] == K, "weight.size(0) == K")
@@ -181,6 +187,8 @@ def fc_Q4A_decode(input, weiq, N_out, norm=None, residual=None, glu=False, sumsq
     _require(not (want_sumsq and glu), "no sumsq with glu")
     if rows > 8:
         x = input if norm is None else rmsnorm_out(input, norm[0], norm[1])
+        if glu_in:
+            x = silu_mul(input)
         if glu:
             _require(N_out % 32 == 0, "F % 32 == 0")
             y = fc_Q4A(x, weiq, 2 * N_out).view(B, M, N_out // 32, 2, 32)
@@ -197,7 +205,7 @@ def fc_Q4A_decode(input, weiq, N_out, norm=None, residual=None, glu=False, sumsq
     sumsq = torch.empty((rows, Ng), dtype=torch.float32, device=input.device) if want_sumsq else None
     _lib.check(lib.llmops_fc_Q4A_decode(_ptr(input), rows, K, _ptr(weiq), Ng, Kg, g, N_out,
                                         _ptr(norm[0]) if norm is not None else None, float(norm[1]) if norm is not None else 0.0,
-                                        _ptr(residual) if residual is not None else None, int(bool(glu)),
+                                        _ptr(residual) if residual is not None else None, 2 if glu_in else int(bool(glu)),
                                         _ptr(sumsq_in) if sumsq_in is not None else None,
                                         sumsq_in.shape[1] if sumsq_in is not None else 0,
                                         _ptr(sumsq) if sumsq is not None else None, _ptr(out), _ptr(ws),

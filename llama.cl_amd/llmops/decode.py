@@ -53,7 +53,13 @@ class LlamaDecoder:
             if plan == "fused":
                 layer["qkv_proj"] = fc(H, H, parts=3)
                 gate, up = fc(F, H), fc(F, H)
-                layer["gate_up_proj"] = llmop_fc_q4a(packed=llmops.interleave_gate_up(gate.weight, up.weight), N=2 * F)
+                # gate and up stacked along N: one FC leaves the row [gate | up] and the down projection takes
+                # silu(gate)*up on its way in.  That needs F to be whole strips; otherwise the strips are
+                # interleaved and silu(gate)*up is the epilogue of the gate|up FC.
+                self.stacked_gate_up = F % 32 == 0
+                gu = torch.cat((gate.weight, up.weight), dim=0) if self.stacked_gate_up else \
+                    llmops.interleave_gate_up(gate.weight, up.weight)
+                layer["gate_up_proj"] = llmop_fc_q4a(packed=gu, N=2 * F)
             else:
                 layer["q_proj"], layer["k_proj"], layer["v_proj"] = fc(H, H), fc(H, H), fc(H, H)
                 layer["gate_proj"], layer["up_proj"] = fc(F, H), fc(F, H)
@@ -113,7 +119,7 @@ class LlamaDecoder:
     def _layer_fused(self, i, ops, hidden_states, sumsq, kv_cache, kv_cache_slots, position_id):
         """Same arithmetic, 6 launches per decode layer instead of 18: rmsnorm inside the q|k|v and
         gate|up FCs (fed with the sums of squares that the FC producing their input leaves behind),
-        silu*up in the gate|up epilogue (interleaved strips), residual adds inside the o and down
+        silu*up on the input side of the down projection, residual adds inside the o and down
         projections, rope + cache update inside the attention kernel."""
         H, F = self.configs["hidden_size"], self.configs["intermediate_size"]
         n1, n2 = ops["input_layernorm"], ops["post_attention_layernorm"]
@@ -123,6 +129,11 @@ class LlamaDecoder:
             q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
         llmops.attention_rope2(q, k, v, self.inv_freq, kv_cache, kv_cache_slots, position_id, i)
         attn_output, ss = llmops.fc_Q4A_decode(q, ops["o_proj"].weight, H, residual=hidden_states, want_sumsq=True)
+        if self.stacked_gate_up:
+            gate_up = llmops.fc_Q4A_decode(attn_output, ops["gate_up_proj"].weight, 2 * F, norm=(n2.weight, n2.eps),
+                                           sumsq_in=ss)
+            return llmops.fc_Q4A_decode(gate_up, ops["down_proj"].weight, H, residual=attn_output, want_sumsq=True,
+                                        glu_in=True)
         act = llmops.fc_Q4A_decode(attn_output, ops["gate_up_proj"].weight, F, norm=(n2.weight, n2.eps), glu=True,
                                    sumsq_in=ss)
         return llmops.fc_Q4A_decode(act, ops["down_proj"].weight, H, residual=attn_output, want_sumsq=True)

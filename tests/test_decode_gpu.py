@@ -35,7 +35,10 @@ def oracle_forward(orc, model, ids, cache, slots, pos):
         q, _, cache = orc.attention(q, k, v, inv, cache, slots, pos, i)
         attn = orc.iadd(fc(ops["o_proj"], q), hidden)
         x = orc.rmsnorm(attn, ops["post_attention_layernorm"].weight.cpu().numpy(), CFG["rms_norm_eps"])
-        if "gate_up_proj" in ops:  # strips alternate gate, up, gate, up ...
+        if "gate_up_proj" in ops and model.stacked_gate_up:  # all gate strips, then all up strips
+            gu = fc(ops["gate_up_proj"], x)
+            gate, up = gu[..., :F].copy(), gu[..., F:].copy()
+        elif "gate_up_proj" in ops:  # strips alternate gate, up, gate, up ...
             gu = fc(ops["gate_up_proj"], x).reshape(x.shape[:-1] + (F // 32, 2, 32))
             gate = gu[..., 0, :].reshape(x.shape[:-1] + (F,)).copy()
             up = gu[..., 1, :].reshape(x.shape[:-1] + (F,)).copy()
@@ -116,8 +119,9 @@ def test_layer_ops_teacher_forced(orc):
         gu = ops["gate_up_proj"](x)
         want_gu = orc.fc(h(x), h(ops["gate_up_proj"].weight), 2 * F)
         close(gu, want_gu, 1e-5)
-        gu5 = gu.view(1, qL, F // 32, 2, 32)
-        gate, up = gu5[..., 0, :].reshape(1, qL, F).contiguous(), gu5[..., 1, :].reshape(1, qL, F).contiguous()
+        assert model.stacked_gate_up  # F is whole strips: all gate strips, then all up strips
+        gu_row = gu.clone()
+        gate, up = gu[..., :F].contiguous(), gu[..., F:].contiguous()
         g0, u0 = h(gate), h(up)
         llmops.itrans(gate, "silu")
         close(gate, orc.silu(g0), 1e-5)
@@ -128,8 +132,13 @@ def test_layer_ops_teacher_forced(orc):
         # the folded forms give the same results as the separate ops above
         n1, n2 = ops["input_layernorm"], ops["post_attention_layernorm"]
         close(llmops.fc_Q4A_decode(hidden, ops["qkv_proj"].weight, 3 * H, norm=(n1.weight, n1.eps)), qkv_saved, 1e-4)
-        close(llmops.fc_Q4A_decode(attn, ops["gate_up_proj"].weight, F, norm=(n2.weight, n2.eps), glu=True), h(up), 1e-4)
+        close(llmops.fc_Q4A_decode(attn, ops["gate_up_proj"].weight, 2 * F, norm=(n2.weight, n2.eps)), h(gu_row), 1e-4)
+        wgu = ops["gate_up_proj"].weight
+        interleaved = llmops.interleave_gate_up(wgu[:F // 32], wgu[F // 32:])
+        close(llmops.fc_Q4A_decode(attn, interleaved, F, norm=(n2.weight, n2.eps), glu=True), h(up), 1e-4)
         close(llmops.fc_Q4A_decode(up, ops["down_proj"].weight, H, residual=attn), orc.iadd(h(down), h(attn)), 1e-5)
+        close(llmops.fc_Q4A_decode(gu_row, ops["down_proj"].weight, H, residual=attn, glu_in=True),
+              orc.iadd(h(down), h(attn)), 1e-5)
 
 
 def test_decode_graph_replay_matches_eager():

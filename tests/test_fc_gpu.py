@@ -286,6 +286,35 @@ def test_fc_decode_sumsq_handover(ops, orc, G, rows, N, K):
         assert max_rel_err(b, orc.fc(orc.rmsnorm(host(y), nw, 1e-5), host(p2), F)) <= 1e-3
 
 
+@pytest.mark.parametrize("G", [32, 128])
+@pytest.mark.parametrize("rows", [1, 2, 4, 8, 20])
+@pytest.mark.parametrize("N,K", [(1000, 1024), (4096, 11008)])
+def test_fc_decode_gate_up_input(ops, orc, G, rows, N, K):
+    """fc_Q4A_decode(glu_in=True): the input row is [gate | up] (2K floats) and the FC runs on
+    silu(gate)*up; against the oracle's silu, imul and fc, with and without the residual and the
+    sums of squares (K = 11008 also takes the split-K hand-off), and bit-equal to silu_mul + FC."""
+    rng = np.random.default_rng(rows + G + N)
+    gu = rng.standard_normal((1, rows, 2 * K)).astype(np.float32)
+    w = (rng.standard_normal((N, K)) * 0.02).astype(np.float32)
+    res = rng.standard_normal((1, rows, N)).astype(np.float32)
+    pw = orc.quant_w(w, G)
+    act = orc.imul(gu[..., K:].copy(), orc.silu(gu[..., :K].copy()))
+    want = orc.fc(act, pw, N)
+    got = ops.fc_Q4A_decode(dev(gu), dev(pw), N, glu_in=True)
+    assert max_rel_err(host(got), want) <= 1e-4  # expf here and exp there: an int8 code may flip
+    two_step = ops.fc_Q4A_decode(ops.silu_mul(dev(gu)), dev(pw), N)
+    assert torch.equal(got, two_step)
+    got, ss = ops.fc_Q4A_decode(dev(gu), dev(pw), N, residual=dev(res), want_sumsq=True, glu_in=True)
+    assert max_rel_err(host(got), want + res) <= 1e-4
+    strips = -(-N // 32)
+    pad = np.zeros((rows, strips * 32))
+    pad[:, :N] = host(got).astype(np.float64).reshape(rows, N)
+    ref_ss = (pad.reshape(rows, strips, 32) ** 2).sum(-1)
+    assert np.abs(host(ss) - ref_ss).max() <= 1e-5 * ref_ss.max()
+    with pytest.raises(RuntimeError):  # no rmsnorm in front of a gate|up row
+        ops.fc_Q4A_decode(dev(gu), dev(pw), N, norm=(torch.ones(K, device="cuda"), 1e-5), glu_in=True)
+
+
 @pytest.mark.parametrize("rows", [9, 12, 16])
 @pytest.mark.parametrize("N,K", [(2070, 1024), (4096, 4096)])
 def test_fc_rows_9_to_16_streaming_mfma(ops, orc, rows, N, K):
