@@ -21,7 +21,7 @@ size_t gemm_workspace_bytes(int64_t rows, int64_t Ng, int64_t Kg, int G);
 int launch_gemm(const uint8_t* w, const int8_t* xq, const float* xd, const float* gs, const float2* xsT, float* y,
                 float* part, int64_t rows, int64_t Ng, int64_t Kg, int G, int64_t N, hipStream_t st);
 int launch_gemm_partials(const uint8_t* w, const int8_t* xq, int32_t* acc, int64_t rows, int64_t Ng, int64_t Kg, int G,
-                         hipStream_t st);
+                         bool two_groups, hipStream_t st);
 int launch_fc_rows(const uint8_t* w, const int8_t* xq, const float2* xsT, float* y, int64_t rows, int64_t Ng, int64_t Kg,
                    int64_t N, const float* residual, hipStream_t st);
 bool gemm_rows_kernel_enabled();
@@ -171,6 +171,7 @@ extern "C" int llmops_fc_Q4A_partials(const int8_t* xq, int64_t rows, const int8
     LLMOPS_REQUIRE(aligned(weiq, 16) && aligned(xq, 16));
     LLMOPS_REQUIRE(Ng * Kg < ((int64_t)1 << 31));
     const uint8_t* w = reinterpret_cast<const uint8_t*>(weiq);
-    if (use_mfma) return launch_gemm_partials(w, xq, acc, rows, Ng, Kg, group_k, as_stream(stream));
+    LLMOPS_REQUIRE(use_mfma >= 0 && use_mfma <= 2 && (use_mfma != 2 || group_k == 128));
+    if (use_mfma) return launch_gemm_partials(w, xq, acc, rows, Ng, Kg, group_k, use_mfma == 2, as_stream(stream));
     return launch_gemv_partials(w, xq, acc, rows, Ng, Kg, group_k, as_stream(stream));
 }

@@ -201,8 +201,27 @@ __global__ __launch_bounds__(256, (RT == 4 ? 2 : (RT == 2 ? 3 : 4))) void fc_gem
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wr = wave >> 1, wc = wave & 1;  // wave's row half / column half
     const int g = lane >> 4, jj = lane & 15, q = jj & 7, sp = jj >> 3;
-    const int strip0 = blockIdx.x * 4;
-    const int row0 = blockIdx.y * BM;
+    // Which tile: workgroups go to the 8 XCDs round robin, each XCD has its own L2, and an XCD runs
+    // about 32 CUs x (workgroups per CU) workgroups at a time.  The tiles are therefore numbered so that
+    // each XCD gets one contiguous run of them and a run walks the tile grid in bands of 8 row blocks,
+    // rows fastest: the workgroups resident on one XCD then cover about 8 row blocks x 8..16 column
+    // blocks and every activation and weight tile is fetched into that L2 once instead of once per
+    // workgroup.  (With column blocks fastest across the whole chip the weights, re-read by every row
+    // block, came from beyond the L2 each time.)
+    const int nbx = (Ng + 3) / 4, nby = (rows + BM - 1) / BM;
+    int bx, by;
+    {
+        const int total = nbx * nby, per_xcd = (total + 7) / 8;
+        const int i = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+        if ((int)(blockIdx.x >> 3) >= per_xcd || i >= total) return;  // uniform for the workgroup
+        constexpr int kBand = 8;
+        const int band = i / (kBand * nbx), in_band = i % (kBand * nbx);
+        const int first = band * kBand, rows_in_band = min(kBand, nby - first);
+        by = first + in_band % rows_in_band;
+        bx = in_band / rows_in_band;
+    }
+    const int strip0 = bx * 4;
+    const int row0 = by * BM;
     const int kb0 = blockIdx.z * kb_per_split, kb1 = min(Kg, kb0 + kb_per_split);
     const int64_t Kp = (int64_t)Kg * 128;
 
@@ -385,6 +404,352 @@ __global__ __launch_bounds__(256, (RT == 4 ? 2 : (RT == 2 ? 3 : 4))) void fc_gem
         }
 }
 
+// ---- two groups of wavefronts in alternating phases (group 128, many rows) -------------------------
+// Per k-group a wavefront has a matrix-core phase (operand reads, 32 int8 MFMAs) and a vector-ALU
+// phase (the fp32 fold: convert, scale product, fma per output element).  Two independent wavefronts
+// on one SIMD drift into the same phase and then simply take turns on the same pipe, so nothing
+// overlaps.  Here a workgroup has 8 wavefronts = two groups of 4, one of each per SIMD, and the phases
+// are separated by workgroup barriers with the second group started one phase late: while one group's
+// MFMAs run, the other group's fold has the vector ALU, by construction.  The vector ALU is the
+// scarcer unit (3 instructions per output element and k-group against 2 MFMAs per 256 elements), so
+// everything else is kept off it:
+//   tile: 256 rows x 128 columns; group p owns rows 128p..128p+127 (wave = 64 x 64, as in the kernel
+//   above); the weights of the tile are staged once and used by both groups.
+//   weights: fetched by group 0 (the one ahead in time) into registers one k-group ahead, unpacked
+//   ONCE per workgroup to int8 and stored to LDS in MFMA operand order ([strip][k half][column
+//   set c][g][q] -> 16 bytes), fp16 scales converted to fp32 on the way; a wave's B operands are
+//   then plain 16-byte LDS reads, no unpacking per wave.
+//   activations and their scales: asynchronous global->LDS copies (no registers, no LDS store
+//   instructions), issued at the top of an iteration for the next k-group and waited for before the
+//   iteration's last barrier; each group copies its own rows.  Tile rows are 128 bytes with the
+//   16-byte chunk c of row r at chunk position c ^ key(r), key(r) = (r + ((r >> 3) & 1)) & 7: the 16
+//   rows that one ds_read_b128 touches then fall on 16 different 16-byte bank groups of the 256-byte
+//   bank line (and any aligned 8 of them on 8 different ones).  The copies land lane by lane, so the
+//   spreading is done by choosing what each lane fetches.  The unpacked weights of a strip take
+//   4096 + 128 bytes for the same reason (a read touches two strips).
+//   Group 1 still folds k-group kb-1 while group 0 overwrites that k-group's weight buffer, which is
+//   why the weight scales are taken into registers in the matrix-core phase.
+//   The A operands are read by hand-placed ds_read_b128 (four row tiles ahead of the MFMAs that use
+//   them) with hand-placed waits: the compiler would issue each read right before its use and leave
+//   the matrix cores waiting for LDS eight times per k-group.
+constexpr int kBuStrip = 2 * 4 * 4 * 8 * 16 + 128;
+struct GemmPPSmem {
+    static constexpr int BM = 256;
+    uint8_t a[2][BM * 128];
+    uint8_t bu[2][4 * kBuStrip];            // unpacked weights: [strip][h][c][g][q][16], strips padded
+    float d[2][4 * 32];                     // weight scale, min per strip column
+    float m[2][4 * 32];
+    float dx[2][BM];
+    float gs[2][BM];
+};
+
+__device__ __forceinline__ uint32_t lds_off(const void* p) {
+    return (uint32_t)(uintptr_t)((const __attribute__((address_space(3))) void*)p);
+}
+// lane i's 16 (4) bytes at base + off (base the same for the whole wave, off a byte offset per lane)
+// land at lds_base + 16*i (4*i); counts in vmcnt like any load
+__device__ __forceinline__ void copy16_to_lds(const void* base, uint32_t off, uint32_t lds_base) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(off), "s"(base), "s"(lds_base) : "memory", "m0");
+}
+__device__ __forceinline__ void copy4_to_lds(const void* base, uint32_t off, uint32_t lds_base) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1" : : "v"(off), "s"(base), "s"(lds_base) : "memory", "m0");
+}
+// 16-byte LDS read whose result may only be used after lds_ready<N>() on it, N = number of LDS
+// operations issued after this one that may still be pending (LDS operations complete in order).
+// Between the two calls the variable must not be touched.
+template <int OFF>
+__device__ __forceinline__ void lds_read16_issue(v4i& r, uint32_t addr) {
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=&v"(r) : "v"(addr), "n"(OFF) : "memory");
+}
+template <int N>
+__device__ __forceinline__ void lds_ready(v4i& r) {
+    asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(r) : "n"(N) : "memory");
+}
+
+template <bool PARTIALS>
+__global__ __launch_bounds__(512, 2) void fc_gemm_pp_kernel(const uint8_t* __restrict__ weiq, const int8_t* __restrict__ xq,
+                                                             const float* __restrict__ xd, const float* __restrict__ gs,
+                                                             const float2* __restrict__ xsT, float* __restrict__ out,
+                                                             int32_t* __restrict__ out_i, int Ng, int Kg, int64_t ldo,
+                                                             int64_t N, int rows, int kb_per_split, int64_t split_stride) {
+    constexpr int RT = 4, BM = 256, GM = 128;
+    extern __shared__ __align__(16) uint8_t smem_raw[];
+    GemmPPSmem& sm = *reinterpret_cast<GemmPPSmem*>(smem_raw);
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int grp = wave >> 2, w4 = wave & 3;
+    const int wr = w4 >> 1, wc = w4 & 1;
+    const int g = lane >> 4, jj = lane & 15, q = jj & 7, sp = jj >> 3;
+    // tile numbering: one contiguous run of tiles per XCD, bands of 8 row blocks, rows fastest
+    const int nbx = (Ng + 3) / 4, nby = (rows + BM - 1) / BM;
+    int bx, by;
+    {
+        const int total = nbx * nby, per_xcd = (total + 7) / 8;
+        const int i = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+        if ((int)(blockIdx.x >> 3) >= per_xcd || i >= total) return;  // uniform for the workgroup
+        constexpr int kBand = 8;
+        const int band = i / (kBand * nbx), in_band = i % (kBand * nbx);
+        const int first = band * kBand, rows_in_band = min(kBand, nby - first);
+        by = first + in_band % rows_in_band;
+        bx = in_band / rows_in_band;
+    }
+    const int strip0 = bx * 4;
+    const int row0 = by * BM + grp * GM;  // first row of this group
+    const int kb0 = blockIdx.z * kb_per_split, kb1 = min(Kg, kb0 + kb_per_split);
+    const int64_t Kp = (int64_t)Kg * 128;
+
+    // ---- what this lane copies per k-group ----
+    // activations: wave w4 of a group copies its row blocks 4*w4 .. 4*w4+3 (8 rows x 128 bytes each)
+    // (all sources are a wave-uniform base pointer, which moves with the k-group, plus a 32-bit byte
+    // offset per lane; the host only launches this kernel when the tensors are below 2 GiB)
+    uint32_t aoff[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int r = (w4 * 4 + i) * 8 + (lane >> 3);  // row within the group (a multiple of 16 rows per group)
+        const int key = (r + ((r >> 3) & 1)) & 7;
+        aoff[i] = (uint32_t)(min(rows - 1, row0 + r) * (int)Kp + (((lane & 7) ^ key) * 16));
+    }
+    // scales: waves 0,1 copy dx of rows 64*w4 + lane, waves 2,3 the group sums of rows 64*(w4-2) + lane
+    const int xr = (w4 & 1) * 64 + lane;
+    const int64_t xrow = min(rows - 1, row0 + xr);
+    const uint8_t* xbase = nullptr;
+    uint32_t xoff = 0;
+    int64_t xstep = 0;  // bytes per k-group
+    if (!PARTIALS) {
+        if (xsT) {
+            xbase = reinterpret_cast<const uint8_t*>(xsT);
+            xoff = (uint32_t)((xrow * 2 + (w4 >> 1)) * 4);
+            xstep = (int64_t)rows * 8;
+        } else {
+            xbase = reinterpret_cast<const uint8_t*>((w4 >> 1) ? gs : xd);
+            xoff = (uint32_t)(xrow * Kg * 4);
+            xstep = 4;
+        }
+    }
+    const uint32_t lds_a = lds_off(&sm.a[0][0]);
+    const uint32_t lds_x = (w4 >> 1) ? lds_off(&sm.gs[0][0]) : lds_off(&sm.dx[0][0]);
+#define LLMOPS_COPY(KB, BUF)                                                                                       \
+    do {                                                                                                           \
+        _Pragma("unroll") for (int i = 0; i < 4; i++)                                                              \
+            copy16_to_lds(xq + (int64_t)(KB) * 128, aoff[i],                                                       \
+                          lds_a + (BUF) * (BM * 128) + (grp * GM + (w4 * 4 + i) * 8) * 128);                       \
+        if (!PARTIALS) copy4_to_lds(xbase + (int64_t)(KB) * xstep, xoff, lds_x + (BUF) * (BM * 4) + (grp * GM + (w4 & 1) * 64) * 4); \
+    } while (0)
+
+    // weights (group 0): thread t of the group takes the 16-byte chunks t and t + 256 of the tile's
+    // 512 (chunk = strip (2 bits) | k8-row (4 bits) | column quad (3 bits)); its first 32 threads also
+    // the 32 chunks of fp16 scales (strip (2 bits) | d or m (1 bit) | column octet (2 bits))
+    const int gtid = tid & 255;
+    uint32_t boff[2];
+    int bdst[2];
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        const int ch = gtid + i * 256, st = ch >> 7, r = (ch >> 3) & 15, q4 = ch & 7;
+        boff[i] = (uint32_t)(min(Ng - 1, strip0 + st) * Kg * kBlk128 + r * 128 + q4 * 16);
+        // [strip][h = r>>3][c][g = (r&7)>>1][q4][8 * (r&1)]; c adds 512 bytes
+        bdst[i] = st * kBuStrip + ((((r >> 3) * 4) * 4 + ((r & 7) >> 1)) * 8 + q4) * 16 + (r & 1) * 8;
+    }
+    const int sst = (gtid >> 3) & 3, spart = gtid & 7;
+    const uint32_t soff = (uint32_t)(min(Ng - 1, strip0 + sst) * Kg * kBlk128 + 2048 + spart * 16);
+    v4u rb[2], rs = {0u, 0u, 0u, 0u};
+#define LLMOPS_FETCH_B(KB)                                                                                 \
+    do {                                                                                                   \
+        if (grp == 0) {                                                                                    \
+            const uint8_t* wkb = weiq + (int64_t)(KB) * kBlk128;                                           \
+            rb[0] = *reinterpret_cast<const v4u*>(wkb + boff[0]);                                          \
+            rb[1] = *reinterpret_cast<const v4u*>(wkb + boff[1]);                                          \
+            if (gtid < 32) rs = *reinterpret_cast<const v4u*>(wkb + soff);                                 \
+        }                                                                                                  \
+    } while (0)
+#define LLMOPS_STASH_B(BUF)                                                                                \
+    do {                                                                                                   \
+        if (grp == 0) {                                                                                    \
+            _Pragma("unroll") for (int i = 0; i < 2; i++)                                                  \
+                _Pragma("unroll") for (int c = 0; c < 4; c++) {                                            \
+                    uint2 u;                                                                               \
+                    u.x = lo4(rb[i][c]);                                                                   \
+                    u.y = hi4(rb[i][c]);                                                                   \
+                    *reinterpret_cast<uint2*>(&sm.bu[BUF][bdst[i] + c * 512]) = u;                         \
+                }                                                                                          \
+            if (gtid < 32) {                                                                               \
+                float* dstf = (spart < 4 ? sm.d[BUF] : sm.m[BUF]) + sst * 32 + (spart & 3) * 8;            \
+                float4 lo, hi;                                                                             \
+                lo.x = f16_bits_to_f32((uint16_t)(rs[0] & 0xFFFFu));                                       \
+                lo.y = f16_bits_to_f32((uint16_t)(rs[0] >> 16));                                           \
+                lo.z = f16_bits_to_f32((uint16_t)(rs[1] & 0xFFFFu));                                       \
+                lo.w = f16_bits_to_f32((uint16_t)(rs[1] >> 16));                                           \
+                hi.x = f16_bits_to_f32((uint16_t)(rs[2] & 0xFFFFu));                                       \
+                hi.y = f16_bits_to_f32((uint16_t)(rs[2] >> 16));                                           \
+                hi.z = f16_bits_to_f32((uint16_t)(rs[3] & 0xFFFFu));                                       \
+                hi.w = f16_bits_to_f32((uint16_t)(rs[3] >> 16));                                           \
+                *reinterpret_cast<float4*>(dstf) = lo;                                                     \
+                *reinterpret_cast<float4*>(dstf + 4) = hi;                                                 \
+            }                                                                                              \
+        }                                                                                                  \
+    } while (0)
+
+    v4f f[RT][4];
+#pragma unroll
+    for (int t = 0; t < RT; t++)
+#pragma unroll
+        for (int c = 0; c < 4; c++) f[t][c] = v4f{0.f, 0.f, 0.f, 0.f};
+    float gk[RT], mk[4];  // min term, four k-groups at a time by fp32 MFMA (see the kernel above)
+#pragma unroll
+    for (int t = 0; t < RT; t++) gk[t] = 0.0f;
+#pragma unroll
+    for (int c = 0; c < 4; c++) mk[c] = 0.0f;
+
+    if (kb0 < kb1) {
+        LLMOPS_COPY(kb0, 0);
+        LLMOPS_FETCH_B(kb0);
+        LLMOPS_STASH_B(0);
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (grp == 1) __syncthreads();  // group 1 runs one phase behind group 0
+
+    const int strip_l = wc * 2 + sp;          // strip (0..3) of the tile this lane's B operands come from
+    const int lrow = grp * GM + wr * 64;      // first tile row of this wave
+    // A operand of row tile t, k half h: row lrow + 16t + jj, chunk 4h + g, swizzled by the row's low bits
+    const int akey = (jj + (jj >> 3)) & 7;
+    const uint32_t a_rd0 = lds_a + (lrow + jj) * 128 + (((0 + g) ^ akey) * 16);
+    const uint32_t a_rd1 = lds_a + (lrow + jj) * 128 + (((4 + g) ^ akey) * 16);
+    const int b_rd = strip_l * kBuStrip + (g * 8 + q) * 16;  // + (4h + c) * 512
+    for (int kb = kb0; kb < kb1; kb++) {
+        const int buf = (kb - kb0) & 1;
+        if (kb + 1 < kb1) {
+            LLMOPS_COPY(kb + 1, buf ^ 1);
+            LLMOPS_FETCH_B(kb + 1);
+        }
+
+        // ---- matrix-core phase ----
+        const uint32_t ar0 = a_rd0 + buf * (BM * 128), ar1 = a_rd1 + buf * (BM * 128);
+        v4i a00, a01, a02, a03, a10, a11, a12, a13;
+        lds_read16_issue<0 * 2048>(a00, ar0);
+        lds_read16_issue<1 * 2048>(a01, ar0);
+        lds_read16_issue<2 * 2048>(a02, ar0);
+        lds_read16_issue<3 * 2048>(a03, ar0);
+        v4i b[2][4];
+#pragma unroll
+        for (int h = 0; h < 2; h++)
+#pragma unroll
+            for (int c = 0; c < 4; c++) b[h][c] = *reinterpret_cast<const v4i*>(&sm.bu[buf][b_rd + (h * 4 + c) * 512]);
+        const float4 d4 = *reinterpret_cast<const float4*>(&sm.d[buf][strip_l * 32 + q * 4]);
+        const float4 m4 = *reinterpret_cast<const float4*>(&sm.m[buf][strip_l * 32 + q * 4]);
+        float gsr[RT];
+        if (!PARTIALS) {
+#pragma unroll
+            for (int t = 0; t < RT; t++) gsr[t] = sm.gs[buf][lrow + t * 16 + jj];
+        }
+        v4i acc[RT][4];
+        const v4i zero4 = v4i{0, 0, 0, 0};
+#define LLMOPS_MMA4(T, H, A)                                                                              \
+    _Pragma("unroll") for (int c = 0; c < 4; c++)                                                         \
+        acc[T][c] = __builtin_amdgcn_mfma_i32_16x16x64_i8(A, b[H][c], (H) == 0 ? zero4 : acc[T][c], 0, 0, 0)
+        lds_ready<3>(a00);
+        LLMOPS_MMA4(0, 0, a00);
+        lds_read16_issue<0 * 2048>(a10, ar1);
+        lds_ready<3>(a01);
+        LLMOPS_MMA4(1, 0, a01);
+        lds_read16_issue<1 * 2048>(a11, ar1);
+        lds_ready<3>(a02);
+        LLMOPS_MMA4(2, 0, a02);
+        lds_read16_issue<2 * 2048>(a12, ar1);
+        lds_ready<3>(a03);
+        LLMOPS_MMA4(3, 0, a03);
+        lds_read16_issue<3 * 2048>(a13, ar1);
+        lds_ready<3>(a10);
+        LLMOPS_MMA4(0, 1, a10);
+        lds_ready<2>(a11);
+        LLMOPS_MMA4(1, 1, a11);
+        lds_ready<1>(a12);
+        LLMOPS_MMA4(2, 1, a12);
+        lds_ready<0>(a13);
+        LLMOPS_MMA4(3, 1, a13);
+#undef LLMOPS_MMA4
+        const float d[4] = {d4.x, d4.y, d4.z, d4.w};
+        if (!PARTIALS) {
+            const float m[4] = {m4.x, m4.y, m4.z, m4.w};
+            const int slot4 = (kb - kb0) & 3;
+            const bool mine4 = slot4 == g;
+#pragma unroll
+            for (int c = 0; c < 4; c++) mk[c] = mine4 ? m[c] : mk[c];
+#pragma unroll
+            for (int t = 0; t < RT; t++) gk[t] = mine4 ? gsr[t] : gk[t];
+            if (slot4 == 3 || kb + 1 == kb1) {
+#pragma unroll
+                for (int t = 0; t < RT; t++) {
+#pragma unroll
+                    for (int c = 0; c < 4; c++) f[t][c] = __builtin_amdgcn_mfma_f32_16x16x4f32(gk[t], mk[c], f[t][c], 0, 0, 0);
+                    gk[t] = 0.0f;
+                }
+#pragma unroll
+                for (int c = 0; c < 4; c++) mk[c] = 0.0f;
+            }
+        }
+        __syncthreads();
+
+        // ---- vector phase: fold the int32 tiles into the fp32 accumulators ----
+        if (PARTIALS) {
+            const int strip = strip0 + strip_l;
+            if (strip < Ng) {
+#pragma unroll
+                for (int t = 0; t < RT; t++)
+#pragma unroll
+                    for (int v = 0; v < 4; v++) {
+                        const int row = row0 + wr * 64 + t * 16 + g * 4 + v;
+                        if (row < rows) {
+#pragma unroll
+                            for (int c = 0; c < 4; c++)
+                                out_i[((int64_t)row * ((int64_t)Ng * kGroupN) + strip * kGroupN + q * 4 + c) * Kg + kb] =
+                                    acc[t][c][v];
+                        }
+                    }
+            }
+        } else {
+#pragma unroll
+            for (int t = 0; t < RT; t++) {
+                // dx of the 4 rows this lane holds results for: rows lrow + t*16 + 4g + v
+                const float4 x4 = *reinterpret_cast<const float4*>(&sm.dx[buf][lrow + t * 16 + g * 4]);
+                const float dxv[4] = {x4.x, x4.y, x4.z, x4.w};
+#pragma unroll
+                for (int v = 0; v < 4; v++)
+#pragma unroll
+                    for (int c = 0; c < 4; c++) f[t][c][v] = fmaf(d[c] * dxv[v], (float)acc[t][c][v], f[t][c][v]);
+            }
+        }
+        if (kb + 1 < kb1) LLMOPS_STASH_B(buf ^ 1);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's copies for the next k-group have landed
+        __syncthreads();
+    }
+    if (grp == 0) __syncthreads();  // pairs with group 1's last barrier
+#undef LLMOPS_COPY
+#undef LLMOPS_FETCH_B
+#undef LLMOPS_STASH_B
+
+    if (PARTIALS) return;
+    const int strip = strip0 + strip_l;
+    if (strip >= Ng) return;
+    float* o = out + (int64_t)blockIdx.z * split_stride;
+    const int64_t n0 = (int64_t)strip * kGroupN + q * 4;
+#pragma unroll
+    for (int t = 0; t < RT; t++)
+#pragma unroll
+        for (int v = 0; v < 4; v++) {
+            const int row = row0 + wr * 64 + t * 16 + g * 4 + v;
+            if (row >= rows) continue;
+            float* dst = o + (int64_t)row * ldo + n0;
+            if (n0 + 3 < N && (ldo & 3) == 0) {
+                *reinterpret_cast<float4*>(dst) = make_float4(f[t][0][v], f[t][1][v], f[t][2][v], f[t][3][v]);
+            } else {
+#pragma unroll
+                for (int c = 0; c < 4; c++)
+                    if (n0 + c < N) dst[c] = f[t][c][v];
+            }
+        }
+}
+
 // y[row][n] = sum over splits (index order) of part[s][row][n]
 __global__ void gemm_reduce_kernel(const float* __restrict__ part, float* __restrict__ y, int64_t rows, int64_t N,
                                    int64_t ldp, int64_t split_stride, int S) {
@@ -433,6 +798,7 @@ struct GemmPlan {
     bool lds;
 };
 
+static int g_gemm_pp_min_rows = 512;
 static int g_gemm_rt = 0;  // 0 = choose per shape; -1 = also keep 9..32 rows on the tiled kernel
 bool gemm_rows_kernel_enabled() { return g_gemm_rt >= 0; }
 
@@ -459,6 +825,14 @@ static GemmPlan plan_gemm(int64_t rows, int64_t Ng, int64_t Kg, int G) {
     // how evenly the tiles fill the machine, so the plan takes the RT with the least estimated time:
     // rounds of resident workgroups x (rows per tile x workgroups sharing a CU / efficiency) x share of
     // K per split.
+    // (its lanes address the tensors with 32-bit byte offsets)
+    const bool small = rows * Kg * 128 < ((int64_t)1 << 31) && Ng * Kg * 2176 < ((int64_t)1 << 31);
+    if (small && (g_gemm_rt == 8 || (g_gemm_rt == 0 && rows >= g_gemm_pp_min_rows))) {
+        // two groups of waves in alternating phases, 256 x 128 tiles, one workgroup per CU
+        p.RT = 8;
+        gemm_split(((Ng + 3) / 4) * ((rows + 255) / 256), 256, Kg, p);
+        return p;
+    }
     static const int kRT[3] = {4, 2, 1};
     static const int kWgPerCu[3] = {2, 3, 4};
     static const double kEff[3] = {1.0, 0.98, 0.77};
@@ -505,9 +879,26 @@ static int launch_gemm_lds_t(const uint8_t* w, const int8_t* xq, const float* xd
                                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(GemmSmem<RT>)));
         configured = true;
     }
-    dim3 grid((unsigned)((Ng + 3) / 4), (unsigned)((rows + RT * 32 - 1) / (RT * 32)), (unsigned)p.S);
+    const int64_t tiles = ((Ng + 3) / 4) * ((rows + RT * 32 - 1) / (RT * 32));
+    dim3 grid((unsigned)(8 * ((tiles + 7) / 8)), 1, (unsigned)p.S);  // one run of tiles per XCD
     fc_gemm_lds_kernel<RT, false><<<grid, 256, sizeof(GemmSmem<RT>), st>>>(w, xq, xd, gs, xsT, out, nullptr, (int)Ng, (int)Kg,
                                                                           ldo, N, (int)rows, p.kb_per_split, split_stride);
+    return LLMOPS_OK;
+}
+
+static int launch_gemm_pp(const uint8_t* w, const int8_t* xq, const float* xd, const float* gs, const float2* xsT, float* out,
+                          int64_t Ng, int64_t Kg, int64_t ldo, int64_t N, int64_t rows, const GemmPlan& p,
+                          int64_t split_stride, hipStream_t st) {
+    static bool configured = false;
+    if (!configured) {
+        LLMOPS_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&fc_gemm_pp_kernel<false>),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(GemmPPSmem)));
+        configured = true;
+    }
+    const int64_t tiles = ((Ng + 3) / 4) * ((rows + 255) / 256);
+    dim3 grid((unsigned)(8 * ((tiles + 7) / 8)), 1, (unsigned)p.S);
+    fc_gemm_pp_kernel<false><<<grid, 512, sizeof(GemmPPSmem), st>>>(w, xq, xd, gs, xsT, out, nullptr, (int)Ng, (int)Kg, ldo, N,
+                                                                   (int)rows, p.kb_per_split, split_stride);
     return LLMOPS_OK;
 }
 
@@ -521,7 +912,8 @@ int launch_gemm(const uint8_t* w, const int8_t* xq, const float* xd, const float
     const int64_t ss = rows * Np;
     if (p.lds) {
         int rc;
-        if (p.RT == 4) rc = launch_gemm_lds_t<4>(w, xq, xd, gs, xsT, out, Ng, Kg, ldo, Nw, rows, p, ss, st);
+        if (p.RT == 8) rc = launch_gemm_pp(w, xq, xd, gs, xsT, out, Ng, Kg, ldo, Nw, rows, p, ss, st);
+        else if (p.RT == 4) rc = launch_gemm_lds_t<4>(w, xq, xd, gs, xsT, out, Ng, Kg, ldo, Nw, rows, p, ss, st);
         else if (p.RT == 2) rc = launch_gemm_lds_t<2>(w, xq, xd, gs, xsT, out, Ng, Kg, ldo, Nw, rows, p, ss, st);
         else rc = launch_gemm_lds_t<1>(w, xq, xd, gs, xsT, out, Ng, Kg, ldo, Nw, rows, p, ss, st);
         if (rc) return rc;
@@ -540,15 +932,29 @@ int launch_gemm(const uint8_t* w, const int8_t* xq, const float* xd, const float
 }
 
 int launch_gemm_partials(const uint8_t* w, const int8_t* xq, int32_t* acc, int64_t rows, int64_t Ng, int64_t Kg, int G,
-                         hipStream_t st) {
-    if (G == 128) {  // the production LDS-tiled loop, writing its int32 tiles instead of folding them
+                         bool two_groups, hipStream_t st) {
+    if (G == 128 && two_groups) {
+        if (!(rows * Kg * 128 < ((int64_t)1 << 31) && Ng * Kg * 2176 < ((int64_t)1 << 31)))
+            return fail(LLMOPS_EINVAL, "the 256-row kernel addresses its operands with 32-bit offsets");
+        static bool configured = false;
+        if (!configured) {
+            LLMOPS_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&fc_gemm_pp_kernel<true>),
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(GemmPPSmem)));
+            configured = true;
+        }
+        const int64_t tiles = ((Ng + 3) / 4) * ((rows + 255) / 256);
+        dim3 grid((unsigned)(8 * ((tiles + 7) / 8)), 1, 1);
+        fc_gemm_pp_kernel<true><<<grid, 512, sizeof(GemmPPSmem), st>>>(w, xq, nullptr, nullptr, nullptr, nullptr, acc, (int)Ng,
+                                                                      (int)Kg, 0, 0, (int)rows, (int)Kg, 0);
+    } else if (G == 128) {  // the production LDS-tiled loop, writing its int32 tiles instead of folding them
         static bool configured = false;
         if (!configured) {
             LLMOPS_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&fc_gemm_lds_kernel<2, true>),
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(GemmSmem<2>)));
             configured = true;
         }
-        dim3 grid((unsigned)((Ng + 3) / 4), (unsigned)((rows + 63) / 64), 1);
+        const int64_t tiles = ((Ng + 3) / 4) * ((rows + 63) / 64);
+        dim3 grid((unsigned)(8 * ((tiles + 7) / 8)), 1, 1);
         fc_gemm_lds_kernel<2, true><<<grid, 256, sizeof(GemmSmem<2>), st>>>(w, xq, nullptr, nullptr, nullptr, nullptr, acc,
                                                                           (int)Ng, (int)Kg, 0, 0, (int)rows, (int)Kg, 0);
     } else {

@@ -303,7 +303,7 @@ def fc_Q4A_partials(xq, weiq, use_mfma=False):
     lead = tuple(xq.shape[:-1])
     rows = xq.numel() // (Kg * g)
     acc = torch.empty(lead + (Ng * 32, Kg), dtype=torch.int32, device=xq.device)
-    _lib.check(_lib.load().llmops_fc_Q4A_partials(_ptr(xq), rows, _ptr(weiq), Ng, Kg, g, _ptr(acc), int(bool(use_mfma)),
+    _lib.check(_lib.load().llmops_fc_Q4A_partials(_ptr(xq), rows, _ptr(weiq), Ng, Kg, g, _ptr(acc), int(use_mfma),
                                                   _stream(xq)))
     return acc
 

@@ -102,9 +102,11 @@ def test_quant_x_rows_variant_vs_oracle(ops, orc, G, rows, K):
 
 
 # ---- int32 partial sums -------------------------------------------------------------------------
-@pytest.mark.parametrize("G", [32, 128])
-@pytest.mark.parametrize("mfma", [False, True])
-@pytest.mark.parametrize("rows,N,K", [(1, 4096, 4096), (3, 352, 2048), (17, 96, 1024), (40, 32, 384)])
+INNER_LOOPS = [(32, 0), (32, 1), (128, 0), (128, 1), (128, 2)]  # (group, use_mfma); 2 = 256-row kernel, group 128 only
+
+
+@pytest.mark.parametrize("G,mfma", INNER_LOOPS)
+@pytest.mark.parametrize("rows,N,K", [(1, 4096, 4096), (3, 352, 2048), (17, 96, 1024), (40, 32, 384), (300, 160, 640)])
 def test_partials_bit_exact(ops, orc, G, mfma, rows, N, K):
     rng = np.random.default_rng(rows * 7 + G)
     wq = orc.quant_w((rng.standard_normal((N, K)) * 0.02).astype(np.float32), G)
@@ -114,8 +116,7 @@ def test_partials_bit_exact(ops, orc, G, mfma, rows, N, K):
     assert np.array_equal(got, orc.fc_partials(xq, wq))
 
 
-@pytest.mark.parametrize("G", [32, 128])
-@pytest.mark.parametrize("mfma", [False, True])
+@pytest.mark.parametrize("G,mfma", INNER_LOOPS)
 def test_partials_extreme_codes(ops, orc, G, mfma):
     w = np.full((32, 2 * G), 15.0, np.float32)
     w[:, 0::G] = 0.0
@@ -313,6 +314,34 @@ def test_fc_decode_gate_up_input(ops, orc, G, rows, N, K):
     assert np.abs(host(ss) - ref_ss).max() <= 1e-5 * ref_ss.max()
     with pytest.raises(RuntimeError):  # no rmsnorm in front of a gate|up row
         ops.fc_Q4A_decode(dev(gu), dev(pw), N, norm=(torch.ones(K, device="cuda"), 1e-5), glu_in=True)
+
+
+@pytest.mark.parametrize("tiling", [1, 2, 4, 8])
+@pytest.mark.parametrize("rows,N,K", [(70, 2070, 1024), (300, 2070, 1024), (515, 352, 4096), (1024, 4096, 512)])
+def test_fc_prefill_every_tiling_vs_oracle(ops, orc, tiling, rows, N, K):
+    """The group-128 MFMA kernels with each row tiling forced in turn (32, 64, 128 rows per workgroup, and
+    the 256-row kernel whose two wave groups alternate phases), on shapes with ragged row and column
+    edges, with and without split-K: output against the oracle, the residual epilogue, and the
+    closed-form construction exactly."""
+    from llmops import _lib
+    lib = _lib.load()
+    rng = np.random.default_rng(rows + N + tiling)
+    x = rng.standard_normal((1, rows, K)).astype(np.float32)
+    w = (rng.standard_normal((N, K)) * 0.02).astype(np.float32)
+    res = rng.standard_normal((1, rows, N)).astype(np.float32)
+    pw = orc.quant_w(w, 128)
+    want = orc.fc(x, pw, N)
+    xe, we = oracle.closed_form_fc_inputs(rows, N, K, seed=rows)
+    lib.llmops_gemm_set_tuning(tiling)
+    try:
+        got = host(ops.fc_Q4A(dev(x), dev(pw), N))
+        got_res = host(ops.fc_Q4A(dev(x), dev(pw), N, residual=dev(res)))
+        ye = host(ops.fc_Q4A(dev(xe.reshape(1, rows, K)), ops.offline_FC_quant_Q4A(dev(we), 128), N))
+    finally:
+        lib.llmops_gemm_set_tuning(0)
+    assert max_rel_err(got, want) <= 1e-5
+    assert max_rel_err(got_res, want + res) <= 1e-5
+    assert np.array_equal(ye, (xe.astype(np.float64) @ we.astype(np.float64).T).astype(np.float32).reshape(1, rows, N))
 
 
 @pytest.mark.parametrize("rows", [9, 12, 16])
