@@ -261,8 +261,9 @@ int llmops_calib_copy(const void* src, void* dst, int64_t bytes, int workgroups,
 void llmops_fc_set_tuning(int target_workgroups, int waves_per_workgroup);
 
 /* prefill GEMM planner knob: force the row-tile factor of the LDS-tiled MFMA kernel (1, 2 or 4:
- * 32, 64 or 128 rows per workgroup); 0 = choose per shape; -1 = choose per shape and send 9..16 rows
- * to the tiled kernel too instead of the weight-streaming MFMA kernel */
+ * 32, 64 or 128 rows per workgroup; 8: the 256-row kernel whose two wave groups alternate between
+ * MFMA and fold phases, which the planner takes from 512 rows on); 0 = choose per shape; -1 = choose
+ * per shape and send 9..16 rows to the tiled kernel too instead of the weight-streaming MFMA kernel */
 void llmops_gemm_set_tuning(int row_tile_factor);
 
 #ifdef __cplusplus

@@ -420,8 +420,10 @@ __global__ __launch_bounds__(256, (RT == 4 ? 2 : (RT == 2 ? 3 : 4))) void fc_gem
 //   set c][g][q] -> 16 bytes), fp16 scales converted to fp32 on the way; a wave's B operands are
 //   then plain 16-byte LDS reads, no unpacking per wave.
 //   activations and their scales: asynchronous global->LDS copies (no registers, no LDS store
-//   instructions), issued at the top of an iteration for the next k-group and waited for before the
-//   iteration's last barrier; each group copies its own rows.  Tile rows are 128 bytes with the
+//   instructions) for the next k-group, issued one at a time between the MFMAs of the matrix-core
+//   phase and waited for before the iteration's last barrier; each group copies its own rows.
+//   (All copies at the top of the phase measured ~500 cycles before the first MFMA: the four waves'
+//   copies queue up in the CU's address unit.)  Tile rows are 128 bytes with the
 //   16-byte chunk c of row r at chunk position c ^ key(r), key(r) = (r + ((r >> 3) & 1)) & 7: the 16
 //   rows that one ds_read_b128 touches then fall on 16 different 16-byte bank groups of the 256-byte
 //   bank line (and any aligned 8 of them on 8 different ones).  The copies land lane by lane, so the
@@ -432,6 +434,14 @@ __global__ __launch_bounds__(256, (RT == 4 ? 2 : (RT == 2 ? 3 : 4))) void fc_gem
 //   The A operands are read by hand-placed ds_read_b128 (four row tiles ahead of the MFMAs that use
 //   them) with hand-placed waits: the compiler would issue each read right before its use and leave
 //   the matrix cores waiting for LDS eight times per k-group.
+//   The fold is register arithmetic and the MFMAs have no side effects, so the compiler is free to
+//   move either across a barrier into the other phase (it did: the fold ended up next to the same
+//   group's MFMAs).  Empty asm statements that name the accumulators as operands pin them.
+// Measured per k-group (2048 x 11008 x 4096, cycles of the shader clock): matrix-core side ~1500
+// (operand reads 450, 32 MFMAs with the copies between them 1000), fold side ~1350-1900 (the fold
+// itself 1350: the vector ALU is shared with the other group's MFMA issue; unpacking the weights on
+// group 0 adds the wait for their fetch), barriers ~400; 4000 per k-group against ~4700 for the
+// four-wave kernel above.
 constexpr int kBuStrip = 2 * 4 * 4 * 8 * 16 + 128;
 struct GemmPPSmem {
     static constexpr int BM = 256;
@@ -457,13 +467,20 @@ __device__ __forceinline__ void copy4_to_lds(const void* base, uint32_t off, uin
 // 16-byte LDS read whose result may only be used after lds_ready<N>() on it, N = number of LDS
 // operations issued after this one that may still be pending (LDS operations complete in order).
 // Between the two calls the variable must not be touched.
-template <int OFF>
+// Between the two calls the variable must not be touched -- which the compiler cannot know, so this
+// pair is only for code that is known not to spill registers (the build of the kernel below that
+// writes int32 tiles does spill, and passes PLAIN = true to get an ordinary load instead).
+template <int OFF, bool PLAIN>
 __device__ __forceinline__ void lds_read16_issue(v4i& r, uint32_t addr) {
-    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=&v"(r) : "v"(addr), "n"(OFF) : "memory");
+    if (PLAIN) {
+        r = *reinterpret_cast<const __attribute__((address_space(3))) v4i*>((uintptr_t)(addr + OFF));
+    } else {
+        asm volatile("ds_read_b128 %0, %1 offset:%2" : "=&v"(r) : "v"(addr), "n"(OFF) : "memory");
+    }
 }
-template <int N>
+template <int N, bool PLAIN>
 __device__ __forceinline__ void lds_ready(v4i& r) {
-    asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(r) : "n"(N) : "memory");
+    if (!PLAIN) asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(r) : "n"(N) : "memory");
 }
 
 template <bool PARTIALS>
@@ -529,12 +546,16 @@ __global__ __launch_bounds__(512, 2) void fc_gemm_pp_kernel(const uint8_t* __res
     }
     const uint32_t lds_a = lds_off(&sm.a[0][0]);
     const uint32_t lds_x = (w4 >> 1) ? lds_off(&sm.gs[0][0]) : lds_off(&sm.dx[0][0]);
+#define LLMOPS_COPY_A(KB, BUF, I)                                                                                  \
+    copy16_to_lds(xq + (int64_t)(KB) * 128, aoff[I], lds_a + (BUF) * (BM * 128) + (grp * GM + (w4 * 4 + (I)) * 8) * 128)
+#define LLMOPS_COPY_X(KB, BUF)                                                                                     \
+    do {                                                                                                           \
+        if (!PARTIALS) copy4_to_lds(xbase + (int64_t)(KB) * xstep, xoff, lds_x + (BUF) * (BM * 4) + (grp * GM + (w4 & 1) * 64) * 4); \
+    } while (0)
 #define LLMOPS_COPY(KB, BUF)                                                                                       \
     do {                                                                                                           \
-        _Pragma("unroll") for (int i = 0; i < 4; i++)                                                              \
-            copy16_to_lds(xq + (int64_t)(KB) * 128, aoff[i],                                                       \
-                          lds_a + (BUF) * (BM * 128) + (grp * GM + (w4 * 4 + i) * 8) * 128);                       \
-        if (!PARTIALS) copy4_to_lds(xbase + (int64_t)(KB) * xstep, xoff, lds_x + (BUF) * (BM * 4) + (grp * GM + (w4 & 1) * 64) * 4); \
+        _Pragma("unroll") for (int i = 0; i < 4; i++) LLMOPS_COPY_A(KB, BUF, i);                                   \
+        LLMOPS_COPY_X(KB, BUF);                                                                                    \
     } while (0)
 
     // weights (group 0): thread t of the group takes the 16-byte chunks t and t + 256 of the tile's
@@ -618,18 +639,18 @@ __global__ __launch_bounds__(512, 2) void fc_gemm_pp_kernel(const uint8_t* __res
     const int b_rd = strip_l * kBuStrip + (g * 8 + q) * 16;  // + (4h + c) * 512
     for (int kb = kb0; kb < kb1; kb++) {
         const int buf = (kb - kb0) & 1;
-        if (kb + 1 < kb1) {
-            LLMOPS_COPY(kb + 1, buf ^ 1);
-            LLMOPS_FETCH_B(kb + 1);
-        }
+        const bool more = kb + 1 < kb1;
 
         // ---- matrix-core phase ----
+        // (the copies for the next k-group are issued between the MFMAs, one per four: four waves
+        // issuing all of theirs at once right after the barrier keep the address unit busy for
+        // several hundred cycles, during which none of them would reach its first MFMA)
         const uint32_t ar0 = a_rd0 + buf * (BM * 128), ar1 = a_rd1 + buf * (BM * 128);
         v4i a00, a01, a02, a03, a10, a11, a12, a13;
-        lds_read16_issue<0 * 2048>(a00, ar0);
-        lds_read16_issue<1 * 2048>(a01, ar0);
-        lds_read16_issue<2 * 2048>(a02, ar0);
-        lds_read16_issue<3 * 2048>(a03, ar0);
+        lds_read16_issue<0 * 2048, PARTIALS>(a00, ar0);
+        lds_read16_issue<1 * 2048, PARTIALS>(a01, ar0);
+        lds_read16_issue<2 * 2048, PARTIALS>(a02, ar0);
+        lds_read16_issue<3 * 2048, PARTIALS>(a03, ar0);
         v4i b[2][4];
 #pragma unroll
         for (int h = 0; h < 2; h++)
@@ -647,25 +668,31 @@ __global__ __launch_bounds__(512, 2) void fc_gemm_pp_kernel(const uint8_t* __res
 #define LLMOPS_MMA4(T, H, A)                                                                              \
     _Pragma("unroll") for (int c = 0; c < 4; c++)                                                         \
         acc[T][c] = __builtin_amdgcn_mfma_i32_16x16x64_i8(A, b[H][c], (H) == 0 ? zero4 : acc[T][c], 0, 0, 0)
-        lds_ready<3>(a00);
+        lds_ready<3, PARTIALS>(a00);
         LLMOPS_MMA4(0, 0, a00);
-        lds_read16_issue<0 * 2048>(a10, ar1);
-        lds_ready<3>(a01);
+        lds_read16_issue<0 * 2048, PARTIALS>(a10, ar1);
+        if (more) LLMOPS_COPY_A(kb + 1, buf ^ 1, 0);
+        lds_ready<3, PARTIALS>(a01);
         LLMOPS_MMA4(1, 0, a01);
-        lds_read16_issue<1 * 2048>(a11, ar1);
-        lds_ready<3>(a02);
+        lds_read16_issue<1 * 2048, PARTIALS>(a11, ar1);
+        if (more) LLMOPS_COPY_A(kb + 1, buf ^ 1, 1);
+        lds_ready<3, PARTIALS>(a02);
         LLMOPS_MMA4(2, 0, a02);
-        lds_read16_issue<2 * 2048>(a12, ar1);
-        lds_ready<3>(a03);
+        lds_read16_issue<2 * 2048, PARTIALS>(a12, ar1);
+        if (more) LLMOPS_COPY_A(kb + 1, buf ^ 1, 2);
+        lds_ready<3, PARTIALS>(a03);
         LLMOPS_MMA4(3, 0, a03);
-        lds_read16_issue<3 * 2048>(a13, ar1);
-        lds_ready<3>(a10);
+        lds_read16_issue<3 * 2048, PARTIALS>(a13, ar1);
+        if (more) LLMOPS_COPY_A(kb + 1, buf ^ 1, 3);
+        lds_ready<3, PARTIALS>(a10);
         LLMOPS_MMA4(0, 1, a10);
-        lds_ready<2>(a11);
+        if (more) LLMOPS_COPY_X(kb + 1, buf ^ 1);
+        lds_ready<2, PARTIALS>(a11);
         LLMOPS_MMA4(1, 1, a11);
-        lds_ready<1>(a12);
+        if (more) LLMOPS_FETCH_B(kb + 1);
+        lds_ready<1, PARTIALS>(a12);
         LLMOPS_MMA4(2, 1, a12);
-        lds_ready<0>(a13);
+        lds_ready<0, PARTIALS>(a13);
         LLMOPS_MMA4(3, 1, a13);
 #undef LLMOPS_MMA4
         const float d[4] = {d4.x, d4.y, d4.z, d4.w};
@@ -688,6 +715,10 @@ __global__ __launch_bounds__(512, 2) void fc_gemm_pp_kernel(const uint8_t* __res
                 for (int c = 0; c < 4; c++) mk[c] = 0.0f;
             }
         }
+        asm volatile("" : "+v"(acc[0][0]), "+v"(acc[0][1]), "+v"(acc[0][2]), "+v"(acc[0][3]), "+v"(acc[1][0]),
+                          "+v"(acc[1][1]), "+v"(acc[1][2]), "+v"(acc[1][3]), "+v"(acc[2][0]), "+v"(acc[2][1]),
+                          "+v"(acc[2][2]), "+v"(acc[2][3]), "+v"(acc[3][0]), "+v"(acc[3][1]), "+v"(acc[3][2]),
+                          "+v"(acc[3][3]));  // likewise: the MFMAs stay in the matrix-core phase
         __syncthreads();
 
         // ---- vector phase: fold the int32 tiles into the fp32 accumulators ----
@@ -719,12 +750,19 @@ __global__ __launch_bounds__(512, 2) void fc_gemm_pp_kernel(const uint8_t* __res
                     for (int c = 0; c < 4; c++) f[t][c][v] = fmaf(d[c] * dxv[v], (float)acc[t][c][v], f[t][c][v]);
             }
         }
+        // the fold is register arithmetic, which the compiler may move across the barrier into the other
+        // phase; naming the accumulators as operands of an (empty) asm statement keeps it on this side
+        asm volatile("" : "+v"(f[0][0]), "+v"(f[0][1]), "+v"(f[0][2]), "+v"(f[0][3]), "+v"(f[1][0]), "+v"(f[1][1]),
+                          "+v"(f[1][2]), "+v"(f[1][3]), "+v"(f[2][0]), "+v"(f[2][1]), "+v"(f[2][2]), "+v"(f[2][3]),
+                          "+v"(f[3][0]), "+v"(f[3][1]), "+v"(f[3][2]), "+v"(f[3][3]));
         if (kb + 1 < kb1) LLMOPS_STASH_B(buf ^ 1);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's copies for the next k-group have landed
         __syncthreads();
     }
     if (grp == 0) __syncthreads();  // pairs with group 1's last barrier
 #undef LLMOPS_COPY
+#undef LLMOPS_COPY_A
+#undef LLMOPS_COPY_X
 #undef LLMOPS_FETCH_B
 #undef LLMOPS_STASH_B
 
