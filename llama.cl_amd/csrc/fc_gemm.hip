@@ -836,7 +836,7 @@ struct GemmPlan {
     bool lds;
 };
 
-static int g_gemm_pp_min_rows = 512;
+static int g_gemm_pp_min_rows = 256;
 static int g_gemm_rt = 0;  // 0 = choose per shape; -1 = also keep 9..32 rows on the tiled kernel
 bool gemm_rows_kernel_enabled() { return g_gemm_rt >= 0; }
 
@@ -857,38 +857,46 @@ static GemmPlan plan_gemm(int64_t rows, int64_t Ng, int64_t Kg, int G) {
         gemm_split((((Ng + 1) / 2 + 3) / 4) * ((rows + p.RT * 16 - 1) / (p.RT * 16)), 512, Kg, p);
         return p;
     }
-    // BM = 32*RT rows per workgroup.  Bigger tiles reuse the unpacked weights over more rows but need
-    // more registers: RT = 4 runs two workgroups per CU, RT = 2 three, RT = 1 four.  Measured rate per
-    // row at full occupancy (M = 2048): 1.0 : 0.98 : 0.77.  What decides between them at smaller M is
-    // how evenly the tiles fill the machine, so the plan takes the RT with the least estimated time:
-    // rounds of resident workgroups x (rows per tile x workgroups sharing a CU / efficiency) x share of
-    // K per split.
-    // (its lanes address the tensors with 32-bit byte offsets)
+    // Candidates: the 256-row kernel with two wave groups (one workgroup per CU) and the four-wave
+    // kernel with 128, 64 or 32 rows per workgroup (two, three, four workgroups per CU: bigger tiles
+    // reuse the unpacked weights over more rows but need more registers).  Measured rate per row at
+    // full occupancy (M = 2048): 1.17 : 1.0 : 0.98 : 0.77.  What decides between them at smaller M is
+    // how evenly the tiles fill the machine, so the plan takes the candidate and split-K factor with
+    // the least estimated time: rounds of resident workgroups x (rows per CU per round / efficiency)
+    // x share of K per split.  Split factors tried: the largest that still runs in one round and the
+    // smallest that fills the machine (a second round of half-length workgroups costs what one round
+    // of full-length ones does, plus the reduction of the partial sums).
+    // (the 256-row kernel's lanes address the tensors with 32-bit byte offsets)
     const bool small = rows * Kg * 128 < ((int64_t)1 << 31) && Ng * Kg * 2176 < ((int64_t)1 << 31);
-    if (small && (g_gemm_rt == 8 || (g_gemm_rt == 0 && rows >= g_gemm_pp_min_rows))) {
-        // two groups of waves in alternating phases, 256 x 128 tiles, one workgroup per CU
-        p.RT = 8;
-        gemm_split(((Ng + 3) / 4) * ((rows + 255) / 256), 256, Kg, p);
-        return p;
-    }
-    static const int kRT[3] = {4, 2, 1};
-    static const int kWgPerCu[3] = {2, 3, 4};
-    static const double kEff[3] = {1.0, 0.98, 0.77};
+    static const int kRT[4] = {8, 4, 2, 1};
+    static const int kRows[4] = {256, 128, 64, 32};
+    static const int kWgPerCu[4] = {1, 2, 3, 4};
+    static const double kEff[4] = {1.17, 1.0, 0.98, 0.77};
     double best = 0.0;
-    for (int i = 0; i < 3; i++) {
+    for (int i = 0; i < 4; i++) {
         if (g_gemm_rt > 0 && kRT[i] != g_gemm_rt) continue;
-        GemmPlan q = p;
-        q.RT = kRT[i];
-        const int64_t bm = 32 * q.RT, slots = 256 * kWgPerCu[i];
+        if (kRT[i] == 8 && (!small || (g_gemm_rt != 8 && rows < g_gemm_pp_min_rows))) continue;
+        const int64_t bm = kRows[i], slots = 256 * kWgPerCu[i];
         const int64_t tiles = ((Ng + 3) / 4) * ((rows + bm - 1) / bm);
-        gemm_split(tiles, slots, Kg, q);
-        const int64_t rounds = (tiles * q.S + slots - 1) / slots;
-        double cost = (double)rounds * (double)(bm * kWgPerCu[i]) / kEff[i] * (double)q.kb_per_split / (double)Kg;
-        if (q.S > 1) cost *= 1.1;  // the partial sums take a second launch
-        if (best == 0.0 || cost < best) {
-            best = cost;
-            p = q;
+        const int64_t s_floor = slots / tiles, s_ceil = (slots + tiles - 1) / tiles;
+        for (int64_t s_try : {s_floor, s_ceil}) {
+            GemmPlan q = p;
+            q.RT = kRT[i];
+            int64_t S = s_try < 1 ? 1 : (s_try > Kg ? Kg : s_try);
+            q.kb_per_split = (int)((Kg + S - 1) / S);
+            q.S = (int)((Kg + q.kb_per_split - 1) / q.kb_per_split);
+            const int64_t rounds = (tiles * q.S + slots - 1) / slots;
+            double cost = (double)rounds * (double)(bm * kWgPerCu[i]) / kEff[i] * (double)q.kb_per_split / (double)Kg;
+            if (q.S > 1) cost *= 1.1;  // the partial sums take a second launch
+            if (best == 0.0 || cost < best) {
+                best = cost;
+                p = q;
+            }
         }
+    }
+    if (best == 0.0) {  // a forced candidate that cannot run here: fall back to the 128-row kernel
+        p.RT = 4;
+        gemm_split(((Ng + 3) / 4) * ((rows + 127) / 128), 512, Kg, p);
     }
     return p;
 }
