@@ -316,6 +316,25 @@ def test_fc_decode_gate_up_input(ops, orc, G, rows, N, K):
         ops.fc_Q4A_decode(dev(gu), dev(pw), N, norm=(torch.ones(K, device="cuda"), 1e-5), glu_in=True)
 
 
+@pytest.mark.parametrize("rows", [17, 48, 100, 128, 129, 200, 256])
+@pytest.mark.parametrize("N,K", [(2070, 1024), (4096, 640), (2048, 2816)])
+def test_fc_prefill_mid_rows_vs_oracle(ops, orc, rows, N, K):
+    """17..256 rows at group 128 as the planner runs them (tiling and split-K factor chosen per shape):
+    ragged rows, N not a multiple of 32, k-group counts 8, 5 and 22 (splits of unequal length): output
+    and residual epilogue against the oracle, the closed-form construction exactly."""
+    rng = np.random.default_rng(rows + N)
+    x = rng.standard_normal((1, rows, K)).astype(np.float32)
+    w = (rng.standard_normal((N, K)) * 0.02).astype(np.float32)
+    res = rng.standard_normal((1, rows, N)).astype(np.float32)
+    pw = orc.quant_w(w, 128)
+    want = orc.fc(x, pw, N)
+    assert max_rel_err(host(ops.fc_Q4A(dev(x), dev(pw), N)), want) <= 1e-5
+    assert max_rel_err(host(ops.fc_Q4A(dev(x), dev(pw), N, residual=dev(res))), want + res) <= 1e-5
+    xe, we = oracle.closed_form_fc_inputs(rows, N, K, seed=rows)
+    ye = host(ops.fc_Q4A(dev(xe.reshape(1, rows, K)), ops.offline_FC_quant_Q4A(dev(we), 128), N))
+    assert np.array_equal(ye, (xe.astype(np.float64) @ we.astype(np.float64).T).astype(np.float32).reshape(1, rows, N))
+
+
 @pytest.mark.parametrize("tiling", [1, 2, 4, 8])
 @pytest.mark.parametrize("rows,N,K", [(70, 2070, 1024), (300, 2070, 1024), (515, 352, 4096), (1024, 4096, 512)])
 def test_fc_prefill_every_tiling_vs_oracle(ops, orc, tiling, rows, N, K):
