@@ -70,8 +70,8 @@ def main():
     if args.calib:
         return calib()
     if args.gpus != 1:
-        print("bench.py: this build runs on ONE GPU (the path is data-parallel per GPU; multi-GPU sharding is design "
-              "only, see DESIGN.md). Re-run with --gpus 1.", file=sys.stderr)
+        print("bench.py: this build runs on ONE GPU (the path is data-parallel per GPU; nothing here uses a second "
+              "one). Re-run with --gpus 1.", file=sys.stderr)
         sys.exit(2)
 
     import torch
