@@ -13,6 +13,7 @@ This is the caller of the hot path, kept as thin as the reference's: every arith
 A decode step (one token, batch 1) has fixed shapes and no host-side decisions, so it can be
 captured once as a HIP graph and replayed (``capture_decode``).
 """
+import numpy as np
 import torch
 
 import llmops
@@ -72,6 +73,69 @@ class LlamaDecoder:
         rd = cfg["head_size"]
         inv_freq = 1.0 / (cfg["rope_base"] ** (torch.arange(0, rd, 2).float() / rd))  # chatllama/main.py:294-296
         self.inv_freq = inv_freq.to(self.device)
+
+    @classmethod
+    def from_reference(cls, path, device="cuda", plan="fused"):
+        """Builds the decoder from a model file written by the reference's ``Model.save``
+        (chatllama/main.py:305-308).  The file is read without executing it (``llmops.ref_pickle``); its
+        packed Q4_1 tensors have the layout this library uses and go to the device as they are."""
+        from llmops import ref_pickle
+
+        t = ref_pickle.model_tensors(ref_pickle.load(path))
+        self = cls.__new__(cls)
+        self.device = torch.device(device)
+        self.plan = plan
+
+        def dev(a):
+            return torch.from_numpy(a).to(self.device)
+
+        def fc(*entries):
+            for e in entries:
+                if e["bias"] is not None:
+                    raise ValueError("FC with bias: not part of the Llama family the reference loads")
+            packed = [dev(e["weight"]) for e in entries]
+            return llmop_fc_q4a(packed=torch.cat(packed, dim=0) if len(packed) > 1 else packed[0],
+                                N=sum(e["N"] for e in entries))
+
+        def norm(e):
+            return llmop_rmsnorm(dev(e["weight"]), e["eps"])
+
+        ref_cfg = t["configs"]
+        first = t["layers"][0]
+        H = ref_cfg["hidden_size"]
+        F = first["mlp.gate_proj"]["N"]
+        self.configs = dict(layer_num=len(t["layers"]), head_num=ref_cfg["head_num"], head_size=ref_cfg["head_size"],
+                            hidden_size=H, intermediate_size=F, vocab_size=t["lm_head"]["N"],
+                            rms_norm_eps=ref_cfg["rms_norm_eps"], rope_base=10000.0)
+        self.layers = []
+        self.stacked_gate_up = F % 32 == 0
+        for e in t["layers"]:
+            layer = {"input_layernorm": norm(e["input_layernorm"]),
+                     "post_attention_layernorm": norm(e["post_attention_layernorm"]),
+                     "o_proj": fc(e["self_attn.o_proj"]), "down_proj": fc(e["mlp.down_proj"])}
+            if plan == "fused":
+                # q|k|v stacked along N needs every part to be whole strips (hidden sizes are)
+                if H % 32 != 0:
+                    raise ValueError("fused plan: hidden_size must be a multiple of 32")
+                layer["qkv_proj"] = fc(e["self_attn.q_proj"], e["self_attn.k_proj"], e["self_attn.v_proj"])
+                gate, up = dev(e["mlp.gate_proj"]["weight"]), dev(e["mlp.up_proj"]["weight"])
+                gu = torch.cat((gate, up), dim=0) if self.stacked_gate_up else llmops.interleave_gate_up(gate, up)
+                layer["gate_up_proj"] = llmop_fc_q4a(packed=gu, N=2 * F)
+            else:
+                layer["q_proj"], layer["k_proj"], layer["v_proj"] = (fc(e["self_attn.q_proj"]), fc(e["self_attn.k_proj"]),
+                                                                     fc(e["self_attn.v_proj"]))
+                layer["gate_proj"], layer["up_proj"] = fc(e["mlp.gate_proj"]), fc(e["mlp.up_proj"])
+            self.layers.append(layer)
+        self.norm = norm(t["norm"])
+        self.lm_head = fc(t["lm_head"])
+        if t["embed"]["scales"] is None:
+            raise ValueError("the reference stores the embedding as int8 rows with per-row scales (embedding_q8c)")
+        self.embed_tokens = llmop_embedding_q8c(packed=(dev(t["embed"]["weight"]), dev(t["embed"]["scales"])))
+        rd = ref_cfg.get("rotary_dims", ref_cfg["head_size"])
+        inv_freq = t["inv_freq"] if t["inv_freq"] is not None else \
+            (1.0 / (10000.0 ** (torch.arange(0, rd, 2).float() / rd))).numpy()
+        self.inv_freq = dev(np.ascontiguousarray(inv_freq, dtype=np.float32))
+        return self
 
     def fc_weight_size(self):
         n = 0

@@ -113,8 +113,9 @@ class llmop_rmsnorm:
 class llmop_embedding_q8c:
     """chatllama/main.py:206-219"""
 
-    def __init__(self, weight):
-        self.weight, self.scales = llmops.embedding_q8c_quant_w(weight.detach())
+    def __init__(self, weight=None, packed=None):
+        # packed = (int8 rows, fp32 per-row scales) as embedding_q8c_quant_w returns them
+        self.weight, self.scales = packed if packed is not None else llmops.embedding_q8c_quant_w(weight.detach())
 
     def __call__(self, input_ids):
         output = llmops.empty(*input_ids.shape, self.weight.shape[1], device=input_ids.device)

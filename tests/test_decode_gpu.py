@@ -163,3 +163,51 @@ def test_decode_graph_replay_matches_eager():
         torch.cuda.synchronize()
         assert torch.equal(dg.logits, eager), rep
         _ = model.forward(ids, kv.cache, slots, 17)  # eager work between replays
+
+
+@pytest.mark.parametrize("plan", ["reference", "fused"])
+def test_decoder_from_reference_format_file(tmp_path, plan):
+    """A model written in the reference's save format (packed tensors as they are, one per projection) is
+    read back without re-quantizing: same logits as the decoder whose tensors were written, bit for bit
+    with the reference launch plan, and with the fused plan (q|k|v and gate|up stacked by the loader)
+    equal to a fused decoder built from the same tensors."""
+    import ref_model_file
+    from llmops.decode import LlamaDecoder
+    from llmops.opset import KVCache
+    src = LlamaDecoder(CFG, group_k=128, seed=9, plan="reference")
+    h = lambda t: t.cpu().numpy()
+    layers = []
+    for ops in src.layers:
+        layers.append({
+            "input_layernorm": (h(ops["input_layernorm"].weight), ops["input_layernorm"].eps),
+            "post_attention_layernorm": (h(ops["post_attention_layernorm"].weight), ops["post_attention_layernorm"].eps),
+            "self_attn.q_proj": (h(ops["q_proj"].weight), ops["q_proj"].N), "self_attn.k_proj": (h(ops["k_proj"].weight), ops["k_proj"].N),
+            "self_attn.v_proj": (h(ops["v_proj"].weight), ops["v_proj"].N), "self_attn.o_proj": (h(ops["o_proj"].weight), ops["o_proj"].N),
+            "mlp.gate_proj": (h(ops["gate_proj"].weight), ops["gate_proj"].N), "mlp.up_proj": (h(ops["up_proj"].weight), ops["up_proj"].N),
+            "mlp.down_proj": (h(ops["down_proj"].weight), ops["down_proj"].N),
+        })
+    configs = {"layer_num": CFG["layer_num"], "head_num": CFG["head_num"], "head_size": CFG["head_size"],
+               "hidden_size": CFG["hidden_size"], "max_position_embeddings": 2048, "rotary_dims": CFG["head_size"],
+               "rms_norm_eps": CFG["rms_norm_eps"]}
+    path = tmp_path / "saved_model.pkl"
+    ref_model_file.write(path, configs=configs, embed=(h(src.embed_tokens.weight), h(src.embed_tokens.scales)), layers=layers,
+                         norm=(h(src.norm.weight), src.norm.eps), lm_head=(h(src.lm_head.weight), src.lm_head.N),
+                         inv_freq=h(src.inv_freq), marker_path=str(tmp_path / "executed"))
+    model = LlamaDecoder.from_reference(str(path), plan=plan)
+    assert not (tmp_path / "executed").exists()
+    assert model.configs["intermediate_size"] == CFG["intermediate_size"] and model.configs["vocab_size"] == CFG["vocab_size"]
+    rng = np.random.default_rng(3)
+    ids = torch.from_numpy(rng.integers(0, CFG["vocab_size"], (1, 5)).astype(np.int64)).cuda()
+
+    def run(m):
+        kv = KVCache(CFG, 1, 32)
+        assert kv.prepare(5, 1, 0)
+        return m.forward(ids, kv.cache, kv.slots, kv.position_id).clone()
+
+    got, want = run(model), run(src)
+    if plan == "reference":
+        assert torch.equal(got, want)
+    else:
+        assert max_rel_err(got.cpu().numpy(), want.cpu().numpy()) <= 5e-2  # fused vs unfused: re-quantized activations drift
+        direct = LlamaDecoder(CFG, group_k=128, seed=9, plan="fused")       # same seed -> same tensors, stacked directly
+        assert torch.equal(got, run(direct))
