@@ -19,7 +19,7 @@ int launch_gemv_partials(const uint8_t* w, const int8_t* xq, int32_t* acc, int64
                          hipStream_t st);
 size_t gemm_workspace_bytes(int64_t rows, int64_t Ng, int64_t Kg, int G);
 int launch_gemm(const uint8_t* w, const int8_t* xq, const float* xd, const float* gs, const float2* xsT, float* y,
-                float* part, int64_t rows, int64_t Ng, int64_t Kg, int G, int64_t N, hipStream_t st);
+                float* part, int64_t rows, int64_t Ng, int64_t Kg, int G, int64_t N, const float* residual, hipStream_t st);
 int launch_gemm_partials(const uint8_t* w, const int8_t* xq, int32_t* acc, int64_t rows, int64_t Ng, int64_t Kg, int G,
                          bool two_groups, hipStream_t st);
 int launch_fc_rows(const uint8_t* w, const int8_t* xq, const float2* xsT, float* y, int64_t rows, int64_t Ng, int64_t Kg,
@@ -93,9 +93,7 @@ static int fc_impl(const float* x, int64_t rows, int64_t K, const int8_t* weiq, 
     // wave, 17..32 rows, the streaming kernel runs out of registers and loses, 32 vs 20 us)
     if (group_k == 128 && rows <= 16 && Ng >= 64 && gemm_rows_kernel_enabled())
         return launch_fc_rows(w, xq, xst, y, rows, Ng, Kg, N, residual, st);
-    rc = launch_gemm(w, xq, xd, gs, xst, y, part, rows, Ng, Kg, group_k, N, st);
-    if (rc || residual == nullptr) return rc;
-    return launch_add(y, residual, rows * N, st);
+    return launch_gemm(w, xq, xd, gs, xst, y, part, rows, Ng, Kg, group_k, N, residual, st);
 }
 
 extern "C" int llmops_fc_Q4A(const float* x, int64_t rows, int64_t K, const int8_t* weiq, int64_t Ng, int64_t Kg,
@@ -160,7 +158,7 @@ extern "C" int llmops_fc_Q4A_prequantized(const int8_t* xq, const float* xd, con
     hipStream_t st = as_stream(stream);
     if (rows <= kMaxGemvRows)
         return launch_gemv(w, xq, xd, gsum, y, part, reinterpret_cast<unsigned*>(ws), rows, Ng, Kg, group_k, N, st);
-    return launch_gemm(w, xq, xd, gsum, nullptr, y, part, rows, Ng, Kg, group_k, N, st);
+    return launch_gemm(w, xq, xd, gsum, nullptr, y, part, rows, Ng, Kg, group_k, N, nullptr, st);
 }
 
 extern "C" int llmops_fc_Q4A_partials(const int8_t* xq, int64_t rows, const int8_t* weiq, int64_t Ng, int64_t Kg,

@@ -189,7 +189,8 @@ __global__ __launch_bounds__(256, (RT == 4 ? 2 : (RT == 2 ? 3 : 4))) void fc_gem
                                                            const float* __restrict__ xd, const float* __restrict__ gs,
                                                            const float2* __restrict__ xsT, float* __restrict__ out,
                                                            int32_t* __restrict__ out_i, int Ng, int Kg, int64_t ldo,
-                                                           int64_t N, int rows, int kb_per_split, int64_t split_stride) {
+                                                           int64_t N, int rows, int kb_per_split, int64_t split_stride,
+                                                           const float* __restrict__ residual) {
     constexpr int BM = RT * 32;
     constexpr int A_CHUNKS = BM * 8;                     // 16-byte chunks of the A tile
     constexpr int A_PER_THREAD = A_CHUNKS / 256;         // RT
@@ -394,12 +395,19 @@ __global__ __launch_bounds__(256, (RT == 4 ? 2 : (RT == 2 ? 3 : 4))) void fc_gem
             const int row = row0 + wr * (BM / 2) + t * 16 + g * 4 + v;
             if (row >= rows) continue;
             float* dst = o + (int64_t)row * ldo + n0;
+            // residual != nullptr only without split-K: then o is the result itself, row stride ldo
+            const float* res = residual ? residual + (int64_t)row * ldo + n0 : nullptr;
             if (n0 + 3 < N && (ldo & 3) == 0) {
-                *reinterpret_cast<float4*>(dst) = make_float4(f[t][0][v], f[t][1][v], f[t][2][v], f[t][3][v]);
+                float4 val = make_float4(f[t][0][v], f[t][1][v], f[t][2][v], f[t][3][v]);
+                if (res) {
+                    const float4 r4 = *reinterpret_cast<const float4*>(res);
+                    val.x += r4.x, val.y += r4.y, val.z += r4.z, val.w += r4.w;
+                }
+                *reinterpret_cast<float4*>(dst) = val;
             } else {
 #pragma unroll
                 for (int c = 0; c < 4; c++)
-                    if (n0 + c < N) dst[c] = f[t][c][v];
+                    if (n0 + c < N) dst[c] = res ? f[t][c][v] + res[c] : f[t][c][v];
             }
         }
 }
@@ -488,7 +496,8 @@ __global__ __launch_bounds__(512, 2) void fc_gemm_pp_kernel(const uint8_t* __res
                                                              const float* __restrict__ xd, const float* __restrict__ gs,
                                                              const float2* __restrict__ xsT, float* __restrict__ out,
                                                              int32_t* __restrict__ out_i, int Ng, int Kg, int64_t ldo,
-                                                             int64_t N, int rows, int kb_per_split, int64_t split_stride) {
+                                                             int64_t N, int rows, int kb_per_split, int64_t split_stride,
+                                                             const float* __restrict__ residual) {
     constexpr int RT = 4, BM = 256, GM = 128;
     extern __shared__ __align__(16) uint8_t smem_raw[];
     GemmPPSmem& sm = *reinterpret_cast<GemmPPSmem*>(smem_raw);
@@ -778,25 +787,49 @@ __global__ __launch_bounds__(512, 2) void fc_gemm_pp_kernel(const uint8_t* __res
             const int row = row0 + wr * 64 + t * 16 + g * 4 + v;
             if (row >= rows) continue;
             float* dst = o + (int64_t)row * ldo + n0;
+            // residual != nullptr only without split-K: then o is the result itself, row stride ldo
+            const float* res = residual ? residual + (int64_t)row * ldo + n0 : nullptr;
             if (n0 + 3 < N && (ldo & 3) == 0) {
-                *reinterpret_cast<float4*>(dst) = make_float4(f[t][0][v], f[t][1][v], f[t][2][v], f[t][3][v]);
+                float4 val = make_float4(f[t][0][v], f[t][1][v], f[t][2][v], f[t][3][v]);
+                if (res) {
+                    const float4 r4 = *reinterpret_cast<const float4*>(res);
+                    val.x += r4.x, val.y += r4.y, val.z += r4.z, val.w += r4.w;
+                }
+                *reinterpret_cast<float4*>(dst) = val;
             } else {
 #pragma unroll
                 for (int c = 0; c < 4; c++)
-                    if (n0 + c < N) dst[c] = f[t][c][v];
+                    if (n0 + c < N) dst[c] = res ? f[t][c][v] + res[c] : f[t][c][v];
             }
         }
 }
 
-// y[row][n] = sum over splits (index order) of part[s][row][n]
+// y[row][n] = sum over splits (index order) of part[s][row][n] (+ residual[row][n]); four columns per
+// thread (the partial sums' row stride ldp is a multiple of 32 floats, so their 16-byte loads are aligned)
 __global__ void gemm_reduce_kernel(const float* __restrict__ part, float* __restrict__ y, int64_t rows, int64_t N,
-                                   int64_t ldp, int64_t split_stride, int S) {
+                                   int64_t ldp, int64_t split_stride, int S, const float* __restrict__ residual) {
+    const int64_t nq = (N + 3) / 4;
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= rows * N) return;
-    const int64_t r = i / N, n = i % N;
-    float a = 0.0f;
-    for (int s = 0; s < S; s++) a += part[(int64_t)s * split_stride + r * ldp + n];
-    y[i] = a;
+    if (i >= rows * nq) return;
+    const int64_t r = i / nq, n = (i % nq) * 4;
+    float4 a = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int s = 0; s < S; s++) {
+        const float4 v = *reinterpret_cast<const float4*>(part + (int64_t)s * split_stride + r * ldp + n);
+        a.x += v.x, a.y += v.y, a.z += v.z, a.w += v.w;
+    }
+    float* dst = y + r * N + n;
+    const float* res = residual ? residual + r * N + n : nullptr;
+    if (n + 3 < N && (N & 3) == 0) {
+        if (res) {
+            const float4 r4 = *reinterpret_cast<const float4*>(res);
+            a.x += r4.x, a.y += r4.y, a.z += r4.z, a.w += r4.w;
+        }
+        *reinterpret_cast<float4*>(dst) = a;
+    } else {
+        const float av[4] = {a.x, a.y, a.z, a.w};
+        for (int c = 0; c < 4; c++)
+            if (n + c < N) dst[c] = res ? av[c] + res[c] : av[c];
+    }
 }
 
 // Integer core only, through the same mma_group: acc[row][n][kb]
@@ -918,7 +951,7 @@ static void launch_gemm_t(const uint8_t* w, const int8_t* xq, const float* xd, c
 template <int RT>
 static int launch_gemm_lds_t(const uint8_t* w, const int8_t* xq, const float* xd, const float* gs, const float2* xsT,
                              float* out, int64_t Ng, int64_t Kg, int64_t ldo, int64_t N, int64_t rows, const GemmPlan& p,
-                             int64_t split_stride, hipStream_t st) {
+                             int64_t split_stride, const float* residual, hipStream_t st) {
     static bool configured = false;  // opt in to more than 64 KiB of dynamic LDS once per kernel
     if (!configured) {
         LLMOPS_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&fc_gemm_lds_kernel<RT, false>),
@@ -928,13 +961,14 @@ static int launch_gemm_lds_t(const uint8_t* w, const int8_t* xq, const float* xd
     const int64_t tiles = ((Ng + 3) / 4) * ((rows + RT * 32 - 1) / (RT * 32));
     dim3 grid((unsigned)(8 * ((tiles + 7) / 8)), 1, (unsigned)p.S);  // one run of tiles per XCD
     fc_gemm_lds_kernel<RT, false><<<grid, 256, sizeof(GemmSmem<RT>), st>>>(w, xq, xd, gs, xsT, out, nullptr, (int)Ng, (int)Kg,
-                                                                          ldo, N, (int)rows, p.kb_per_split, split_stride);
+                                                                          ldo, N, (int)rows, p.kb_per_split, split_stride,
+                                                                          residual);
     return LLMOPS_OK;
 }
 
 static int launch_gemm_pp(const uint8_t* w, const int8_t* xq, const float* xd, const float* gs, const float2* xsT, float* out,
                           int64_t Ng, int64_t Kg, int64_t ldo, int64_t N, int64_t rows, const GemmPlan& p,
-                          int64_t split_stride, hipStream_t st) {
+                          int64_t split_stride, const float* residual, hipStream_t st) {
     static bool configured = false;
     if (!configured) {
         LLMOPS_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&fc_gemm_pp_kernel<false>),
@@ -944,13 +978,19 @@ static int launch_gemm_pp(const uint8_t* w, const int8_t* xq, const float* xd, c
     const int64_t tiles = ((Ng + 3) / 4) * ((rows + 255) / 256);
     dim3 grid((unsigned)(8 * ((tiles + 7) / 8)), 1, (unsigned)p.S);
     fc_gemm_pp_kernel<false><<<grid, 512, sizeof(GemmPPSmem), st>>>(w, xq, xd, gs, xsT, out, nullptr, (int)Ng, (int)Kg, ldo, N,
-                                                                   (int)rows, p.kb_per_split, split_stride);
+                                                                   (int)rows, p.kb_per_split, split_stride, residual);
     return LLMOPS_OK;
 }
 
+int launch_add(float* a, const float* b, int64_t total, hipStream_t st);  // misc.hip
+
+// y = product (+ residual, fp32 [rows, N], may be y itself)
 int launch_gemm(const uint8_t* w, const int8_t* xq, const float* xd, const float* gs, const float2* xsT, float* y,
-                float* part, int64_t rows, int64_t Ng, int64_t Kg, int G, int64_t N, hipStream_t st) {
+                float* part, int64_t rows, int64_t Ng, int64_t Kg, int G, int64_t N, const float* residual, hipStream_t st) {
     const GemmPlan p = plan_gemm(rows, Ng, Kg, G);
+    // the residual is added where the result is written: in the kernel's stores without split-K, in
+    // the reduction of the partial sums with it
+    const float* kres = p.S > 1 ? nullptr : residual;
     const int64_t Np = Ng * kGroupN;
     float* out = p.S > 1 ? part : y;
     const int64_t ldo = p.S > 1 ? Np : N;
@@ -958,10 +998,10 @@ int launch_gemm(const uint8_t* w, const int8_t* xq, const float* xd, const float
     const int64_t ss = rows * Np;
     if (p.lds) {
         int rc;
-        if (p.RT == 8) rc = launch_gemm_pp(w, xq, xd, gs, xsT, out, Ng, Kg, ldo, Nw, rows, p, ss, st);
-        else if (p.RT == 4) rc = launch_gemm_lds_t<4>(w, xq, xd, gs, xsT, out, Ng, Kg, ldo, Nw, rows, p, ss, st);
-        else if (p.RT == 2) rc = launch_gemm_lds_t<2>(w, xq, xd, gs, xsT, out, Ng, Kg, ldo, Nw, rows, p, ss, st);
-        else rc = launch_gemm_lds_t<1>(w, xq, xd, gs, xsT, out, Ng, Kg, ldo, Nw, rows, p, ss, st);
+        if (p.RT == 8) rc = launch_gemm_pp(w, xq, xd, gs, xsT, out, Ng, Kg, ldo, Nw, rows, p, ss, kres, st);
+        else if (p.RT == 4) rc = launch_gemm_lds_t<4>(w, xq, xd, gs, xsT, out, Ng, Kg, ldo, Nw, rows, p, ss, kres, st);
+        else if (p.RT == 2) rc = launch_gemm_lds_t<2>(w, xq, xd, gs, xsT, out, Ng, Kg, ldo, Nw, rows, p, ss, kres, st);
+        else rc = launch_gemm_lds_t<1>(w, xq, xd, gs, xsT, out, Ng, Kg, ldo, Nw, rows, p, ss, kres, st);
         if (rc) return rc;
     } else {
         if (p.RT == 4) launch_gemm_t<32, 4>(w, xq, xd, gs, out, Ng, Kg, ldo, Nw, rows, p, ss, st);
@@ -970,9 +1010,11 @@ int launch_gemm(const uint8_t* w, const int8_t* xq, const float* xd, const float
     }
     LLMOPS_LAUNCH_CHECK();
     if (p.S > 1) {
-        const int64_t total = rows * N;
-        gemm_reduce_kernel<<<(unsigned)((total + 255) / 256), 256, 0, st>>>(part, y, rows, N, Np, ss, p.S);
+        const int64_t total = rows * ((N + 3) / 4);
+        gemm_reduce_kernel<<<(unsigned)((total + 255) / 256), 256, 0, st>>>(part, y, rows, N, Np, ss, p.S, residual);
         LLMOPS_LAUNCH_CHECK();
+    } else if (residual != nullptr && !p.lds) {
+        return launch_add(y, residual, rows * N, st);  // the group-32 kernel has no residual in its stores
     }
     return LLMOPS_OK;
 }
@@ -991,7 +1033,7 @@ int launch_gemm_partials(const uint8_t* w, const int8_t* xq, int32_t* acc, int64
         const int64_t tiles = ((Ng + 3) / 4) * ((rows + 255) / 256);
         dim3 grid((unsigned)(8 * ((tiles + 7) / 8)), 1, 1);
         fc_gemm_pp_kernel<true><<<grid, 512, sizeof(GemmPPSmem), st>>>(w, xq, nullptr, nullptr, nullptr, nullptr, acc, (int)Ng,
-                                                                      (int)Kg, 0, 0, (int)rows, (int)Kg, 0);
+                                                                      (int)Kg, 0, 0, (int)rows, (int)Kg, 0, nullptr);
     } else if (G == 128) {  // the production LDS-tiled loop, writing its int32 tiles instead of folding them
         static bool configured = false;
         if (!configured) {
@@ -1002,7 +1044,7 @@ int launch_gemm_partials(const uint8_t* w, const int8_t* xq, int32_t* acc, int64
         const int64_t tiles = ((Ng + 3) / 4) * ((rows + 63) / 64);
         dim3 grid((unsigned)(8 * ((tiles + 7) / 8)), 1, 1);
         fc_gemm_lds_kernel<2, true><<<grid, 256, sizeof(GemmSmem<2>), st>>>(w, xq, nullptr, nullptr, nullptr, nullptr, acc,
-                                                                          (int)Ng, (int)Kg, 0, 0, (int)rows, (int)Kg, 0);
+                                                                          (int)Ng, (int)Kg, 0, 0, (int)rows, (int)Kg, 0, nullptr);
     } else {
         dim3 grid((unsigned)(((Ng + 1) / 2 + 3) / 4), (unsigned)((rows + 15) / 16), (unsigned)Kg);
         fc_gemm_partials_kernel<32><<<grid, 256, 0, st>>>(w, xq, acc, (int)Ng, (int)Kg, (int)rows);
