@@ -24,7 +24,7 @@ __device__ __forceinline__ float dpp(float v) {
 __device__ __forceinline__ float lane_bcast(float v, int lane) {
     return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), lane));
 }
-constexpr int kQuadXor1 = 0xB1, kQuadXor2 = 0x4E, kRowHalfMirror = 0x141, kRowMirror = 0x140, kRowRor8 = 0x128;
+constexpr int kQuadXor1 = 0xB1, kQuadXor2 = 0x4E, kRowHalfMirror = 0x141, kRowMirror = 0x140, kRowRor8 = 0x128, kRowRor4 = 0x124;
 
 // max and sum over each row of 16 lanes, result in every lane of the row
 __device__ __forceinline__ void row16_max_sum(float& mx, float& sm) {
@@ -54,12 +54,14 @@ template <int G>
 __device__ __forceinline__ void load_step(Step<G>& st, const uint8_t* strip, int step, int kb_end, int lane) {
     const int quad = lane & 7, rs = lane >> 3;
     if (G == 128) {
+        // uniform block address + 32-bit lane offsets: the loads take the (scalar base, vector offset) form
         const uint8_t* blk = strip + (int64_t)step * block_bytes(128);
+        const uint32_t wo = (uint32_t)lane * 16u, so = (uint32_t)quad * 8u;
         st.valid = true;
-        st.w[0] = ldg16(blk + lane * 16);
-        st.w[Step<G>::kLoads - 1] = ldg16(blk + 1024 + lane * 16);
-        st.dh = ldg8(blk + 2048 + quad * 8);
-        st.mh = ldg8(blk + 2048 + 64 + quad * 8);
+        st.w[0] = ldg16(blk + wo);
+        st.w[Step<G>::kLoads - 1] = ldg16(blk + 1024 + wo);
+        st.dh = ldg8(blk + 2048 + so);
+        st.mh = ldg8(blk + 2048 + 64 + so);
     } else {
         const int kb = step * 2 + (rs >> 2);
         st.valid = kb < kb_end;
@@ -74,6 +76,27 @@ __device__ __forceinline__ void load_step(Step<G>& st, const uint8_t* strip, int
             st.mh = make_uint2(0, 0);
         }
     }
+}
+
+// Half-strip form of a group-128 step: the wave covers the block's 16 k8-rows x 16 of the strip's 32
+// columns with one 16 B load per lane (lane = row*4 + quad, quad = 4 adjacent columns of the half):
+// 64 B of every 128-byte row.  The other half of each row is read by the workgroup that owns the
+// strip's other 16 columns; the launch numbers the two so that they land on the same XCD and share
+// the line in its L2.
+__device__ __forceinline__ void load_half_step(Step<128>& st, const uint8_t* strip, int step, int half, int lane) {
+    const uint8_t* blk = strip + (int64_t)step * block_bytes(128);
+    const uint32_t q = (uint32_t)(half * 4 + (lane & 3));
+    st.valid = true;
+    st.w[0] = ldg16(blk + ((uint32_t)(lane >> 2) * kRowBytes + q * 16u));
+    st.dh = ldg8(blk + 2048 + q * 8u);
+    st.mh = ldg8(blk + 2048 + 64 + q * 8u);
+}
+
+__device__ __forceinline__ void dot_half_step(const Step<128>& st, const int8_t* codes, int lane, int acc[4]) {
+    const int2 xa = *reinterpret_cast<const int2*>(codes + (lane >> 2) * 8);
+    const uint32_t* w0 = reinterpret_cast<const uint32_t*>(&st.w[0]);
+#pragma unroll
+    for (int j = 0; j < 4; j++) acc[j] = dot8_q4(w0[j], xa.x, xa.y, 0);
 }
 
 // int32 partial dot products of the lane's 4 columns over the lane's k8-rows of this step;
@@ -143,6 +166,12 @@ struct XSlot {
     float2 scale[Step<G>::kBlocksPerStep];
 };
 
+// The same for a pair of group-128 blocks quantized in one pass
+struct XPairSlot {
+    int8_t codes[256];
+    float2 scale[2];
+};
+
 // FC_dynamic_quantize_x for one step (/root/reference/ops/op_fc.hpp:246-268): amax -> d = amax/127 ->
 // id = 1/d -> RNE codes; raw sum of the group
 template <int G>
@@ -172,6 +201,58 @@ __device__ __forceinline__ void quantize_step(const XRaw<G>& xr, XSlot<G>* slot,
         slot->codes[lane] = (int8_t)q8_code_rne(xr.v[0], id);
         if ((lane & 31) == 0) slot->scale[(G == 128) ? 0 : (lane >> 5)] = make_float2(d, hi ? s_hi : s_lo);
     }
+}
+
+// max and sum over each row of 16 lanes with the lane exchange folded into the arithmetic instruction
+// (one instruction per level and quantity).  A DPP operand must not be read within two wait states of
+// the instruction that wrote it: the two chains alternate and an s_nop fills the remaining slot.
+__device__ __forceinline__ void row16_max_sum_fused(float& mx, float& sm) {
+    asm("s_nop 1\n\t"
+        "v_max_f32_dpp %0, %0, %0 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf\n\t"
+        "v_add_f32_dpp %1, %1, %1 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 0\n\t"
+        "v_max_f32_dpp %0, %0, %0 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf\n\t"
+        "v_add_f32_dpp %1, %1, %1 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 0\n\t"
+        "v_max_f32_dpp %0, %0, %0 row_half_mirror row_mask:0xf bank_mask:0xf\n\t"
+        "v_add_f32_dpp %1, %1, %1 row_half_mirror row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 0\n\t"
+        "v_max_f32_dpp %0, %0, %0 row_mirror row_mask:0xf bank_mask:0xf\n\t"
+        "v_add_f32_dpp %1, %1, %1 row_mirror row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1"
+        : "+v"(mx), "+v"(sm));
+}
+
+// The same for two groups of 128 at once: lanes 0-31 hold the first group (four consecutive values per
+// lane), lanes 32-63 the second.  Same operations per value as the reference (amax -> d = amax/127 ->
+// id = 1/d -> round to nearest even, clamp), written for instruction count: the rows of 16 lanes are
+// combined pairwise with v_permlane16_swap, rounding and conversion are one addition of 1.5*2^23 (whose
+// low byte is then the two's-complement code), four codes are packed with two byte permutes.  The raw
+// group sum is a tree sum.
+__device__ __forceinline__ void quantize_pair(const float4& v, XPairSlot* slot, int lane) {
+    float amax;
+    float sum = (v.x + v.y) + (v.z + v.w);
+    asm("v_max3_f32 %0, |%1|, |%2|, |%3|\n\t"
+        "v_max_f32_e64 %0, %0, |%4|"
+        : "=&v"(amax)
+        : "v"(v.x), "v"(v.y), "v"(v.z), "v"(v.w));
+    row16_max_sum_fused(amax, sum);
+    // rows (0,1) -> lanes 0-31, rows (2,3) -> lanes 32-63: after the swap one register holds rows
+    // [0,0,2,2] and the other [1,1,3,3]
+    const auto ra = __builtin_amdgcn_permlane16_swap(__float_as_uint(amax), __float_as_uint(amax), false, false);
+    const auto rs = __builtin_amdgcn_permlane16_swap(__float_as_uint(sum), __float_as_uint(sum), false, false);
+    amax = __uint_as_float(ra[0] > ra[1] ? ra[0] : ra[1]);  // non-negative floats order like their bit patterns
+    sum = __uint_as_float(rs[0]) + __uint_as_float(rs[1]);
+    const float d = amax / 127.0f;
+    const float id = (d != 0.0f) ? (1.0f / d) : 0.0f;
+    constexpr float kRound = 12582912.0f;  // 1.5 * 2^23
+    const uint32_t u0 = __float_as_uint(__builtin_amdgcn_fmed3f(v.x * id, -128.0f, 127.0f) + kRound);
+    const uint32_t u1 = __float_as_uint(__builtin_amdgcn_fmed3f(v.y * id, -128.0f, 127.0f) + kRound);
+    const uint32_t u2 = __float_as_uint(__builtin_amdgcn_fmed3f(v.z * id, -128.0f, 127.0f) + kRound);
+    const uint32_t u3 = __float_as_uint(__builtin_amdgcn_fmed3f(v.w * id, -128.0f, 127.0f) + kRound);
+    const uint32_t lo = __builtin_amdgcn_perm(u1, u0, 0x0c0c0400u), hi = __builtin_amdgcn_perm(u3, u2, 0x04000c0cu);
+    *reinterpret_cast<uint32_t*>(&slot->codes[lane * 4]) = lo | hi;
+    slot->scale[lane >> 5] = make_float2(d, sum);  // every lane of the half writes the same pair
 }
 
 __device__ __forceinline__ float wave_sum_dpp(float v) {
