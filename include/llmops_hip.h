@@ -116,8 +116,8 @@ int llmops_fc_Q4A_residual(const float* x, int64_t rows, int64_t K, const int8_t
  *   glu == 2    : the same two ops on the input side: x is fp32 [rows,2K], a gate|up row (gate in columns
  *                 [0,K), up in [K,2K)), and the FC's input is silu(gate)*up; not with norm_w.  The FC in front
  *                 then runs without glu on the gate and up weights stacked along N.
- *   sumsq_out   : fp32 [rows,2*Ng], receives the sum of squares of every 16 adjacent outputs (after the
- *                 residual add; padding columns count as 0); not with glu == 1
+ *   sumsq_out   : fp32 [rows,Ng], receives the sum of squares of every strip's 32 outputs (after the
+ *                 residual add); not with glu == 1
  *   sumsq_in, sumsq_parts : with norm_w: fp32 [rows,sumsq_parts] whose row sums are sum(x^2) -- what the
  *                 FC that produced x left in its sumsq_out -- so that the rmsnorm does not read the row again
  * N_out is the number of output columns (Ng*32-ish; Ng/2*32-ish with glu == 1). */
@@ -259,10 +259,6 @@ int llmops_calib_copy(const void* src, void* dst, int64_t bytes, int workgroups,
 /* split-K planner knobs of the streaming FC kernel: number of workgroups to aim for and
  * wavefronts per workgroup (4, 8, 16; 0 = default).  Values <= 0 / < 0 leave a knob unchanged. */
 void llmops_fc_set_tuning(int target_workgroups, int waves_per_workgroup);
-
-/* rows <= 8, group 128, 96..255 strips: two workgroups per strip with 16 columns each instead of
- * split-K (default on; 0 switches it off, for comparisons) */
-void llmops_fc_set_half_strips(int on);
 
 /* prefill GEMM planner knob: force the row-tile factor of the LDS-tiled MFMA kernel (1, 2 or 4:
  * 32, 64 or 128 rows per workgroup; 8: the 256-row kernel whose two wave groups alternate between

@@ -30,9 +30,11 @@ def sources():
     return sorted(glob.glob(os.path.join(CSRC, "*.hip")) + glob.glob(os.path.join(CSRC, "*.cpp")))
 
 
-# Kernels that read LDS with hand-placed ds_read / s_waitcnt pairs: a register spilled between the
-# two would be saved before its data has arrived, so these must compile without VGPR spills.
-NO_SPILL = ["fc_gemm_pp_kernelILb0E"]
+# Kernels that must compile without VGPR spills: the 256-row GEMM reads LDS with hand-placed ds_read /
+# s_waitcnt pairs (a register spilled between the two would be saved before its data has arrived); the
+# one-row group-128 decode kernels are written to fit the 64 registers that two 16-wave workgroups per
+# CU leave each wave, and scratch traffic in their loop costs what the rewrite gained.
+NO_SPILL = ["fc_gemm_pp_kernelILb0E", "fc_gemv_fused_kernelILi128ELi1E"]
 
 
 def check_spills(remarks):
@@ -44,7 +46,7 @@ def check_spills(remarks):
         elif "VGPRs Spill:" in line and name is not None:
             spilled = int(line.split("VGPRs Spill:")[1].split()[0])
             if spilled and any(k in name for k in NO_SPILL):
-                raise RuntimeError(f"{name} spills {spilled} VGPRs; its hand-placed LDS reads do not allow that")
+                raise RuntimeError(f"{name} spills {spilled} VGPRs; this kernel must not spill (see NO_SPILL)")
 
 
 def build(verbose=False):

@@ -44,8 +44,13 @@ template <int G, int NW>
 __device__ __forceinline__ TileRange tile_range(int Kg, int S, int steps_per_split, int wave) {
     constexpr int BPS = Step<G>::kBlocksPerStep;
     TileRange r;
-    r.nb = blockIdx.x / S;
-    r.s = blockIdx.x % S;
+    if (S == 1) {  // no division for the common case
+        r.nb = blockIdx.x;
+        r.s = 0;
+    } else {
+        r.nb = blockIdx.x / S;
+        r.s = blockIdx.x % S;
+    }
     const int T = (Kg + BPS - 1) / BPS;  // steps in a strip
     const int t_lo = r.s * steps_per_split;
     const int t_hi = min(T, t_lo + steps_per_split);
@@ -55,35 +60,26 @@ __device__ __forceinline__ TileRange tile_range(int Kg, int S, int steps_per_spl
     return r;
 }
 
-// Sums of squares of a strip's outputs, one per 16 columns (16 adjacent threads hold them, zeros for
-// padding); `part` = 2*strip + (which half).  The next FC's rmsnorm adds these partial sums instead of
-// re-reading the whole row.
-__device__ __forceinline__ void half_strip_sumsq(float out, bool mine, int tr, int part, int strips, float* __restrict__ sumsq_out) {
+// Sum of squares of a strip's 32 outputs (threads tr*32 .. tr*32+31 hold them, zeros for padding):
+// the next FC's rmsnorm adds these per-strip sums instead of re-reading the whole row.
+__device__ __forceinline__ void strip_sumsq(float out, bool mine, int tr, int nb, int strips, float* __restrict__ sumsq_out) {
     float sq = out * out;
 #pragma unroll
-    for (int o = 8; o > 0; o >>= 1) sq += __shfl_xor(sq, o, 64);
-    if (mine && (threadIdx.x & 15) == 0) sumsq_out[(int64_t)tr * 2 * strips + part] = sq;
+    for (int o = 16; o > 0; o >>= 1) sq += __shfl_xor(sq, o, 64);
+    if (mine && (lane_id_now() & 31) == 0) sumsq_out[(int64_t)tr * strips + nb] = sq;
 }
 
 // Sum the lanes' running sums over row slots, waves and k-splits and store the strip's outputs.
 template <int MT, int NW>
-__device__ __forceinline__ void finish_strip(float f[MT][4], float (*red)[MT][kGroupN], unsigned* ticket_sh, int nb, int s,
+__device__ __forceinline__ void finish_strip(float f[MT][4], float (*red)[MT][kGroupN], unsigned* ticket_sh, int wave, int nb, int s,
                                              int S, int rows, int64_t N, float* __restrict__ y, float* part,
-                                             unsigned* counters, const float* __restrict__ residual,
+                                             unsigned* counters, bool has_residual, float residual_value,
                                              float* __restrict__ sumsq_out = nullptr) {
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = lane_id_now(), tid = wave * 64 + lane;  // `wave` is uniform (a scalar register)
     const int quad = lane & 7, rs = lane >> 3;
     // sum the 8 row slots (lane bits 3..5)
 #pragma unroll
-    for (int r = 0; r < MT; r++)
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-            float v = f[r][j];
-            v += dpp<kRowRor8>(v);
-            v += __shfl_xor(v, 16, 64);
-            v += __shfl_xor(v, 32, 64);
-            f[r][j] = v;
-        }
+    for (int r = 0; r < MT; r++) rowslot_sum4(f[r]);
     if (rs == 0) {
 #pragma unroll
         for (int r = 0; r < MT; r++)
@@ -92,7 +88,7 @@ __device__ __forceinline__ void finish_strip(float f[MT][4], float (*red)[MT][kG
     }
     __syncthreads();
 
-    const int tr = threadIdx.x >> 5, tn = threadIdx.x & 31;  // (row, column) this thread finalises
+    const int tr = tid >> 5, tn = tid & 31;  // (row, column) this thread finalises
     const bool mine = tr < MT && tr < rows;
     if (S == 1 && !mine && sumsq_out == nullptr) return;
     const int64_t n = (int64_t)nb * kGroupN + tn;
@@ -103,9 +99,9 @@ __device__ __forceinline__ void finish_strip(float f[MT][4], float (*red)[MT][kG
         for (int w = 0; w < NW; w++) v += red[w][tr][tn];
     }
     if (S == 1) {
-        const float out = (mine && n < N) ? (residual ? v + residual[(int64_t)tr * N + n] : v) : 0.0f;
+        const float out = (mine && n < N) ? (has_residual ? v + residual_value : v) : 0.0f;
         if (mine && n < N) y[(int64_t)tr * N + n] = out;
-        if (sumsq_out != nullptr) half_strip_sumsq(out, mine, tr, 2 * nb + (tn >> 4), (int)(gridDim.x / S), sumsq_out);
+        if (sumsq_out != nullptr) strip_sumsq(out, mine, tr, nb, (int)(gridDim.x / S), sumsq_out);
         return;
     }
     // Cross-workgroup hand-off without cache-wide fences: partial sums are written and read with
@@ -117,7 +113,7 @@ __device__ __forceinline__ void finish_strip(float f[MT][4], float (*red)[MT][kG
     if (mine) __hip_atomic_store(&part[((int64_t)s * rows + tr) * Np + n], v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
-    if (threadIdx.x == 0)
+    if (tid == 0)
         *ticket_sh = __hip_atomic_fetch_add(&counters[nb], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __syncthreads();
     if (*ticket_sh != (unsigned)(S - 1)) return;
@@ -126,50 +122,11 @@ __device__ __forceinline__ void finish_strip(float f[MT][4], float (*red)[MT][kG
         float acc = 0.0f;
         for (int i = 0; i < S; i++)
             acc += __hip_atomic_load(&part[((int64_t)i * rows + tr) * Np + n], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        out = residual ? acc + residual[(int64_t)tr * N + n] : acc;
+        out = has_residual ? acc + residual_value : acc;
         y[(int64_t)tr * N + n] = out;
     }
-    if (sumsq_out != nullptr) half_strip_sumsq(out, mine, tr, 2 * nb + (tn >> 4), (int)(gridDim.x / S), sumsq_out);
-    if (threadIdx.x == 0) __hip_atomic_store(&counters[nb], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // next launch
-}
-
-// The same for a workgroup that owns 16 of the strip's 32 columns over all of K (lane = row slot*4 + quad).
-template <int MT, int NW>
-__device__ __forceinline__ void finish_half_strip(float f[MT][4], float (*red)[MT][kGroupN], int nb, int half, int strips,
-                                                  int rows, int64_t N, float* __restrict__ y,
-                                                  const float* __restrict__ residual, float* __restrict__ sumsq_out) {
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    // sum the 16 row slots (lane bits 2..5)
-#pragma unroll
-    for (int r = 0; r < MT; r++)
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-            float v = f[r][j];
-            v += dpp<kRowRor8>(v);
-            v += dpp<kRowRor4>(v);
-            v += __shfl_xor(v, 16, 64);
-            v += __shfl_xor(v, 32, 64);
-            f[r][j] = v;
-        }
-    if (lane < 4) {
-#pragma unroll
-        for (int r = 0; r < MT; r++)
-#pragma unroll
-            for (int j = 0; j < 4; j++) red[wave][r][lane * 4 + j] = f[r][j];
-    }
-    __syncthreads();
-    const int tr = threadIdx.x >> 4, tn = threadIdx.x & 15;  // (row, column of the half) this thread finalises
-    const bool mine = tr < MT && tr < rows;
-    if (!mine && sumsq_out == nullptr) return;
-    const int64_t n = (int64_t)nb * kGroupN + half * 16 + tn;
-    float v = 0.0f;
-    if (mine) {
-#pragma unroll
-        for (int w = 0; w < NW; w++) v += red[w][tr][tn];
-    }
-    const float out = (mine && n < N) ? (residual ? v + residual[(int64_t)tr * N + n] : v) : 0.0f;
-    if (mine && n < N) y[(int64_t)tr * N + n] = out;
-    if (sumsq_out != nullptr) half_strip_sumsq(out, mine, tr, 2 * nb + half, strips, sumsq_out);
+    if (sumsq_out != nullptr) strip_sumsq(out, mine, tr, nb, (int)(gridDim.x / S), sumsq_out);
+    if (tid == 0) __hip_atomic_store(&counters[nb], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // next launch
 }
 
 // ---- variant 1: activations already quantized (xq, xd, gs in global memory) -------------------
@@ -214,7 +171,7 @@ __global__ __launch_bounds__(NW * 64) void fc_gemv_kernel(const uint8_t* __restr
         }
         cur = nxt;
     }
-    finish_strip<MT, NW>(f, red, &ticket_sh, tr.nb, tr.s, S, rows, N, y, part, counters, residual);
+    finish_strip<MT, NW>(f, red, &ticket_sh, wave, tr.nb, tr.s, S, rows, N, y, part, counters, false, 0.0f);
 }
 
 // ---- variant 2: raw fp32 activations, quantized by the wavefront that consumes them -----------
@@ -232,11 +189,7 @@ __global__ __launch_bounds__(NW * 64) void fc_gemv_kernel(const uint8_t* __restr
 //          FC's input is silu(gate)*up, formed as the two halves are loaded.  The FC that produces
 //          the row then keeps one strip per workgroup (no pairing of gate and up strips), which
 //          spreads its strips more evenly over the compute units.
-//   kHalf: (group 128) a workgroup owns 16 of a strip's 32 columns over all of K: twice the workgroups
-//          without a hand-off between them, for tensors with fewer strips than the chip has compute
-//          units.  Workgroups b and b+8 share a strip; workgroups are dealt to the 8 XCDs in turn, so
-//          the two halves of every 128-byte row are served from the same L2 (a matter of speed only).
-constexpr int kNorm = 1, kGlu = 2, kSums = 4, kGluIn = 8, kHalf = 16;
+constexpr int kNorm = 1, kGlu = 2, kSums = 4, kGluIn = 8;
 
 // One activation row needs few registers; asking for eight waves per SIMD (two workgroups of 16 waves
 // per CU) keeps every variant at or below 64 registers, so that grids of 257..512 workgroups are
@@ -256,9 +209,8 @@ __global__ __launch_bounds__(NW * 64, (MT == 1 ? NW / 2 : 1)) void fc_gemv_fused
                                                                  const float* __restrict__ sumsq_in, int sumsq_parts,
                                                                  float* __restrict__ sumsq_out) {
     constexpr bool NORM = (MODE & kNorm) != 0, GLU = (MODE & kGlu) != 0, SUMS = (MODE & kSums) != 0;
-    constexpr bool GLUIN = (MODE & kGluIn) != 0, HALF = (MODE & kHalf) != 0;
+    constexpr bool GLUIN = (MODE & kGluIn) != 0;
     static_assert(!(GLUIN && NORM), "the gate|up input has no rmsnorm");
-    static_assert(!HALF || (G == 128 && !GLU), "half strips: group 128, no gate/up epilogue");
     const int64_t xstride = GLUIN ? 2 * K : K;  // floats between activation rows
     constexpr int NWS = GLU ? NW / 2 : NW;  // waves per strip
     __shared__ float red[NW][MT][kGroupN];
@@ -268,18 +220,9 @@ __global__ __launch_bounds__(NW * 64, (MT == 1 ? NW / 2 : 1)) void fc_gemv_fused
     __shared__ unsigned ticket_sh;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int rs = HALF ? lane >> 2 : lane >> 3;
+    const int rs = lane >> 3;
     TileRange tr;
-    int half = 0;
-    if (HALF) {  // S == 1: 16 consecutive workgroup ids = both halves of 8 strips
-        const int b = blockIdx.x;
-        const int per_wave = (Kg + NW - 1) / NW;
-        tr.nb = ((b >> 4) << 3) | (b & 7);
-        half = (b >> 3) & 1;
-        tr.s = 0;
-        tr.t0 = min(Kg, wave * per_wave);
-        tr.t1 = min(Kg, tr.t0 + per_wave);
-    } else if (GLU) {  // S == 1: blockIdx.x is the strip pair, each half of the workgroup owns one strip
+    if (GLU) {  // S == 1: blockIdx.x is the strip pair, each half of the workgroup owns one strip
         constexpr int BPS = Step<G>::kBlocksPerStep;
         const int T = (Kg + BPS - 1) / BPS;
         const int per_wave = (T + NWS - 1) / NWS;
@@ -292,6 +235,19 @@ __global__ __launch_bounds__(NW * 64, (MT == 1 ? NW / 2 : 1)) void fc_gemv_fused
     }
     const uint8_t* strip = weiq + (int64_t)tr.nb * Kg * block_bytes(G);
     const bool first_row = (G == 128) ? (rs == 0) : ((rs & 3) == 0);
+    // The residual element this thread will add at the very end (thread = (row, column) of the strip) is
+    // asked for now: at the end it would put a memory round trip behind the last barrier.  (With the
+    // rmsnorm prologue the main loop has no register to spare; there it is asked for after the loop.)
+    float resv = 0.0f;
+#define LLMOPS_LOAD_RESIDUAL(TID)                                                          \
+    if (!GLU && residual != nullptr) {                                                     \
+        const int fr_ = (TID) >> 5;                                                        \
+        const int64_t n_ = (int64_t)tr.nb * kGroupN + ((TID) & 31);                        \
+        if (fr_ < MT && fr_ < rows && n_ < N) resv = residual[(int64_t)fr_ * N + n_];      \
+    }
+    if (!NORM) {
+        LLMOPS_LOAD_RESIDUAL(threadIdx.x)
+    }
 
     float f[MT][4];
 #pragma unroll
@@ -324,37 +280,42 @@ __global__ __launch_bounds__(NW * 64, (MT == 1 ? NW / 2 : 1)) void fc_gemv_fused
                                                          : make_float4(0.f, 0.f, 0.f, 0.f);
             }
     }
-    // two weight blocks in flight per wave, each with its activations (and norm weights):
+    // weight blocks in flight per wave, each with its activations (and norm weights):
     //   group 32 : cur/nxt, one step (two blocks) each, the activations of a step fetched one step ahead
-    //   group 128: sa/sb alternate; xv/uv/wv hold the activations of a pair of blocks, four per lane
+    //   group 128: a pair of blocks; the activations of a pair are four per lane
     Step<G> cur, nxt;
     XRaw<G> xcur[MT], xnxt[MT], wcur, wnxt;
     XRaw<G> ucur[GLUIN ? MT : 1], unxt[GLUIN ? MT : 1];  // the up half of a gate|up row
-    float4 xv[MT], uv[GLUIN ? MT : 1], wv;
-    const int pair_h = lane >> 5;  // group 128: which block of the pair this lane's four activations belong to
-    // the pair's 256 activations are contiguous: uniform base + lane*16 bytes
-#define LLMOPS_LOAD_PAIR(TP)                                                                                     \
+    struct PairBuf {
+        Step<G> a, b;
+        float4 xv[MT], uv[GLUIN ? MT : 1], wv;
+    };
+    PairBuf P0;
+    const bool first_of_pair = lane < 32;  // group 128: which block of the pair this lane's four activations belong to
+    // the pair's 256 activations are contiguous: uniform base + lane*16 bytes; activations are asked for
+    // before the weights (loads return in issue order and the quantization comes first)
+    // group 128 loads go through buffer descriptors (scalar base + scalar block offset + lane offset)
+    const buffer_rsrc strip_rs = make_rsrc(strip, (uint32_t)Kg * (uint32_t)block_bytes(G));
+    const buffer_rsrc x_rs = make_rsrc(x, (uint32_t)rows * (uint32_t)xstride * 4u);
+    const buffer_rsrc nw_rs = make_rsrc(NORM ? norm_w : x, NORM ? (uint32_t)K * 4u : 0u);
+#define LLMOPS_LOAD_BLOCK(ST, T) load_step_buf(ST, strip_rs, (T), lane)
+#define LLMOPS_LOAD_PAIR(P, TP)                                                                                  \
     do {                                                                                                         \
-        const bool ok_ = (TP) + pair_h < tr.t1;                                                                  \
-        const uint32_t lo_ = (uint32_t)lane * 4u;                                                                \
+        const bool ok_ = first_of_pair || (TP) + 1 < tr.t1;                                                      \
+        const uint32_t lo_ = (uint32_t)lane * 16u, so_ = (uint32_t)(TP) * 512u;                                  \
         _Pragma("unroll") for (int r = 0; r < MT; r++) {                                                         \
-            const float* xr_ = x + (int64_t)r * xstride + (int64_t)(TP) * 128;                                   \
+            const uint32_t ro_ = so_ + (uint32_t)r * (uint32_t)xstride * 4u;                                     \
             const bool okr_ = ok_ && r < rows;                                                                   \
-            xv[r] = okr_ ? *reinterpret_cast<const float4*>(xr_ + lo_) : make_float4(0.f, 0.f, 0.f, 0.f);        \
-            if (GLUIN) uv[GLUIN ? r : 0] = okr_ ? *reinterpret_cast<const float4*>(xr_ + K + lo_) : make_float4(0.f, 0.f, 0.f, 0.f); \
+            P.xv[r] = okr_ ? buf_ldf4(x_rs, lo_, ro_) : make_float4(0.f, 0.f, 0.f, 0.f);                         \
+            if (GLUIN) P.uv[GLUIN ? r : 0] = okr_ ? buf_ldf4(x_rs, lo_, ro_ + (uint32_t)K * 4u) : make_float4(0.f, 0.f, 0.f, 0.f); \
         }                                                                                                        \
-        if (NORM) wv = ok_ ? *reinterpret_cast<const float4*>(norm_w + (int64_t)(TP) * 128 + lo_) : make_float4(0.f, 0.f, 0.f, 0.f); \
-    } while (0)
-#define LLMOPS_LOAD_BLOCK(ST, T)                                              \
-    do {                                                                      \
-        if constexpr (HALF) load_half_step(ST, strip, (T), half, lane);       \
-        else load_step<G>(ST, strip, (T), Kg, lane);                          \
+        if (NORM) P.wv = ok_ ? buf_ldf4(nw_rs, lo_, so_) : make_float4(0.f, 0.f, 0.f, 0.f);                      \
+        LLMOPS_LOAD_BLOCK(P.a, (TP));                                                                            \
+        if ((TP) + 1 < tr.t1) LLMOPS_LOAD_BLOCK(P.b, (TP) + 1);                                                  \
     } while (0)
     if (tr.t0 < tr.t1) {
         if constexpr (G == 128) {
-            LLMOPS_LOAD_PAIR(tr.t0);
-            LLMOPS_LOAD_BLOCK(cur, tr.t0);
-            if (tr.t0 + 1 < tr.t1) LLMOPS_LOAD_BLOCK(nxt, tr.t0 + 1);
+            LLMOPS_LOAD_PAIR(P0, tr.t0);
         } else {
 #pragma unroll
             for (int r = 0; r < MT; r++)
@@ -416,46 +377,43 @@ __global__ __launch_bounds__(NW * 64, (MT == 1 ? NW / 2 : 1)) void fc_gemv_fused
     _Pragma("unroll") for (int r = 0; r < MT; r++) if (r < rows) {                                    \
         const Slot* slot = &xs[wave][r];                                                              \
         int acc[4];                                                                                   \
-        if constexpr (HALF) dot_half_step(ST, slot->codes + (J) * 128, lane, acc);                    \
-        else dot_step<G>(ST, slot->codes + (J) * 128, lane, acc);                                     \
+        dot_step<G>(ST, slot->codes + (J) * 128, lane, acc);                                          \
         const float2 sc = slot->scale[J];                                                             \
         fold(f[r], acc, ST.dh, ST.mh, sc.x, first_row ? sc.y : 0.0f);                                 \
     }
+#define LLMOPS_PAIR(P, TP)                                                                            \
+    do {                                                                                              \
+        _Pragma("unroll") for (int r = 0; r < MT; r++) if (r < rows) {                                \
+            float4 v = P.xv[r];                                                                       \
+            if (NORM) {                                                                               \
+                v.x = v.x * rsn[r] * P.wv.x;                                                          \
+                v.y = v.y * rsn[r] * P.wv.y;                                                          \
+                v.z = v.z * rsn[r] * P.wv.z;                                                          \
+                v.w = v.w * rsn[r] * P.wv.w;                                                          \
+            }                                                                                         \
+            if (GLUIN) { /* silu(gate)*up, the arithmetic of silu_mul_kernel */                       \
+                const float4 u = P.uv[GLUIN ? r : 0];                                                 \
+                v.x = u.x * (v.x * (1.0f / (1.0f + expf(-v.x))));                                     \
+                v.y = u.y * (v.y * (1.0f / (1.0f + expf(-v.y))));                                     \
+                v.z = u.z * (v.z * (1.0f / (1.0f + expf(-v.z))));                                     \
+                v.w = u.w * (v.w * (1.0f / (1.0f + expf(-v.w))));                                     \
+            }                                                                                         \
+            quantize_pair(v, &xs[wave][r], lane);                                                     \
+        }                                                                                             \
+        __builtin_amdgcn_wave_barrier(); /* LDS writes stay ahead of the reads below */               \
+        LLMOPS_BLOCK(P.a, 0)                                                                          \
+        if ((TP) + 1 < tr.t1) {                                                                       \
+            LLMOPS_BLOCK(P.b, 1)                                                                      \
+        }                                                                                             \
+        __builtin_amdgcn_wave_barrier(); /* reads stay ahead of the next pair's writes */             \
+    } while (0)
+        // Most shapes give a wave one pair; a longer run asks for the next pair only when this one is done,
+        // which keeps the registers of the two from overlapping (64 in all).
         for (int tp = tr.t0; tp < tr.t1; tp += 2) {
-#pragma unroll
-            for (int r = 0; r < MT; r++) {
-                if (r < rows) {
-                    float4 v = xv[r];
-                    if (NORM) {
-                        v.x = v.x * rsn[r] * wv.x;
-                        v.y = v.y * rsn[r] * wv.y;
-                        v.z = v.z * rsn[r] * wv.z;
-                        v.w = v.w * rsn[r] * wv.w;
-                    }
-                    if (GLUIN) {  // silu(gate)*up, the arithmetic of silu_mul_kernel
-                        const float4 u = uv[GLUIN ? r : 0];
-                        v.x = u.x * (v.x * (1.0f / (1.0f + expf(-v.x))));
-                        v.y = u.y * (v.y * (1.0f / (1.0f + expf(-v.y))));
-                        v.z = u.z * (v.z * (1.0f / (1.0f + expf(-v.z))));
-                        v.w = u.w * (v.w * (1.0f / (1.0f + expf(-v.w))));
-                    }
-                    quantize_pair(v, &xs[wave][r], lane);
-                }
-            }
-            __builtin_amdgcn_wave_barrier();  // LDS writes stay ahead of the reads below
-            LLMOPS_BLOCK(cur, 0)
-            if (tp + 1 < tr.t1) {
-                LLMOPS_BLOCK(nxt, 1)
-            }
-            __builtin_amdgcn_wave_barrier();  // reads stay ahead of the next pair's writes
-            // Most shapes give a wave one pair; a longer run asks for the next pair only now, which keeps
-            // the registers of the pair in flight and of the pair in use from overlapping (64 in all).
-            if (tp + 2 < tr.t1) {
-                LLMOPS_LOAD_PAIR(tp + 2);
-                LLMOPS_LOAD_BLOCK(cur, tp + 2);
-                if (tp + 3 < tr.t1) LLMOPS_LOAD_BLOCK(nxt, tp + 3);
-            }
+            LLMOPS_PAIR(P0, tp);
+            if (tp + 2 < tr.t1) LLMOPS_LOAD_PAIR(P0, tp + 2);
         }
+#undef LLMOPS_PAIR
 #undef LLMOPS_BLOCK
     } else {
         for (int t = tr.t0; t < tr.t1; t++) {
@@ -502,26 +460,19 @@ __global__ __launch_bounds__(NW * 64, (MT == 1 ? NW / 2 : 1)) void fc_gemv_fused
 #undef LLMOPS_LOAD_PAIR
 #undef LLMOPS_LOAD_BLOCK
 
-    if (HALF) {
-        finish_half_strip<MT, NW>(f, red, tr.nb, half, (int)(gridDim.x / 2), rows, N, y, residual, sumsq_out);
-        return;
-    }
     if (!GLU) {
-        finish_strip<MT, NW>(f, red, &ticket_sh, tr.nb, tr.s, S, rows, N, y, part, counters, residual, sumsq_out);
+        if (NORM) {
+            LLMOPS_LOAD_RESIDUAL(wave * 64 + lane_id_now())
+        }
+#undef LLMOPS_LOAD_RESIDUAL
+        finish_strip<MT, NW>(f, red, &ticket_sh, wave, tr.nb, tr.s, S, rows, N, y, part, counters, residual != nullptr, resv,
+                             sumsq_out);
         return;
     }
     // gate/up epilogue: sum row slots, then the two halves of the workgroup, then silu(gate)*up
     const int quad = lane & 7;
 #pragma unroll
-    for (int r = 0; r < MT; r++)
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-            float v = f[r][j];
-            v += dpp<kRowRor8>(v);
-            v += __shfl_xor(v, 16, 64);
-            v += __shfl_xor(v, 32, 64);
-            f[r][j] = v;
-        }
+    for (int r = 0; r < MT; r++) rowslot_sum4(f[r]);
     if (rs == 0) {
 #pragma unroll
         for (int r = 0; r < MT; r++)
@@ -529,7 +480,8 @@ __global__ __launch_bounds__(NW * 64, (MT == 1 ? NW / 2 : 1)) void fc_gemv_fused
             for (int j = 0; j < 4; j++) red[wave][r][quad * 4 + j] = f[r][j];
     }
     __syncthreads();
-    const int trow = threadIdx.x >> 5, tn = threadIdx.x & 31;
+    const int tid = wave * 64 + lane_id_now();
+    const int trow = tid >> 5, tn = tid & 31;
     if (trow < MT && trow < rows) {
         float g = 0.0f, u = 0.0f;
 #pragma unroll
@@ -581,11 +533,8 @@ __global__ __launch_bounds__(64) void fc_gemv_partials_kernel(const uint8_t* __r
 static int g_target_workgroups = 256;  // split-K planner aims for this many workgroups
 static int g_waves_per_workgroup = 0;  // 0 = choose per shape (pre-quantized variant only)
 
-static int g_half_strips = 1;  // 0: never split strips into column halves
-
 struct GemvPlan {
     int S, steps_per_split, NW;
-    bool half;  // two workgroups per strip, 16 columns each, no split-K
 };
 
 static GemvPlan plan_gemv(int64_t rows, int64_t Ng, int64_t Kg, int G, bool fused) {
@@ -601,7 +550,7 @@ static GemvPlan plan_gemv(int64_t rows, int64_t Ng, int64_t Kg, int G, bool fuse
     if (S < 1) S = 1;
     int sps = (T + S - 1) / S;
     S = (T + sps - 1) / sps;  // drop empty splits
-    return {S, sps, NW, false};
+    return {S, sps, NW};
 }
 
 size_t gemv_workspace_bytes(int64_t rows, int64_t Ng, int64_t Kg, int G) {
@@ -633,15 +582,6 @@ static void launch_fused_t(const uint8_t* w, const float* x, float* y, float* pa
         w, x, y, part, counters, (int)Kg, K, N, rows, p.S, p.steps_per_split, o.residual, o.norm_w, o.eps, o.sumsq_in, \
         o.sumsq_parts, o.sumsq_out)
     const bool sums = o.norm_w != nullptr && o.sumsq_in != nullptr;
-    if constexpr (G == 128) {
-        if (p.half) {
-            if (o.glu_in) LLMOPS_FUSED(kGluIn | kHalf, Ng * 2);
-            else if (sums) LLMOPS_FUSED(kNorm | kSums | kHalf, Ng * 2);
-            else if (o.norm_w) LLMOPS_FUSED(kNorm | kHalf, Ng * 2);
-            else LLMOPS_FUSED(kHalf, Ng * 2);
-            return;
-        }
-    }
     if (o.glu_in) {
         LLMOPS_FUSED(kGluIn, Ng * p.S);
     } else if (o.glu) {
@@ -662,14 +602,6 @@ int launch_gemv_fused(const uint8_t* w, const float* x, float* y, float* part, u
                       const float* sumsq_in, int sumsq_parts, float* sumsq_out, hipStream_t st) {
     GemvPlan p = plan_gemv(rows, Ng, Kg, G, true);
     if (glu == 1) p.S = 1;
-    // Tensors with fewer strips than compute units and a K that gives a wave one pair of blocks: column
-    // halves give every unit a workgroup without the split-K hand-off (4096x4096: 4.8 against 5.2 us).  With
-    // a longer K the second quantization of every activation group costs what the hand-off does (4096x11008:
-    // 9.4 against 9.1 us), so those keep split-K.
-    if (g_half_strips && G == 128 && glu != 1 && Ng % 8 == 0 && Ng >= 96 && Ng < 256 && Kg <= 2 * p.NW) {
-        p.half = true;
-        p.S = 1;
-    }
     const FusedOps o{residual, norm_w, eps, glu == 1, glu == 2, sumsq_in, sumsq_parts, sumsq_out};
 #define LLMOPS_CASE(GG, MT, NWW) launch_fused_t<GG, MT, NWW>(w, x, y, part, counters, Ng, Kg, N, (int)rows, p, o, st)
     if (G == 128) {
@@ -740,8 +672,6 @@ int launch_gemv_partials(const uint8_t* w, const int8_t* xq, int32_t* acc, int64
 }
 
 }  // namespace llmops
-
-extern "C" void llmops_fc_set_half_strips(int on) { llmops::g_half_strips = on != 0; }
 
 extern "C" void llmops_fc_set_tuning(int target_workgroups, int waves_per_workgroup) {
     if (target_workgroups > 0) llmops::g_target_workgroups = target_workgroups > 4096 ? 4096 : target_workgroups;

@@ -24,7 +24,7 @@ __device__ __forceinline__ float dpp(float v) {
 __device__ __forceinline__ float lane_bcast(float v, int lane) {
     return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), lane));
 }
-constexpr int kQuadXor1 = 0xB1, kQuadXor2 = 0x4E, kRowHalfMirror = 0x141, kRowMirror = 0x140, kRowRor8 = 0x128, kRowRor4 = 0x124;
+constexpr int kQuadXor1 = 0xB1, kQuadXor2 = 0x4E, kRowHalfMirror = 0x141, kRowMirror = 0x140, kRowRor8 = 0x128;
 
 // max and sum over each row of 16 lanes, result in every lane of the row
 __device__ __forceinline__ void row16_max_sum(float& mx, float& sm) {
@@ -78,25 +78,36 @@ __device__ __forceinline__ void load_step(Step<G>& st, const uint8_t* strip, int
     }
 }
 
-// Half-strip form of a group-128 step: the wave covers the block's 16 k8-rows x 16 of the strip's 32
-// columns with one 16 B load per lane (lane = row*4 + quad, quad = 4 adjacent columns of the half):
-// 64 B of every 128-byte row.  The other half of each row is read by the workgroup that owns the
-// strip's other 16 columns; the launch numbers the two so that they land on the same XCD and share
-// the line in its L2.
-__device__ __forceinline__ void load_half_step(Step<128>& st, const uint8_t* strip, int step, int half, int lane) {
-    const uint8_t* blk = strip + (int64_t)step * block_bytes(128);
-    const uint32_t q = (uint32_t)(half * 4 + (lane & 3));
-    st.valid = true;
-    st.w[0] = ldg16(blk + ((uint32_t)(lane >> 2) * kRowBytes + q * 16u));
-    st.dh = ldg8(blk + 2048 + q * 8u);
-    st.mh = ldg8(blk + 2048 + 64 + q * 8u);
+// The same group-128 step through a buffer descriptor: scalar base (the strip), scalar offset (the block)
+// and one 32-bit lane offset, so that a loop over blocks keeps no 64-bit addresses in vector registers.
+// Reads past the descriptor's size return 0.
+typedef __amdgpu_buffer_rsrc_t buffer_rsrc;
+__device__ __forceinline__ buffer_rsrc make_rsrc(const void* base, uint32_t bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
 }
-
-__device__ __forceinline__ void dot_half_step(const Step<128>& st, const int8_t* codes, int lane, int acc[4]) {
-    const int2 xa = *reinterpret_cast<const int2*>(codes + (lane >> 2) * 8);
-    const uint32_t* w0 = reinterpret_cast<const uint32_t*>(&st.w[0]);
-#pragma unroll
-    for (int j = 0; j < 4; j++) acc[j] = dot8_q4(w0[j], xa.x, xa.y, 0);
+// weights: non-temporal (cache policy bit 1)
+__device__ __forceinline__ uint4 buf_ldg16_nt(buffer_rsrc r, uint32_t voff, uint32_t soff) {
+    const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 2);
+    return make_uint4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ uint2 buf_ldg8(buffer_rsrc r, uint32_t voff, uint32_t soff) {
+    typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+    const u32x2 v = __builtin_amdgcn_raw_buffer_load_b64(r, voff, soff, 0);
+    return make_uint2(v.x, v.y);
+}
+__device__ __forceinline__ float4 buf_ldf4(buffer_rsrc r, uint32_t voff, uint32_t soff) {
+    const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 0);
+    return make_float4(__uint_as_float(v.x), __uint_as_float(v.y), __uint_as_float(v.z), __uint_as_float(v.w));
+}
+__device__ __forceinline__ void load_step_buf(Step<128>& st, buffer_rsrc strip, int step, int lane) {
+    const uint32_t so = (uint32_t)step * (uint32_t)block_bytes(128);
+    const uint32_t wo = (uint32_t)lane * 16u, qo = (uint32_t)(lane & 7) * 8u;
+    st.valid = true;
+    // constant parts go to the scalar offset: the lane offsets stay two registers for the whole loop
+    st.w[0] = buf_ldg16_nt(strip, wo, so);
+    st.w[1] = buf_ldg16_nt(strip, wo, so + 1024u);
+    st.dh = buf_ldg8(strip, qo, so + 2048u);
+    st.mh = buf_ldg8(strip, qo, so + 2048u + 64u);
 }
 
 // int32 partial dot products of the lane's 4 columns over the lane's k8-rows of this step;
@@ -123,15 +134,43 @@ __device__ __forceinline__ void unpack_h4(uint2 h, float out[4]) {
     out[3] = f16_bits_to_f32((uint16_t)(h.y >> 16));
 }
 
-// f[r][j] += (d*dx)*acc + m*gsum for the lane's 4 columns
+// The lane id computed on the spot (2 instructions) instead of kept in a register since the kernel began:
+// the epilogue of a kernel that is short of registers in its main loop uses this.
+__device__ __forceinline__ int lane_id_now() {
+    int l;
+    asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(l));
+    return l;
+}
+
+// f[r][j] += d*(dx*acc) + m*gsum for the lane's 4 columns (d and m enter the fused multiply-adds as
+// fp16 operands: no separate conversions)
 __device__ __forceinline__ void fold(float f[4], const int acc[4], uint2 dh, uint2 mh, float dx, float g) {
     float d[4], m[4];
     unpack_h4(dh, d);
     unpack_h4(mh, m);
 #pragma unroll
     for (int j = 0; j < 4; j++) {
-        f[j] = fmaf(d[j] * dx, (float)acc[j], f[j]);
+        f[j] = fmaf(d[j], dx * (float)acc[j], f[j]);
         f[j] = fmaf(m[j], g, f[j]);
+    }
+}
+
+// Sum over the 8 row slots of a wave (lane bits 3, 4, 5), result in every lane: one DPP-fused add inside the
+// rows of 16 lanes, then the rows pairwise (v_permlane16_swap) and the wave's halves (v_permlane32_swap).
+__device__ __forceinline__ void rowslot_sum4(float f[4]) {
+    asm("s_nop 1\n\t"
+        "v_add_f32_dpp %0, %0, %0 row_ror:8 row_mask:0xf bank_mask:0xf\n\t"
+        "v_add_f32_dpp %1, %1, %1 row_ror:8 row_mask:0xf bank_mask:0xf\n\t"
+        "v_add_f32_dpp %2, %2, %2 row_ror:8 row_mask:0xf bank_mask:0xf\n\t"
+        "v_add_f32_dpp %3, %3, %3 row_ror:8 row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1"
+        : "+v"(f[0]), "+v"(f[1]), "+v"(f[2]), "+v"(f[3]));
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(f[j]), __float_as_uint(f[j]), false, false);
+        const float v = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+        const auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+        f[j] = __uint_as_float(b[0]) + __uint_as_float(b[1]);
     }
 }
 
@@ -256,8 +295,16 @@ __device__ __forceinline__ void quantize_pair(const float4& v, XPairSlot* slot, 
 }
 
 __device__ __forceinline__ float wave_sum_dpp(float v) {
-    float dummy = 0.0f;
-    row16_max_sum(dummy, v);
+    asm("s_nop 1\n\t"
+        "v_add_f32_dpp %0, %0, %0 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\t"
+        "v_add_f32_dpp %0, %0, %0 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\t"
+        "v_add_f32_dpp %0, %0, %0 row_half_mirror row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\t"
+        "v_add_f32_dpp %0, %0, %0 row_mirror row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1"
+        : "+v"(v));
     return (lane_bcast(v, 0) + lane_bcast(v, 16)) + (lane_bcast(v, 32) + lane_bcast(v, 48));
 }
 

@@ -162,7 +162,7 @@ def fc_Q4A_decode(input, weiq, N_out, norm=None, residual=None, glu=False, sumsq
     silu(gate)*up with N_out = F columns.  glu_in=True: ``input`` is a gate|up row [B, M, 2K] (what an FC
     over the gate and up weights stacked along N leaves behind) and the FC runs on silu(gate)*up.
     want_sumsq=True returns ``(out, sumsq)`` where ``sumsq``
-    [B*M, 2*strips] holds the sum of squares of every 16 outputs; passed as ``sumsq_in`` to the FC that
+    [B*M, strips] holds the sum of squares of every 32 outputs; passed as ``sumsq_in`` to the FC that
     rmsnorms ``out`` it saves that FC the pass over the row.  With more than 8 rows the same
     arithmetic is composed from the separate ops."""
     _dev(input, torch.float32, 3, "input")
@@ -197,12 +197,12 @@ def fc_Q4A_decode(input, weiq, N_out, norm=None, residual=None, glu=False, sumsq
         out = fc_Q4A(x, weiq, N_out, residual=residual)
         if want_sumsq:
             pad = torch.nn.functional.pad(out.reshape(rows, N_out), (0, Ng * 32 - N_out))
-            return out, pad.view(rows, 2 * Ng, 16).square().sum(-1)
+            return out, pad.view(rows, Ng, 32).square().sum(-1)
         return out
     lib = _lib.load()
     ws = _workspace(input.device, lib.llmops_fc_Q4A_workspace_bytes(rows, K, Ng, Kg, g))
     out = torch.empty((B, M, N_out), dtype=torch.float32, device=input.device)
-    sumsq = torch.empty((rows, 2 * Ng), dtype=torch.float32, device=input.device) if want_sumsq else None
+    sumsq = torch.empty((rows, Ng), dtype=torch.float32, device=input.device) if want_sumsq else None
     _lib.check(lib.llmops_fc_Q4A_decode(_ptr(input), rows, K, _ptr(weiq), Ng, Kg, g, N_out,
                                         _ptr(norm[0]) if norm is not None else None, float(norm[1]) if norm is not None else 0.0,
                                         _ptr(residual) if residual is not None else None, 2 if glu_in else int(bool(glu)),

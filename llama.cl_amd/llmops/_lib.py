@@ -59,7 +59,6 @@ SIGNATURES = {
     "llmops_calib_read": (c_int, [c_ptr, c_i64, c_int, c_ptr, c_ptr]),
     "llmops_calib_copy": (c_int, [c_ptr, c_ptr, c_i64, c_int, c_ptr]),
     "llmops_fc_set_tuning": (None, [c_int, c_int]),
-    "llmops_fc_set_half_strips": (None, [c_int]),
     "llmops_gemm_set_tuning": (None, [c_int]),
 }
 

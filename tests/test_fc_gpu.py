@@ -19,17 +19,6 @@ def ops():
     return llmops
 
 
-@pytest.fixture(params=[1, 0], ids=["column-halves", "split-k"])
-def few_strips_mode(request):
-    """Tensors of 96..255 strips at group 128 and <= 8 rows: two workgroups per strip with 16 columns each
-    (the default) or split-K with the hand-off through memory; tests that take this fixture run both."""
-    from llmops import _lib
-    lib = _lib.load()
-    lib.llmops_fc_set_half_strips(request.param)
-    yield request.param
-    lib.llmops_fc_set_half_strips(1)
-
-
 def dev(a):
     return torch.from_numpy(np.ascontiguousarray(a)).cuda()
 
@@ -268,9 +257,9 @@ def test_fc_decode_folded_ops_vs_oracle(ops, orc, G, rows):
 @pytest.mark.parametrize("G", [32, 128])
 @pytest.mark.parametrize("rows", [1, 3, 8, 20])
 @pytest.mark.parametrize("N,K", [(1000, 1024), (4096, 11008)])
-def test_fc_decode_sumsq_handover(ops, orc, few_strips_mode, G, rows, N, K):
-    """The sums of squares per 16 outputs an FC leaves behind (N = 4096: column halves or the split-K
-    hand-off), and the rmsnorm of the next FC fed with them instead of reading its input row."""
+def test_fc_decode_sumsq_handover(ops, orc, G, rows, N, K):
+    """The per-strip sums of squares an FC leaves behind (also through the split-K hand-off: K = 11008),
+    and the rmsnorm of the next FC fed with them instead of reading its input row."""
     rng = np.random.default_rng(rows + G + N)
     x = rng.standard_normal((1, rows, K)).astype(np.float32)
     w = (rng.standard_normal((N, K)) * 0.02).astype(np.float32)
@@ -281,8 +270,8 @@ def test_fc_decode_sumsq_handover(ops, orc, few_strips_mode, G, rows, N, K):
     strips = -(-N // 32)
     pad = np.zeros((rows, strips * 32))
     pad[:, :N] = yh
-    want = (pad.reshape(rows, 2 * strips, 16) ** 2).sum(-1)
-    assert host(ss).shape == (rows, 2 * strips)
+    want = (pad.reshape(rows, strips, 32) ** 2).sum(-1)
+    assert host(ss).shape == (rows, strips)
     assert np.abs(host(ss) - want).max() <= 1e-5 * want.max()
     # consumer: rmsnorm(y) @ W2 with and without the handed-over sums must agree to rounding
     if N % G == 0:
@@ -301,10 +290,10 @@ def test_fc_decode_sumsq_handover(ops, orc, few_strips_mode, G, rows, N, K):
 @pytest.mark.parametrize("G", [32, 128])
 @pytest.mark.parametrize("rows", [1, 2, 4, 8, 20])
 @pytest.mark.parametrize("N,K", [(1000, 1024), (4096, 11008)])
-def test_fc_decode_gate_up_input(ops, orc, few_strips_mode, G, rows, N, K):
+def test_fc_decode_gate_up_input(ops, orc, G, rows, N, K):
     """fc_Q4A_decode(glu_in=True): the input row is [gate | up] (2K floats) and the FC runs on
     silu(gate)*up; against the oracle's silu, imul and fc, with and without the residual and the
-    sums of squares (N = 4096: column halves or the split-K hand-off), and bit-equal to silu_mul + FC."""
+    sums of squares (K = 11008 also takes the split-K hand-off), and bit-equal to silu_mul + FC."""
     rng = np.random.default_rng(rows + G + N)
     gu = rng.standard_normal((1, rows, 2 * K)).astype(np.float32)
     w = (rng.standard_normal((N, K)) * 0.02).astype(np.float32)
@@ -321,40 +310,10 @@ def test_fc_decode_gate_up_input(ops, orc, few_strips_mode, G, rows, N, K):
     strips = -(-N // 32)
     pad = np.zeros((rows, strips * 32))
     pad[:, :N] = host(got).astype(np.float64).reshape(rows, N)
-    ref_ss = (pad.reshape(rows, 2 * strips, 16) ** 2).sum(-1)
+    ref_ss = (pad.reshape(rows, strips, 32) ** 2).sum(-1)
     assert np.abs(host(ss) - ref_ss).max() <= 1e-5 * ref_ss.max()
     with pytest.raises(RuntimeError):  # no rmsnorm in front of a gate|up row
         ops.fc_Q4A_decode(dev(gu), dev(pw), N, norm=(torch.ones(K, device="cuda"), 1e-5), glu_in=True)
-
-
-@pytest.mark.parametrize("rows", [1, 2, 3, 4, 5, 8])
-@pytest.mark.parametrize("N,K", [(4096, 4096), (3060, 1280), (7920, 384), (4090, 11008)])
-def test_fc_decode_few_strips_vs_oracle(ops, orc, few_strips_mode, rows, N, K):
-    """96..255 strips at group 128, 1..8 rows, both ways of spreading them over the chip: plain fc_Q4A,
-    the residual epilogue, the rmsnorm prologue, the sums of squares; ragged N (3060 = 95.6 strips: the
-    last half strip is part padding, 7920: the last half strip is all padding, 4090), k-block counts 3..86
-    (fewer blocks than waves, more blocks than waves; the planner keeps split-K at K = 11008 either way);
-    and the closed-form construction exactly."""
-    rng = np.random.default_rng(rows + N)
-    x = rng.standard_normal((1, rows, K)).astype(np.float32)
-    w = (rng.standard_normal((N, K)) * 0.02).astype(np.float32)
-    res = rng.standard_normal((1, rows, N)).astype(np.float32)
-    nw = (1.0 + 0.1 * rng.standard_normal(K)).astype(np.float32)
-    pw = orc.quant_w(w, 128)
-    want = orc.fc(x, pw, N)
-    assert max_rel_err(host(ops.fc_Q4A(dev(x), dev(pw), N)), want) <= 1e-5
-    got, ss = ops.fc_Q4A_decode(dev(x), dev(pw), N, residual=dev(res), want_sumsq=True)
-    assert max_rel_err(host(got), want + res) <= 1e-5
-    strips = -(-N // 32)
-    pad = np.zeros((rows, strips * 32))
-    pad[:, :N] = host(got).astype(np.float64).reshape(rows, N)
-    ref_ss = (pad.reshape(rows, 2 * strips, 16) ** 2).sum(-1)
-    assert np.abs(host(ss) - ref_ss).max() <= 1e-5 * ref_ss.max()
-    got = host(ops.fc_Q4A_decode(dev(x), dev(pw), N, norm=(dev(nw), 1e-5)))
-    assert max_rel_err(got, orc.fc(orc.rmsnorm(x, nw, 1e-5), pw, N)) <= 1e-4
-    xe, we = oracle.closed_form_fc_inputs(rows, N, K, seed=rows)
-    ye = host(ops.fc_Q4A(dev(xe.reshape(1, rows, K)), ops.offline_FC_quant_Q4A(dev(we), 128), N))
-    assert np.array_equal(ye, (xe.astype(np.float64) @ we.astype(np.float64).T).astype(np.float32).reshape(1, rows, N))
 
 
 @pytest.mark.parametrize("rows", [17, 48, 100, 128, 129, 200, 256])
