@@ -84,10 +84,11 @@ int llmops_FC_dynamic_quantize_x_rows(const float* x, int64_t rows, int64_t K, i
  * ------------------------------------------------------------------------------------------ */
 
 /* workspace bytes llmops_fc_Q4A needs for these sizes (activation codes, split-K partial sums and
- * arrival counters).  The first LLMOPS_FC_COUNTER_BYTES bytes of the workspace must be zero when
- * the library first sees it; the library leaves them zero after every call.  One workspace must
- * not be shared by calls that can overlap on the device. */
-#define LLMOPS_FC_COUNTER_BYTES 65536
+ * the hand-off area of the k-splits: arrival counters and exchange slots).  The first
+ * LLMOPS_FC_COUNTER_BYTES bytes of the workspace must be zero when the library first sees it; the
+ * library leaves them zero after every call.  One workspace must not be shared by calls that can
+ * overlap on the device. */
+#define LLMOPS_FC_COUNTER_BYTES 1048576
 size_t llmops_fc_Q4A_workspace_bytes(int64_t rows, int64_t K, int64_t Ng, int64_t Kg, int group_k);
 
 /* fc_Q4A (ops/op_fc.hpp:286-426, bound at ops/main.cpp:160).
@@ -257,7 +258,9 @@ int llmops_calib_read(const void* src, int64_t bytes, int workgroups, void* out4
 int llmops_calib_copy(const void* src, void* dst, int64_t bytes, int workgroups, llmops_stream_t stream);
 
 /* split-K planner knobs of the streaming FC kernel: number of workgroups to aim for and
- * wavefronts per workgroup (4, 8, 16; 0 = default).  Values <= 0 / < 0 leave a knob unchanged. */
+ * wavefronts per workgroup (4, 8, 16; 0 = default).  Values <= 0 / < 0 leave a knob unchanged.
+ * target_workgroups == -2 / -3 instead selects how two k-splits of a strip meet: through one 64-bit
+ * exchange per output (default) / through the arrival ticket like larger split counts. */
 void llmops_fc_set_tuning(int target_workgroups, int waves_per_workgroup);
 
 /* prefill GEMM planner knob: force the row-tile factor of the LDS-tiled MFMA kernel (1, 2 or 4:

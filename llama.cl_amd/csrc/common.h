@@ -15,6 +15,9 @@ namespace llmops {
 
 constexpr int kGroupN = 32;   // columns per packed strip (q4_1_block::group_n, ops/op_fc.hpp:17)
 constexpr int kRowBytes = 128;  // one k8-row of a block: 32 columns x 4 bytes
+// zeroed head of the FC workspace (LLMOPS_FC_COUNTER_BYTES): arrival counters of the k-splits, one per
+// strip, then the exchange slots of the two-split hand-off
+constexpr int kTicketBytes = 65536;
 
 __host__ __device__ constexpr int64_t block_bytes(int G) { return (int64_t)(G / 8) * kRowBytes + 64 + 64; }
 

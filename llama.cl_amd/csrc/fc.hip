@@ -67,7 +67,7 @@ static int fc_impl(const float* x, int64_t rows, int64_t K, const int8_t* weiq, 
     LLMOPS_REQUIRE(rows > 0 && K > 0 && Ng > 0 && Kg > 0);
     LLMOPS_REQUIRE(K == Kg * group_k);  // the reference reads past K otherwise (ops/op_fc.hpp:184)
     LLMOPS_REQUIRE(N > (Ng - 1) * kGroupN && N <= Ng * kGroupN);
-    LLMOPS_REQUIRE(Ng <= LLMOPS_FC_COUNTER_BYTES / 4);
+    LLMOPS_REQUIRE(Ng <= kTicketBytes / 4);
     LLMOPS_REQUIRE(Ng * 64 < ((int64_t)1 << 31));
     LLMOPS_REQUIRE(aligned(weiq, 16) && aligned(workspace, 256) && aligned(x, 8));
     const FcWorkspace lay = fc_layout(rows, Ng, Kg, group_k);
@@ -117,7 +117,7 @@ extern "C" int llmops_fc_Q4A_decode(const float* x, int64_t rows, int64_t K, con
     LLMOPS_REQUIRE(x != nullptr && weiq != nullptr && y != nullptr && workspace != nullptr);
     LLMOPS_REQUIRE(rows > 0 && rows <= kMaxGemvRows);
     LLMOPS_REQUIRE(K > 0 && Ng > 0 && Kg > 0 && K == Kg * group_k);
-    LLMOPS_REQUIRE(Ng <= LLMOPS_FC_COUNTER_BYTES / 4 && Ng * 64 < ((int64_t)1 << 31));
+    LLMOPS_REQUIRE(Ng <= kTicketBytes / 4 && Ng * 64 < ((int64_t)1 << 31));
     LLMOPS_REQUIRE(aligned(weiq, 16) && aligned(workspace, 256) && aligned(x, 8));
     LLMOPS_REQUIRE(glu >= 0 && glu <= 2);
     if (glu == 1) {
@@ -147,7 +147,7 @@ extern "C" int llmops_fc_Q4A_prequantized(const int8_t* xq, const float* xd, con
     LLMOPS_REQUIRE(workspace != nullptr);
     LLMOPS_REQUIRE(rows > 0 && Ng > 0 && Kg > 0);
     LLMOPS_REQUIRE(N > (Ng - 1) * kGroupN && N <= Ng * kGroupN);
-    LLMOPS_REQUIRE(Ng <= LLMOPS_FC_COUNTER_BYTES / 4);
+    LLMOPS_REQUIRE(Ng <= kTicketBytes / 4);
     LLMOPS_REQUIRE(aligned(weiq, 16) && aligned(xq, 16) && aligned(workspace, 256));
     const FcWorkspace lay = fc_layout(rows, Ng, Kg, group_k);
     if (workspace_bytes < lay.total)

@@ -74,7 +74,7 @@ template <int MT, int NW>
 __device__ __forceinline__ void finish_strip(float f[MT][4], float (*red)[MT][kGroupN], unsigned* ticket_sh, int wave, int nb, int s,
                                              int S, int rows, int64_t N, float* __restrict__ y, float* part,
                                              unsigned* counters, bool has_residual, float residual_value,
-                                             float* __restrict__ sumsq_out = nullptr) {
+                                             float* __restrict__ sumsq_out = nullptr, unsigned long long* slots = nullptr) {
     const int lane = lane_id_now(), tid = wave * 64 + lane;  // `wave` is uniform (a scalar register)
     const int quad = lane & 7, rs = lane >> 3;
     // sum the 8 row slots (lane bits 3..5)
@@ -102,6 +102,23 @@ __device__ __forceinline__ void finish_strip(float f[MT][4], float (*red)[MT][kG
         const float out = (mine && n < N) ? (has_residual ? v + residual_value : v) : 0.0f;
         if (mine && n < N) y[(int64_t)tr * N + n] = out;
         if (sumsq_out != nullptr) strip_sumsq(out, mine, tr, nb, (int)(gridDim.x / S), sumsq_out);
+        return;
+    }
+    // Two k-splits and nobody waiting for the strip's sum of squares: the hand-off is one 64-bit exchange
+    // per output.  A slot is empty (0) or holds (1 << 32 | value bits); whoever finds the other split's
+    // value there adds the two (a + b: the same bits whichever came first), stores the output and empties
+    // the slot for the next launch; whoever finds it empty has parked its own value and is done.  The value
+    // travels inside the atomic, so there is nothing to order, and the cost is one round trip to memory
+    // instead of three (store and acknowledgement, ticket, loads).
+    if (slots != nullptr) {
+        if (!(mine && n < N)) return;
+        unsigned long long* slot = slots + ((int64_t)tr * Np + n);
+        const unsigned long long parked = (1ull << 32) | (unsigned long long)__float_as_uint(v);
+        const unsigned long long old = __hip_atomic_exchange(slot, parked, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if ((old >> 32) == 0ull) return;
+        const float both = v + __uint_as_float((unsigned)(old & 0xFFFFFFFFull));
+        y[(int64_t)tr * N + n] = has_residual ? both + residual_value : both;
+        __hip_atomic_store(slot, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         return;
     }
     // Cross-workgroup hand-off without cache-wide fences: partial sums are written and read with
@@ -207,7 +224,7 @@ __global__ __launch_bounds__(NW * 64, (MT == 1 ? NW / 2 : 1)) void fc_gemv_fused
                                                                  int steps_per_split, const float* __restrict__ residual,
                                                                  const float* __restrict__ norm_w, float eps,
                                                                  const float* __restrict__ sumsq_in, int sumsq_parts,
-                                                                 float* __restrict__ sumsq_out) {
+                                                                 float* __restrict__ sumsq_out, int exchange) {
     constexpr bool NORM = (MODE & kNorm) != 0, GLU = (MODE & kGlu) != 0, SUMS = (MODE & kSums) != 0;
     constexpr bool GLUIN = (MODE & kGluIn) != 0;
     static_assert(!(GLUIN && NORM), "the gate|up input has no rmsnorm");
@@ -465,8 +482,9 @@ __global__ __launch_bounds__(NW * 64, (MT == 1 ? NW / 2 : 1)) void fc_gemv_fused
             LLMOPS_LOAD_RESIDUAL(wave * 64 + lane_id_now())
         }
 #undef LLMOPS_LOAD_RESIDUAL
+        // exchange: two k-splits meet through 64-bit slots (which `part` then points at) instead of the ticket
         finish_strip<MT, NW>(f, red, &ticket_sh, wave, tr.nb, tr.s, S, rows, N, y, part, counters, residual != nullptr, resv,
-                             sumsq_out);
+                             sumsq_out, exchange ? reinterpret_cast<unsigned long long*>(part) : nullptr);
         return;
     }
     // gate/up epilogue: sum row slots, then the two halves of the workgroup, then silu(gate)*up
@@ -531,6 +549,7 @@ __global__ __launch_bounds__(64) void fc_gemv_partials_kernel(const uint8_t* __r
 }
 
 static int g_target_workgroups = 256;  // split-K planner aims for this many workgroups
+static int g_exchange_handoff = 1;     // 0: two k-splits also meet through the arrival ticket
 static int g_waves_per_workgroup = 0;  // 0 = choose per shape (pre-quantized variant only)
 
 struct GemvPlan {
@@ -577,10 +596,16 @@ template <int G, int MT, int NW>
 static void launch_fused_t(const uint8_t* w, const float* x, float* y, float* part, unsigned* counters, int64_t Ng,
                            int64_t Kg, int64_t N, int rows, GemvPlan p, const FusedOps& o, hipStream_t st) {
     const int64_t K = Kg * G;
+    // Two k-splits and no sums of squares wanted: the splits meet through one 64-bit exchange per output, in
+    // slots behind the arrival counters in the zeroed head of the workspace (if they fit there).
+    const int64_t slot_bytes = (int64_t)rows * Ng * kGroupN * 8;
+    const int exchange = g_exchange_handoff && p.S == 2 && !o.glu && o.sumsq_out == nullptr &&
+                         slot_bytes <= LLMOPS_FC_COUNTER_BYTES - kTicketBytes;
+    if (exchange) part = reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(counters) + kTicketBytes);
 #define LLMOPS_FUSED(MODE, GRID)                                                                                      \
     fc_gemv_fused_kernel<G, MT, NW, MODE><<<(unsigned)(GRID), NW * 64, 0, st>>>(                                      \
         w, x, y, part, counters, (int)Kg, K, N, rows, p.S, p.steps_per_split, o.residual, o.norm_w, o.eps, o.sumsq_in, \
-        o.sumsq_parts, o.sumsq_out)
+        o.sumsq_parts, o.sumsq_out, exchange)
     const bool sums = o.norm_w != nullptr && o.sumsq_in != nullptr;
     if (o.glu_in) {
         LLMOPS_FUSED(kGluIn, Ng * p.S);
@@ -674,6 +699,10 @@ int launch_gemv_partials(const uint8_t* w, const int8_t* xq, int32_t* acc, int64
 }  // namespace llmops
 
 extern "C" void llmops_fc_set_tuning(int target_workgroups, int waves_per_workgroup) {
+    if (target_workgroups == -2 || target_workgroups == -3) {  // hand-off of two k-splits: -2 exchange slots, -3 ticket
+        llmops::g_exchange_handoff = target_workgroups == -2;
+        return;
+    }
     if (target_workgroups > 0) llmops::g_target_workgroups = target_workgroups > 4096 ? 4096 : target_workgroups;
     if (waves_per_workgroup >= 0) llmops::g_waves_per_workgroup = waves_per_workgroup;
 }

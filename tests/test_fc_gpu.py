@@ -316,6 +316,38 @@ def test_fc_decode_gate_up_input(ops, orc, G, rows, N, K):
         ops.fc_Q4A_decode(dev(gu), dev(pw), N, norm=(torch.ones(K, device="cuda"), 1e-5), glu_in=True)
 
 
+@pytest.mark.parametrize("rows", [1, 2, 4, 5, 8])
+@pytest.mark.parametrize("N,K", [(4096, 11008), (4090, 11008), (3000, 5632)])
+def test_fc_two_k_splits_both_handoffs(ops, orc, rows, N, K):
+    """Shapes the planner cuts into two k-splits per strip (fewer strips than compute units, long K): the
+    splits meet through one 64-bit exchange per output (default) or through the arrival ticket.  Both
+    against the oracle, bit-equal to each other, bit-equal over repeated launches (the slots are left
+    empty), with and without the residual; ragged N (the padding columns never touch a slot)."""
+    from llmops import _lib
+    lib = _lib.load()
+    rng = np.random.default_rng(rows + N)
+    x = rng.standard_normal((1, rows, K)).astype(np.float32)
+    w = (rng.standard_normal((N, K)) * 0.02).astype(np.float32)
+    res = rng.standard_normal((1, rows, N)).astype(np.float32)
+    pw = dev(orc.quant_w(w, 128))
+    want = orc.fc(x, host(pw), N)
+    got = {}
+    try:
+        for knob in (-2, -3, -2):
+            lib.llmops_fc_set_tuning(knob, -1)
+            a = ops.fc_Q4A(dev(x), pw, N)
+            b = ops.fc_Q4A(dev(x), pw, N)
+            c = ops.fc_Q4A_decode(dev(x), pw, N, residual=dev(res))
+            assert torch.equal(a, b)
+            assert max_rel_err(host(a), want) <= 1e-5
+            assert max_rel_err(host(c), want + res) <= 1e-5
+            if got:
+                assert torch.equal(a, got["a"]) and torch.equal(c, got["c"])
+            got = {"a": a, "c": c}
+    finally:
+        lib.llmops_fc_set_tuning(-2, -1)
+
+
 @pytest.mark.parametrize("rows", [17, 48, 100, 128, 129, 200, 256])
 @pytest.mark.parametrize("N,K", [(2070, 1024), (4096, 640), (2048, 2816)])
 def test_fc_prefill_mid_rows_vs_oracle(ops, orc, rows, N, K):
