@@ -280,13 +280,14 @@ __global__ __launch_bounds__(NW * 64, (MT == 1 ? NW / 2 : 1)) void fc_gemv_fused
     // They are only added up after the first weight loads have been issued (below): using them here
     // would make the wave wait for them before it asks for anything else.
     float p4[(NORM && SUMS) ? MT : 1][4];
-    if (NORM && SUMS) {
+    if (NORM && SUMS) {  // at most 256 parts (the launcher sees to it); what lies beyond a row's parts reads as 0
 #pragma unroll
-        for (int r = 0; r < MT; r++)
+        for (int r = 0; r < MT; r++) {
+            const buffer_rsrc ss_rs = make_rsrc(sumsq_in + (int64_t)r * sumsq_parts, r < rows ? (uint32_t)sumsq_parts * 4u : 0u);
 #pragma unroll
-            for (int u = 0; u < 4; u++)
-                p4[(NORM && SUMS) ? r : 0][u] =
-                    (r < rows && lane + 64 * u < sumsq_parts) ? sumsq_in[(int64_t)r * sumsq_parts + lane + 64 * u] : 0.0f;
+            for (int u = 0; u < 4; u++) p4[(NORM && SUMS) ? r : 0][u] = buf_ldf1(ss_rs, (uint32_t)(lane + 64 * u) * 4u, 0u);
+        }
+        __builtin_amdgcn_sched_barrier(0);  // asked for first, used after everything else has been asked for
     } else if (NORM) {
 #pragma unroll
         for (int r = 0; r < MT; r++)
@@ -315,45 +316,54 @@ __global__ __launch_bounds__(NW * 64, (MT == 1 ? NW / 2 : 1)) void fc_gemv_fused
     const buffer_rsrc strip_rs = make_rsrc(strip, (uint32_t)Kg * (uint32_t)block_bytes(G));
     const buffer_rsrc x_rs = make_rsrc(x, (uint32_t)rows * (uint32_t)xstride * 4u);
     const buffer_rsrc nw_rs = make_rsrc(NORM ? norm_w : x, NORM ? (uint32_t)K * 4u : 0u);
-#define LLMOPS_LOAD_BLOCK(ST, T) load_step_buf(ST, strip_rs, (T), lane)
-#define LLMOPS_LOAD_PAIR(P, TP)                                                                                  \
-    do {                                                                                                         \
-        const bool ok_ = first_of_pair || (TP) + 1 < tr.t1;                                                      \
-        const uint32_t lo_ = (uint32_t)lane * 16u, so_ = (uint32_t)(TP) * 512u;                                  \
+#define LLMOPS_LOAD_PAIR(P, TP, WANT)                                                                            \
+    do { /* branch-free: what is not wanted is asked for at an offset that returns 0 (see kNoLoad) */            \
+        const bool ok_ = (WANT) && (first_of_pair || (TP) + 1 < tr.t1);                                          \
+        const uint32_t so_ = (uint32_t)(TP) * 512u;                                                              \
         _Pragma("unroll") for (int r = 0; r < MT; r++) {                                                         \
             const uint32_t ro_ = so_ + (uint32_t)r * (uint32_t)xstride * 4u;                                     \
-            const bool okr_ = ok_ && r < rows;                                                                   \
-            P.xv[r] = okr_ ? buf_ldf4(x_rs, lo_, ro_) : make_float4(0.f, 0.f, 0.f, 0.f);                         \
-            if (GLUIN) P.uv[GLUIN ? r : 0] = okr_ ? buf_ldf4(x_rs, lo_, ro_ + (uint32_t)K * 4u) : make_float4(0.f, 0.f, 0.f, 0.f); \
+            const uint32_t lo_ = (ok_ && r < rows) ? (uint32_t)lane * 16u : kNoLoad;                             \
+            P.xv[r] = buf_ldf4(x_rs, lo_, ro_);                                                                  \
+            if (GLUIN) P.uv[GLUIN ? r : 0] = buf_ldf4(x_rs, lo_, ro_ + (uint32_t)K * 4u);                        \
         }                                                                                                        \
-        if (NORM) P.wv = ok_ ? buf_ldf4(nw_rs, lo_, so_) : make_float4(0.f, 0.f, 0.f, 0.f);                      \
-        LLMOPS_LOAD_BLOCK(P.a, (TP));                                                                            \
-        if ((TP) + 1 < tr.t1) LLMOPS_LOAD_BLOCK(P.b, (TP) + 1);                                                  \
+        if (NORM) P.wv = buf_ldf4(nw_rs, ok_ ? (uint32_t)lane * 16u : kNoLoad, so_);                             \
+        __builtin_amdgcn_sched_barrier(0); /* the compiler's scheduler must not move the weights ahead */       \
+        load_step_buf(P.a, strip_rs, (TP), lane, (WANT));                                                        \
+        load_step_buf(P.b, strip_rs, (TP) + 1, lane, (WANT) && (TP) + 1 < tr.t1);                                \
+        __builtin_amdgcn_sched_barrier(0);                                                                       \
     } while (0)
-    if (tr.t0 < tr.t1) {
-        if constexpr (G == 128) {
-            LLMOPS_LOAD_PAIR(P0, tr.t0);
-        } else {
+    // Group 128: the first pair is asked for inside the region that uses it (below), so that loads,
+    // statistic and loop stay in one block in this order; only the statistic that needs a workgroup
+    // barrier (rmsnorm from the row) must run in every wave, and its loads are issued here.
+    constexpr bool kBarrierStat = NORM && !SUMS;
+    if constexpr (G == 128) {
+        if constexpr (kBarrierStat) LLMOPS_LOAD_PAIR(P0, tr.t0, tr.t0 < tr.t1);
+    } else if (tr.t0 < tr.t1) {
 #pragma unroll
-            for (int r = 0; r < MT; r++)
-                if (r < rows) {
-                    load_x<G>(xcur[r], x + (int64_t)r * xstride, tr.t0, K, lane);
-                    if (GLUIN) load_x<G>(ucur[GLUIN ? r : 0], x + (int64_t)r * xstride + K, tr.t0, K, lane);
-                }
-            if (NORM) load_x<G>(wcur, norm_w, tr.t0, K, lane);
-            load_step<G>(cur, strip, tr.t0, Kg, lane);
-        }
+        for (int r = 0; r < MT; r++)
+            if (r < rows) {
+                load_x<G>(xcur[r], x + (int64_t)r * xstride, tr.t0, K, lane);
+                if (GLUIN) load_x<G>(ucur[GLUIN ? r : 0], x + (int64_t)r * xstride + K, tr.t0, K, lane);
+            }
+        if (NORM) load_x<G>(wcur, norm_w, tr.t0, K, lane);
+        load_step<G>(cur, strip, tr.t0, Kg, lane);
     }
 
     float rsn[MT];
+    // statistic from the handed-over sums; the empty statement the partial sums pass through keeps the
+    // compiler from adding them up, and therefore waiting for them, before the loads issued after them
+#define LLMOPS_SUMS_STAT                                                                                         \
+    _Pragma("unroll") for (int r = 0; r < MT; r++) {                                                             \
+        const int rr = (NORM && SUMS) ? r : 0;                                                                   \
+        asm volatile("" : "+v"(p4[rr][0]), "+v"(p4[rr][1]), "+v"(p4[rr][2]), "+v"(p4[rr][3])::"memory");        \
+        const float a = (p4[rr][0] + p4[rr][1]) + (p4[rr][2] + p4[rr][3]);                                       \
+        rsn[r] = 1.0f / sqrtf(wave_sum_dpp(a) / (float)K + eps);                                                 \
+    }
     if (NORM && SUMS) {
 #pragma unroll
-        for (int r = 0; r < MT; r++) {
-            const int rr = (NORM && SUMS) ? r : 0;
-            float a = (p4[rr][0] + p4[rr][1]) + (p4[rr][2] + p4[rr][3]);
-            if (r < rows)
-                for (int i = lane + 256; i < sumsq_parts; i += 64) a += sumsq_in[(int64_t)r * sumsq_parts + i];
-            rsn[r] = 1.0f / sqrtf(wave_sum_dpp(a) / (float)K + eps);
+        for (int r = 0; r < MT; r++) rsn[r] = 0.0f;
+        if constexpr (G != 128) {
+            LLMOPS_SUMS_STAT
         }
     } else if (NORM) {
 #pragma unroll
@@ -424,11 +434,19 @@ __global__ __launch_bounds__(NW * 64, (MT == 1 ? NW / 2 : 1)) void fc_gemv_fused
         }                                                                                             \
         __builtin_amdgcn_wave_barrier(); /* reads stay ahead of the next pair's writes */             \
     } while (0)
-        // Most shapes give a wave one pair; a longer run asks for the next pair only when this one is done,
-        // which keeps the registers of the two from overlapping (64 in all).
-        for (int tp = tr.t0; tp < tr.t1; tp += 2) {
-            LLMOPS_PAIR(P0, tp);
-            if (tp + 2 < tr.t1) LLMOPS_LOAD_PAIR(P0, tp + 2);
+        if (tr.t0 < tr.t1) {
+            if constexpr (!kBarrierStat) {
+                LLMOPS_LOAD_PAIR(P0, tr.t0, true);
+                if constexpr (NORM && SUMS) {
+                    LLMOPS_SUMS_STAT
+                }
+            }
+            // Most shapes give a wave one pair; a longer run asks for the next pair only when this one is
+            // done, which keeps the registers of the two from overlapping (64 in all).
+            for (int tp = tr.t0; tp < tr.t1; tp += 2) {
+                LLMOPS_PAIR(P0, tp);
+                if (tp + 2 < tr.t1) LLMOPS_LOAD_PAIR(P0, tp + 2, true);
+            }
         }
 #undef LLMOPS_PAIR
 #undef LLMOPS_BLOCK
@@ -475,7 +493,7 @@ __global__ __launch_bounds__(NW * 64, (MT == 1 ? NW / 2 : 1)) void fc_gemv_fused
         }
     }
 #undef LLMOPS_LOAD_PAIR
-#undef LLMOPS_LOAD_BLOCK
+#undef LLMOPS_SUMS_STAT
 
     if (!GLU) {
         if (NORM) {
@@ -606,7 +624,8 @@ static void launch_fused_t(const uint8_t* w, const float* x, float* y, float* pa
     fc_gemv_fused_kernel<G, MT, NW, MODE><<<(unsigned)(GRID), NW * 64, 0, st>>>(                                      \
         w, x, y, part, counters, (int)Kg, K, N, rows, p.S, p.steps_per_split, o.residual, o.norm_w, o.eps, o.sumsq_in, \
         o.sumsq_parts, o.sumsq_out, exchange)
-    const bool sums = o.norm_w != nullptr && o.sumsq_in != nullptr;
+    // (the kernel reads up to 256 handed-over partial sums per row; with more, the statistic is recomputed)
+    const bool sums = o.norm_w != nullptr && o.sumsq_in != nullptr && o.sumsq_parts <= 256;
     if (o.glu_in) {
         LLMOPS_FUSED(kGluIn, Ng * p.S);
     } else if (o.glu) {

@@ -99,9 +99,17 @@ __device__ __forceinline__ float4 buf_ldf4(buffer_rsrc r, uint32_t voff, uint32_
     const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 0);
     return make_float4(__uint_as_float(v.x), __uint_as_float(v.y), __uint_as_float(v.z), __uint_as_float(v.w));
 }
-__device__ __forceinline__ void load_step_buf(Step<128>& st, buffer_rsrc strip, int step, int lane) {
+__device__ __forceinline__ float buf_ldf1(buffer_rsrc r, uint32_t voff, uint32_t soff) {
+    return __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 0));
+}
+// A lane offset no descriptor covers: the load returns 0 without touching memory.  Loads that are not
+// wanted are issued with it instead of being branched around: the hardware counts outstanding loads
+// in issue order, and only a wave whose every path issues the same loads can wait for exactly the one
+// it needs (a branch around a younger load makes the compiler wait for all of them).
+constexpr uint32_t kNoLoad = 0xFFFFFF00u;
+__device__ __forceinline__ void load_step_buf(Step<128>& st, buffer_rsrc strip, int step, int lane, bool wanted = true) {
     const uint32_t so = (uint32_t)step * (uint32_t)block_bytes(128);
-    const uint32_t wo = (uint32_t)lane * 16u, qo = (uint32_t)(lane & 7) * 8u;
+    const uint32_t wo = wanted ? (uint32_t)lane * 16u : kNoLoad, qo = wanted ? (uint32_t)(lane & 7) * 8u : kNoLoad;
     st.valid = true;
     // constant parts go to the scalar offset: the lane offsets stay two registers for the whole loop
     st.w[0] = buf_ldg16_nt(strip, wo, so);
