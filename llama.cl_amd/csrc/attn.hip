@@ -292,6 +292,20 @@ __device__ __forceinline__ float4 rope4(const float* base, int e4, const float* 
     return make_float4(r[0], r[1], r[2], r[3]);
 }
 
+// the same on values already in registers: `own` = the lane's 4 elements at e4, `other` = their partners
+__device__ __forceinline__ float4 rope4_regs(float4 own, float4 other, int e4, const float* cs, const float* sn, int half) {
+    if (e4 >= 2 * half) return own;
+    const bool low = e4 < half;
+    const int f0 = low ? e4 : e4 - half;
+    float o[4] = {own.x, own.y, own.z, own.w}, p[4] = {other.x, other.y, other.z, other.w}, r[4];
+#pragma unroll
+    for (int c = 0; c < 4; c++) r[c] = low ? cs[f0 + c] * o[c] - sn[f0 + c] * p[c] : sn[f0 + c] * p[c] + cs[f0 + c] * o[c];
+    return make_float4(r[0], r[1], r[2], r[3]);
+}
+__device__ __forceinline__ int rope_partner(int e4, int half) {
+    return e4 >= 2 * half ? e4 : (e4 < half ? e4 + half : e4 - half);
+}
+
 template <typename T, int PW>
 __global__ __launch_bounds__(256) void attn_decode_kernel(float* q, float* k, const float* __restrict__ v,
                                                            const float* __restrict__ inv_freq, int half, T* kc, T* vc,
@@ -311,45 +325,59 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(float* q, float* k, co
     T* kbase = kc + bh * maxlen * S;
     T* vbase = vc + bh * maxlen * S;
 
+    // Loads return in issue order and a wave can only wait for "all but the youngest n".  So the small
+    // loads whose data the rotation needs go first, then the K rows, then the V rows: the cos/sin table,
+    // the rotation of q (and k) and the scores are then computed while the rows behind them are still in
+    // flight, instead of after the last V row has landed.
+    const int slot = slots[0];
+    const bool slot_ok = slot >= 0 && slot < maxlen;
+    // the workgroup that owns the new token's row (or the last chunk, if the row lies beyond kvLen)
+    const int owner = (slot_ok && slot / C < nchunks) ? slot / C : nchunks - 1;
+    const int e4 = e * 4, ep = rope_partner(e4, half);
+    const float freq = inv_freq[min((int)threadIdx.x, half - 1)];
+    const float4 q_own = *reinterpret_cast<const float4*>(q + bh * S + e4);
+    const float4 q_oth = *reinterpret_cast<const float4*>(q + bh * S + ep);
+    float4 kn = make_float4(0.f, 0.f, 0.f, 0.f), k_oth = kn, vn = kn;
+    if (chunk == owner) {  // (uniform; older than the cache rows, so it does not blur the waits for them)
+        kn = *reinterpret_cast<const float4*>(k + bh * S + e4);
+        k_oth = *reinterpret_cast<const float4*>(k + bh * S + ep);
+        vn = *reinterpret_cast<const float4*>(v + bh * S + e4);
+    }
+    __builtin_amdgcn_sched_barrier(0);
     float4 kv[NL], vv[NL];
 #pragma unroll
     for (int i = 0; i < NL; i++) {
         const int64_t p = p0 + wave * PW + i * 2 + hf;
         const int64_t pc = p < kvLen ? p : kvLen - 1;
-        kv[i] = load4(kbase + pc * S + e * 4);
-        vv[i] = load4(vbase + pc * S + e * 4);
+        kv[i] = load4(kbase + pc * S + e4);
     }
-    const int slot = slots[0];
-    const bool slot_ok = slot >= 0 && slot < maxlen;
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < NL; i++) {
+        const int64_t p = p0 + wave * PW + i * 2 + hf;
+        const int64_t pc = p < kvLen ? p : kvLen - 1;
+        vv[i] = load4(vbase + pc * S + e4);
+    }
+    __builtin_amdgcn_sched_barrier(0);
     if (threadIdx.x < half) {
-        const float xita = inv_freq[threadIdx.x] * (float)position_id;
+        const float xita = freq * (float)position_id;
         cs_sh[threadIdx.x] = cosf(xita);
         sn_sh[threadIdx.x] = sinf(xita);
     }
     __syncthreads();
-    const float4 qv = rope4(q + bh * S, e * 4, cs_sh, sn_sh, half);
-    // the workgroup that owns the new token's row (or the last chunk, if the row lies beyond kvLen)
-    const int owner = (slot_ok && slot / C < nchunks) ? slot / C : nchunks - 1;
+    const float4 qv = rope4_regs(q_own, q_oth, e4, cs_sh, sn_sh, half);
     if (chunk == owner) {
-        float4 kn = rope4(k + bh * S, e * 4, cs_sh, sn_sh, half);
-        float4 vn = *reinterpret_cast<const float4*>(v + bh * S + e * 4);
+        kn = rope4_regs(kn, k_oth, e4, cs_sh, sn_sh, half);
         __syncthreads();  // every wave has read the raw k before it is overwritten
         if (wave == 0 && hf == 0) {
-            *reinterpret_cast<float4*>(k + bh * S + e * 4) = kn;
+            *reinterpret_cast<float4*>(k + bh * S + e4) = kn;
             if (slot_ok) {
-                store4<T>(kbase + (int64_t)slot * S + e * 4, kn);
-                store4<T>(vbase + (int64_t)slot * S + e * 4, vn);
+                store4<T>(kbase + (int64_t)slot * S + e4, kn);
+                store4<T>(vbase + (int64_t)slot * S + e4, vn);
             }
         }
         kn = make_float4(cache_round<T>(kn.x), cache_round<T>(kn.y), cache_round<T>(kn.z), cache_round<T>(kn.w));
         vn = make_float4(cache_round<T>(vn.x), cache_round<T>(vn.y), cache_round<T>(vn.z), cache_round<T>(vn.w));
-#pragma unroll
-        for (int i = 0; i < NL; i++) {
-            if (p0 + wave * PW + i * 2 + hf == slot) {
-                kv[i] = kn;
-                vv[i] = vn;
-            }
-        }
     }
     const float d_scale = 1.0f / sqrtf((float)S);
     // NL partial dot products per lane, each to be summed over the 32 lanes of a half-wave.  Summing
@@ -357,6 +385,11 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(float* q, float* k, co
     // they add: at every exchange a lane keeps one half of its rows and hands the other half to its
     // partner, so NL rows cost NL/2 + NL/4 + .. + 1 exchanges plus one per remaining lane bit.
     float sp[NL];
+    if (chunk == owner) {  // the new token's row comes from registers (K here, V where the V rows are used)
+#pragma unroll
+        for (int i = 0; i < NL; i++)
+            if (p0 + wave * PW + i * 2 + hf == slot) kv[i] = kn;
+    }
 #pragma unroll
     for (int i = 0; i < NL; i++) {
         float s = qv.x * kv[i].x;
@@ -402,6 +435,11 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(float* q, float* k, co
         }
     }
     __syncthreads();
+    if (chunk == owner) {
+#pragma unroll
+        for (int i = 0; i < NL; i++)
+            if (p0 + wave * PW + i * 2 + hf == slot) vv[i] = vn;
+    }
     float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
     for (int i = 0; i < NL; i++) {
