@@ -236,10 +236,38 @@ __device__ __forceinline__ float merge_chunks(const float* rec, int nchunks, int
 __global__ __launch_bounds__(128) void attn_merge_kernel(float* __restrict__ q, const float* __restrict__ part, int64_t qL,
                                                           int64_t H, int nchunks) {
     constexpr int S = 128;
+    __shared__ float wsh[2][64];
     const int64_t bhq = blockIdx.x;
     const int64_t pq = bhq % qL, h = (bhq / qL) % H, b = bhq / (qL * H);
     const float* rec = part + (int64_t)bhq * nchunks * (S + 2);
-    const float r = merge_chunks(rec, nchunks, threadIdx.x, [](const float* p) { return *p; });
+    float r;
+    if (nchunks <= 64) {
+        // The chunk weights exp(m_c - M) / sum are the same for all 128 output elements: each wave computes
+        // them once, one chunk per lane (one expf per lane instead of one per chunk and thread), and every
+        // thread then only accumulates its element over the chunks.  Loads in order of use (statistics, then
+        // the partial outputs, 16 in flight), addresses clamped instead of branched around.
+        const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+        const float* rc = rec + (int64_t)min(lane, nchunks - 1) * (S + 2);
+        const float m = rc[0], sm0 = rc[1];
+        float acc = 0.0f;
+        const float mm = lane < nchunks ? m : -FLT_MAX;
+        const float sm = lane < nchunks ? sm0 : 0.0f;
+        const float M = wave_max(mm);
+        const float w = (sm == 0.0f) ? 0.0f : expf(mm - M);
+        const float den = wave_sum(w * sm);
+        wsh[wave][lane] = w * (1.0f / den);
+        __builtin_amdgcn_wave_barrier();
+        for (int c0 = 0; c0 < nchunks; c0 += 16) {
+            float o[16];
+#pragma unroll
+            for (int u = 0; u < 16; u++) o[u] = rec[(int64_t)min(c0 + u, nchunks - 1) * (S + 2) + 2 + threadIdx.x];
+#pragma unroll
+            for (int u = 0; u < 16; u++) acc = fmaf(c0 + u < nchunks ? wsh[wave][c0 + u] : 0.0f, o[u], acc);
+        }
+        r = acc;
+    } else {
+        r = merge_chunks(rec, nchunks, threadIdx.x, [](const float* p) { return *p; });
+    }
     q[((b * qL + pq) * H + h) * S + threadIdx.x] = r;
 }
 
