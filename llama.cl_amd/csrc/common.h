@@ -61,6 +61,14 @@ __device__ __forceinline__ int dot8_q4(uint32_t w, int xlo, int xhi, int acc) {
     return acc;
 }
 
+// silu(gate) * up (itrans "silu" + imul, ops/op_misc.hpp:83-138) as every fused form of it computes it:
+// the sigmoid's reciprocal is the hardware's (1 ulp) rather than an IEEE division -- the reference's own
+// uses the 12-bit rcpps (ops/utils.hpp:373-378) -- and all fused forms share this one expression so that
+// they agree bit for bit.
+__device__ __forceinline__ float silu_times(float gate, float up) {
+    return up * (gate * __builtin_amdgcn_rcpf(1.0f + expf(-gate)));
+}
+
 __device__ __forceinline__ float wave_max(float v) {
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));

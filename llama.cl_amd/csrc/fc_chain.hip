@@ -363,7 +363,7 @@ __global__ __launch_bounds__(kChainThreads) void fc_chain_kernel(const ChainOpDe
                     }
                 }
                 float v = sum[0];
-                if (us == 2) v = sum[1] * (v * (1.0f / (1.0f + expf(-v))));  // silu(gate)*up (ops/op_misc.hpp:83-138)
+                if (us == 2) v = silu_times(v, sum[1]);  // silu(gate)*up (ops/op_misc.hpp:83-138)
                 v += resv;
                 st_pair(op.y_pairs + n, v, epoch);
                 if (n < op.N_out) *(gfloat*)(op.y + n) = v;

@@ -420,10 +420,10 @@ __global__ __launch_bounds__(NW * 64, (MT == 1 ? NW / 2 : 1)) void fc_gemv_fused
             }                                                                                         \
             if (GLUIN) { /* silu(gate)*up, the arithmetic of silu_mul_kernel */                       \
                 const float4 u = P.uv[GLUIN ? r : 0];                                                 \
-                v.x = u.x * (v.x * (1.0f / (1.0f + expf(-v.x))));                                     \
-                v.y = u.y * (v.y * (1.0f / (1.0f + expf(-v.y))));                                     \
-                v.z = u.z * (v.z * (1.0f / (1.0f + expf(-v.z))));                                     \
-                v.w = u.w * (v.w * (1.0f / (1.0f + expf(-v.w))));                                     \
+                v.x = silu_times(v.x, u.x);                                                           \
+                v.y = silu_times(v.y, u.y);                                                           \
+                v.z = silu_times(v.z, u.z);                                                           \
+                v.w = silu_times(v.w, u.w);                                                           \
             }                                                                                         \
             quantize_pair(v, &xs[wave][r], lane);                                                     \
         }                                                                                             \
@@ -468,7 +468,7 @@ __global__ __launch_bounds__(NW * 64, (MT == 1 ? NW / 2 : 1)) void fc_gemv_fused
                     if (NORM) xcur[r].v[0] = xcur[r].v[0] * rsn[r] * wcur.v[0];
                     if (GLUIN) {  // silu(gate)*up, the arithmetic of silu_mul_kernel
                         const float g = xcur[r].v[0];
-                        xcur[r].v[0] = ucur[GLUIN ? r : 0].v[0] * (g * (1.0f / (1.0f + expf(-g))));
+                        xcur[r].v[0] = silu_times(g, ucur[GLUIN ? r : 0].v[0]);
                     }
                     Slot* slot = &xs[wave][r];
                     quantize_step<G>(xcur[r], slot, lane);
@@ -526,7 +526,7 @@ __global__ __launch_bounds__(NW * 64, (MT == 1 ? NW / 2 : 1)) void fc_gemv_fused
             u += red[GLU ? w + NWS : w][trow][tn];
         }
         const int64_t n = (int64_t)blockIdx.x * kGroupN + tn;  // N = number of output columns (F)
-        if (n < N) y[(int64_t)trow * N + n] = u * (g * (1.0f / (1.0f + expf(-g))));
+        if (n < N) y[(int64_t)trow * N + n] = silu_times(g, u);
     }
 }
 

@@ -68,7 +68,7 @@ __global__ void silu_mul_kernel(const float* __restrict__ gu, float* __restrict_
     if (i >= rows * F) return;
     const int64_t r = i / F, c = i % F;
     const float g = gu[r * 2 * F + c], u = gu[r * 2 * F + F + c];
-    out[i] = u * (g * (1.0f / (1.0f + expf(-g))));
+    out[i] = silu_times(g, u);
 }
 
 template <bool MUL>
