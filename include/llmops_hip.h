@@ -121,6 +121,7 @@ int llmops_fc_Q4A_residual(const float* x, int64_t rows, int64_t K, const int8_t
  *                 residual add); not with glu == 1
  *   sumsq_in, sumsq_parts : with norm_w: fp32 [rows,sumsq_parts] whose row sums are sum(x^2) -- what the
  *                 FC that produced x left in its sumsq_out -- so that the rmsnorm does not read the row again
+ *                 (up to 256 parts; with more the statistic is computed from the row as without sumsq_in)
  * N_out is the number of output columns (Ng*32-ish; Ng/2*32-ish with glu == 1). */
 int llmops_fc_Q4A_decode(const float* x, int64_t rows, int64_t K, const int8_t* weiq, int64_t Ng, int64_t Kg,
                          int group_k, int64_t N_out, const float* norm_w, float eps, const float* residual, int glu,

@@ -287,6 +287,25 @@ def test_fc_decode_sumsq_handover(ops, orc, G, rows, N, K):
         assert max_rel_err(b, orc.fc(orc.rmsnorm(host(y), nw, 1e-5), host(p2), F)) <= 1e-3
 
 
+@pytest.mark.parametrize("rows", [1, 3])
+def test_fc_decode_sumsq_handover_many_parts(ops, orc, rows):
+    """A producer with more than 256 strips (N = 16384: 512 partial sums): the consumer does not take the
+    handed-over sums (it reads at most 256) but computes the statistic from the row -- same result as
+    without them, and against the oracle."""
+    rng = np.random.default_rng(rows)
+    K1, N1, F = 256, 16384, 96
+    x = rng.standard_normal((1, rows, K1)).astype(np.float32)
+    p1 = dev(orc.quant_w((rng.standard_normal((N1, K1)) * 0.05).astype(np.float32), 128))
+    y, ss = ops.fc_Q4A_decode(dev(x), p1, N1, want_sumsq=True)
+    assert ss.shape == (rows, 512)
+    nw = (1.0 + 0.1 * rng.standard_normal(N1)).astype(np.float32)
+    p2 = dev(orc.quant_w((rng.standard_normal((F, N1)) * 0.02).astype(np.float32), 128))
+    a = ops.fc_Q4A_decode(y, p2, F, norm=(dev(nw), 1e-5))
+    b = ops.fc_Q4A_decode(y, p2, F, norm=(dev(nw), 1e-5), sumsq_in=ss)
+    assert torch.equal(a, b)
+    assert max_rel_err(host(b), orc.fc(orc.rmsnorm(host(y), nw, 1e-5), host(p2), F)) <= 1e-3
+
+
 @pytest.mark.parametrize("G", [32, 128])
 @pytest.mark.parametrize("rows", [1, 2, 4, 8, 20])
 @pytest.mark.parametrize("N,K", [(1000, 1024), (4096, 11008)])
