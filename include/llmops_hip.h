@@ -94,8 +94,9 @@ size_t llmops_fc_Q4A_workspace_bytes(int64_t rows, int64_t K, int64_t Ng, int64_
 /* fc_Q4A (ops/op_fc.hpp:286-426, bound at ops/main.cpp:160).
  * x fp32 [rows,K] (rows = B*M), weiq [Ng,Kg,blk] -> y fp32 [rows,N]:
  *   y[r,n] = sum_kb  fp32(d[n,kb])*dx[r,kb] * float(acc[r,n,kb]) + fp32(m[n,kb])*gsum[r,kb]
- * with acc the exact int32 dot product of 4-bit codes and int8 activation codes.  rows <= 8 runs
- * the HBM-streaming dot4 kernel, larger row counts the int8 MFMA kernel.  Requires K == Kg*G
+ * with acc the exact int32 dot product of 4-bit codes and int8 activation codes.  One or two rows (at
+ * group 32 up to 8; at group 128 3-4 rows of tensors with fewer than 256 strips as well) run the
+ * HBM-streaming dot4 kernel, larger row counts the int8 MFMA kernels.  Requires K == Kg*G
  * (every shape the reference is used with); N may be any value in (Ng*32-32, Ng*32]. */
 int llmops_fc_Q4A(const float* x, int64_t rows, int64_t K, const int8_t* weiq, int64_t Ng, int64_t Kg,
                   int group_k, int64_t N, float* y, void* workspace, size_t workspace_bytes,

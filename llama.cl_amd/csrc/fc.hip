@@ -81,8 +81,14 @@ static int fc_impl(const float* x, int64_t rows, int64_t K, const int8_t* weiq, 
     float* part = reinterpret_cast<float*>(ws + lay.off_part);
     hipStream_t st = as_stream(stream);
     const uint8_t* w = reinterpret_cast<const uint8_t*>(weiq);
-    // few rows: one launch, the streaming kernel quantizes the activations it needs on the fly
-    if (rows <= kMaxGemvRows)
+    // few rows: one launch, the streaming kernel quantizes the activations it needs on the fly.  Its work per
+    // weight byte grows with the row count (every row is quantized and dotted separately), while the time of
+    // the weight-streaming MFMA kernel below hardly depends on it, separate quantization launch included:
+    //   12288x4096 (384 strips): 3 rows 13.8 against 13.2 us, 4 rows 15.4 / 13.2, 6 rows 18.5 / 13.3, 8 rows 22.6 / 13.8
+    //   4096x11008 (128 strips, one per workgroup there): 3 rows 11.8 / 15.0, 4 rows 13.2 / 15.4, 5 rows 15.6 / 15.3
+    const bool rows_kernel = group_k == 128 && Ng >= 64 && gemm_rows_kernel_enabled();
+    const bool gemv = rows <= kMaxGemvRows && !(rows_kernel && (rows >= 5 || (rows >= 3 && Ng >= 256)));
+    if (gemv)
         return launch_gemv_fused(w, x, y, part, counters, rows, Ng, Kg, group_k, N, residual, nullptr, 0.0f, 0, nullptr, 0,
                                  nullptr, st);
     float2* xst = reinterpret_cast<float2*>(ws + lay.off_xst);
@@ -91,8 +97,7 @@ static int fc_impl(const float* x, int64_t rows, int64_t K, const int8_t* weiq, 
     // up to 16 rows are still bound by the weight stream: one strip per workgroup, MFMA inner product
     // (measured against the tiled kernel: 15 vs 18 us at 16 rows, 11008x4096; with two row tiles per
     // wave, 17..32 rows, the streaming kernel runs out of registers and loses, 32 vs 20 us)
-    if (group_k == 128 && rows <= 16 && Ng >= 64 && gemm_rows_kernel_enabled())
-        return launch_fc_rows(w, xq, xst, y, rows, Ng, Kg, N, residual, st);
+    if (rows_kernel && rows <= 16) return launch_fc_rows(w, xq, xst, y, rows, Ng, Kg, N, residual, st);
     return launch_gemm(w, xq, xd, gs, xst, y, part, rows, Ng, Kg, group_k, N, residual, st);
 }
 
