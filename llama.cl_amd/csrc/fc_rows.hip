@@ -15,6 +15,7 @@
 // The activations come pre-quantized (llmops_FC_dynamic_quantize_x_rows, with the (scale, sum)
 // pairs transposed to [Kg][rows]); the int32 sums are the same as in every other path.
 #include "common.h"
+#include "gemv_device.h"
 
 namespace llmops {
 
@@ -27,36 +28,59 @@ constexpr int kRowsBlk = 2176;
 template <int RT>
 struct RowsStage {
     uint32_t w[2][2][2];  // [64-k half][16-column tile][k8-row of the pair]
-    uint16_t d[2], m[2];  // fp16 scale and min of the lane's column in either tile
+    uint32_t d[2], m[2];  // the dword that holds the fp16 scale / min of the lane's column in either tile
     v4i_r a[RT][2];       // activation codes: row tile, 64-k half
     float2 xs[RT][4];     // (dx, gsum) of the 4 rows this lane holds results for
 };
 
+// Loads of one k-group through buffer descriptors (scalar base + scalar offset + 32-bit lane offset).
+// A stage that is not wanted (past the wave's last k-group) is asked for through descriptors of size 0,
+// which return 0 without touching memory, instead of being branched around: loads complete in issue
+// order and are counted, so only a loop whose every iteration issues the same loads lets the wave wait
+// for exactly the stage it is about to use while the next one is still in flight.
+struct RowsBufs {
+    const void *w_base, *xq_base, *xs_base;
+    uint32_t w_bytes, xq_bytes, xs_bytes;
+    uint32_t lane_w, lane_s, lane_a[2], lane_x[2];  // lane offsets (bytes); RT <= 2
+};
+
 template <int RT>
-__device__ __forceinline__ void rows_load(RowsStage<RT>& st, const uint8_t* __restrict__ strip, const int8_t* __restrict__ xq,
-                                          const float2* __restrict__ xsT, int kb, int64_t Kp, int rows, int g, int jj) {
-    const uint8_t* blk = strip + (int64_t)kb * kRowsBlk;
+__device__ __forceinline__ void rows_load(RowsStage<RT>& st, const RowsBufs& bf, int kb, int rows, bool wanted) {
+    const uint32_t sw = (uint32_t)kb * (uint32_t)kRowsBlk;
+    // (the size is chosen with scalar instructions; per-lane offsets stay loop invariants)
+    const buffer_rsrc rw = make_rsrc(bf.w_base, wanted ? bf.w_bytes : 0u);
+    const buffer_rsrc rq = make_rsrc(bf.xq_base, wanted ? bf.xq_bytes : 0u);
+    const buffer_rsrc rx = make_rsrc(bf.xs_base, wanted ? bf.xs_bytes : 0u);
+    const uint32_t lw = bf.lane_w, ls = bf.lane_s;
 #pragma unroll
     for (int h = 0; h < 2; h++)
 #pragma unroll
         for (int tau = 0; tau < 2; tau++)
 #pragma unroll
             for (int p = 0; p < 2; p++)
-                st.w[h][tau][p] = __builtin_nontemporal_load(
-                    reinterpret_cast<const uint32_t*>(blk + (8 * h + 2 * g + p) * kRowBytes + (16 * tau + jj) * 4));
+                st.w[h][tau][p] = __builtin_amdgcn_raw_buffer_load_b32(rw, lw, sw + (uint32_t)((8 * h + p) * kRowBytes + 64 * tau), 2);
 #pragma unroll
     for (int tau = 0; tau < 2; tau++) {
-        st.d[tau] = *reinterpret_cast<const uint16_t*>(blk + 2048 + 2 * (16 * tau + jj));
-        st.m[tau] = *reinterpret_cast<const uint16_t*>(blk + 2048 + 64 + 2 * (16 * tau + jj));
+        st.d[tau] = __builtin_amdgcn_raw_buffer_load_b32(rw, ls, sw + 2048u + 32u * tau, 0);
+        st.m[tau] = __builtin_amdgcn_raw_buffer_load_b32(rw, ls, sw + 2048u + 64u + 32u * tau, 0);
     }
 #pragma unroll
     for (int t = 0; t < RT; t++) {
-        const int ra = min(rows - 1, 16 * t + jj);
+        const uint32_t la = bf.lane_a[t];
 #pragma unroll
-        for (int h = 0; h < 2; h++)
-            st.a[t][h] = *reinterpret_cast<const v4i_r*>(xq + (int64_t)ra * Kp + (int64_t)kb * 128 + 64 * h + 16 * g);
+        for (int h = 0; h < 2; h++) {
+            const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rq, la, (uint32_t)kb * 128u + 64u * h, 0);
+            st.a[t][h] = v4i_r{(int)v.x, (int)v.y, (int)v.z, (int)v.w};
+        }
+        // the (scale, sum) pairs of the lane's 4 rows are contiguous: two 16-byte loads.  Rows past `rows`
+        // read the next k-group's pairs (or 0 past the end of the buffer); their results are never stored.
+        const uint32_t lx = bf.lane_x[t];
 #pragma unroll
-        for (int v = 0; v < 4; v++) st.xs[t][v] = xsT[(int64_t)kb * rows + min(rows - 1, 16 * t + 4 * g + v)];
+        for (int v2 = 0; v2 < 2; v2++) {
+            const u32x4 q = __builtin_amdgcn_raw_buffer_load_b128(rx, lx, (uint32_t)kb * (uint32_t)rows * 8u + 16u * v2, 0);
+            st.xs[t][2 * v2] = make_float2(__uint_as_float(q.x), __uint_as_float(q.y));
+            st.xs[t][2 * v2 + 1] = make_float2(__uint_as_float(q.z), __uint_as_float(q.w));
+        }
     }
 }
 
@@ -68,7 +92,8 @@ __global__ __launch_bounds__(kRowsWaves * 64, 4) void fc_rows_mfma_kernel(const 
                                                                          const float* __restrict__ residual) {
     constexpr int NW = kRowsWaves;
     __shared__ float red[NW][16 * RT][kGroupN];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // uniform: block offsets stay scalar
     const int g = lane >> 4, jj = lane & 15;
     const uint8_t* strip = weiq + (int64_t)blockIdx.x * Kg * kRowsBlk;
     const int64_t Kp = (int64_t)Kg * 128;
@@ -80,36 +105,64 @@ __global__ __launch_bounds__(kRowsWaves * 64, 4) void fc_rows_mfma_kernel(const 
 #pragma unroll
         for (int tau = 0; tau < 2; tau++) f[t][tau] = v4f_r{0.f, 0.f, 0.f, 0.f};
 
-    RowsStage<RT> cur, nxt;
-    if (t0 < t1) rows_load<RT>(cur, strip, xq, xsT, t0, Kp, rows, g, jj);
-    for (int kb = t0; kb < t1; kb++) {
-        if (kb + 1 < t1) rows_load<RT>(nxt, strip, xq, xsT, kb + 1, Kp, rows, g, jj);
-        v4i_r b[2][2];
+    RowsBufs bf;
+    bf.w_base = strip, bf.w_bytes = (uint32_t)Kg * (uint32_t)kRowsBlk;
+    bf.xq_base = xq, bf.xq_bytes = (uint32_t)rows * (uint32_t)Kp;
+    bf.xs_base = xsT, bf.xs_bytes = (uint32_t)Kg * (uint32_t)rows * 8u;
+    bf.lane_w = (uint32_t)(2 * g * kRowBytes + jj * 4);
+    bf.lane_s = (uint32_t)((jj >> 1) * 4);  // the dword with this column's fp16 scale; half_sh picks the half
+    const int half_sh = (jj & 1) * 16;
 #pragma unroll
-        for (int h = 0; h < 2; h++)
-#pragma unroll
-            for (int tau = 0; tau < 2; tau++) {
-                const uint32_t pa = cur.w[h][tau][0], pb = cur.w[h][tau][1];
-                b[h][tau] = v4i_r{(int)(pa & 0x0F0F0F0Fu), (int)((pa >> 4) & 0x0F0F0F0Fu), (int)(pb & 0x0F0F0F0Fu),
-                                  (int)((pb >> 4) & 0x0F0F0F0Fu)};
-            }
-#pragma unroll
-        for (int tau = 0; tau < 2; tau++) {
-            const float d = f16_bits_to_f32(cur.d[tau]), m = f16_bits_to_f32(cur.m[tau]);
-#pragma unroll
-            for (int t = 0; t < RT; t++) {
-                v4i_r acc = v4i_r{0, 0, 0, 0};
-                acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(cur.a[t][0], b[0][tau], acc, 0, 0, 0);
-                acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(cur.a[t][1], b[1][tau], acc, 0, 0, 0);
-#pragma unroll
-                for (int v = 0; v < 4; v++) {
-                    f[t][tau][v] = fmaf(d * cur.xs[t][v].x, (float)acc[v], f[t][tau][v]);
-                    f[t][tau][v] = fmaf(m, cur.xs[t][v].y, f[t][tau][v]);
-                }
-            }
-        }
-        cur = nxt;
+    for (int t = 0; t < RT; t++) {
+        bf.lane_a[t] = (uint32_t)min(rows - 1, 16 * t + jj) * (uint32_t)Kp + 16u * g;
+        bf.lane_x[t] = (uint32_t)(16 * t + 4 * g) * 8u;
     }
+
+    // Two stages used alternately (no register copies: a copy would have to wait for the loads it copies):
+    // the k-group being multiplied waits for exactly its own loads while the next one's are in flight.
+#define LLMOPS_ROWS_COMPUTE(ST)                                                                              \
+    do {                                                                                                     \
+        v4i_r b[2][2];                                                                                       \
+        _Pragma("unroll") for (int h = 0; h < 2; h++) _Pragma("unroll") for (int tau = 0; tau < 2; tau++) {  \
+            const uint32_t pa = ST.w[h][tau][0], pb = ST.w[h][tau][1];                                       \
+            b[h][tau] = v4i_r{(int)(pa & 0x0F0F0F0Fu), (int)((pa >> 4) & 0x0F0F0F0Fu), (int)(pb & 0x0F0F0F0Fu), \
+                              (int)((pb >> 4) & 0x0F0F0F0Fu)};                                               \
+        }                                                                                                    \
+        _Pragma("unroll") for (int tau = 0; tau < 2; tau++) {                                                \
+            const float d = f16_bits_to_f32((uint16_t)(ST.d[tau] >> half_sh));                               \
+            const float m = f16_bits_to_f32((uint16_t)(ST.m[tau] >> half_sh));                               \
+            _Pragma("unroll") for (int t = 0; t < RT; t++) {                                                 \
+                v4i_r acc = v4i_r{0, 0, 0, 0};                                                               \
+                acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(ST.a[t][0], b[0][tau], acc, 0, 0, 0);            \
+                acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(ST.a[t][1], b[1][tau], acc, 0, 0, 0);            \
+                _Pragma("unroll") for (int v = 0; v < 4; v++) {                                              \
+                    f[t][tau][v] = fmaf(d * ST.xs[t][v].x, (float)acc[v], f[t][tau][v]);                     \
+                    f[t][tau][v] = fmaf(m, ST.xs[t][v].y, f[t][tau][v]);                                     \
+                }                                                                                            \
+            }                                                                                                \
+        }                                                                                                    \
+    } while (0)
+    // Four k-groups per pass, two stages in flight, nothing loaded is live across the loop's back edge (a
+    // value that is would be copied there by the register allocator, and the copy waits for its load).  A
+    // hidden size of 4096 gives a wave exactly one pass; longer runs start each pass with a fresh pair.
+    RowsStage<RT> sa, sb;
+    for (int kb = t0; kb < t1; kb += 4) {
+        rows_load<RT>(sa, bf, kb, rows, true);
+        rows_load<RT>(sb, bf, kb + 1, rows, kb + 1 < t1);
+        __builtin_amdgcn_sched_barrier(0);
+        LLMOPS_ROWS_COMPUTE(sa);
+        __builtin_amdgcn_sched_barrier(0);
+        rows_load<RT>(sa, bf, kb + 2, rows, kb + 2 < t1);
+        __builtin_amdgcn_sched_barrier(0);
+        LLMOPS_ROWS_COMPUTE(sb);  // (a stage that was not wanted holds zeros and adds nothing)
+        __builtin_amdgcn_sched_barrier(0);
+        rows_load<RT>(sb, bf, kb + 3, rows, kb + 3 < t1);
+        __builtin_amdgcn_sched_barrier(0);
+        LLMOPS_ROWS_COMPUTE(sa);
+        __builtin_amdgcn_sched_barrier(0);
+        LLMOPS_ROWS_COMPUTE(sb);
+    }
+#undef LLMOPS_ROWS_COMPUTE
 
     // the waves' sums meet in LDS; one thread finishes each output
 #pragma unroll
