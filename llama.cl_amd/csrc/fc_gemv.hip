@@ -214,9 +214,9 @@ constexpr int kNorm = 1, kGlu = 2, kSums = 4, kGluIn = 8;
 //
 // The kernel is bound by vector-ALU issue as much as by memory (a wave64 instruction occupies its SIMD
 // for 4 cycles; at ~130-200 instructions per 2 KB block a CU streams 20-30 GB/s), so the loop is written
-// for instruction count: at group 128 a wave quantizes the activations of two blocks with one pass of all
-// 64 lanes (lanes 0-31 the first block's group, lanes 32-63 the second's) and the two weight buffers
-// alternate without register copies.
+// for instruction count: a wave quantizes 256 activations with one pass of all 64 lanes (group 128: lanes
+// 0-31 the first block's group, lanes 32-63 the second's; group 32: eight groups of 8 lanes) and uses the
+// weight buffers of the pass in place, without register copies.
 template <int G, int MT, int NW, int MODE>
 __global__ __launch_bounds__(NW * 64, (MT == 1 ? NW / 2 : 1)) void fc_gemv_fused_kernel(const uint8_t* __restrict__ weiq, const float* __restrict__ x,
                                                                  float* __restrict__ y, float* part, unsigned* counters,
@@ -231,7 +231,7 @@ __global__ __launch_bounds__(NW * 64, (MT == 1 ? NW / 2 : 1)) void fc_gemv_fused
     const int64_t xstride = GLUIN ? 2 * K : K;  // floats between activation rows
     constexpr int NWS = GLU ? NW / 2 : NW;  // waves per strip
     __shared__ float red[NW][MT][kGroupN];
-    using Slot = typename std::conditional<G == 128, XPairSlot, XSlot<G>>::type;  // a pair of blocks / a step of two
+    using Slot = XPairSlot;  // codes and scales of one pass (256 k-values)
     __shared__ __align__(16) Slot xs[NW][MT];
     __shared__ float nred[NORM ? NW : 1][MT];
     __shared__ unsigned ticket_sh;
@@ -298,28 +298,27 @@ __global__ __launch_bounds__(NW * 64, (MT == 1 ? NW / 2 : 1)) void fc_gemv_fused
                                                          : make_float4(0.f, 0.f, 0.f, 0.f);
             }
     }
-    // weight blocks in flight per wave, each with its activations (and norm weights):
-    //   group 32 : cur/nxt, one step (two blocks) each, the activations of a step fetched one step ahead
-    //   group 128: a pair of blocks; the activations of a pair are four per lane
-    Step<G> cur, nxt;
-    XRaw<G> xcur[MT], xnxt[MT], wcur, wnxt;
-    XRaw<G> ucur[GLUIN ? MT : 1], unxt[GLUIN ? MT : 1];  // the up half of a gate|up row
+    // A wave works in passes of 256 k-values: SPP steps (group 128: two blocks, one per step; group 32: four
+    // steps of two blocks each) whose weights are in flight together with the pass's activations (and norm
+    // weights), four per lane.  A wave's tile range is rounded to whole passes by its owner: steps
+    // TP .. TP+SPP-1 of a pass that lie at or beyond t1 belong to nobody here and are not asked for.
+    constexpr int SPP = (G == 128) ? 2 : 4;
     struct PairBuf {
-        Step<G> a, b;
+        Step<G> s[SPP];
         float4 xv[MT], uv[GLUIN ? MT : 1], wv;
     };
     PairBuf P0;
-    const bool first_of_pair = lane < 32;  // group 128: which block of the pair this lane's four activations belong to
-    // the pair's 256 activations are contiguous: uniform base + lane*16 bytes; activations are asked for
-    // before the weights (loads return in issue order and the quantization comes first)
-    // group 128 loads go through buffer descriptors (scalar base + scalar block offset + lane offset)
+    const int lane_step = lane / (64 / SPP);  // which step of the pass this lane's four activations belong to
+    // the pass's 256 activations are contiguous: uniform base + lane*16 bytes; activations are asked for
+    // before the weights (loads return in issue order and the quantization comes first); all loads go
+    // through buffer descriptors (scalar base + scalar block offset + lane offset)
     const buffer_rsrc strip_rs = make_rsrc(strip, (uint32_t)Kg * (uint32_t)block_bytes(G));
     const buffer_rsrc x_rs = make_rsrc(x, (uint32_t)rows * (uint32_t)xstride * 4u);
     const buffer_rsrc nw_rs = make_rsrc(NORM ? norm_w : x, NORM ? (uint32_t)K * 4u : 0u);
 #define LLMOPS_LOAD_PAIR(P, TP, WANT)                                                                            \
     do { /* branch-free: what is not wanted is asked for at an offset that returns 0 (see kNoLoad) */            \
-        const bool ok_ = (WANT) && (first_of_pair || (TP) + 1 < tr.t1);                                          \
-        const uint32_t so_ = (uint32_t)(TP) * 512u;                                                              \
+        const bool ok_ = (WANT) && (TP) + lane_step < tr.t1 && (int64_t)(TP) * Step<G>::kK + lane * 4 < K;       \
+        const uint32_t so_ = (uint32_t)(TP) * (uint32_t)(Step<G>::kK * 4);                                       \
         _Pragma("unroll") for (int r = 0; r < MT; r++) {                                                         \
             const uint32_t ro_ = so_ + (uint32_t)r * (uint32_t)xstride * 4u;                                     \
             const uint32_t lo_ = (ok_ && r < rows) ? (uint32_t)lane * 16u : kNoLoad;                             \
@@ -328,26 +327,17 @@ __global__ __launch_bounds__(NW * 64, (MT == 1 ? NW / 2 : 1)) void fc_gemv_fused
         }                                                                                                        \
         if (NORM) P.wv = buf_ldf4(nw_rs, ok_ ? (uint32_t)lane * 16u : kNoLoad, so_);                             \
         __builtin_amdgcn_sched_barrier(0); /* the compiler's scheduler must not move the weights ahead */       \
-        load_step_buf(P.a, strip_rs, (TP), lane, (WANT));                                                        \
-        load_step_buf(P.b, strip_rs, (TP) + 1, lane, (WANT) && (TP) + 1 < tr.t1);                                \
+        _Pragma("unroll") for (int i_ = 0; i_ < SPP; i_++) {                                                     \
+            if constexpr (G == 128) load_step_buf(P.s[i_], strip_rs, (TP) + i_, lane, (WANT) && (TP) + i_ < tr.t1); \
+            else load_step_buf(P.s[i_], strip_rs, (TP) + i_, Kg, lane, (WANT) && (TP) + i_ < tr.t1);             \
+        }                                                                                                        \
         __builtin_amdgcn_sched_barrier(0);                                                                       \
     } while (0)
-    // Group 128: the first pair is asked for inside the region that uses it (below), so that loads,
-    // statistic and loop stay in one block in this order; only the statistic that needs a workgroup
-    // barrier (rmsnorm from the row) must run in every wave, and its loads are issued here.
+    // The first pass is asked for inside the region that uses it (below), so that loads, statistic and
+    // loop stay in one block in this order; only the statistic that needs a workgroup barrier (rmsnorm
+    // from the row) must run in every wave, and its loads are issued here.
     constexpr bool kBarrierStat = NORM && !SUMS;
-    if constexpr (G == 128) {
-        if constexpr (kBarrierStat) LLMOPS_LOAD_PAIR(P0, tr.t0, tr.t0 < tr.t1);
-    } else if (tr.t0 < tr.t1) {
-#pragma unroll
-        for (int r = 0; r < MT; r++)
-            if (r < rows) {
-                load_x<G>(xcur[r], x + (int64_t)r * xstride, tr.t0, K, lane);
-                if (GLUIN) load_x<G>(ucur[GLUIN ? r : 0], x + (int64_t)r * xstride + K, tr.t0, K, lane);
-            }
-        if (NORM) load_x<G>(wcur, norm_w, tr.t0, K, lane);
-        load_step<G>(cur, strip, tr.t0, Kg, lane);
-    }
+    if constexpr (kBarrierStat) LLMOPS_LOAD_PAIR(P0, tr.t0, tr.t0 < tr.t1);
 
     float rsn[MT];
     // statistic from the handed-over sums; the empty statement the partial sums pass through keeps the
@@ -362,9 +352,6 @@ __global__ __launch_bounds__(NW * 64, (MT == 1 ? NW / 2 : 1)) void fc_gemv_fused
     if (NORM && SUMS) {
 #pragma unroll
         for (int r = 0; r < MT; r++) rsn[r] = 0.0f;
-        if constexpr (G != 128) {
-            LLMOPS_SUMS_STAT
-        }
     } else if (NORM) {
 #pragma unroll
         for (int r = 0; r < MT; r++) {
@@ -399,13 +386,12 @@ __global__ __launch_bounds__(NW * 64, (MT == 1 ? NW / 2 : 1)) void fc_gemv_fused
         }
     }
 
-    if constexpr (G == 128) {
 #define LLMOPS_BLOCK(ST, J)                                                                           \
     _Pragma("unroll") for (int r = 0; r < MT; r++) if (r < rows) {                                    \
         const Slot* slot = &xs[wave][r];                                                              \
         int acc[4];                                                                                   \
-        dot_step<G>(ST, slot->codes + (J) * 128, lane, acc);                                          \
-        const float2 sc = slot->scale[J];                                                             \
+        dot_step<G>(ST, slot->codes + (J) * Step<G>::kK, lane, acc);                                  \
+        const float2 sc = slot->scale[(G == 128) ? (J) : (J) * 2 + (rs >> 2)];                        \
         fold(f[r], acc, ST.dh, ST.mh, sc.x, first_row ? sc.y : 0.0f);                                 \
     }
 #define LLMOPS_PAIR(P, TP)                                                                            \
@@ -425,73 +411,34 @@ __global__ __launch_bounds__(NW * 64, (MT == 1 ? NW / 2 : 1)) void fc_gemv_fused
                 v.z = silu_times(v.z, u.z);                                                           \
                 v.w = silu_times(v.w, u.w);                                                           \
             }                                                                                         \
-            quantize_pair(v, &xs[wave][r], lane);                                                     \
+            if constexpr (G == 128) quantize_pair(v, &xs[wave][r], lane);                             \
+            else quantize_pass32(v, &xs[wave][r], lane);                                              \
         }                                                                                             \
         __builtin_amdgcn_wave_barrier(); /* LDS writes stay ahead of the reads below */               \
-        LLMOPS_BLOCK(P.a, 0)                                                                          \
-        if ((TP) + 1 < tr.t1) {                                                                       \
-            LLMOPS_BLOCK(P.b, 1)                                                                      \
+        LLMOPS_BLOCK(P.s[0], 0)                                                                       \
+        _Pragma("unroll") for (int i_ = 1; i_ < SPP; i_++) {                                          \
+            if ((TP) + i_ < tr.t1) {                                                                  \
+                LLMOPS_BLOCK(P.s[i_], i_)                                                             \
+            }                                                                                         \
         }                                                                                             \
-        __builtin_amdgcn_wave_barrier(); /* reads stay ahead of the next pair's writes */             \
+        __builtin_amdgcn_wave_barrier(); /* reads stay ahead of the next pass's writes */             \
     } while (0)
-        if (tr.t0 < tr.t1) {
-            if constexpr (!kBarrierStat) {
-                LLMOPS_LOAD_PAIR(P0, tr.t0, true);
-                if constexpr (NORM && SUMS) {
-                    LLMOPS_SUMS_STAT
-                }
-            }
-            // Most shapes give a wave one pair; a longer run asks for the next pair only when this one is
-            // done, which keeps the registers of the two from overlapping (64 in all).
-            for (int tp = tr.t0; tp < tr.t1; tp += 2) {
-                LLMOPS_PAIR(P0, tp);
-                if (tp + 2 < tr.t1) LLMOPS_LOAD_PAIR(P0, tp + 2, true);
+    if (tr.t0 < tr.t1) {
+        if constexpr (!kBarrierStat) {
+            LLMOPS_LOAD_PAIR(P0, tr.t0, true);
+            if constexpr (NORM && SUMS) {
+                LLMOPS_SUMS_STAT
             }
         }
-#undef LLMOPS_PAIR
-#undef LLMOPS_BLOCK
-    } else {
-        for (int t = tr.t0; t < tr.t1; t++) {
-            if (t + 1 < tr.t1) {
-                load_step<G>(nxt, strip, t + 1, Kg, lane);
-#pragma unroll
-                for (int r = 0; r < MT; r++)
-                    if (r < rows) {
-                        load_x<G>(xnxt[r], x + (int64_t)r * xstride, t + 1, K, lane);
-                        if (GLUIN) load_x<G>(unxt[GLUIN ? r : 0], x + (int64_t)r * xstride + K, t + 1, K, lane);
-                    }
-                if (NORM) load_x<G>(wnxt, norm_w, t + 1, K, lane);
-            }
-#pragma unroll
-            for (int r = 0; r < MT; r++) {
-                if (r < rows) {
-                    if (NORM) xcur[r].v[0] = xcur[r].v[0] * rsn[r] * wcur.v[0];
-                    if (GLUIN) {  // silu(gate)*up, the arithmetic of silu_mul_kernel
-                        const float g = xcur[r].v[0];
-                        xcur[r].v[0] = silu_times(g, ucur[GLUIN ? r : 0].v[0]);
-                    }
-                    Slot* slot = &xs[wave][r];
-                    quantize_step<G>(xcur[r], slot, lane);
-                    __builtin_amdgcn_wave_barrier();  // LDS writes stay ahead of the reads below
-                    if (cur.valid) {
-                        int acc[4];
-                        dot_step<G>(cur, slot->codes, lane, acc);
-                        const float2 sc = slot->scale[rs >> 2];
-                        fold(f[r], acc, cur.dh, cur.mh, sc.x, first_row ? sc.y : 0.0f);
-                    }
-                    __builtin_amdgcn_wave_barrier();  // reads stay ahead of the next step's writes
-                }
-            }
-            cur = nxt;
-#pragma unroll
-            for (int r = 0; r < MT; r++) xcur[r] = xnxt[r];
-            if (GLUIN) {
-#pragma unroll
-                for (int r = 0; r < MT; r++) ucur[GLUIN ? r : 0] = unxt[GLUIN ? r : 0];
-            }
-            if (NORM) wcur = wnxt;
+        // Most shapes give a wave one pass; a longer run asks for the next pass only when this one is done,
+        // which keeps the registers of the two from overlapping (64 in all).
+        for (int tp = tr.t0; tp < tr.t1; tp += SPP) {
+            LLMOPS_PAIR(P0, tp);
+            if (tp + SPP < tr.t1) LLMOPS_LOAD_PAIR(P0, tp + SPP, true);
         }
     }
+#undef LLMOPS_PAIR
+#undef LLMOPS_BLOCK
 #undef LLMOPS_LOAD_PAIR
 #undef LLMOPS_SUMS_STAT
 

@@ -118,6 +118,22 @@ __device__ __forceinline__ void load_step_buf(Step<128>& st, buffer_rsrc strip, 
     st.mh = buf_ldg8(strip, qo, so + 2048u + 64u);
 }
 
+// A group-32 step (two adjacent blocks, lane = rs*8 + quad, rs>>2 = block of the step, rs&3 = k8-row)
+// through a buffer descriptor.  A block past the strip's last (odd block count) or an unwanted step is
+// asked for at kNoLoad: zeros, which add nothing.
+__device__ __forceinline__ void load_step_buf(Step<32>& st, buffer_rsrc strip, int step, int kb_end, int lane, bool wanted = true) {
+    const int rs = lane >> 3, quad = lane & 7;
+    const bool ok = wanted && step * 2 + (rs >> 2) < kb_end;
+    const uint32_t so = (uint32_t)step * 2u * (uint32_t)block_bytes(32);
+    const uint32_t bo = (uint32_t)(rs >> 2) * (uint32_t)block_bytes(32);
+    const uint32_t wo = ok ? bo + (uint32_t)(rs & 3) * kRowBytes + (uint32_t)quad * 16u : kNoLoad;
+    const uint32_t qo = ok ? bo + (uint32_t)quad * 8u : kNoLoad;
+    st.valid = true;
+    st.w[0] = buf_ldg16_nt(strip, wo, so);
+    st.dh = buf_ldg8(strip, qo, so + 512u);
+    st.mh = buf_ldg8(strip, qo, so + 512u + 64u);
+}
+
 // int32 partial dot products of the lane's 4 columns over the lane's k8-rows of this step;
 // `codes` points at the step's activation codes (Step<G>::kK of them)
 template <int G>
@@ -213,10 +229,10 @@ struct XSlot {
     float2 scale[Step<G>::kBlocksPerStep];
 };
 
-// The same for a pair of group-128 blocks quantized in one pass
+// The same for a pass of 256 k-values quantized at once: two blocks of group 128 or eight of group 32
 struct XPairSlot {
     int8_t codes[256];
-    float2 scale[2];
+    float2 scale[8];
 };
 
 // FC_dynamic_quantize_x for one step (/root/reference/ops/op_fc.hpp:246-268): amax -> d = amax/127 ->
@@ -300,6 +316,38 @@ __device__ __forceinline__ void quantize_pair(const float4& v, XPairSlot* slot, 
     const uint32_t lo = __builtin_amdgcn_perm(u1, u0, 0x0c0c0400u), hi = __builtin_amdgcn_perm(u3, u2, 0x04000c0cu);
     *reinterpret_cast<uint32_t*>(&slot->codes[lane * 4]) = lo | hi;
     slot->scale[lane >> 5] = make_float2(d, sum);  // every lane of the half writes the same pair
+}
+
+// Eight groups of 32 at once (group g = lanes 8g..8g+7, four consecutive values per lane): the same
+// operations per value; the reduction stays inside the 8 lanes of a group (three DPP levels).
+__device__ __forceinline__ void quantize_pass32(const float4& v, XPairSlot* slot, int lane) {
+    float amax;
+    float sum = (v.x + v.y) + (v.z + v.w);
+    asm("v_max3_f32 %0, |%1|, |%2|, |%3|\n\t"
+        "v_max_f32_e64 %0, %0, |%4|"
+        : "=&v"(amax)
+        : "v"(v.x), "v"(v.y), "v"(v.z), "v"(v.w));
+    asm("s_nop 1\n\t"
+        "v_max_f32_dpp %0, %0, %0 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf\n\t"
+        "v_add_f32_dpp %1, %1, %1 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 0\n\t"
+        "v_max_f32_dpp %0, %0, %0 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf\n\t"
+        "v_add_f32_dpp %1, %1, %1 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 0\n\t"
+        "v_max_f32_dpp %0, %0, %0 row_half_mirror row_mask:0xf bank_mask:0xf\n\t"
+        "v_add_f32_dpp %1, %1, %1 row_half_mirror row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1"
+        : "+v"(amax), "+v"(sum));
+    const float d = amax / 127.0f;
+    const float id = (d != 0.0f) ? (1.0f / d) : 0.0f;
+    constexpr float kRound = 12582912.0f;  // 1.5 * 2^23
+    const uint32_t u0 = __float_as_uint(__builtin_amdgcn_fmed3f(v.x * id, -128.0f, 127.0f) + kRound);
+    const uint32_t u1 = __float_as_uint(__builtin_amdgcn_fmed3f(v.y * id, -128.0f, 127.0f) + kRound);
+    const uint32_t u2 = __float_as_uint(__builtin_amdgcn_fmed3f(v.z * id, -128.0f, 127.0f) + kRound);
+    const uint32_t u3 = __float_as_uint(__builtin_amdgcn_fmed3f(v.w * id, -128.0f, 127.0f) + kRound);
+    const uint32_t lo = __builtin_amdgcn_perm(u1, u0, 0x0c0c0400u), hi = __builtin_amdgcn_perm(u3, u2, 0x04000c0cu);
+    *reinterpret_cast<uint32_t*>(&slot->codes[lane * 4]) = lo | hi;
+    slot->scale[lane >> 3] = make_float2(d, sum);  // every lane of the group writes the same pair
 }
 
 __device__ __forceinline__ float wave_sum_dpp(float v) {
