@@ -176,6 +176,7 @@ def main():
     if not args.no_decode:
         out["decode_step"] = decode_step(torch, stream)
     if not args.no_extra:
+        out["decode_fc_g32"] = decode_fc_g32(torch, llmops, stream)
         out["prefill_gemm"] = prefill_gemm(torch, llmops, stream)
         out["decode_attention"] = decode_attention(torch, llmops, stream)
         out["prefill_attention"] = prefill_attention(torch, llmops, stream)
@@ -347,6 +348,26 @@ def prefill_gemm(torch, llmops, stream):
                                           "GB/s": round(fc_bytes(N, K, M) / us / 1e3, 1)}
             del ws, w0
     return out
+
+
+def decode_fc_g32(torch, llmops, stream):
+    """BASELINE config 1: the reference's own CPU-runnable case, one 4096x4096 FC at Q4_1 group 32, M=1
+    (seed 1), cycling 32 distinct weight copies in a replayed graph."""
+    gen = torch.Generator(device="cpu").manual_seed(1)
+    N = K = 4096
+    with torch.cuda.stream(stream):
+        w0 = llmops.offline_FC_quant_Q4A((torch.randn(N, K, generator=gen) * 0.02).cuda(), 32)
+        ws = [torch.roll(w0, i + 1, 0).contiguous() for i in range(32)]
+        x = torch.randn(1, 1, K, generator=gen).cuda()
+
+        def run():
+            for w in ws:
+                llmops.fc_Q4A(x, w, N)
+
+        us = _time_graph(torch, stream, run) * 1e3 / len(ws)
+    b = fc_bytes(N, K, 1, 32)
+    return {"4096x4096 g32 M=1": {"us": round(us, 2), "GB/s": round(b / us / 1e3, 1), "bytes": b,
+                                   "pct_hbm_peak": round(b / us / 1e3 / HBM_PEAK_GBS * 100, 2)}}
 
 
 def decode_attention(torch, llmops, stream):
