@@ -271,6 +271,10 @@ void llmops_fc_set_tuning(int target_workgroups, int waves_per_workgroup);
  * per shape and send 9..16 rows to the tiled kernel too instead of the weight-streaming MFMA kernel */
 void llmops_gemm_set_tuning(int row_tile_factor);
 
+/* weight-streaming MFMA kernel (3..16 rows): two workgroups per strip with half of K each for tensors of
+ * fewer than 256 strips (default on; 0 switches it off, for comparisons and tests) */
+void llmops_fc_rows_set_split(int on);
+
 #ifdef __cplusplus
 }
 #endif

@@ -23,7 +23,7 @@ int launch_gemm(const uint8_t* w, const int8_t* xq, const float* xd, const float
 int launch_gemm_partials(const uint8_t* w, const int8_t* xq, int32_t* acc, int64_t rows, int64_t Ng, int64_t Kg, int G,
                          bool two_groups, hipStream_t st);
 int launch_fc_rows(const uint8_t* w, const int8_t* xq, const float2* xsT, float* y, int64_t rows, int64_t Ng, int64_t Kg,
-                   int64_t N, const float* residual, hipStream_t st);
+                   int64_t N, const float* residual, unsigned long long* slots, size_t slot_bytes, hipStream_t st);
 bool gemm_rows_kernel_enabled();
 
 static inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
@@ -97,7 +97,9 @@ static int fc_impl(const float* x, int64_t rows, int64_t K, const int8_t* weiq, 
     // up to 16 rows are still bound by the weight stream: one strip per workgroup, MFMA inner product
     // (measured against the tiled kernel: 15 vs 18 us at 16 rows, 11008x4096; with two row tiles per
     // wave, 17..32 rows, the streaming kernel runs out of registers and loses, 32 vs 20 us)
-    if (rows_kernel && rows <= 16) return launch_fc_rows(w, xq, xst, y, rows, Ng, Kg, N, residual, st);
+    if (rows_kernel && rows <= 16)
+        return launch_fc_rows(w, xq, xst, y, rows, Ng, Kg, N, residual, reinterpret_cast<unsigned long long*>(ws + kTicketBytes),
+                              LLMOPS_FC_COUNTER_BYTES - kTicketBytes, st);
     return launch_gemm(w, xq, xd, gs, xst, y, part, rows, Ng, Kg, group_k, N, residual, st);
 }
 

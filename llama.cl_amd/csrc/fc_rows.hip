@@ -23,6 +23,7 @@ typedef int v4i_r __attribute__((ext_vector_type(4)));
 typedef float v4f_r __attribute__((ext_vector_type(4)));
 
 constexpr int kRowsWaves = 8;
+static int g_rows_split = 1;  // 0: never cut K in two for tensors with few strips
 constexpr int kRowsBlk = 2176;
 
 template <int RT>
@@ -89,15 +90,20 @@ __global__ __launch_bounds__(kRowsWaves * 64, 4) void fc_rows_mfma_kernel(const 
                                                                          const int8_t* __restrict__ xq,
                                                                          const float2* __restrict__ xsT,
                                                                          float* __restrict__ y, int Kg, int64_t N, int rows,
-                                                                         const float* __restrict__ residual) {
+                                                                         const float* __restrict__ residual,
+                                                                         unsigned long long* slots) {
     constexpr int NW = kRowsWaves;
     __shared__ float red[NW][16 * RT][kGroupN];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // uniform: block offsets stay scalar
     const int g = lane >> 4, jj = lane & 15;
-    const uint8_t* strip = weiq + (int64_t)blockIdx.x * Kg * kRowsBlk;
+    // slots != nullptr: two workgroups per strip, each with half of K (tensors with fewer strips than the
+    // chip has compute units); the halves meet through one 64-bit exchange per output (below)
+    const int nb = slots ? blockIdx.x >> 1 : blockIdx.x, split = slots ? blockIdx.x & 1 : 0;
+    const uint8_t* strip = weiq + (int64_t)nb * Kg * kRowsBlk;
     const int64_t Kp = (int64_t)Kg * 128;
-    const int t0 = (wave * Kg) / NW, t1 = ((wave + 1) * Kg) / NW;  // this wave's k-groups
+    const int k_lo = slots ? (split * Kg) / 2 : 0, k_n = slots ? ((split + 1) * Kg) / 2 - k_lo : Kg;
+    const int t0 = k_lo + (wave * k_n) / NW, t1 = k_lo + ((wave + 1) * k_n) / NW;  // this wave's k-groups
 
     v4f_r f[RT][2];
 #pragma unroll
@@ -176,23 +182,40 @@ __global__ __launch_bounds__(kRowsWaves * 64, 4) void fc_rows_mfma_kernel(const 
     for (int i = 0; i < RT; i++) {
         const int idx = threadIdx.x + NW * 64 * i;
         const int row = idx >> 5, col = idx & 31;
-        const int64_t n = (int64_t)blockIdx.x * kGroupN + col;
+        const int64_t n = (int64_t)nb * kGroupN + col;
         if (row < rows && n < N) {
             float v = 0.0f;
 #pragma unroll
             for (int w = 0; w < NW; w++) v += red[w][row][col];
+            if (slots != nullptr) {
+                // A slot is empty (0) or holds (1 << 32 | value bits).  Whoever finds the other half's value
+                // adds the two (a + b: the same bits whichever came first), stores the output and empties the
+                // slot for the next launch; whoever finds it empty has parked its own value and is done.
+                unsigned long long* slot = slots + ((int64_t)row * gridDim.x / 2 * kGroupN + n);
+                const unsigned long long parked = (1ull << 32) | (unsigned long long)__float_as_uint(v);
+                const unsigned long long old = __hip_atomic_exchange(slot, parked, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                if ((old >> 32) == 0ull) continue;
+                v += __uint_as_float((unsigned)(old & 0xFFFFFFFFull));
+                __hip_atomic_store(slot, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
             y[(int64_t)row * N + n] = residual ? v + residual[(int64_t)row * N + n] : v;
         }
     }
 }
 
 // rows <= 16, group 128, activations already quantized (codes [rows, Kg*128], pairs [Kg][rows])
+// `slots`: the zeroed exchange area of the FC workspace (`slot_bytes` of it), or nullptr
 int launch_fc_rows(const uint8_t* w, const int8_t* xq, const float2* xsT, float* y, int64_t rows, int64_t Ng, int64_t Kg,
-                   int64_t N, const float* residual, hipStream_t st) {
+                   int64_t N, const float* residual, unsigned long long* slots, size_t slot_bytes, hipStream_t st) {
     if (rows > 16) return fail(LLMOPS_EINVAL, "the streaming MFMA kernel takes at most 16 rows, got %lld", (long long)rows);
-    fc_rows_mfma_kernel<1><<<(unsigned)Ng, kRowsWaves * 64, 0, st>>>(w, xq, xsT, y, (int)Kg, N, (int)rows, residual);
+    // fewer strips than compute units and a K worth cutting: two workgroups per strip
+    const bool split = slots != nullptr && g_rows_split && Ng < 256 && Kg >= 16 && (size_t)rows * Ng * kGroupN * 8 <= slot_bytes;
+    fc_rows_mfma_kernel<1><<<(unsigned)(split ? 2 * Ng : Ng), kRowsWaves * 64, 0, st>>>(w, xq, xsT, y, (int)Kg, N, (int)rows, residual,
+                                                                                     split ? slots : nullptr);
     LLMOPS_LAUNCH_CHECK();
     return LLMOPS_OK;
 }
 
 }  // namespace llmops
+
+extern "C" void llmops_fc_rows_set_split(int on) { llmops::g_rows_split = on != 0; }

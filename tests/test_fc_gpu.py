@@ -367,6 +367,34 @@ def test_fc_two_k_splits_both_handoffs(ops, orc, rows, N, K):
         lib.llmops_fc_set_tuning(-2, -1)
 
 
+@pytest.mark.parametrize("rows", [3, 5, 8, 9, 13, 16])
+@pytest.mark.parametrize("N,K", [(4096, 11008), (4090, 4096), (2070, 2048), (3000, 2176)])
+def test_fc_rows_kernel_two_k_halves(ops, orc, rows, N, K):
+    """The weight-streaming MFMA kernel on tensors with fewer than 256 strips: two workgroups per strip with
+    half of K each, meeting through one 64-bit exchange per output, against one workgroup per strip: both
+    against the oracle, bit-equal over repeated launches, with and without the residual; ragged N, odd
+    k-group counts (17 = 8 + 9)."""
+    from llmops import _lib
+    lib = _lib.load()
+    rng = np.random.default_rng(rows + N)
+    x = rng.standard_normal((1, rows, K)).astype(np.float32)
+    w = (rng.standard_normal((N, K)) * 0.02).astype(np.float32)
+    res = rng.standard_normal((1, rows, N)).astype(np.float32)
+    pw = dev(orc.quant_w(w, 128))
+    want = orc.fc(x, host(pw), N)
+    try:
+        for on in (1, 0, 1):
+            lib.llmops_fc_rows_set_split(on)
+            a = ops.fc_Q4A(dev(x), pw, N)
+            b = ops.fc_Q4A(dev(x), pw, N)
+            c = ops.fc_Q4A(dev(x), pw, N, residual=dev(res))
+            assert torch.equal(a, b)
+            assert max_rel_err(host(a), want) <= 1e-5
+            assert max_rel_err(host(c), want + res) <= 1e-5
+    finally:
+        lib.llmops_fc_rows_set_split(1)
+
+
 @pytest.mark.parametrize("rows", [17, 48, 100, 128, 129, 200, 256])
 @pytest.mark.parametrize("N,K", [(2070, 1024), (4096, 640), (2048, 2816)])
 def test_fc_prefill_mid_rows_vs_oracle(ops, orc, rows, N, K):
