@@ -95,7 +95,7 @@ size_t llmops_fc_Q4A_workspace_bytes(int64_t rows, int64_t K, int64_t Ng, int64_
  * x fp32 [rows,K] (rows = B*M), weiq [Ng,Kg,blk] -> y fp32 [rows,N]:
  *   y[r,n] = sum_kb  fp32(d[n,kb])*dx[r,kb] * float(acc[r,n,kb]) + fp32(m[n,kb])*gsum[r,kb]
  * with acc the exact int32 dot product of 4-bit codes and int8 activation codes.  One or two rows (at
- * group 32 up to 8; at group 128 3-4 rows of tensors with fewer than 256 strips as well) run the
+ * group 32 up to 8; at group 128 three rows of tensors of up to 256 strips as well) run the
  * HBM-streaming dot4 kernel, larger row counts the int8 MFMA kernels.  Requires K == Kg*G
  * (every shape the reference is used with); N may be any value in (Ng*32-32, Ng*32]. */
 int llmops_fc_Q4A(const float* x, int64_t rows, int64_t K, const int8_t* weiq, int64_t Ng, int64_t Kg,
@@ -274,6 +274,11 @@ void llmops_gemm_set_tuning(int row_tile_factor);
 /* weight-streaming MFMA kernel (3..16 rows): two workgroups per strip with half of K each for tensors of
  * fewer than 256 strips (default on; 0 switches it off, for comparisons and tests) */
 void llmops_fc_rows_set_split(int on);
+
+/* llmops_fc_Q4A with 2..8 rows, group 128: from how many rows the weight-streaming MFMA kernel (separate
+ * quantization launch) replaces the streaming kernel that quantizes on the fly, for tensors of up to
+ * 256 strips and for larger ones (defaults 4 and 3; values below 2 restore them) */
+void llmops_fc_set_row_routing(int rows_from_small, int rows_from_large);
 
 #ifdef __cplusplus
 }

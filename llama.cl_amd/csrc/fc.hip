@@ -59,6 +59,10 @@ extern "C" size_t llmops_fc_Q4A_workspace_bytes(int64_t rows, int64_t K, int64_t
     return fc_layout(rows, Ng, Kg, group_k).total;
 }
 
+// from how many rows the weight-streaming MFMA kernel takes over from the streaming kernel that quantizes
+// on the fly: tensors of up to 256 strips / of more
+static int g_rows_from_small = 4, g_rows_from_large = 3;
+
 static int fc_impl(const float* x, int64_t rows, int64_t K, const int8_t* weiq, int64_t Ng, int64_t Kg, int group_k,
                    int64_t N, const float* residual, float* y, void* workspace, size_t workspace_bytes,
                    llmops_stream_t stream) {
@@ -83,11 +87,15 @@ static int fc_impl(const float* x, int64_t rows, int64_t K, const int8_t* weiq, 
     const uint8_t* w = reinterpret_cast<const uint8_t*>(weiq);
     // few rows: one launch, the streaming kernel quantizes the activations it needs on the fly.  Its work per
     // weight byte grows with the row count (every row is quantized and dotted separately), while the time of
-    // the weight-streaming MFMA kernel below hardly depends on it, separate quantization launch included:
-    //   12288x4096 (384 strips): 3 rows 13.8 against 13.2 us, 4 rows 15.4 / 13.2, 6 rows 18.5 / 13.3, 8 rows 22.6 / 13.8
-    //   4096x11008 (128 strips, one per workgroup there): 3 rows 11.8 / 15.0, 4 rows 13.2 / 15.4, 5 rows 15.6 / 15.3
+    // the weight-streaming MFMA kernel below hardly depends on it, separate quantization launch included
+    // (us, streaming / MFMA):
+    //   4096x4096 (128 strips):    2 rows  6.0 /  8.0, 3 rows  7.5 /  8.2, 4 rows  8.3 /  8.2, 8 rows 10.2 /  8.4
+    //   4096x11008 (128 strips):   2 rows  9.3 / 11.6, 3 rows 11.5 / 11.8, 4 rows 13.0 / 12.0, 8 rows 20.3 / 12.5
+    //   8192x4096 (256 strips):    2 rows  6.7 /  8.9, 3 rows  8.1 /  8.6, 4 rows  8.8 /  8.6, 8 rows 14.5 /  8.9
+    //   12288x4096 (384 strips):   2 rows  9.3 / 12.0, 3 rows 13.4 / 11.6, 4 rows 15.6 / 11.7, 8 rows 22.4 / 12.2
+    //   22016x4096 (688 strips):   2 rows 12.8 / 16.1, 3 rows 20.1 / 16.0, 4 rows 22.2 / 15.3, 8 rows 31.0 / 16.1
     const bool rows_kernel = group_k == 128 && Ng >= 64 && gemm_rows_kernel_enabled();
-    const bool gemv = rows <= kMaxGemvRows && !(rows_kernel && (rows >= 5 || (rows >= 3 && Ng >= 256)));
+    const bool gemv = rows <= kMaxGemvRows && !(rows_kernel && rows >= (Ng > 256 ? g_rows_from_large : g_rows_from_small));
     if (gemv)
         return launch_gemv_fused(w, x, y, part, counters, rows, Ng, Kg, group_k, N, residual, nullptr, 0.0f, 0, nullptr, 0,
                                  nullptr, st);
@@ -179,4 +187,9 @@ extern "C" int llmops_fc_Q4A_partials(const int8_t* xq, int64_t rows, const int8
     LLMOPS_REQUIRE(use_mfma >= 0 && use_mfma <= 2 && (use_mfma != 2 || group_k == 128));
     if (use_mfma) return launch_gemm_partials(w, xq, acc, rows, Ng, Kg, group_k, use_mfma == 2, as_stream(stream));
     return launch_gemv_partials(w, xq, acc, rows, Ng, Kg, group_k, as_stream(stream));
+}
+
+extern "C" void llmops_fc_set_row_routing(int rows_from_small, int rows_from_large) {
+    g_rows_from_small = rows_from_small >= 2 ? rows_from_small : 4;
+    g_rows_from_large = rows_from_large >= 2 ? rows_from_large : 3;
 }

@@ -395,6 +395,32 @@ def test_fc_rows_kernel_two_k_halves(ops, orc, rows, N, K):
         lib.llmops_fc_rows_set_split(1)
 
 
+@pytest.mark.parametrize("rows", [2, 3, 4, 6, 8])
+@pytest.mark.parametrize("N,K", [(4096, 1024), (9000, 512)])
+def test_fc_few_rows_either_kernel(ops, orc, rows, N, K):
+    """2..8 rows at group 128 can run the streaming kernel that quantizes on the fly or the weight-streaming
+    MFMA kernel behind a quantization launch (the row count at which the second takes over is a tuning
+    knob): both against the oracle, with and without the residual, for a tensor on either side of 256
+    strips."""
+    from llmops import _lib
+    lib = _lib.load()
+    rng = np.random.default_rng(rows * 7 + N)
+    x = rng.standard_normal((1, rows, K)).astype(np.float32)
+    w = (rng.standard_normal((N, K)) * 0.02).astype(np.float32)
+    res = rng.standard_normal((1, rows, N)).astype(np.float32)
+    pw = dev(orc.quant_w(w, 128))
+    want = orc.fc(x, host(pw), N)
+    try:
+        for first in (9, 2, 0):  # streaming kernel for all of 2..8 rows; MFMA kernel from 2 rows; defaults
+            lib.llmops_fc_set_row_routing(first, first)
+            a = ops.fc_Q4A(dev(x), pw, N)
+            c = ops.fc_Q4A(dev(x), pw, N, residual=dev(res))
+            assert max_rel_err(host(a), want) <= 1e-5
+            assert max_rel_err(host(c), want + res) <= 1e-5
+    finally:
+        lib.llmops_fc_set_row_routing(0, 0)
+
+
 @pytest.mark.parametrize("rows", [17, 48, 100, 128, 129, 200, 256])
 @pytest.mark.parametrize("N,K", [(2070, 1024), (4096, 640), (2048, 2816)])
 def test_fc_prefill_mid_rows_vs_oracle(ops, orc, rows, N, K):
