@@ -1,8 +1,8 @@
-// Q4_1 x Q8 fully-connected product for 9..16 activation rows (group 128): weight streaming like
+// Q4_1 x Q8 fully-connected product for 3..16 activation rows (group 128): weight streaming like
 // the one-row kernel, inner product on the int8 matrix cores.
 //
 // With this few rows the FC is still bound by the weight stream, so the work is cut like the
-// decode kernel's: one workgroup per strip of 32 output columns, its 8 waves split K into
+// decode kernel's: one workgroup per strip of 32 output columns, its 8 or 16 waves split K into
 // contiguous runs of k-groups, every wave reads each packed weight byte once, and the waves'
 // fp32 results meet in LDS.  Nothing is staged through LDS on the way in: a lane fetches exactly
 // the two dwords per (64-k half, 16-column tile) that make up its B operand of
@@ -22,7 +22,6 @@ namespace llmops {
 typedef int v4i_r __attribute__((ext_vector_type(4)));
 typedef float v4f_r __attribute__((ext_vector_type(4)));
 
-constexpr int kRowsWaves = 8;
 static int g_rows_split = 1;  // 0: never cut K in two for tensors with few strips
 constexpr int kRowsBlk = 2176;
 
@@ -85,14 +84,13 @@ __device__ __forceinline__ void rows_load(RowsStage<RT>& st, const RowsBufs& bf,
     }
 }
 
-template <int RT>
-__global__ __launch_bounds__(kRowsWaves * 64, 4) void fc_rows_mfma_kernel(const uint8_t* __restrict__ weiq,
+template <int RT, int NW>
+__global__ __launch_bounds__(NW * 64, 4) void fc_rows_mfma_kernel(const uint8_t* __restrict__ weiq,
                                                                          const int8_t* __restrict__ xq,
                                                                          const float2* __restrict__ xsT,
                                                                          float* __restrict__ y, int Kg, int64_t N, int rows,
                                                                          const float* __restrict__ residual,
                                                                          unsigned long long* slots) {
-    constexpr int NW = kRowsWaves;
     __shared__ float red[NW][16 * RT][kGroupN];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // uniform: block offsets stay scalar
@@ -164,9 +162,14 @@ __global__ __launch_bounds__(kRowsWaves * 64, 4) void fc_rows_mfma_kernel(const 
         __builtin_amdgcn_sched_barrier(0);
         rows_load<RT>(sb, bf, kb + 3, rows, kb + 3 < t1);
         __builtin_amdgcn_sched_barrier(0);
-        LLMOPS_ROWS_COMPUTE(sa);
+        // (the loads above are issued whatever the run's length; only the arithmetic on zeros is skipped)
+        if (kb + 2 < t1) {
+            LLMOPS_ROWS_COMPUTE(sa);
+        }
         __builtin_amdgcn_sched_barrier(0);
-        LLMOPS_ROWS_COMPUTE(sb);
+        if (kb + 3 < t1) {
+            LLMOPS_ROWS_COMPUTE(sb);
+        }
     }
 #undef LLMOPS_ROWS_COMPUTE
 
@@ -210,8 +213,16 @@ int launch_fc_rows(const uint8_t* w, const int8_t* xq, const float2* xsT, float*
     if (rows > 16) return fail(LLMOPS_EINVAL, "the streaming MFMA kernel takes at most 16 rows, got %lld", (long long)rows);
     // fewer strips than compute units and a K worth cutting: two workgroups per strip
     const bool split = slots != nullptr && g_rows_split && Ng < 256 && Kg >= 16 && (size_t)rows * Ng * kGroupN * 8 <= slot_bytes;
-    fc_rows_mfma_kernel<1><<<(unsigned)(split ? 2 * Ng : Ng), kRowsWaves * 64, 0, st>>>(w, xq, xsT, y, (int)Kg, N, (int)rows, residual,
-                                                                                     split ? slots : nullptr);
+    // A wave has four k-groups in flight per pass: 8 waves cover 32 k-groups per workgroup in one pass (a hidden
+    // size of 4096); longer runs take 16 waves rather than a second pass (4096x11008 in two halves, 16 rows:
+    // 13.3 against 13.8 us; with 32 k-groups 16 waves are slower, 15.7 against 14.1 us at 11008x4096)
+    const int64_t k_per_wg = split ? (Kg + 1) / 2 : Kg;
+    if (k_per_wg > 32)
+        fc_rows_mfma_kernel<1, 16><<<(unsigned)(split ? 2 * Ng : Ng), 1024, 0, st>>>(w, xq, xsT, y, (int)Kg, N, (int)rows, residual,
+                                                                                  split ? slots : nullptr);
+    else
+        fc_rows_mfma_kernel<1, 8><<<(unsigned)(split ? 2 * Ng : Ng), 512, 0, st>>>(w, xq, xsT, y, (int)Kg, N, (int)rows, residual,
+                                                                                split ? slots : nullptr);
     LLMOPS_LAUNCH_CHECK();
     return LLMOPS_OK;
 }

@@ -396,12 +396,12 @@ def test_fc_rows_kernel_two_k_halves(ops, orc, rows, N, K):
 
 
 @pytest.mark.parametrize("rows", [2, 3, 4, 6, 8])
-@pytest.mark.parametrize("N,K", [(4096, 1024), (9000, 512)])
+@pytest.mark.parametrize("N,K", [(4096, 1024), (9000, 512), (8224, 4480)])
 def test_fc_few_rows_either_kernel(ops, orc, rows, N, K):
     """2..8 rows at group 128 can run the streaming kernel that quantizes on the fly or the weight-streaming
     MFMA kernel behind a quantization launch (the row count at which the second takes over is a tuning
     knob): both against the oracle, with and without the residual, for a tensor on either side of 256
-    strips."""
+    strips and one whose 35 k-groups per workgroup take the MFMA kernel's 16-wave form."""
     from llmops import _lib
     lib = _lib.load()
     rng = np.random.default_rng(rows * 7 + N)
