@@ -528,7 +528,10 @@ static GemvPlan plan_gemv(int64_t rows, int64_t Ng, int64_t Kg, int G, bool fuse
     if (NW == 0) NW = 16;
     if (rows > 4 && NW > 8) NW = 8;  // one (row, column) finaliser thread per output of the strip
     int S = (int)((g_target_workgroups + Ng - 1) / Ng);
-    if ((T + NW - 1) / NW <= 2) S = 1;    // a wave already has only 1-2 blocks: splitting buys nothing
+    // a wave already has at most one pass of 256 k-values (2 steps at group 128, 4 at group 32 in the kernel
+    // that quantizes on the fly): splitting would leave passes half empty (4096x4096 at group 32: 5.5 us
+    // whole against 5.9 us in two splits)
+    if ((T + NW - 1) / NW <= ((G == 32 && fused) ? 4 : 2)) S = 1;
     const int max_s = (T + NW - 1) / NW;  // at least one step per wave
     if (S > max_s) S = max_s;
     if (S < 1) S = 1;
