@@ -83,37 +83,48 @@ __global__ __launch_bounds__(256) void quant_x_kernel(const float* __restrict__ 
 }
 
 // Prefill variant (many rows): G/4 threads per group, each with one 16-byte load and one packed
-// 4-code store, so a workgroup quantizes 256/(G/4) groups with fully coalesced traffic.  Codes and
-// scales are the same bits as above; the raw group sum is a tree sum (it only feeds the fp32 output).
-template <int G>
-__global__ __launch_bounds__(256) void quant_x_rows_kernel(const float* __restrict__ x, int64_t items, int64_t K, int64_t Kg,
+// 4-code store per group, so a workgroup quantizes 256/(G/4) groups at a time with fully coalesced traffic.
+// With many groups a team of G/4 threads takes U consecutive ones and asks for all of them before it uses
+// the first (more bytes in flight per thread).  Codes and scales are the same bits as above; the raw group
+// sum is a tree sum (it only feeds the fp32 output).  Whole groups only (K == Kg*G), so group i starts at
+// float i*G of the dense [rows, K] array.
+template <int G, int U>
+__global__ __launch_bounds__(256) void quant_x_rows_kernel(const float* __restrict__ x, int64_t items, int64_t Kg,
                                                             int64_t rows, int8_t* __restrict__ xq, float* __restrict__ xd,
                                                             float* __restrict__ gsum, float2* __restrict__ xsT) {
     constexpr int TPG = G / 4;        // threads per group
-    constexpr int GPW = 256 / TPG;    // groups per workgroup
+    constexpr int GPW = 256 / TPG;    // teams per workgroup
     const int sub = threadIdx.x % TPG;
-    const int64_t item = (int64_t)blockIdx.x * GPW + threadIdx.x / TPG;
-    const bool live = item < items;   // a group's threads are all live or all idle: the shuffles below stay inside a group
-    const int64_t it = live ? item : items - 1;
-    const int64_t r = it / Kg, kb = it % Kg;
-    const float4 v = *reinterpret_cast<const float4*>(x + r * K + kb * G + sub * 4);
-    float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
-    float s = (v.x + v.y) + (v.z + v.w);
+    const int64_t first = ((int64_t)blockIdx.x * GPW + threadIdx.x / TPG) * U;
+    // a team's threads are all live or all idle for a group: the shuffles below stay inside a team
+    float4 v[U];
 #pragma unroll
-    for (int o = TPG / 2; o > 0; o >>= 1) {
-        amax = fmaxf(amax, __shfl_xor(amax, o, 64));
-        s += __shfl_xor(s, o, 64);
+    for (int u = 0; u < U; u++) {
+        const int64_t it = first + u < items ? first + u : items - 1;
+        v[u] = *reinterpret_cast<const float4*>(x + it * G + sub * 4);
     }
-    const float d = amax / 127.0f;
-    const float id = (d != 0.0f) ? (1.0f / d) : 0.0f;
-    const uint32_t c = ((uint32_t)q8_code(v.x, id) & 0xFFu) | (((uint32_t)q8_code(v.y, id) & 0xFFu) << 8) |
-                       (((uint32_t)q8_code(v.z, id) & 0xFFu) << 16) | (((uint32_t)q8_code(v.w, id) & 0xFFu) << 24);
-    if (!live) return;
-    *reinterpret_cast<uint32_t*>(xq + (r * Kg + kb) * G + sub * 4) = c;
-    if (sub == 0) {
-        xd[r * Kg + kb] = d;
-        gsum[r * Kg + kb] = s;
-        if (xsT != nullptr) xsT[kb * rows + r] = make_float2(d, s);
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+        const int64_t item = first + u;
+        float amax = fmaxf(fmaxf(fabsf(v[u].x), fabsf(v[u].y)), fmaxf(fabsf(v[u].z), fabsf(v[u].w)));
+        float s = (v[u].x + v[u].y) + (v[u].z + v[u].w);
+#pragma unroll
+        for (int o = TPG / 2; o > 0; o >>= 1) {
+            amax = fmaxf(amax, __shfl_xor(amax, o, 64));
+            s += __shfl_xor(s, o, 64);
+        }
+        const float d = amax / 127.0f;
+        const float id = (d != 0.0f) ? (1.0f / d) : 0.0f;
+        const uint32_t c = ((uint32_t)q8_code(v[u].x, id) & 0xFFu) | (((uint32_t)q8_code(v[u].y, id) & 0xFFu) << 8) |
+                           (((uint32_t)q8_code(v[u].z, id) & 0xFFu) << 16) | (((uint32_t)q8_code(v[u].w, id) & 0xFFu) << 24);
+        if (item < items) {
+            *reinterpret_cast<uint32_t*>(xq + item * G + sub * 4) = c;
+            if (sub == 0) {
+                xd[item] = d;
+                gsum[item] = s;
+                if (xsT != nullptr) xsT[(item % Kg) * rows + item / Kg] = make_float2(d, s);
+            }
+        }
     }
 }
 
@@ -128,10 +139,16 @@ int launch_quant_x(const float* x, int64_t rows, int64_t K, int group_k, int8_t*
     const int64_t Kg = (K + group_k - 1) / group_k;
     const int64_t items = rows * Kg;
     if (!exact_sum && K == Kg * group_k && aligned(x, 16) && aligned(xq, 4)) {  // whole groups only: vector loads
-        if (group_k == 32)
-            quant_x_rows_kernel<32><<<(unsigned)((items + 31) / 32), 256, 0, stream>>>(x, items, K, Kg, rows, xq, xd, gsum, xsT);
-        else
-            quant_x_rows_kernel<128><<<(unsigned)((items + 7) / 8), 256, 0, stream>>>(x, items, K, Kg, rows, xq, xd, gsum, xsT);
+        const int64_t teams = (group_k == 32) ? 32 : 8;  // per workgroup
+        if (items >= 32768) {  // enough groups to fill the chip with four per team
+            const unsigned grid = (unsigned)((items + teams * 4 - 1) / (teams * 4));
+            if (group_k == 32) quant_x_rows_kernel<32, 4><<<grid, 256, 0, stream>>>(x, items, Kg, rows, xq, xd, gsum, xsT);
+            else quant_x_rows_kernel<128, 4><<<grid, 256, 0, stream>>>(x, items, Kg, rows, xq, xd, gsum, xsT);
+        } else {
+            const unsigned grid = (unsigned)((items + teams - 1) / teams);
+            if (group_k == 32) quant_x_rows_kernel<32, 1><<<grid, 256, 0, stream>>>(x, items, Kg, rows, xq, xd, gsum, xsT);
+            else quant_x_rows_kernel<128, 1><<<grid, 256, 0, stream>>>(x, items, Kg, rows, xq, xd, gsum, xsT);
+        }
         LLMOPS_LAUNCH_CHECK();
         return LLMOPS_OK;
     }
