@@ -813,17 +813,23 @@ __global__ void gemm_reduce_kernel(const float* __restrict__ part, float* __rest
     if (i >= rows * nq) return;
     const int64_t r = i / nq, n = (i % nq) * 4;
     float4 a = make_float4(0.f, 0.f, 0.f, 0.f);
-    for (int s = 0; s < S; s++) {
-        const float4 v = *reinterpret_cast<const float4*>(part + (int64_t)s * split_stride + r * ldp + n);
-        a.x += v.x, a.y += v.y, a.z += v.z, a.w += v.w;
-    }
     float* dst = y + r * N + n;
     const float* res = residual ? residual + r * N + n : nullptr;
-    if (n + 3 < N && (N & 3) == 0) {
-        if (res) {
-            const float4 r4 = *reinterpret_cast<const float4*>(res);
-            a.x += r4.x, a.y += r4.y, a.z += r4.z, a.w += r4.w;
-        }
+    const bool whole = n + 3 < N && (N & 3) == 0;
+    float4 r4 = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (whole && res) r4 = *reinterpret_cast<const float4*>(res);
+    // four splits' loads in flight at a time (a split past the last re-reads the last and is not added)
+    for (int s0 = 0; s0 < S; s0 += 4) {
+        float4 v[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++)
+            v[u] = *reinterpret_cast<const float4*>(part + (int64_t)min(s0 + u, S - 1) * split_stride + r * ldp + n);
+#pragma unroll
+        for (int u = 0; u < 4; u++)
+            if (s0 + u < S) a.x += v[u].x, a.y += v[u].y, a.z += v[u].z, a.w += v[u].w;
+    }
+    if (whole) {
+        if (res) a.x += r4.x, a.y += r4.y, a.z += r4.z, a.w += r4.w;
         *reinterpret_cast<float4*>(dst) = a;
     } else {
         const float av[4] = {a.x, a.y, a.z, a.w};
