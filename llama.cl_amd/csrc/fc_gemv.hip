@@ -288,15 +288,6 @@ __global__ __launch_bounds__(NW * 64, (MT == 1 ? NW / 2 : 1)) void fc_gemv_fused
             for (int u = 0; u < 4; u++) p4[(NORM && SUMS) ? r : 0][u] = buf_ldf1(ss_rs, (uint32_t)(lane + 64 * u) * 4u, 0u);
         }
         __builtin_amdgcn_sched_barrier(0);  // asked for first, used after everything else has been asked for
-    } else if (NORM) {
-#pragma unroll
-        for (int r = 0; r < MT; r++)
-#pragma unroll
-            for (int i = 0; i < NV; i++) {
-                const int64_t e = ((int64_t)i * NW * 64 + threadIdx.x) * 4;
-                nv[NORM ? r : 0][i] = (r < rows && e < K) ? *reinterpret_cast<const float4*>(x + (int64_t)r * K + e)
-                                                         : make_float4(0.f, 0.f, 0.f, 0.f);
-            }
     }
     // A wave works in passes of 256 k-values: SPP steps (group 128: two blocks, one per step; group 32: four
     // steps of two blocks each) whose weights are in flight together with the pass's activations (and norm
@@ -315,6 +306,19 @@ __global__ __launch_bounds__(NW * 64, (MT == 1 ? NW / 2 : 1)) void fc_gemv_fused
     const buffer_rsrc strip_rs = make_rsrc(strip, (uint32_t)Kg * (uint32_t)block_bytes(G));
     const buffer_rsrc x_rs = make_rsrc(x, (uint32_t)rows * (uint32_t)xstride * 4u);
     const buffer_rsrc nw_rs = make_rsrc(NORM ? norm_w : x, NORM ? (uint32_t)K * 4u : 0u);
+    if constexpr (NORM && !SUMS) {
+        // the row for the statistic, four floats per thread and slice of NW*256: asked for unconditionally (a
+        // slice beyond K at an offset that returns 0) and first, so that the statistic waits for these only
+#pragma unroll
+        for (int r = 0; r < MT; r++)
+#pragma unroll
+            for (int i = 0; i < NV; i++) {
+                const int64_t e = ((int64_t)i * NW * 64 + threadIdx.x) * 4;
+                nv[NORM ? r : 0][i] = buf_ldf4(x_rs, (r < rows && e < K) ? (uint32_t)threadIdx.x * 16u : kNoLoad,
+                                               (uint32_t)(r * K + (int64_t)i * NW * 256) * 4u);
+            }
+        __builtin_amdgcn_sched_barrier(0);
+    }
 #define LLMOPS_LOAD_PAIR(P, TP, WANT)                                                                            \
     do { /* branch-free: what is not wanted is asked for at an offset that returns 0 (see kNoLoad) */            \
         const bool ok_ = (WANT) && (TP) + lane_step < tr.t1 && (int64_t)(TP) * Step<G>::kK + lane * 4 < K;       \
