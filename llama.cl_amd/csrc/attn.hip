@@ -245,10 +245,15 @@ __global__ __launch_bounds__(128) void attn_merge_kernel(float* __restrict__ q, 
         // The chunk weights exp(m_c - M) / sum are the same for all 128 output elements: each wave computes
         // them once, one chunk per lane (one expf per lane instead of one per chunk and thread), and every
         // thread then only accumulates its element over the chunks.  Loads in order of use (statistics, then
-        // the partial outputs, 16 in flight), addresses clamped instead of branched around.
+        // the partial outputs, the first 32 in flight together with the statistics), addresses clamped instead of branched around.
         const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
         const float* rc = rec + (int64_t)min(lane, nchunks - 1) * (S + 2);
         const float m = rc[0], sm0 = rc[1];
+        // (the first 32 partial outputs do not depend on the weights: asked for before the weights are computed)
+        float o0[32];
+#pragma unroll
+        for (int u = 0; u < 32; u++) o0[u] = rec[(int64_t)min(u, nchunks - 1) * (S + 2) + 2 + threadIdx.x];
+        __builtin_amdgcn_sched_barrier(0);
         float acc = 0.0f;
         const float mm = lane < nchunks ? m : -FLT_MAX;
         const float sm = lane < nchunks ? sm0 : 0.0f;
@@ -257,7 +262,9 @@ __global__ __launch_bounds__(128) void attn_merge_kernel(float* __restrict__ q, 
         const float den = wave_sum(w * sm);
         wsh[wave][lane] = w * (1.0f / den);
         __builtin_amdgcn_wave_barrier();
-        for (int c0 = 0; c0 < nchunks; c0 += 16) {
+#pragma unroll
+        for (int u = 0; u < 32; u++) acc = fmaf(u < nchunks ? wsh[wave][u] : 0.0f, o0[u], acc);
+        for (int c0 = 32; c0 < nchunks; c0 += 16) {
             float o[16];
 #pragma unroll
             for (int u = 0; u < 16; u++) o[u] = rec[(int64_t)min(c0 + u, nchunks - 1) * (S + 2) + 2 + threadIdx.x];
