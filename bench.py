@@ -136,6 +136,7 @@ def main():
                 per_shape = measure_shapes(torch, llmops, plan, dims, weights, xs, stream)
             del weights, graph
         floor_us = dispatch_floor(torch, stream)
+    ceiling_gbs = read_ceiling(torch, llmops)
     setup_s = time.time() - t0
 
     main_r = results["fused"]
@@ -148,6 +149,9 @@ def main():
             "avg_launch_us": round(avg_us, 3), "launches_per_step": main_r["launches"],
             "bytes_per_launch_avg": int(step_bytes / main_r["launches"]), "per_shape": per_shape,
             "dispatch_floor_us": round(floor_us, 3),
+            "read_ceiling": {"GB/s": round(ceiling_gbs, 1), "frac_of_it": round(achieved / ceiling_gbs, 4),
+                             "what": "plain read kernel (16-byte loads) over 2 GiB, one launch: what this part's HBM "
+                                     "delivers to a kernel that does nothing else"},
             "timing": "HIP events on the launch stream around the timed graph replays; every node of the graph is this "
                       "kernel, so the average includes the dispatch gap between dependent launches (dispatch_floor_us)"}
     out = {
@@ -275,6 +279,24 @@ def decode_step(torch, stream, kv_len=2048, reps=20):
         del dg, kv
     out["config"] = "Llama-2-7B shape, 32 layers, Q4_1(128) FCs incl. 55296x4096 lm_head, kv-len 2048, batch 1, HIP graph"
     return out
+
+
+def read_ceiling(torch, llmops, nbytes=2 << 30, reps=4):
+    """GB/s of a plain read kernel over a buffer far larger than the caches (the measured ceiling beside the nominal peak)."""
+    import ctypes
+    lib = llmops._lib.load()
+    src = torch.zeros(nbytes, dtype=torch.uint8, device="cuda")
+    out4 = torch.zeros(4, dtype=torch.int32, device="cuda")
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    llmops._lib.check(lib.llmops_calib_read(src.data_ptr(), nbytes, 8192, out4.data_ptr(), st))
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        llmops._lib.check(lib.llmops_calib_read(src.data_ptr(), nbytes, 8192, out4.data_ptr(), st))
+    e1.record()
+    torch.cuda.synchronize()
+    return nbytes * reps / (e0.elapsed_time(e1) * 1e-3) / 1e9
 
 
 def calib(nbytes=1 << 30, reps=5):
