@@ -120,6 +120,24 @@ __global__ void emb_q8c_kernel(float* __restrict__ out, const int64_t* __restric
     for (int64_t e = threadIdx.x; e < E; e += blockDim.x) out[(int64_t)blockIdx.x * E + e] = s * (float)q[id * E + e];
 }
 
+// The same with E a multiple of 4 and 4-byte aligned rows: four codes per thread, blockIdx.y walks the row, so a
+// single token's row is one round of independent loads instead of a loop in one workgroup.
+__global__ __launch_bounds__(256) void emb_q8c_vec_kernel(float* __restrict__ out, const int64_t* __restrict__ ids,
+                                                          const int8_t* __restrict__ q, const float* __restrict__ scales,
+                                                          int64_t E) {
+    const int64_t e = ((int64_t)blockIdx.y * 256 + threadIdx.x) * 4;
+    if (e >= E) return;
+    const int64_t id = ids[blockIdx.x];
+    const float s = scales[id];
+    const uint32_t c = *reinterpret_cast<const uint32_t*>(q + id * E + e);
+    float4 v;
+    v.x = s * (float)(int8_t)(c & 0xFFu);
+    v.y = s * (float)(int8_t)((c >> 8) & 0xFFu);
+    v.z = s * (float)(int8_t)((c >> 16) & 0xFFu);
+    v.w = s * (float)(int8_t)(c >> 24);
+    *reinterpret_cast<float4*>(out + (int64_t)blockIdx.x * E + e) = v;
+}
+
 // embedding (ops/op_embedding.hpp:24-49): out[i,:] = w[ids[i],:]
 __global__ void emb_kernel(float* __restrict__ out, const int64_t* __restrict__ ids, const float* __restrict__ w, int64_t E) {
     const int64_t id = ids[blockIdx.x];
@@ -213,7 +231,10 @@ extern "C" int llmops_embedding_q8c(float* out, const int64_t* ids, int64_t n, c
     (void)V;
     LLMOPS_REQUIRE(out != nullptr && ids != nullptr && q != nullptr && scales != nullptr && n > 0 && E > 0);
     LLMOPS_REQUIRE(n < ((int64_t)1 << 31));
-    emb_q8c_kernel<<<(unsigned)n, 256, 0, as_stream(stream)>>>(out, ids, q, scales, E);
+    if ((E % 4) == 0 && aligned(q, 4) && aligned(out, 16) && (E + 1023) / 1024 < 65536)
+        emb_q8c_vec_kernel<<<dim3((unsigned)n, (unsigned)((E + 1023) / 1024)), 256, 0, as_stream(stream)>>>(out, ids, q, scales, E);
+    else
+        emb_q8c_kernel<<<(unsigned)n, 256, 0, as_stream(stream)>>>(out, ids, q, scales, E);
     LLMOPS_LAUNCH_CHECK();
     return LLMOPS_OK;
 }
