@@ -232,6 +232,20 @@ def test_neighbours_golden(ops):
         ops.itrans(x, "gelu")
 
 
+@pytest.mark.parametrize("V,E,n", [(50, 30, 7), (9, 4096, 1), (300, 5000, 3), (20, 1026, 4)])
+def test_embedding_q8c_vs_oracle(ops, orc, V, E, n):
+    """embedding_q8c lookup, bit-equal to the oracle: row lengths that take the four-codes-per-thread kernel
+    (a multiple of 4, one or several workgroups per row) and ones that take the byte-wise one."""
+    rng = np.random.default_rng(V + E)
+    w = rng.standard_normal((V, E)).astype(np.float32)
+    ids = rng.integers(0, V, size=(1, n)).astype(np.int64)
+    q, s = orc.embedding_q8c_quant_w(w)
+    want = orc.embedding_q8c(ids, q, s)
+    out = ops.empty(1, n, E)
+    ops.embedding_q8c(out, dev(ids), dev(q), dev(s))
+    assert np.array_equal(host(out), want)
+
+
 def test_fused_neighbours_vs_oracle(ops, orc):
     """Extensions used by the decode step: rmsnorm_out == clone+rmsnorm, silu_mul == silu then imul,
     fc_Q4A(residual=) == fc_Q4A then iadd."""
