@@ -88,7 +88,7 @@ int llmops_FC_dynamic_quantize_x_rows(const float* x, int64_t rows, int64_t K, i
  * LLMOPS_FC_COUNTER_BYTES bytes of the workspace must be zero when the library first sees it; the
  * library leaves them zero after every call.  One workspace must not be shared by calls that can
  * overlap on the device. */
-#define LLMOPS_FC_COUNTER_BYTES 1048576
+#define LLMOPS_FC_COUNTER_BYTES 3145728
 size_t llmops_fc_Q4A_workspace_bytes(int64_t rows, int64_t K, int64_t Ng, int64_t Kg, int group_k);
 
 /* fc_Q4A (ops/op_fc.hpp:286-426, bound at ops/main.cpp:160).
@@ -271,7 +271,7 @@ void llmops_fc_set_tuning(int target_workgroups, int waves_per_workgroup);
  * per shape and send 9..16 rows to the tiled kernel too instead of the weight-streaming MFMA kernel */
 void llmops_gemm_set_tuning(int row_tile_factor);
 
-/* weight-streaming MFMA kernel (3..16 rows): two workgroups per strip with half of K each for tensors of
+/* weight-streaming MFMA kernel (3..16 rows, 17..32 for tensors of fewer than 256 strips): two workgroups per strip with half of K each for tensors of
  * fewer than 256 strips (default on; 0 switches it off, for comparisons and tests) */
 void llmops_fc_rows_set_split(int on);
 

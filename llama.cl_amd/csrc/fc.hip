@@ -42,7 +42,8 @@ static FcWorkspace fc_layout(int64_t rows, int64_t Ng, int64_t Kg, int G) {
     w.off_gs = o;
     o = align_up(o + (size_t)rows * Kg * sizeof(float), 256);
     w.off_xst = o;
-    o = align_up(o + (size_t)rows * Kg * 2 * sizeof(float), 256);
+    // (+256: the weight-streaming MFMA kernel fetches the pairs of whole 16-row tiles, up to 31 pairs past the last row)
+    o = align_up(o + (size_t)rows * Kg * 2 * sizeof(float) + 256, 256);
     w.off_part = o;
     o = align_up(o + (rows <= kMaxGemvRows ? gemv_workspace_bytes(rows, Ng, Kg, G) : gemm_workspace_bytes(rows, Ng, Kg, G)), 256);
     w.total = o;
@@ -103,9 +104,11 @@ static int fc_impl(const float* x, int64_t rows, int64_t K, const int8_t* weiq, 
     int rc = launch_quant_x(x, rows, K, group_k, xq, xd, gs, xst, false, st);
     if (rc) return rc;
     // up to 16 rows are still bound by the weight stream: one strip per workgroup, MFMA inner product
-    // (measured against the tiled kernel: 15 vs 18 us at 16 rows, 11008x4096; with two row tiles per
-    // wave, 17..32 rows, the streaming kernel runs out of registers and loses, 32 vs 20 us)
-    if (rows_kernel && rows <= 16)
+    // (measured against the tiled kernel: 15 vs 18 us at 16 rows, 11008x4096).  17..32 rows (two row tiles
+    // per wave) only win for tensors of fewer than 256 strips, where the tiled kernel has too few tiles
+    // (us, tiled / streaming: 4096x4096 at 17 rows 20.2 / 9.9, at 32 rows 24.3 / 11.9; 4096x11008 at 24 rows
+    // 22.0 / 15.7; 11008x4096 at 24 rows 19.3 / 18.8; 12288x4096 17.9 / 19.0; 22016x4096 23.0 / 27.4)
+    if (rows_kernel && (rows <= 16 || (rows <= 32 && Ng < 256)))
         return launch_fc_rows(w, xq, xst, y, rows, Ng, Kg, N, residual, reinterpret_cast<unsigned long long*>(ws + kTicketBytes),
                               LLMOPS_FC_COUNTER_BYTES - kTicketBytes, st);
     return launch_gemm(w, xq, xd, gs, xst, y, part, rows, Ng, Kg, group_k, N, residual, st);

@@ -1,4 +1,4 @@
-// Q4_1 x Q8 fully-connected product for 3..16 activation rows (group 128): weight streaming like
+// Q4_1 x Q8 fully-connected product for 3..32 activation rows (group 128): weight streaming like
 // the one-row kernel, inner product on the int8 matrix cores.
 //
 // With this few rows the FC is still bound by the weight stream, so the work is cut like the
@@ -85,7 +85,7 @@ __device__ __forceinline__ void rows_load(RowsStage<RT>& st, const RowsBufs& bf,
 }
 
 template <int RT, int NW>
-__global__ __launch_bounds__(NW * 64, 4) void fc_rows_mfma_kernel(const uint8_t* __restrict__ weiq,
+__global__ __launch_bounds__(NW * 64, RT == 2 ? 3 : 4) void fc_rows_mfma_kernel(const uint8_t* __restrict__ weiq,
                                                                          const int8_t* __restrict__ xq,
                                                                          const float2* __restrict__ xsT,
                                                                          float* __restrict__ y, int Kg, int64_t N, int rows,
@@ -206,23 +206,26 @@ __global__ __launch_bounds__(NW * 64, 4) void fc_rows_mfma_kernel(const uint8_t*
     }
 }
 
-// rows <= 16, group 128, activations already quantized (codes [rows, Kg*128], pairs [Kg][rows])
+// rows <= 32 (two row tiles per wave from 17 on), group 128, activations already quantized (codes [rows, Kg*128], pairs [Kg][rows])
 // `slots`: the zeroed exchange area of the FC workspace (`slot_bytes` of it), or nullptr
 int launch_fc_rows(const uint8_t* w, const int8_t* xq, const float2* xsT, float* y, int64_t rows, int64_t Ng, int64_t Kg,
                    int64_t N, const float* residual, unsigned long long* slots, size_t slot_bytes, hipStream_t st) {
-    if (rows > 16) return fail(LLMOPS_EINVAL, "the streaming MFMA kernel takes at most 16 rows, got %lld", (long long)rows);
+    if (rows > 32) return fail(LLMOPS_EINVAL, "the streaming MFMA kernel takes at most 32 rows, got %lld", (long long)rows);
     // fewer strips than compute units and a K worth cutting: two workgroups per strip
     const bool split = slots != nullptr && g_rows_split && Ng < 256 && Kg >= 16 && (size_t)rows * Ng * kGroupN * 8 <= slot_bytes;
+    const unsigned grid = (unsigned)(split ? 2 * Ng : Ng);
+    unsigned long long* sl = split ? slots : nullptr;
     // A wave has four k-groups in flight per pass: 8 waves cover 32 k-groups per workgroup in one pass (a hidden
     // size of 4096); longer runs take 16 waves rather than a second pass (4096x11008 in two halves, 16 rows:
-    // 13.3 against 13.8 us; with 32 k-groups 16 waves are slower, 15.7 against 14.1 us at 11008x4096)
+    // 13.3 against 13.8 us; with 32 k-groups 16 waves are slower, 15.7 against 14.1 us at 11008x4096).
+    // 17..32 rows: two row tiles per wave, 8 waves (16 would not have the registers).
     const int64_t k_per_wg = split ? (Kg + 1) / 2 : Kg;
-    if (k_per_wg > 32)
-        fc_rows_mfma_kernel<1, 16><<<(unsigned)(split ? 2 * Ng : Ng), 1024, 0, st>>>(w, xq, xsT, y, (int)Kg, N, (int)rows, residual,
-                                                                                  split ? slots : nullptr);
+    if (rows > 16)
+        fc_rows_mfma_kernel<2, 8><<<grid, 512, 0, st>>>(w, xq, xsT, y, (int)Kg, N, (int)rows, residual, sl);
+    else if (k_per_wg > 32)
+        fc_rows_mfma_kernel<1, 16><<<grid, 1024, 0, st>>>(w, xq, xsT, y, (int)Kg, N, (int)rows, residual, sl);
     else
-        fc_rows_mfma_kernel<1, 8><<<(unsigned)(split ? 2 * Ng : Ng), 512, 0, st>>>(w, xq, xsT, y, (int)Kg, N, (int)rows, residual,
-                                                                                split ? slots : nullptr);
+        fc_rows_mfma_kernel<1, 8><<<grid, 512, 0, st>>>(w, xq, xsT, y, (int)Kg, N, (int)rows, residual, sl);
     LLMOPS_LAUNCH_CHECK();
     return LLMOPS_OK;
 }

@@ -367,7 +367,7 @@ def test_fc_two_k_splits_both_handoffs(ops, orc, rows, N, K):
         lib.llmops_fc_set_tuning(-2, -1)
 
 
-@pytest.mark.parametrize("rows", [3, 5, 8, 9, 13, 16])
+@pytest.mark.parametrize("rows", [3, 5, 8, 9, 13, 16, 17, 24, 32])
 @pytest.mark.parametrize("N,K", [(4096, 11008), (4090, 4096), (2070, 2048), (3000, 2176)])
 def test_fc_rows_kernel_two_k_halves(ops, orc, rows, N, K):
     """The weight-streaming MFMA kernel on tensors with fewer than 256 strips: two workgroups per strip with
