@@ -174,6 +174,16 @@ int llmops_attention_rope(float* q, float* k, const float* v, int64_t B, int64_t
 /* softmax (ops/op_misc.hpp:183-194, ops/utils.hpp:484-490): in place over rows of length K */
 int llmops_softmax(float* x, int64_t rows, int64_t K, llmops_stream_t stream);
 
+/* mm_qk, mm_qk42, mm_qk81, mm_qk24 (ops/op_attn.hpp:149-193, 195-298, 300-422, 424-515; bound at
+ * ops/main.cpp:163-166): the reference's four benchmark variants of one product,
+ *   attn_w[b,h,pq,pk] = dot(q[b,h,pq,:], kcache[b,h,pk,:]) / sqrt(S),   pk < kvLen <= kv_max.
+ * q is addressed as q + b*q_stride_b + h*q_stride_h + pq*q_stride_q (elements, multiples of 4):
+ * [B,qL,H*S] for mm_qk/81/24 -> (qL*H*S, S, H*S); [B,H,qL,S] for mm_qk42 -> (H*qL*S, qL*S, S).
+ * kcache fp32 [B,H,kv_max,S]; attn_w fp32 [B,H,qL,kvLen] dense; S % 8 == 0 (ops/op_attn.hpp:205). */
+int llmops_mm_qk(const float* q, int64_t q_stride_b, int64_t q_stride_h, int64_t q_stride_q, const float* kcache,
+                 int64_t kv_max, float* attn_w, int64_t B, int64_t H, int64_t qL, int64_t kvLen, int64_t S,
+                 llmops_stream_t stream);
+
 /* ------------------------------------------------------------------------------------------
  * Neighbours needed for one decode step (ops/op_misc.hpp, ops/op_embedding.hpp)
  * ------------------------------------------------------------------------------------------ */

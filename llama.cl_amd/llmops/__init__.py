@@ -355,6 +355,49 @@ def softmax(x):
     _lib.check(_lib.load().llmops_softmax(_ptr(x), x.numel() // K, K, _stream(x)))
 
 
+def _mm_qk(q, kcache, attn_w, q_is_bhqs):
+    _dev(kcache, torch.float32, 4, "kcache")
+    _dev(q, torch.float32, 4 if q_is_bhqs else 3, "q")
+    B, H, kmax, S = kcache.shape
+    _require(q.shape[0] == B, "kcache.size(-4) == B")
+    if q_is_bhqs:
+        qL = q.shape[2]
+        _require(tuple(q.shape) == (B, H, qL, S), "q is [B,H,qL,S]")
+        strides = (H * qL * S, qL * S, S)
+    else:
+        qL = q.shape[1]
+        _require(q.shape[2] == H * S, "q is [B,qL,H*S]")
+        strides = (qL * H * S, S, H * S)
+    if attn_w is None:
+        attn_w = torch.empty((B, H, qL, kmax), dtype=torch.float32, device=q.device)
+    else:
+        _dev(attn_w, torch.float32, 4, "attn_w")
+        _require(tuple(attn_w.shape[:3]) == (B, H, qL) and attn_w.shape[3] <= kmax, "attn_w is [B,H,qL,kvLen<=max]")
+    _lib.check(_lib.load().llmops_mm_qk(_ptr(q), *strides, _ptr(kcache), kmax, _ptr(attn_w), B, H, qL, attn_w.shape[3], S,
+                                        _stream(q)))
+    return attn_w
+
+
+def mm_qk(q, kcache):
+    """q [B,qL,H*S], kcache [B,H,kvLen,S] -> (q.k)/sqrt(S) as [B,H,qL,kvLen] (ops/op_attn.hpp:149-193)."""
+    return _mm_qk(q, kcache, None, False)
+
+
+def mm_qk81(q, kcache):
+    """Same contract as mm_qk (ops/op_attn.hpp:300-422)."""
+    return _mm_qk(q, kcache, None, False)
+
+
+def mm_qk24(q, kcache):
+    """Same contract as mm_qk (ops/op_attn.hpp:424-515)."""
+    return _mm_qk(q, kcache, None, False)
+
+
+def mm_qk42(q, kcache, attn_w):
+    """q [B,H,qL,S], kcache [B,H,max-kv-len,S]; fills attn_w [B,H,qL,kvLen] (ops/op_attn.hpp:195-298)."""
+    _mm_qk(q, kcache, attn_w, True)
+
+
 # ---- neighbours -------------------------------------------------------------------------------
 def rmsnorm(input, weight, variance_epsilon):
     _dev(input, torch.float32, 3, "input")

@@ -40,6 +40,7 @@ SIGNATURES = {
     "llmops_attention_rope": (c_int, [c_ptr, c_ptr, c_ptr, c_i64, c_i64, c_i64, c_i64, c_ptr, c_i64, c_ptr, c_int,
                                       c_i64, c_i64, c_ptr, c_int, c_int, c_ptr, c_size, c_ptr]),
     "llmops_softmax": (c_int, [c_ptr, c_i64, c_i64, c_ptr]),
+    "llmops_mm_qk": (c_int, [c_ptr, c_i64, c_i64, c_i64, c_ptr, c_i64, c_ptr, c_i64, c_i64, c_i64, c_i64, c_i64, c_ptr]),
     "llmops_rmsnorm": (c_int, [c_ptr, c_i64, c_i64, c_ptr, c_f32, c_ptr]),
     "llmops_rmsnorm_out": (c_int, [c_ptr, c_ptr, c_i64, c_i64, c_ptr, c_f32, c_ptr]),
     "llmops_silu_mul": (c_int, [c_ptr, c_ptr, c_i64, c_i64, c_ptr]),

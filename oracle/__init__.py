@@ -162,6 +162,23 @@ class Oracle:
                                _p(cache), _i64(planes), _i64(maxlen), _p(s), _int(position_id), _int(layer_id))
         return q, k, cache
 
+    def mm_qk(self, q, kcache, kvLen=None, q_is_bhqs=False):
+        """attn_w [B,H,qL,kvLen]; q is [B,qL,H*S] (mm_qk, mm_qk81, mm_qk24) or [B,H,qL,S] (mm_qk42)"""
+        q = _c32(q)
+        kc = _c32(kcache)
+        B, H, kmax, S = kc.shape
+        kvLen = kmax if kvLen is None else int(kvLen)
+        if q_is_bhqs:
+            qL = q.shape[2]
+            st = (H * qL * S, qL * S, S)
+        else:
+            qL = q.shape[1]
+            st = (qL * H * S, S, H * S)
+        out = np.empty((B, H, qL, kvLen), dtype=np.float32)
+        self.lib.orc_mm_qk(_p(q), _i64(st[0]), _i64(st[1]), _i64(st[2]), _p(kc), _i64(kmax), _p(out), _i64(B), _i64(H),
+                           _i64(qL), _i64(kvLen), _i64(S))
+        return out
+
     def softmax(self, x):
         x = _c32(x).copy()
         K = x.shape[-1]
@@ -340,6 +357,20 @@ class Reference:
                                               _p(f), _i64(f.shape[0]), _p(cache), _i64(planes), _i64(maxlen), _p(s),
                                               _int(position_id), _int(layer_id)))
         return q, k, cache
+
+    def mm_qk(self, q, kcache, kvLen=None, q_is_bhqs=False, variant=None):
+        """variant: 0 mm_qk, 1 mm_qk42, 2 mm_qk81, 3 mm_qk24 (default: 1 for a [B,H,qL,S] query, else 0)"""
+        q = _c32(q).copy()
+        kc = _c32(kcache).copy()
+        B, H, kmax, S = kc.shape
+        kvLen = kmax if kvLen is None else int(kvLen)
+        variant = (1 if q_is_bhqs else 0) if variant is None else variant
+        assert (variant == 1) == bool(q_is_bhqs) and (variant == 1 or kvLen == kmax)
+        qL = q.shape[2] if q_is_bhqs else q.shape[1]
+        out = np.zeros((B, H, qL, kvLen), dtype=np.float32)
+        self._chk(self.lib.ref_mm_qk(_int(variant), _p(q), _p(kc), _p(out), _i64(B), _i64(H), _i64(qL), _i64(kmax),
+                                     _i64(kvLen), _i64(S)))
+        return out
 
     def softmax(self, x):
         x = _c32(x).copy()

@@ -17,6 +17,8 @@
  *   orc_quant_x             reference build bit-for-bit, golden vectors, RNE tie cases
  *   orc_fc_partials         int64 brute-force einsum over unpacked nibbles (pure integers)
  *   orc_fc                  reference build bit-for-bit (same fma order), closed-form x@W.T
+ *   orc_mm_qk               fp64 einsum (the check the reference's own perf script makes,
+ *                           ops/perf_ops.py:168-175), strided and padded-plane cases
  *   orc_rope / orc_attention / orc_softmax / orc_rmsnorm / orc_silu / orc_embedding_q8c
  *                           reference build within 1e-5 (float op order differs), fp64 textbook
  *                           formulas, literal softmax vectors of ops/test_ops.py:171-172
@@ -355,6 +357,27 @@ static void softmax_row(float* a, int64_t n) {
 void orc_softmax(float* x, int64_t rows, int64_t K) {
 #pragma omp parallel for schedule(static)
     for (int64_t r = 0; r < rows; r++) softmax_row(x + r * K, K);
+}
+
+/* mm_qk / mm_qk42 / mm_qk81 / mm_qk24 (ops/op_attn.hpp:149-193, 195-298, 300-422, 424-515): the four
+ *      benchmark ops compute one product, attn_w[b,h,pq,pk] = dot(q[b,h,pq,:], k[b,h,pk,:]) * (1/sqrt(S)),
+ *      with q addressed through strides (elements) and the cache plane holding kv_max rows per head. */
+void orc_mm_qk(const float* q, int64_t qs_b, int64_t qs_h, int64_t qs_q, const float* kcache, int64_t kv_max,
+               float* attn_w, int64_t B, int64_t H, int64_t qL, int64_t kvLen, int64_t S) {
+    const float d_scale = 1.0f / sqrtf((float)S);
+#pragma omp parallel for schedule(static)
+    for (int64_t bh = 0; bh < B * H; bh++) {
+        const int64_t b = bh / H, h = bh % H;
+        for (int64_t pq = 0; pq < qL; pq++) {
+            const float* qr = q + b * qs_b + h * qs_h + pq * qs_q;
+            for (int64_t pk = 0; pk < kvLen; pk++) {
+                const float* kr = kcache + (bh * kv_max + pk) * S;
+                float sum = 0.0f;
+                for (int64_t s = 0; s < S; s++) sum += qr[s] * kr[s];
+                attn_w[(bh * qL + pq) * kvLen + pk] = sum * d_scale;
+            }
+        }
+    }
 }
 
 /* ---- attention_rope2 / attention_rope (ops/op_attn.hpp:721-1029 / :518-718; same contract).

@@ -133,6 +133,31 @@ int ref_attention_rope(int version, float* q, float* k, float* v, int64_t B, int
     });
 }
 
+// variant 0: mm_qk, 1: mm_qk42, 2: mm_qk81, 3: mm_qk24 (ops/op_attn.hpp:149-515).  q is [B,qL,H*S] for
+// 0/2/3 and [B,H,qL,S] for 1; kcache [B,H,kv_max,S]; attn_w [B,H,qL,kvLen].  Variants 0/2/3 take kvLen from
+// the cache's shape, so they are given kv_max == kvLen.
+int ref_mm_qk(int variant, float* q, float* kcache, float* attn_w, int64_t B, int64_t H, int64_t qL, int64_t kv_max,
+              int64_t kvLen, int64_t S) {
+    return guarded([&] {
+        tensor tk = view(kcache, {B, H, kv_max, S});
+        tensor out;
+        if (variant == 1) {
+            tensor tq = view(q, {B, H, qL, S});
+            tensor tw = view(attn_w, {B, H, qL, kvLen});
+            mm_qk42(tq, tk, tw);
+            return;
+        }
+        tensor tq = view(q, {B, qL, H * S});
+        if (variant == 0)
+            out = mm_qk(tq, tk);
+        else if (variant == 2)
+            out = mm_qk81(tq, tk);
+        else
+            out = mm_qk24(tq, tk);
+        std::memcpy(attn_w, out.data<float>(), sizeof(float) * B * H * qL * kvLen);
+    });
+}
+
 // in place, rows of length K
 int ref_softmax(float* x, int64_t rows, int64_t K) {
     return guarded([&] { softmax(view(x, {rows, K})); });

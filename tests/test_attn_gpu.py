@@ -270,3 +270,34 @@ def test_fused_neighbours_vs_oracle(ops, orc):
         got = host(ops.fc_Q4A(dev(x), dev(wq), N, residual=dev(res)))
         want = orc.iadd(orc.fc(x, wq, N), res)
         assert max_rel_err(got, want) <= 1e-5
+
+
+# ---- mm_qk / mm_qk42 / mm_qk81 / mm_qk24: the reference's benchmark names for the scaled q.k product ---------
+@pytest.mark.parametrize("B,H,qL,kv,S", [(1, 2, 1, 7, 16), (2, 3, 5, 33, 128), (1, 4, 37, 130, 64), (1, 32, 8, 2048, 128),
+                                          (1, 2, 129, 257, 128)])
+def test_mm_qk_against_oracle(ops, orc, B, H, qL, kv, S):
+    rng = np.random.default_rng(qL * 7 + kv)
+    q = rng.random((B, qL, H * S), dtype=np.float32)              # ops/perf_ops.py:165-166
+    kc = rng.random((B, H, kv, S), dtype=np.float32)
+    want = orc.mm_qk(q, kc)
+    for name in ("mm_qk", "mm_qk81", "mm_qk24"):
+        got = host(getattr(ops, name)(dev(q), dev(kc)))
+        assert got.shape == (B, H, qL, kv)
+        assert max_rel_err(got, want) <= 1e-5, name
+    # mm_qk42: [B,H,qL,S] query, caller's output, cache plane longer than the rows asked for
+    q_bhqs = np.ascontiguousarray(q.reshape(B, qL, H, S).transpose(0, 2, 1, 3))
+    part = max(1, kv - 3)
+    out = torch.full((B, H, qL, part), float("nan"), device="cuda")
+    assert ops.mm_qk42(dev(q_bhqs), dev(kc), out) is None
+    assert max_rel_err(host(out), orc.mm_qk(q_bhqs, kc, kvLen=part, q_is_bhqs=True)) <= 1e-5
+    assert np.isfinite(host(out)).all()                           # every element of the caller's buffer was written
+
+
+def test_mm_qk_rejects_what_the_reference_asserts(ops):
+    q = torch.zeros(1, 4, 2 * 12, device="cuda")
+    with pytest.raises(RuntimeError):                              # S % 8 (ops/op_attn.hpp:205)
+        ops.mm_qk(q, torch.zeros(1, 2, 5, 12, device="cuda"))
+    with pytest.raises(RuntimeError):                              # kcache.size(-4) == B (ops/op_attn.hpp:154)
+        ops.mm_qk(torch.zeros(1, 4, 32, device="cuda"), torch.zeros(2, 2, 5, 16, device="cuda"))
+    with pytest.raises(RuntimeError):
+        ops.mm_qk(torch.zeros(1, 4, 32), torch.zeros(1, 2, 5, 16))  # host tensors: there is no CPU path

@@ -324,3 +324,47 @@ def test_attention_vs_reference_build(orc):
     b = R.attention(g["q"], g["k"], g["v"], g["inv_freq"], g["cache"], g["slots"], pos, layer)
     for u, v in zip(a, b):
         assert max_rel_err(u, v) < 1e-5
+
+
+# ---- mm_qk (the four benchmark variants of the scaled q.k product, ops/op_attn.hpp:149-515) -----------
+def _qk_fp64(q_bhqs, kc, kvLen):
+    return np.einsum("bhqs,bhks->bhqk", q_bhqs.astype(np.float64), kc[:, :, :kvLen].astype(np.float64)) / math.sqrt(kc.shape[-1])
+
+
+@pytest.mark.parametrize("B,H,qL,kv,S", [(1, 2, 1, 7, 16), (2, 3, 5, 33, 128), (1, 1, 37, 130, 64)])
+def test_mm_qk_oracle_against_fp64_einsum(orc, B, H, qL, kv, S):
+    rng = np.random.default_rng(B * 1000 + qL)
+    q = rng.random((B, qL, H * S), dtype=np.float32)          # ops/perf_ops.py:165-166 draws both from U[0,1)
+    kc = rng.standard_normal((B, H, kv, S)).astype(np.float32)
+    q_bhqs = np.ascontiguousarray(q.reshape(B, qL, H, S).transpose(0, 2, 1, 3))
+    ref = _qk_fp64(q_bhqs, kc, kv)
+    assert np.allclose(orc.mm_qk(q, kc), ref, rtol=1e-5, atol=1e-5)
+    # the [B,H,qL,S] form with a cache plane longer than the rows asked for (mm_qk42)
+    part = max(1, kv - 3)
+    got = orc.mm_qk(q_bhqs, kc, kvLen=part, q_is_bhqs=True)
+    assert got.shape == (B, H, qL, part)
+    assert np.allclose(got, _qk_fp64(q_bhqs, kc, part), rtol=1e-5, atol=1e-5)
+    # a transposed operand or a dropped scale would show here: one-hot rows pick single cache entries
+    e = np.zeros((B, qL, H * S), np.float32)
+    e[:, :, ::S] = 1.0                                          # s = 0 of every head
+    assert np.allclose(orc.mm_qk(e, kc), np.broadcast_to((kc[:, :, None, :, 0] / math.sqrt(S)), (B, H, qL, kv)), rtol=1e-6)
+
+
+@pytest.mark.parametrize("variant", [0, 1, 2, 3])
+def test_mm_qk_oracle_against_reference_build(orc, variant):
+    ref = _ref(32)
+    # crosses the 64-blocks of the AVX variants; those have no tail loops (mm_qk42 steps 4 queries x 2 cache rows,
+    # ops/op_attn.hpp:216-218, and writes past the end otherwise), so the sizes are multiples of 8
+    B, H, qL, kv, S = 2, 4, 72, 200, 128
+    rng = np.random.default_rng(variant)
+    kc = rng.standard_normal((B, H, kv, S)).astype(np.float32)
+    q = rng.standard_normal((B, qL, H * S)).astype(np.float32)
+    q_bhqs = np.ascontiguousarray(q.reshape(B, qL, H, S).transpose(0, 2, 1, 3))
+    if variant == 1:
+        got = ref.mm_qk(q_bhqs, kc, kvLen=kv - 8, q_is_bhqs=True, variant=1)
+        mine = orc.mm_qk(q_bhqs, kc, kvLen=kv - 8, q_is_bhqs=True)
+    else:
+        got = ref.mm_qk(q, kc, variant=variant)
+        mine = orc.mm_qk(q, kc)
+    assert got.shape == mine.shape
+    assert np.abs(got - mine).max() <= 1e-5 * np.abs(mine).max()
