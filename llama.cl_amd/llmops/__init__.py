@@ -46,8 +46,13 @@ def _ptr(t):
     return ctypes.c_void_p(t.data_ptr())
 
 
+def _raw_stream(device):
+    """hipStream_t of torch's current stream on `device`, as an int"""
+    return torch._C._cuda_getCurrentRawStream(device.index if device.index is not None else torch.cuda.current_device())
+
+
 def _stream(t):
-    return ctypes.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+    return ctypes.c_void_p(_raw_stream(t.device))
 
 
 def _dev(t, dtype, rank=None, name="tensor"):
@@ -60,9 +65,11 @@ def _dev(t, dtype, rank=None, name="tensor"):
 
 
 def _workspace(device, nbytes, kind="fc"):
-    """Persistent per-device scratch, one per op family.  Its first bytes hold arrival counters,
+    """Persistent scratch, one per op family, device and stream: ops enqueued on different streams may run
+    at the same time and must not share counters or partial sums.  Its first bytes hold arrival counters,
     which must start at zero and which the kernels leave at zero."""
-    key = (kind, device.type, device.index if device.index is not None else torch.cuda.current_device())
+    index = device.index if device.index is not None else torch.cuda.current_device()
+    key = (kind, device.type, index, torch._C._cuda_getCurrentRawStream(index))
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
         size = max(int(nbytes), 16 << 20)

@@ -481,3 +481,27 @@ def test_fc_rows_9_to_16_streaming_mfma(ops, orc, rows, N, K):
     want = orc.fc(x, pw, N)
     assert max_rel_err(host(ops.fc_Q4A(dev(x), dev(pw), N)), want) <= 1e-5
     assert max_rel_err(host(ops.fc_Q4A(dev(x), dev(pw), N, residual=dev(res))), want + res) <= 1e-5
+
+
+# ---- ops enqueued on different streams run at the same time and must not share scratch ------------------
+def test_fc_on_concurrent_streams_matches_serial(ops):
+    G = 128
+    rng = np.random.default_rng(11)
+    # 4096x11008 is the shape whose k-splits meet through the workspace; 8 rows goes through the prefill pieces
+    cases = []
+    for N, K, M in [(4096, 11008, 1), (4096, 4096, 1), (4096, 11008, 8), (1024, 11008, 16)]:
+        w = dev((rng.standard_normal((N, K)) * 0.02).astype(np.float32))
+        cases.append((ops.offline_FC_quant_Q4A(w, G), dev(rng.standard_normal((1, M, K)).astype(np.float32)), N))
+    serial = [ops.fc_Q4A(x, wq, N) for wq, x, N in cases]
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream() for _ in range(3)]
+    got = [[] for _ in streams]
+    for rep in range(20):
+        for si, s in enumerate(streams):
+            with torch.cuda.stream(s):
+                wq, x, N = cases[(rep + si) % len(cases)]
+                got[si].append(((rep + si) % len(cases), ops.fc_Q4A(x, wq, N)))
+    torch.cuda.synchronize()
+    for per_stream in got:
+        for ci, y in per_stream:
+            assert torch.equal(y, serial[ci]), ci
