@@ -30,7 +30,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 # of `--calib` (one FETCH_SIZE count = 2.000 KiB, one WRITE_SIZE count = 1.000 KiB on this part); the summary with
 # the per-shape figures is profiles/fc_gemv_fused_kernel__hbm_traffic_pmc.md.  Counters cannot be read from inside
 # this process, so the figure is the recorded one and only holds for the fused plan at group 128, M=1.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 27188733
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 27188725
 G = 128
 LAYERS = 32
 # (name, N, K) of one layer's FCs, in the order the model calls them (chatllama/main.py:344-375)
@@ -63,6 +63,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-decode", action="store_true", help="skip the full decode-step timing (BASELINE config 5)")
     ap.add_argument("--no-extra", action="store_true", help="skip the prefill GEMM (config 3) and attention (config 4) legs")
+    ap.add_argument("--no-concurrent", action="store_true",
+                    help="skip the leg that runs the FC set on 2-4 concurrent streams (profiler runs skip it so that every "
+                         "traced launch of the kernel ran alone on the chip)")
     ap.add_argument("--calib", action="store_true",
                     help="only run the plain copy/read kernels over 1 GiB (reference points for traffic counters and "
                          "for the attainable HBM rate) and print their rates")
@@ -134,7 +137,8 @@ def main():
                               "launches": LAYERS * len(plan)}
             if label == "fused":
                 per_shape = measure_shapes(torch, llmops, plan, dims, weights, xs, stream)
-                overlapped = concurrent_streams(torch, llmops, dims, weights, xs, stream, step_bytes)
+                overlapped = None if args.no_concurrent else concurrent_streams(torch, llmops, dims, weights, xs, stream,
+                                                                                step_bytes)
             del weights, graph
         floor_us = dispatch_floor(torch, stream)
     ceiling_gbs = read_ceiling(torch, llmops)
