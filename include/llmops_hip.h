@@ -281,6 +281,11 @@ void llmops_fc_set_tuning(int target_workgroups, int waves_per_workgroup);
  * per shape and send 9..16 rows to the tiled kernel too instead of the weight-streaming MFMA kernel */
 void llmops_gemm_set_tuning(int row_tile_factor);
 
+/* prefill GEMM with split-K: the product kernel adds the partial sums itself (the last split of a tile to
+ * arrive adds all of them in index order) when the split count is at most 12 x in_kernel; otherwise, and
+ * always with 0, a second launch adds them.  Default 1.  Same result either way; kept for comparisons and tests. */
+void llmops_gemm_set_reduce(int in_kernel);
+
 /* weight-streaming MFMA kernel (3..16 rows, 17..32 for tensors of fewer than 256 strips): two workgroups per strip with half of K each for tensors of
  * fewer than 256 strips (default on; 0 switches it off, for comparisons and tests) */
 void llmops_fc_rows_set_split(int on);

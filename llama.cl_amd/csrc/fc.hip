@@ -19,7 +19,8 @@ int launch_gemv_partials(const uint8_t* w, const int8_t* xq, int32_t* acc, int64
                          hipStream_t st);
 size_t gemm_workspace_bytes(int64_t rows, int64_t Ng, int64_t Kg, int G);
 int launch_gemm(const uint8_t* w, const int8_t* xq, const float* xd, const float* gs, const float2* xsT, float* y,
-                float* part, int64_t rows, int64_t Ng, int64_t Kg, int G, int64_t N, const float* residual, hipStream_t st);
+                float* part, unsigned* counters, int64_t rows, int64_t Ng, int64_t Kg, int G, int64_t N, const float* residual,
+                hipStream_t st);
 int launch_gemm_partials(const uint8_t* w, const int8_t* xq, int32_t* acc, int64_t rows, int64_t Ng, int64_t Kg, int G,
                          bool two_groups, hipStream_t st);
 int launch_fc_rows(const uint8_t* w, const int8_t* xq, const float2* xsT, float* y, int64_t rows, int64_t Ng, int64_t Kg,
@@ -111,7 +112,7 @@ static int fc_impl(const float* x, int64_t rows, int64_t K, const int8_t* weiq, 
     if (rows_kernel && (rows <= 16 || (rows <= 32 && Ng < 256)))
         return launch_fc_rows(w, xq, xst, y, rows, Ng, Kg, N, residual, reinterpret_cast<unsigned long long*>(ws + kTicketBytes),
                               LLMOPS_FC_COUNTER_BYTES - kTicketBytes, st);
-    return launch_gemm(w, xq, xd, gs, xst, y, part, rows, Ng, Kg, group_k, N, residual, st);
+    return launch_gemm(w, xq, xd, gs, xst, y, part, counters, rows, Ng, Kg, group_k, N, residual, st);
 }
 
 extern "C" int llmops_fc_Q4A(const float* x, int64_t rows, int64_t K, const int8_t* weiq, int64_t Ng, int64_t Kg,
@@ -176,7 +177,7 @@ extern "C" int llmops_fc_Q4A_prequantized(const int8_t* xq, const float* xd, con
     hipStream_t st = as_stream(stream);
     if (rows <= kMaxGemvRows)
         return launch_gemv(w, xq, xd, gsum, y, part, reinterpret_cast<unsigned*>(ws), rows, Ng, Kg, group_k, N, st);
-    return launch_gemm(w, xq, xd, gsum, nullptr, y, part, rows, Ng, Kg, group_k, N, nullptr, st);
+    return launch_gemm(w, xq, xd, gsum, nullptr, y, part, reinterpret_cast<unsigned*>(ws), rows, Ng, Kg, group_k, N, nullptr, st);
 }
 
 extern "C" int llmops_fc_Q4A_partials(const int8_t* xq, int64_t rows, const int8_t* weiq, int64_t Ng, int64_t Kg,

@@ -16,6 +16,7 @@
 //   /root/reference/ops/op_fc.hpp:381-412; min term is m * raw group sum).
 // Result tile layout of the 16x16 MFMAs: lane holds column jj, rows 4*g+v in register v.
 #include "common.h"
+#include "gemv_device.h"
 
 namespace llmops {
 
@@ -190,7 +191,8 @@ __global__ __launch_bounds__(256, (RT == 4 ? 2 : (RT == 2 ? 3 : 4))) void fc_gem
                                                            const float2* __restrict__ xsT, float* __restrict__ out,
                                                            int32_t* __restrict__ out_i, int Ng, int Kg, int64_t ldo,
                                                            int64_t N, int rows, int kb_per_split, int64_t split_stride,
-                                                           const float* __restrict__ residual) {
+                                                           const float* __restrict__ residual, float* __restrict__ y_final,
+                                                           int64_t Ny, unsigned* __restrict__ counters) {
     constexpr int BM = RT * 32;
     constexpr int A_CHUNKS = BM * 8;                     // 16-byte chunks of the A tile
     constexpr int A_PER_THREAD = A_CHUNKS / 256;         // RT
@@ -385,6 +387,92 @@ __global__ __launch_bounds__(256, (RT == 4 ? 2 : (RT == 2 ? 3 : 4))) void fc_gem
 
     if (PARTIALS) return;
     const int strip = strip0 + strip_l;
+    if (counters != nullptr) {
+        // Split-K without a second launch: every split stores its tile of partial sums with device-scope
+        // (write-through) stores, waits for them and takes a ticket on the tile's counter; the split that
+        // draws the last ticket adds all splits' tiles in index order (so the sum does not depend on who
+        // arrives when), adds the residual and writes the result.  Nobody waits for anybody.  The partial
+        // sums' row stride is a multiple of 32 floats and strips beyond Ng, rows beyond `rows` fall outside
+        // the buffer descriptor (loads return 0, stores are dropped); they are skipped anyway.
+        constexpr int kAgent = 16;  // sc1: coherent at device scope, as a relaxed atomic store / load would be
+        const int S = (int)gridDim.z;
+        const int tile_rows = min(BM, rows - row0);
+        const uint32_t tile_bytes = (uint32_t)tile_rows * (uint32_t)ldo * 4u;
+        const uint32_t col_off = (uint32_t)(strip * kGroupN + q * 4) * 4u;
+        const bool strip_ok = strip < Ng;
+        {
+            const buffer_rsrc rs = make_rsrc(out + (int64_t)blockIdx.z * split_stride + (int64_t)row0 * ldo, strip_ok ? tile_bytes : 0u);
+#pragma unroll
+            for (int t = 0; t < RT; t++)
+#pragma unroll
+                for (int v = 0; v < 4; v++) {
+                    const int r = wr * (BM / 2) + t * 16 + g * 4 + v;
+                    const u32x4 val = {__float_as_uint(f[t][0][v]), __float_as_uint(f[t][1][v]), __float_as_uint(f[t][2][v]),
+                                       __float_as_uint(f[t][3][v])};
+                    __builtin_amdgcn_raw_buffer_store_b128(val, rs, (uint32_t)r * (uint32_t)ldo * 4u + col_off, 0, kAgent);
+                }
+        }
+        __shared__ unsigned ticket_sh;
+        __builtin_amdgcn_s_waitcnt(0);  // this wave's stores have been acknowledged
+        __syncthreads();
+        if (tid == 0) ticket_sh = __hip_atomic_fetch_add(&counters[by * nbx + bx], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();
+        if (ticket_sh != (unsigned)(S - 1)) return;
+        if (tid == 0) __hip_atomic_store(&counters[by * nbx + bx], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // next launch
+        if (!strip_ok) return;
+        const int64_t n0 = (int64_t)strip * kGroupN + q * 4;
+        // One row tile at a time, all of its loads (up to SU splits x 4 rows) in flight together: the
+        // reduction then costs about RT round trips to memory whatever the split count.  A split past the
+        // last is asked for through an empty descriptor: it returns 0 without touching memory.
+        constexpr int SU = RT == 4 ? 12 : (RT == 2 ? 6 : 4);
+#pragma unroll
+        for (int t = 0; t < RT; t++) {
+            float4 a[4];
+#pragma unroll
+            for (int v = 0; v < 4; v++) a[v] = make_float4(0.f, 0.f, 0.f, 0.f);
+            for (int s0 = 0; s0 < S; s0 += SU) {
+                u32x4 pv[SU][4];
+#pragma unroll
+                for (int u = 0; u < SU; u++) {
+                    const int sidx = min(s0 + u, S - 1);
+                    const buffer_rsrc rs =
+                        make_rsrc(out + (int64_t)sidx * split_stride + (int64_t)row0 * ldo, s0 + u < S ? tile_bytes : 0u);
+#pragma unroll
+                    for (int v = 0; v < 4; v++)
+                        pv[u][v] = __builtin_amdgcn_raw_buffer_load_b128(
+                            rs, (uint32_t)(wr * (BM / 2) + t * 16 + g * 4 + v) * (uint32_t)ldo * 4u + col_off, 0, kAgent);
+                }
+#pragma unroll
+                for (int u = 0; u < SU; u++)
+#pragma unroll
+                    for (int v = 0; v < 4; v++) {
+                        a[v].x += __uint_as_float(pv[u][v][0]), a[v].y += __uint_as_float(pv[u][v][1]);
+                        a[v].z += __uint_as_float(pv[u][v][2]), a[v].w += __uint_as_float(pv[u][v][3]);
+                    }
+            }
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                const int row = row0 + wr * (BM / 2) + t * 16 + g * 4 + v;
+                if (row >= rows) continue;
+                float* dst = y_final + (int64_t)row * Ny + n0;
+                const float* res = residual ? residual + (int64_t)row * Ny + n0 : nullptr;
+                if (n0 + 3 < Ny && (Ny & 3) == 0) {
+                    float4 val = a[v];
+                    if (res) {
+                        const float4 r4 = *reinterpret_cast<const float4*>(res);
+                        val.x += r4.x, val.y += r4.y, val.z += r4.z, val.w += r4.w;
+                    }
+                    *reinterpret_cast<float4*>(dst) = val;
+                } else {
+                    const float av[4] = {a[v].x, a[v].y, a[v].z, a[v].w};
+#pragma unroll
+                    for (int c = 0; c < 4; c++)
+                        if (n0 + c < Ny) dst[c] = res ? av[c] + res[c] : av[c];
+                }
+            }
+        }
+        return;
+    }
     if (strip >= Ng) return;
     float* o = out + (int64_t)blockIdx.z * split_stride;
     const int64_t n0 = (int64_t)strip * kGroupN + q * 4;
@@ -877,6 +965,7 @@ struct GemmPlan {
 
 static int g_gemm_pp_min_rows = 256;
 static int g_gemm_rt = 0;  // 0 = choose per shape; -1 = also keep 9..32 rows on the tiled kernel
+static int g_gemm_fused_reduce = 1;  // split-K partial sums added by the product kernel itself (0: by a second launch)
 bool gemm_rows_kernel_enabled() { return g_gemm_rt >= 0; }
 
 // Split-K factor for `tiles` output tiles on a machine with `slots` resident workgroups.
@@ -957,7 +1046,8 @@ static void launch_gemm_t(const uint8_t* w, const int8_t* xq, const float* xd, c
 template <int RT>
 static int launch_gemm_lds_t(const uint8_t* w, const int8_t* xq, const float* xd, const float* gs, const float2* xsT,
                              float* out, int64_t Ng, int64_t Kg, int64_t ldo, int64_t N, int64_t rows, const GemmPlan& p,
-                             int64_t split_stride, const float* residual, hipStream_t st) {
+                             int64_t split_stride, const float* residual, float* y_final, int64_t Ny, unsigned* counters,
+                             hipStream_t st) {
     static bool configured = false;  // opt in to more than 64 KiB of dynamic LDS once per kernel
     if (!configured) {
         LLMOPS_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&fc_gemm_lds_kernel<RT, false>),
@@ -968,7 +1058,7 @@ static int launch_gemm_lds_t(const uint8_t* w, const int8_t* xq, const float* xd
     dim3 grid((unsigned)(8 * ((tiles + 7) / 8)), 1, (unsigned)p.S);  // one run of tiles per XCD
     fc_gemm_lds_kernel<RT, false><<<grid, 256, sizeof(GemmSmem<RT>), st>>>(w, xq, xd, gs, xsT, out, nullptr, (int)Ng, (int)Kg,
                                                                           ldo, N, (int)rows, p.kb_per_split, split_stride,
-                                                                          residual);
+                                                                          residual, y_final, Ny, counters);
     return LLMOPS_OK;
 }
 
@@ -992,11 +1082,21 @@ int launch_add(float* a, const float* b, int64_t total, hipStream_t st);  // mis
 
 // y = product (+ residual, fp32 [rows, N], may be y itself)
 int launch_gemm(const uint8_t* w, const int8_t* xq, const float* xd, const float* gs, const float2* xsT, float* y,
-                float* part, int64_t rows, int64_t Ng, int64_t Kg, int G, int64_t N, const float* residual, hipStream_t st) {
+                float* part, unsigned* counters, int64_t rows, int64_t Ng, int64_t Kg, int G, int64_t N, const float* residual,
+                hipStream_t st) {
     const GemmPlan p = plan_gemm(rows, Ng, Kg, G);
+    // With up to 12 splits the four-wave kernel adds the partial sums itself (the last split of a tile to arrive
+    // does), given one zeroed arrival counter per tile; otherwise a second launch adds them.  Measured (us, second
+    // launch / in kernel): 11008x4096 at 128 rows 29.3 / 25.7, at 256 rows 43.9 / 38.8; 4096x11008 at 384 rows
+    // 61.0 / 53.9, at 96 rows (11 splits) 28.6 / 24.6 - but at 128 rows (16 splits of a 128-row tile) 31.9 / 38.8:
+    // the one workgroup that adds 16 tiles takes longer than a launch that spreads them over the chip.
+    const int64_t lds_tiles = ((Ng + 3) / 4) * ((rows + p.RT * 32 - 1) / (p.RT * 32));
+    const bool fused_reduce = g_gemm_fused_reduce && p.S > 1 && p.lds && p.RT != 8 && counters != nullptr &&
+                              p.S <= 12 * g_gemm_fused_reduce && lds_tiles <= kTicketBytes / 4 && (int64_t)p.RT * 32 * Ng * kGroupN * 4 < ((int64_t)1 << 31);
     // the residual is added where the result is written: in the kernel's stores without split-K, in
     // the reduction of the partial sums with it
-    const float* kres = p.S > 1 ? nullptr : residual;
+    const float* kres = (p.S > 1 && !fused_reduce) ? nullptr : residual;
+    unsigned* kcnt = fused_reduce ? counters : nullptr;
     const int64_t Np = Ng * kGroupN;
     float* out = p.S > 1 ? part : y;
     const int64_t ldo = p.S > 1 ? Np : N;
@@ -1005,9 +1105,9 @@ int launch_gemm(const uint8_t* w, const int8_t* xq, const float* xd, const float
     if (p.lds) {
         int rc;
         if (p.RT == 8) rc = launch_gemm_pp(w, xq, xd, gs, xsT, out, Ng, Kg, ldo, Nw, rows, p, ss, kres, st);
-        else if (p.RT == 4) rc = launch_gemm_lds_t<4>(w, xq, xd, gs, xsT, out, Ng, Kg, ldo, Nw, rows, p, ss, kres, st);
-        else if (p.RT == 2) rc = launch_gemm_lds_t<2>(w, xq, xd, gs, xsT, out, Ng, Kg, ldo, Nw, rows, p, ss, kres, st);
-        else rc = launch_gemm_lds_t<1>(w, xq, xd, gs, xsT, out, Ng, Kg, ldo, Nw, rows, p, ss, kres, st);
+        else if (p.RT == 4) rc = launch_gemm_lds_t<4>(w, xq, xd, gs, xsT, out, Ng, Kg, ldo, Nw, rows, p, ss, kres, y, N, kcnt, st);
+        else if (p.RT == 2) rc = launch_gemm_lds_t<2>(w, xq, xd, gs, xsT, out, Ng, Kg, ldo, Nw, rows, p, ss, kres, y, N, kcnt, st);
+        else rc = launch_gemm_lds_t<1>(w, xq, xd, gs, xsT, out, Ng, Kg, ldo, Nw, rows, p, ss, kres, y, N, kcnt, st);
         if (rc) return rc;
     } else {
         if (p.RT == 4) launch_gemm_t<32, 4>(w, xq, xd, gs, out, Ng, Kg, ldo, Nw, rows, p, ss, st);
@@ -1015,7 +1115,7 @@ int launch_gemm(const uint8_t* w, const int8_t* xq, const float* xd, const float
         else launch_gemm_t<32, 1>(w, xq, xd, gs, out, Ng, Kg, ldo, Nw, rows, p, ss, st);
     }
     LLMOPS_LAUNCH_CHECK();
-    if (p.S > 1) {
+    if (p.S > 1 && !fused_reduce) {
         const int64_t total = rows * ((N + 3) / 4);
         gemm_reduce_kernel<<<(unsigned)((total + 255) / 256), 256, 0, st>>>(part, y, rows, N, Np, ss, p.S, residual);
         LLMOPS_LAUNCH_CHECK();
@@ -1050,7 +1150,7 @@ int launch_gemm_partials(const uint8_t* w, const int8_t* xq, int32_t* acc, int64
         const int64_t tiles = ((Ng + 3) / 4) * ((rows + 63) / 64);
         dim3 grid((unsigned)(8 * ((tiles + 7) / 8)), 1, 1);
         fc_gemm_lds_kernel<2, true><<<grid, 256, sizeof(GemmSmem<2>), st>>>(w, xq, nullptr, nullptr, nullptr, nullptr, acc,
-                                                                          (int)Ng, (int)Kg, 0, 0, (int)rows, (int)Kg, 0, nullptr);
+                                                                          (int)Ng, (int)Kg, 0, 0, (int)rows, (int)Kg, 0, nullptr, nullptr, 0, nullptr);
     } else {
         dim3 grid((unsigned)(((Ng + 1) / 2 + 3) / 4), (unsigned)((rows + 15) / 16), (unsigned)Kg);
         fc_gemm_partials_kernel<32><<<grid, 256, 0, st>>>(w, xq, acc, (int)Ng, (int)Kg, (int)rows);
@@ -1062,3 +1162,4 @@ int launch_gemm_partials(const uint8_t* w, const int8_t* xq, int32_t* acc, int64
 }  // namespace llmops
 
 extern "C" void llmops_gemm_set_tuning(int rows_per_wave_tile) { llmops::g_gemm_rt = rows_per_wave_tile; }
+extern "C" void llmops_gemm_set_reduce(int in_kernel) { llmops::g_gemm_fused_reduce = in_kernel < 0 ? 0 : in_kernel; }

@@ -61,6 +61,7 @@ SIGNATURES = {
     "llmops_calib_copy": (c_int, [c_ptr, c_ptr, c_i64, c_int, c_ptr]),
     "llmops_fc_set_tuning": (None, [c_int, c_int]),
     "llmops_gemm_set_tuning": (None, [c_int]),
+    "llmops_gemm_set_reduce": (None, [c_int]),
     "llmops_fc_set_row_routing": (None, [c_int, c_int]),
     "llmops_fc_rows_set_split": (None, [c_int]),
 }

@@ -505,3 +505,29 @@ def test_fc_on_concurrent_streams_matches_serial(ops):
     for per_stream in got:
         for ci, y in per_stream:
             assert torch.equal(y, serial[ci]), ci
+
+
+# ---- split-K of the prefill GEMM: partial sums added by the product kernel itself or by a second launch ------
+@pytest.mark.parametrize("M,N,K", [(128, 11008, 4096), (128, 4096, 11008), (96, 4090, 4096), (40, 1000, 11008), (256, 4096, 11008),
+                                   (512, 4096, 11008), (33, 352, 2048)])
+def test_gemm_split_k_reduced_in_kernel_equals_second_launch(ops, M, N, K):
+    from llmops import _lib
+    lib = _lib.load()
+    rng = np.random.default_rng(M + N)
+    wq = ops.offline_FC_quant_Q4A(dev((rng.standard_normal((N, K)) * 0.02).astype(np.float32)), 128)
+    x = dev(rng.standard_normal((1, M, K)).astype(np.float32))
+    res = dev(rng.standard_normal((1, M, N)).astype(np.float32))
+    try:
+        lib.llmops_gemm_set_reduce(0)
+        want, want_res = ops.fc_Q4A(x, wq, N), ops.fc_Q4A(x, wq, N, residual=res)
+        for mode in (1, 100):                                     # default rule; every split count (several load batches)
+            lib.llmops_gemm_set_reduce(mode)
+            for _ in range(3):                                    # the arrival counters are left at zero for the next call
+                assert torch.equal(ops.fc_Q4A(x, wq, N), want)
+                assert torch.equal(ops.fc_Q4A(x, wq, N, residual=res), want_res)
+    finally:
+        lib.llmops_gemm_set_reduce(1)
+    # and the decode kernels, which share the counters, still find them at zero
+    y1 = ops.fc_Q4A(x[:, :1].contiguous(), wq, N)
+    assert torch.equal(y1, ops.fc_Q4A(x[:, :1].contiguous(), wq, N))
+    assert max_rel_err(host(y1)[0, 0], host(want)[0, 0]) <= TOL
