@@ -164,6 +164,97 @@ __global__ __launch_bounds__(256) void fc_gemm_kernel(const uint8_t* __restrict_
         }
 }
 
+// ---- split-K without a second launch -------------------------------------------------------------------
+// Every split stores its tile of partial sums with device-scope (write-through) stores, waits for them and
+// takes a ticket on the tile's counter; the split that draws the last ticket adds all splits' tiles in
+// index order (so the sum does not depend on who arrives when), adds the residual and writes the result.
+// Nobody waits for anybody.  The partial sums' row stride is a multiple of 32 floats; strips beyond Ng and
+// rows beyond `rows` fall outside the buffer descriptor (loads return 0, stores are dropped).
+// Called by every thread of the workgroup.  row0 / tile_rows: first row and row count of the rows this
+// thread's wave group owns; wave_row: the wave's first row inside them; a thread holds rows
+// wave_row + 16t + 4g + v, columns 32*strip + 4q .. + 3 in f[t][c][v].
+// The last arrival works one row tile at a time with all of its loads (up to SU splits x 4 rows) in flight
+// together: the reduction then costs about RT round trips to memory whatever the split count.  A split past
+// the last is asked for through an empty descriptor: it returns 0 without touching memory.
+template <int RT, int SU>
+__device__ __forceinline__ void splitk_finish(const v4f (&f)[RT][4], float* __restrict__ out, int64_t split_stride, int64_t ldo,
+                                              int row0, int tile_rows, int wave_row, int strip, int Ng, int q, int g, int rows,
+                                              float* __restrict__ y_final, int64_t Ny, const float* __restrict__ residual,
+                                              unsigned* counter, int tid) {
+    constexpr int kAgent = 16;  // sc1: coherent at device scope, as a relaxed atomic store / load would be
+    const int S = (int)gridDim.z;
+    const uint32_t tile_bytes = tile_rows > 0 ? (uint32_t)tile_rows * (uint32_t)ldo * 4u : 0u;
+    const uint32_t col_off = (uint32_t)(strip * kGroupN + q * 4) * 4u;
+    const bool strip_ok = strip < Ng;
+    {
+        const buffer_rsrc rs = make_rsrc(out + (int64_t)blockIdx.z * split_stride + (int64_t)row0 * ldo, strip_ok ? tile_bytes : 0u);
+#pragma unroll
+        for (int t = 0; t < RT; t++)
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                const int r = wave_row + t * 16 + g * 4 + v;
+                const u32x4 val = {__float_as_uint(f[t][0][v]), __float_as_uint(f[t][1][v]), __float_as_uint(f[t][2][v]),
+                                   __float_as_uint(f[t][3][v])};
+                __builtin_amdgcn_raw_buffer_store_b128(val, rs, (uint32_t)r * (uint32_t)ldo * 4u + col_off, 0, kAgent);
+            }
+    }
+    __shared__ unsigned ticket_sh;
+    __builtin_amdgcn_s_waitcnt(0);  // this wave's stores have been acknowledged
+    __syncthreads();
+    if (tid == 0) ticket_sh = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    if (ticket_sh != (unsigned)(S - 1)) return;
+    if (tid == 0) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // next launch
+    if (!strip_ok) return;
+    const int64_t n0 = (int64_t)strip * kGroupN + q * 4;
+#pragma unroll
+    for (int t = 0; t < RT; t++) {
+        float4 a[4];
+#pragma unroll
+        for (int v = 0; v < 4; v++) a[v] = make_float4(0.f, 0.f, 0.f, 0.f);
+        for (int s0 = 0; s0 < S; s0 += SU) {
+            u32x4 pv[SU][4];
+#pragma unroll
+            for (int u = 0; u < SU; u++) {
+                const int sidx = min(s0 + u, S - 1);
+                const buffer_rsrc rs =
+                    make_rsrc(out + (int64_t)sidx * split_stride + (int64_t)row0 * ldo, s0 + u < S ? tile_bytes : 0u);
+#pragma unroll
+                for (int v = 0; v < 4; v++)
+                    pv[u][v] = __builtin_amdgcn_raw_buffer_load_b128(
+                        rs, (uint32_t)(wave_row + t * 16 + g * 4 + v) * (uint32_t)ldo * 4u + col_off, 0, kAgent);
+            }
+#pragma unroll
+            for (int u = 0; u < SU; u++)
+#pragma unroll
+                for (int v = 0; v < 4; v++) {
+                    a[v].x += __uint_as_float(pv[u][v][0]), a[v].y += __uint_as_float(pv[u][v][1]);
+                    a[v].z += __uint_as_float(pv[u][v][2]), a[v].w += __uint_as_float(pv[u][v][3]);
+                }
+        }
+#pragma unroll
+        for (int v = 0; v < 4; v++) {
+            const int row = row0 + wave_row + t * 16 + g * 4 + v;
+            if (row >= rows) continue;
+            float* dst = y_final + (int64_t)row * Ny + n0;
+            const float* res = residual ? residual + (int64_t)row * Ny + n0 : nullptr;
+            if (n0 + 3 < Ny && (Ny & 3) == 0) {
+                float4 val = a[v];
+                if (res) {
+                    const float4 r4 = *reinterpret_cast<const float4*>(res);
+                    val.x += r4.x, val.y += r4.y, val.z += r4.z, val.w += r4.w;
+                }
+                *reinterpret_cast<float4*>(dst) = val;
+            } else {
+                const float av[4] = {a[v].x, a[v].y, a[v].z, a[v].w};
+#pragma unroll
+                for (int c = 0; c < 4; c++)
+                    if (n0 + c < Ny) dst[c] = res ? av[c] + res[c] : av[c];
+            }
+        }
+    }
+}
+
 // ---- LDS-tiled kernel for group 128 ---------------------------------------------------------------
 // Workgroup = 4 wavefronts (2 x 2), tile = BM rows x 128 columns (4 strips), one k-group per
 // iteration.  Per iteration the workgroup stages into LDS, through registers and double buffered:
@@ -388,89 +479,8 @@ __global__ __launch_bounds__(256, (RT == 4 ? 2 : (RT == 2 ? 3 : 4))) void fc_gem
     if (PARTIALS) return;
     const int strip = strip0 + strip_l;
     if (counters != nullptr) {
-        // Split-K without a second launch: every split stores its tile of partial sums with device-scope
-        // (write-through) stores, waits for them and takes a ticket on the tile's counter; the split that
-        // draws the last ticket adds all splits' tiles in index order (so the sum does not depend on who
-        // arrives when), adds the residual and writes the result.  Nobody waits for anybody.  The partial
-        // sums' row stride is a multiple of 32 floats and strips beyond Ng, rows beyond `rows` fall outside
-        // the buffer descriptor (loads return 0, stores are dropped); they are skipped anyway.
-        constexpr int kAgent = 16;  // sc1: coherent at device scope, as a relaxed atomic store / load would be
-        const int S = (int)gridDim.z;
-        const int tile_rows = min(BM, rows - row0);
-        const uint32_t tile_bytes = (uint32_t)tile_rows * (uint32_t)ldo * 4u;
-        const uint32_t col_off = (uint32_t)(strip * kGroupN + q * 4) * 4u;
-        const bool strip_ok = strip < Ng;
-        {
-            const buffer_rsrc rs = make_rsrc(out + (int64_t)blockIdx.z * split_stride + (int64_t)row0 * ldo, strip_ok ? tile_bytes : 0u);
-#pragma unroll
-            for (int t = 0; t < RT; t++)
-#pragma unroll
-                for (int v = 0; v < 4; v++) {
-                    const int r = wr * (BM / 2) + t * 16 + g * 4 + v;
-                    const u32x4 val = {__float_as_uint(f[t][0][v]), __float_as_uint(f[t][1][v]), __float_as_uint(f[t][2][v]),
-                                       __float_as_uint(f[t][3][v])};
-                    __builtin_amdgcn_raw_buffer_store_b128(val, rs, (uint32_t)r * (uint32_t)ldo * 4u + col_off, 0, kAgent);
-                }
-        }
-        __shared__ unsigned ticket_sh;
-        __builtin_amdgcn_s_waitcnt(0);  // this wave's stores have been acknowledged
-        __syncthreads();
-        if (tid == 0) ticket_sh = __hip_atomic_fetch_add(&counters[by * nbx + bx], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __syncthreads();
-        if (ticket_sh != (unsigned)(S - 1)) return;
-        if (tid == 0) __hip_atomic_store(&counters[by * nbx + bx], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // next launch
-        if (!strip_ok) return;
-        const int64_t n0 = (int64_t)strip * kGroupN + q * 4;
-        // One row tile at a time, all of its loads (up to SU splits x 4 rows) in flight together: the
-        // reduction then costs about RT round trips to memory whatever the split count.  A split past the
-        // last is asked for through an empty descriptor: it returns 0 without touching memory.
-        constexpr int SU = RT == 4 ? 12 : (RT == 2 ? 6 : 4);
-#pragma unroll
-        for (int t = 0; t < RT; t++) {
-            float4 a[4];
-#pragma unroll
-            for (int v = 0; v < 4; v++) a[v] = make_float4(0.f, 0.f, 0.f, 0.f);
-            for (int s0 = 0; s0 < S; s0 += SU) {
-                u32x4 pv[SU][4];
-#pragma unroll
-                for (int u = 0; u < SU; u++) {
-                    const int sidx = min(s0 + u, S - 1);
-                    const buffer_rsrc rs =
-                        make_rsrc(out + (int64_t)sidx * split_stride + (int64_t)row0 * ldo, s0 + u < S ? tile_bytes : 0u);
-#pragma unroll
-                    for (int v = 0; v < 4; v++)
-                        pv[u][v] = __builtin_amdgcn_raw_buffer_load_b128(
-                            rs, (uint32_t)(wr * (BM / 2) + t * 16 + g * 4 + v) * (uint32_t)ldo * 4u + col_off, 0, kAgent);
-                }
-#pragma unroll
-                for (int u = 0; u < SU; u++)
-#pragma unroll
-                    for (int v = 0; v < 4; v++) {
-                        a[v].x += __uint_as_float(pv[u][v][0]), a[v].y += __uint_as_float(pv[u][v][1]);
-                        a[v].z += __uint_as_float(pv[u][v][2]), a[v].w += __uint_as_float(pv[u][v][3]);
-                    }
-            }
-#pragma unroll
-            for (int v = 0; v < 4; v++) {
-                const int row = row0 + wr * (BM / 2) + t * 16 + g * 4 + v;
-                if (row >= rows) continue;
-                float* dst = y_final + (int64_t)row * Ny + n0;
-                const float* res = residual ? residual + (int64_t)row * Ny + n0 : nullptr;
-                if (n0 + 3 < Ny && (Ny & 3) == 0) {
-                    float4 val = a[v];
-                    if (res) {
-                        const float4 r4 = *reinterpret_cast<const float4*>(res);
-                        val.x += r4.x, val.y += r4.y, val.z += r4.z, val.w += r4.w;
-                    }
-                    *reinterpret_cast<float4*>(dst) = val;
-                } else {
-                    const float av[4] = {a[v].x, a[v].y, a[v].z, a[v].w};
-#pragma unroll
-                    for (int c = 0; c < 4; c++)
-                        if (n0 + c < Ny) dst[c] = res ? av[c] + res[c] : av[c];
-                }
-            }
-        }
+        splitk_finish<RT, (RT == 4 ? 12 : (RT == 2 ? 6 : 4))>(f, out, split_stride, ldo, row0, min(BM, rows - row0), wr * (BM / 2), strip,
+                                                             Ng, q, g, rows, y_final, Ny, residual, &counters[by * nbx + bx], tid);
         return;
     }
     if (strip >= Ng) return;
@@ -1089,7 +1099,9 @@ int launch_gemm(const uint8_t* w, const int8_t* xq, const float* xd, const float
     // does), given one zeroed arrival counter per tile; otherwise a second launch adds them.  Measured (us, second
     // launch / in kernel): 11008x4096 at 128 rows 29.3 / 25.7, at 256 rows 43.9 / 38.8; 4096x11008 at 384 rows
     // 61.0 / 53.9, at 96 rows (11 splits) 28.6 / 24.6 - but at 128 rows (16 splits of a 128-row tile) 31.9 / 38.8:
-    // the one workgroup that adds 16 tiles takes longer than a launch that spreads them over the chip.
+    // the one workgroup that adds 16 tiles takes longer than a launch that spreads them over the chip.  The
+    // 256-row kernel keeps the second launch: with one workgroup per CU nothing covers the last arrival's tail
+    // (4096x11008, 256 rows: 42.2 / 49.1; 512 rows: 66.1 / 70.4).
     const int64_t lds_tiles = ((Ng + 3) / 4) * ((rows + p.RT * 32 - 1) / (p.RT * 32));
     const bool fused_reduce = g_gemm_fused_reduce && p.S > 1 && p.lds && p.RT != 8 && counters != nullptr &&
                               p.S <= 12 * g_gemm_fused_reduce && lds_tiles <= kTicketBytes / 4 && (int64_t)p.RT * 32 * Ng * kGroupN * 4 < ((int64_t)1 << 31);

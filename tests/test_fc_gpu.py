@@ -509,7 +509,7 @@ def test_fc_on_concurrent_streams_matches_serial(ops):
 
 # ---- split-K of the prefill GEMM: partial sums added by the product kernel itself or by a second launch ------
 @pytest.mark.parametrize("M,N,K", [(128, 11008, 4096), (128, 4096, 11008), (96, 4090, 4096), (40, 1000, 11008), (256, 4096, 11008),
-                                   (512, 4096, 11008), (33, 352, 2048)])
+                                   (512, 4096, 11008), (33, 352, 2048), (300, 4090, 11008), (700, 1000, 4096)])
 def test_gemm_split_k_reduced_in_kernel_equals_second_launch(ops, M, N, K):
     from llmops import _lib
     lib = _lib.load()
