@@ -1025,7 +1025,13 @@ static GemmPlan plan_gemm(int64_t rows, int64_t Ng, int64_t Kg, int G) {
             q.S = (int)((Kg + q.kb_per_split - 1) / q.kb_per_split);
             const int64_t rounds = (tiles * q.S + slots - 1) / slots;
             double cost = (double)rounds * (double)(bm * kWgPerCu[i]) / kEff[i] * (double)q.kb_per_split / (double)Kg;
-            if (q.S > 1) cost *= 1.1;  // the partial sums take a second launch
+            // Split-K is not free.  In the unit of this estimate (rows x share of K; about 0.014 us x Kg) the last
+            // split of a tile to arrive adds S tiles of bm rows at ~150 GB/s (0.24 * S * bm / Kg); a second launch
+            // over the partial sums costs about 8 us whatever the shape (570 / Kg).
+            if (q.S > 1) {
+                const bool in_kernel = g_gemm_fused_reduce && q.S <= 12 * g_gemm_fused_reduce && kRT[i] != 8;
+                cost += in_kernel ? 0.24 * (double)q.S * (double)bm / (double)Kg : 570.0 / (double)Kg;
+            }
             if (best == 0.0 || cost < best) {
                 best = cost;
                 p = q;

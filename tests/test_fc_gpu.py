@@ -522,9 +522,15 @@ def test_gemm_split_k_reduced_in_kernel_equals_second_launch(ops, M, N, K):
         want, want_res = ops.fc_Q4A(x, wq, N), ops.fc_Q4A(x, wq, N, residual=res)
         for mode in (1, 100):                                     # default rule; every split count (several load batches)
             lib.llmops_gemm_set_reduce(mode)
+            # The planner prices the two ways of adding differently, so the tile size and split count, and with
+            # them the order of the fp32 additions, may differ from the second-launch run: equal to rounding.
+            # Within a mode the result must not depend on which split arrives last: bit-identical repeats.
+            first, first_res = ops.fc_Q4A(x, wq, N), ops.fc_Q4A(x, wq, N, residual=res)
+            assert max_rel_err(host(first), host(want)) <= 1e-5
+            assert max_rel_err(host(first_res), host(want_res)) <= 1e-5
             for _ in range(3):                                    # the arrival counters are left at zero for the next call
-                assert torch.equal(ops.fc_Q4A(x, wq, N), want)
-                assert torch.equal(ops.fc_Q4A(x, wq, N, residual=res), want_res)
+                assert torch.equal(ops.fc_Q4A(x, wq, N), first)
+                assert torch.equal(ops.fc_Q4A(x, wq, N, residual=res), first_res)
     finally:
         lib.llmops_gemm_set_reduce(1)
     # and the decode kernels, which share the counters, still find them at zero
