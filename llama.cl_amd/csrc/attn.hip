@@ -284,7 +284,10 @@ __global__ __launch_bounds__(128) void attn_merge_kernel(float* __restrict__ q, 
 // chunk holds the new token's cache row rotates k, writes the rotated k back in place and k, v
 // into the cache, and attends to the new row from registers; attn_merge_kernel then combines the
 // chunk records into q.  (Merging inside this kernel through an arrival ticket was measured
-// slower: the last workgroup's device-scope loads of 32 chunk records cost more than a launch.)
+// slower, also with all of the last workgroup's record loads in flight at once: kv 2048 21.5 against
+// 18.4 us, kv 4096 39.9 against 30.9 us.  Every workgroup then waits for the acknowledgement of its
+// device-scope stores and for its ticket, 3-4 us during which it holds its place on the CU, and the
+// workgroups of the next round start that much later; a launch costs less.)
 template <typename T>
 __device__ __forceinline__ float cache_round(float v);
 template <>
