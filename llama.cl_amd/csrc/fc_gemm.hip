@@ -1017,7 +1017,9 @@ static GemmPlan plan_gemm(int64_t rows, int64_t Ng, int64_t Kg, int G) {
         const int64_t bm = kRows[i], slots = 256 * kWgPerCu[i];
         const int64_t tiles = ((Ng + 3) / 4) * ((rows + bm - 1) / bm);
         const int64_t s_floor = slots / tiles, s_ceil = (slots + tiles - 1) / tiles;
-        for (int64_t s_try : {s_floor, s_ceil}) {
+        // (a third candidate where the machine would take more: the most splits the product kernel still adds itself)
+        const int64_t s_cap = 12 * (int64_t)g_gemm_fused_reduce;
+        for (int64_t s_try : {s_floor, s_ceil, (s_cap > 0 && s_cap < s_floor && kRT[i] != 8) ? s_cap : s_floor}) {
             GemmPlan q = p;
             q.RT = kRT[i];
             int64_t S = s_try < 1 ? 1 : (s_try > Kg ? Kg : s_try);
@@ -1027,10 +1029,11 @@ static GemmPlan plan_gemm(int64_t rows, int64_t Ng, int64_t Kg, int G) {
             double cost = (double)rounds * (double)(bm * kWgPerCu[i]) / kEff[i] * (double)q.kb_per_split / (double)Kg;
             // Split-K is not free.  In the unit of this estimate (rows x share of K; about 0.014 us x Kg) the last
             // split of a tile to arrive adds S tiles of bm rows at ~150 GB/s (0.24 * S * bm / Kg); a second launch
-            // over the partial sums costs about 8 us whatever the shape (570 / Kg).
+            // over the partial sums costs 8-11 us whatever the shape (800 / Kg: the price at which the measured
+            // choices came out best; 4096x11008 at 40-64 rows 24-25.5 -> 21-21.8 us against 570 / Kg).
             if (q.S > 1) {
                 const bool in_kernel = g_gemm_fused_reduce && q.S <= 12 * g_gemm_fused_reduce && kRT[i] != 8;
-                cost += in_kernel ? 0.24 * (double)q.S * (double)bm / (double)Kg : 570.0 / (double)Kg;
+                cost += in_kernel ? 0.24 * (double)q.S * (double)bm / (double)Kg : 800.0 / (double)Kg;
             }
             if (best == 0.0 || cost < best) {
                 best = cost;
