@@ -30,7 +30,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 # of `--calib` (one FETCH_SIZE count = 2.000 KiB, one WRITE_SIZE count = 1.000 KiB on this part); the summary with
 # the per-shape figures is profiles/fc_gemv_fused_kernel__hbm_traffic_pmc.md.  Counters cannot be read from inside
 # this process, so the figure is the recorded one and only holds for the fused plan at group 128, M=1.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 27188748
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 27188727
 G = 128
 LAYERS = 32
 # (name, N, K) of one layer's FCs, in the order the model calls them (chatllama/main.py:344-375)
