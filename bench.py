@@ -335,12 +335,12 @@ def read_ceiling(torch, llmops, nbytes=2 << 30, reps=4):
     src = torch.zeros(nbytes, dtype=torch.uint8, device="cuda")
     out4 = torch.zeros(4, dtype=torch.int32, device="cuda")
     st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
-    llmops._lib.check(lib.llmops_calib_read(src.data_ptr(), nbytes, 8192, out4.data_ptr(), st))
+    llmops._lib.check(lib.llmops_test_calib_read(src.data_ptr(), nbytes, 8192, out4.data_ptr(), st))
     torch.cuda.synchronize()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     e0.record()
     for _ in range(reps):
-        llmops._lib.check(lib.llmops_calib_read(src.data_ptr(), nbytes, 8192, out4.data_ptr(), st))
+        llmops._lib.check(lib.llmops_test_calib_read(src.data_ptr(), nbytes, 8192, out4.data_ptr(), st))
     e1.record()
     torch.cuda.synchronize()
     return nbytes * reps / (e0.elapsed_time(e1) * 1e-3) / 1e9
@@ -357,8 +357,8 @@ def calib(nbytes=1 << 30, reps=5):
     out4 = torch.zeros(4, dtype=torch.int32, device="cuda")
     st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
     res = {"bytes": nbytes}
-    for name, fn in (("copy", lambda: lib.llmops_calib_copy(src.data_ptr(), dst.data_ptr(), nbytes, 4096, st)),
-                     ("read", lambda: lib.llmops_calib_read(src.data_ptr(), nbytes, 8192, out4.data_ptr(), st))):
+    for name, fn in (("copy", lambda: lib.llmops_test_calib_copy(src.data_ptr(), dst.data_ptr(), nbytes, 4096, st)),
+                     ("read", lambda: lib.llmops_test_calib_read(src.data_ptr(), nbytes, 8192, out4.data_ptr(), st))):
         fn()
         torch.cuda.synchronize()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)

@@ -209,92 +209,6 @@ int llmops_embedding_q8c(float* out, const int64_t* ids, int64_t n, const int8_t
 /* embedding (ops/op_embedding.hpp:24-49): out[i,:] = w[ids[i],:]; ids int64 */
 int llmops_embedding(float* out, const int64_t* ids, int64_t n, const float* w, int64_t V, int64_t E, llmops_stream_t stream);
 
-/* ------------------------------------------------------------------------------------------
- * A chain of dependent single-row FCs in one persistent launch
- * ------------------------------------------------------------------------------------------
- * What a decoder layer does between two attention calls (chatllama/main.py:344-375): rmsnorm ->
- * fc_Q4A (q|k|v) ... fc_Q4A (o) -> iadd -> rmsnorm -> fc_Q4A (gate, up) -> itrans("silu"), imul ->
- * fc_Q4A (down) -> iadd.  Each op is llmops_fc_Q4A_decode with rows = 1.  An op's x and residual
- * may be buffers written before the launch or the y of an earlier op of the chain (x = NULL is
- * short for the previous op's y); the kernel then waits for exactly the values it needs.  One
- * resident grid runs all ops and keeps weights streaming across op boundaries.  Outputs equal
- * llmops_fc_Q4A_decode's within fp32 summation order (the int32 dot products are the same).
- *
- * Rules: K = Kg*group_k <= 16384; Ng <= 8 * (compute units) (4 * with glu); group 32 needs an even
- * Kg; glu excludes residual; every op has its own y; a buffer that is read as written before the
- * launch (x or residual that is no earlier op's y) must not be the y of that op or a later one,
- * except that a residual may be the op's own y (in place).  */
-typedef struct llmops_chain_op {
-    const int8_t* weiq;    /* packed [Ng][Kg][block]; glu: gate/up strips interleaved */
-    int64_t Ng, Kg;
-    int64_t N_out;         /* outputs (glu: of silu(gate)*up) */
-    const float* x;        /* fp32 [K], or NULL = output of the previous op */
-    const float* norm_w;   /* optional fp32 [K]: rmsnorm(x)*norm_w first */
-    const float* residual; /* optional fp32 [N_out], added to the output */
-    float* y;              /* fp32 [N_out], always written */
-    float eps;
-    int32_t glu;
-} llmops_chain_op;
-
-/* bytes of device memory for the plan (op table) of n_ops ops */
-size_t llmops_fc_chain_plan_bytes(int n_ops);
-/* workspace bytes (sync words + one partial-sum region per op) for this chain on the current device */
-int llmops_fc_chain_workspace_bytes(const llmops_chain_op* ops, int n_ops, int group_k, size_t* bytes);
-/* Validates the chain, cuts every op over the device's compute units and writes the op table to
- * `plan` (device memory) with a synchronous copy: call it outside stream capture.  The first 256
- * bytes of `workspace` must be zero when the library first sees it and are left zero by every
- * launch that ends with status 0.  `ops` itself is not referenced after the call. */
-int llmops_fc_chain_build(const llmops_chain_op* ops, int n_ops, int group_k, void* plan, size_t plan_bytes,
-                          void* workspace, size_t workspace_bytes);
-/* Enqueues the chain (one kernel; capturable).  Two launches that share a workspace must not overlap. */
-int llmops_fc_chain_run(const void* plan, int n_ops, int group_k, void* workspace, llmops_stream_t stream);
-/* Synchronous read of the chain's status word: 0 = ok, 1 = a barrier wait ran out (the grid was
- * not co-resident or a launch overlapped another), 2 = plan built for another grid.  After a
- * non-zero status the outputs are invalid and the first 256 workspace bytes must be zeroed again. */
-int llmops_fc_chain_status(const void* workspace, int32_t* status);
-/* knobs: LDS ring depth in steps per wavefront (2..4, 0 = default), workgroups (0 = one per CU),
- * barrier wait limit in 100 MHz ticks (<= 0 keeps it) */
-void llmops_fc_chain_set_tuning(int ring_depth, int grid, long long spin_limit_ticks);
-/* diagnostics: when `buffer` (device, int64 [grid][n_ops][4]) is set, the first service wave of every
- * workgroup records the 100 MHz wall clock at four points of every op (op start, input row
- * quantized, all sums in LDS, outputs published).  NULL switches it off. */
-void llmops_fc_chain_set_trace(void* buffer);
-
-/* ------------------------------------------------------------------------------------------
- * Measurement helpers (no counterpart in the reference; used by bench.py and the profiles)
- * ------------------------------------------------------------------------------------------ */
-
-/* read / copy `bytes` (multiple of 16) with `workgroups` workgroups of 256 threads streaming
- * contiguous slabs: the machine's measured HBM ceiling and the calibration of traffic counters */
-int llmops_calib_read(const void* src, int64_t bytes, int workgroups, void* out4, llmops_stream_t stream);
-int llmops_calib_copy(const void* src, void* dst, int64_t bytes, int workgroups, llmops_stream_t stream);
-
-/* split-K planner knobs of the streaming FC kernel: number of workgroups to aim for and
- * wavefronts per workgroup (4, 8, 16; 0 = default).  Values <= 0 / < 0 leave a knob unchanged.
- * target_workgroups == -2 / -3 instead selects how two k-splits of a strip meet: through one 64-bit
- * exchange per output (default) / through the arrival ticket like larger split counts. */
-void llmops_fc_set_tuning(int target_workgroups, int waves_per_workgroup);
-
-/* prefill GEMM planner knob: force the row-tile factor of the LDS-tiled MFMA kernel (1, 2 or 4:
- * 32, 64 or 128 rows per workgroup; 8: the 256-row kernel whose two wave groups alternate between
- * MFMA and fold phases, which the planner takes from 512 rows on); 0 = choose per shape; -1 = choose
- * per shape and send 9..16 rows to the tiled kernel too instead of the weight-streaming MFMA kernel */
-void llmops_gemm_set_tuning(int row_tile_factor);
-
-/* prefill GEMM with split-K: the product kernel adds the partial sums itself (the last split of a tile to
- * arrive adds all of them in index order) when the split count is at most 12 x in_kernel; otherwise, and
- * always with 0, a second launch adds them.  Default 1.  Same result either way; kept for comparisons and tests. */
-void llmops_gemm_set_reduce(int in_kernel);
-
-/* weight-streaming MFMA kernel (3..16 rows, 17..32 for tensors of fewer than 256 strips): two workgroups per strip with half of K each for tensors of
- * fewer than 256 strips (default on; 0 switches it off, for comparisons and tests) */
-void llmops_fc_rows_set_split(int on);
-
-/* llmops_fc_Q4A with 2..8 rows, group 128: from how many rows the weight-streaming MFMA kernel (separate
- * quantization launch) replaces the streaming kernel that quantizes on the fly, for tensors of up to
- * 256 strips and for larger ones (defaults 4 and 3; values below 2 restore them) */
-void llmops_fc_set_row_routing(int rows_from_small, int rows_from_large);
-
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,56 @@
+/* llmops_hip_test.h -- hooks for tests and benchmarks of libllmops_hip.so.
+ *
+ * None of these has a counterpart in the reference and none is part of the product ABI
+ * (include/llmops_hip.h): they change process-wide planner state or run measurement kernels, so a
+ * program that serves requests must not call them.  Tests flip a knob, run one op, and restore the
+ * default in a finally block; bench.py uses the read/copy kernels for the measured HBM ceiling and
+ * to calibrate the traffic counters.
+ */
+#ifndef LLMOPS_HIP_TEST_H
+#define LLMOPS_HIP_TEST_H
+
+#include "llmops_hip.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ------------------------------------------------------------------------------------------
+ * Measurement helpers (used by bench.py and the profiles)
+ * ------------------------------------------------------------------------------------------ */
+
+/* read / copy `bytes` (multiple of 16) with `workgroups` workgroups of 256 threads streaming
+ * contiguous slabs: the machine's measured HBM ceiling and the calibration of traffic counters */
+int llmops_test_calib_read(const void* src, int64_t bytes, int workgroups, void* out4, llmops_stream_t stream);
+int llmops_test_calib_copy(const void* src, void* dst, int64_t bytes, int workgroups, llmops_stream_t stream);
+
+/* split-K planner knobs of the streaming FC kernel: number of workgroups to aim for and
+ * wavefronts per workgroup (4, 8, 16; 0 = default).  Values <= 0 / < 0 leave a knob unchanged.
+ * target_workgroups == -2 / -3 instead selects how two k-splits of a strip meet: through one 64-bit
+ * exchange per output (default) / through the arrival ticket like larger split counts. */
+void llmops_test_fc_set_tuning(int target_workgroups, int waves_per_workgroup);
+
+/* prefill GEMM planner knob: force the row-tile factor of the LDS-tiled MFMA kernel (1, 2 or 4:
+ * 32, 64 or 128 rows per workgroup; 8: the 256-row kernel whose two wave groups alternate between
+ * MFMA and fold phases, which the planner takes from 512 rows on); 0 = choose per shape; -1 = choose
+ * per shape and send 9..16 rows to the tiled kernel too instead of the weight-streaming MFMA kernel */
+void llmops_test_gemm_set_tuning(int row_tile_factor);
+
+/* prefill GEMM with split-K: the product kernel adds the partial sums itself (the last split of a tile to
+ * arrive adds all of them in index order) when the split count is at most 12 x in_kernel; otherwise, and
+ * always with 0, a second launch adds them.  Default 1.  Same result either way; kept for comparisons and tests. */
+void llmops_test_gemm_set_reduce(int in_kernel);
+
+/* weight-streaming MFMA kernel (3..16 rows, 17..32 for tensors of fewer than 256 strips): two workgroups per strip with half of K each for tensors of
+ * fewer than 256 strips (default on; 0 switches it off, for comparisons and tests) */
+void llmops_test_fc_rows_set_split(int on);
+
+/* llmops_fc_Q4A with 2..8 rows, group 128: from how many rows the weight-streaming MFMA kernel (separate
+ * quantization launch) replaces the streaming kernel that quantizes on the fly, for tensors of up to
+ * 256 strips and for larger ones (defaults 4 and 3; values below 2 restore them) */
+void llmops_test_fc_set_row_routing(int rows_from_small, int rows_from_large);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LLMOPS_HIP_TEST_H */

@@ -49,15 +49,15 @@ def check_spills(remarks):
                 raise RuntimeError(f"{name} spills {spilled} VGPRs; this kernel must not spill (see NO_SPILL)")
 
 
-def build(verbose=False):
-    cmd = [HIPCC] + FLAGS + ["-Rpass-analysis=kernel-resource-usage", "-o", OUT] + sources()
-    if verbose:
-        print(" ".join(cmd))
+def _compile(src, obj):
+    cmd = [HIPCC] + [f for f in FLAGS if f != "-shared"] + ["-Rpass-analysis=kernel-resource-usage", "-c", "-o", obj, src]
     proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
-    lines = proc.stdout.splitlines()
-    remarks = [l for l in lines if "[-Rpass-analysis=kernel-resource-usage]" in l]
-    # the host pass does not know the AMDGPU feature name and says so; that line is noise, and so are
-    # the resource remarks and the source lines the compiler quotes under each of them
+    return src, proc.returncode, proc.stdout.splitlines()
+
+
+def _readable(lines):
+    """the host pass does not know the AMDGPU feature name and says so; that line is noise, and so are
+    the resource remarks and the source lines the compiler quotes under each of them"""
     keep, skip = [], 0
     for l in lines:
         if "[-Rpass-analysis=kernel-resource-usage]" in l:
@@ -68,12 +68,40 @@ def build(verbose=False):
             continue
         if "is not a recognized feature for this target" not in l:
             keep.append(l)
-    log = "\n".join(keep)
-    if proc.returncode != 0:
-        raise RuntimeError("hipcc failed:\n" + log)
-    check_spills(remarks)
-    if verbose and log.strip():
-        print(log)
+    return "\n".join(keep)
+
+
+def build(verbose=False, jobs=None):
+    """Compiles every source to an object of its own (in parallel) and links the shared library.  Always
+    recompiles everything: the objects live in a scratch directory that is emptied first."""
+    import concurrent.futures
+    import shutil
+    import tempfile
+
+    objdir = tempfile.mkdtemp(prefix="llmops_build_")
+    try:
+        srcs = sources()
+        jobs = jobs or min(len(srcs), max(1, (os.cpu_count() or 2) - 1), 16)
+        objs = [os.path.join(objdir, os.path.basename(s) + ".o") for s in srcs]
+        with concurrent.futures.ThreadPoolExecutor(jobs) as ex:
+            results = list(ex.map(lambda so: _compile(*so), zip(srcs, objs)))
+        remarks, logs = [], []
+        for src, rc, lines in results:
+            remarks += [l for l in lines if "[-Rpass-analysis=kernel-resource-usage]" in l]
+            log = _readable(lines)
+            if rc != 0:
+                raise RuntimeError(f"hipcc failed on {src}:\n" + log)
+            if log.strip():
+                logs.append(log)
+        check_spills(remarks)
+        link = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", OUT] + objs
+        proc = subprocess.run(link, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+        if proc.returncode != 0:
+            raise RuntimeError("link failed:\n" + proc.stdout)
+        if verbose and logs:
+            print("\n".join(logs))
+    finally:
+        shutil.rmtree(objdir, ignore_errors=True)
     return OUT
 
 

@@ -10,6 +10,7 @@
 #include <string>
 
 #include "../../include/llmops_hip.h"
+#include "../../include/llmops_hip_test.h"
 
 namespace llmops {
 

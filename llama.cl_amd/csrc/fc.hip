@@ -193,7 +193,7 @@ extern "C" int llmops_fc_Q4A_partials(const int8_t* xq, int64_t rows, const int8
     return launch_gemv_partials(w, xq, acc, rows, Ng, Kg, group_k, as_stream(stream));
 }
 
-extern "C" void llmops_fc_set_row_routing(int rows_from_small, int rows_from_large) {
+extern "C" void llmops_test_fc_set_row_routing(int rows_from_small, int rows_from_large) {
     g_rows_from_small = rows_from_small >= 2 ? rows_from_small : 4;
     g_rows_from_large = rows_from_large >= 2 ? rows_from_large : 3;
 }

@@ -1182,5 +1182,5 @@ int launch_gemm_partials(const uint8_t* w, const int8_t* xq, int32_t* acc, int64
 
 }  // namespace llmops
 
-extern "C" void llmops_gemm_set_tuning(int rows_per_wave_tile) { llmops::g_gemm_rt = rows_per_wave_tile; }
-extern "C" void llmops_gemm_set_reduce(int in_kernel) { llmops::g_gemm_fused_reduce = in_kernel < 0 ? 0 : in_kernel; }
+extern "C" void llmops_test_gemm_set_tuning(int rows_per_wave_tile) { llmops::g_gemm_rt = rows_per_wave_tile; }
+extern "C" void llmops_test_gemm_set_reduce(int in_kernel) { llmops::g_gemm_fused_reduce = in_kernel < 0 ? 0 : in_kernel; }

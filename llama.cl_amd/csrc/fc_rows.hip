@@ -232,4 +232,4 @@ int launch_fc_rows(const uint8_t* w, const int8_t* xq, const float2* xsT, float*
 
 }  // namespace llmops
 
-extern "C" void llmops_fc_rows_set_split(int on) { llmops::g_rows_split = on != 0; }
+extern "C" void llmops_test_fc_rows_set_split(int on) { llmops::g_rows_split = on != 0; }

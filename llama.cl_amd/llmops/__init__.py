@@ -220,86 +220,6 @@ def fc_Q4A_decode(input, weiq, N_out, norm=None, residual=None, glu=False, sumsq
     return (out, sumsq) if want_sumsq else out
 
 
-class FcChain:
-    """A chain of dependent single-row FCs run by one persistent launch (extension; see
-    ``llmops_fc_chain_*`` in include/llmops_hip.h).
-
-    ``ops`` is a list of dicts with the arguments of ``fc_Q4A_decode`` for one row:
-    ``weiq`` (packed tensor), ``N_out``, ``x`` (fp32 [K] tensor or None = output of the previous op),
-    ``norm`` ((weight, eps) or None), ``residual`` (fp32 [N_out] tensor or None), ``glu`` (bool) and
-    ``y`` (fp32 [N_out] output tensor; allocated when missing).  ``run()`` enqueues the chain on
-    the current stream; ``outputs`` holds the y tensors in op order.  The object keeps every tensor
-    it references alive, so a HIP graph that captured ``run()`` stays valid as long as it does."""
-
-    def __init__(self, ops):
-        _require(len(ops) > 0, "n_ops > 0")
-        lib = _lib.load()
-        dev = ops[0]["weiq"].device
-        self.group_k = group_k_of(ops[0]["weiq"])
-        self.n_ops = len(ops)
-        self.outputs = []
-        self._keep = []
-        arr = (_lib.ChainOp * self.n_ops)()
-        for i, o in enumerate(ops):
-            w = o["weiq"]
-            _dev(w, torch.int8, 3, "wei_quantized")
-            _require(group_k_of(w) == self.group_k, "one group size per chain")
-            _require(w.device == dev, "one device per chain")
-            Ng, Kg, _ = w.shape
-            N_out = int(o["N_out"])
-            x, norm, res, y = o.get("x"), o.get("norm"), o.get("residual"), o.get("y")
-            if x is not None:
-                _dev(x, torch.float32, None, "x")
-                _require(x.numel() == Kg * self.group_k, "x.numel() == K")
-            if norm is not None:
-                _dev(norm[0], torch.float32, 1, "norm weight")
-                _require(norm[0].shape[0] == Kg * self.group_k, "weight.size(0) == K")
-            if res is not None:
-                _dev(res, torch.float32, None, "residual")
-                _require(res.numel() == N_out, "residual.numel() == N_out")
-            if y is None:
-                y = torch.empty(N_out, dtype=torch.float32, device=dev)
-            else:
-                _dev(y, torch.float32, None, "y")
-                _require(y.numel() == N_out, "y.numel() == N_out")
-            arr[i].weiq, arr[i].Ng, arr[i].Kg, arr[i].N_out = _ptr(w), Ng, Kg, N_out
-            arr[i].x = _ptr(x) if x is not None else None
-            arr[i].norm_w = _ptr(norm[0]) if norm is not None else None
-            arr[i].eps = float(norm[1]) if norm is not None else 0.0
-            arr[i].residual = _ptr(res) if res is not None else None
-            arr[i].y = _ptr(y)
-            arr[i].glu = int(bool(o.get("glu", False)))
-            self.outputs.append(y)
-            self._keep.append((w, x, norm, res, y))
-        need = ctypes.c_size_t(0)
-        with torch.cuda.device(dev):
-            _lib.check(lib.llmops_fc_chain_workspace_bytes(arr, self.n_ops, self.group_k, ctypes.byref(need)))
-            self.workspace = torch.zeros(need.value, dtype=torch.uint8, device=dev)
-            self.plan = torch.zeros(lib.llmops_fc_chain_plan_bytes(self.n_ops), dtype=torch.uint8, device=dev)
-            torch.cuda.synchronize(dev)
-            _lib.check(lib.llmops_fc_chain_build(arr, self.n_ops, self.group_k, _ptr(self.plan), self.plan.numel(),
-                                                 _ptr(self.workspace), self.workspace.numel()))
-        self.device = dev
-
-    def run(self):
-        with torch.cuda.device(self.device):
-            _lib.check(_lib.load().llmops_fc_chain_run(_ptr(self.plan), self.n_ops, self.group_k, _ptr(self.workspace),
-                                                       torch.cuda.current_stream(self.device).cuda_stream))
-        return self.outputs
-
-    def status(self):
-        """Synchronises and returns the chain's status word (0 = ok); raises on a failed launch."""
-        st = ctypes.c_int32(0)
-        with torch.cuda.device(self.device):
-            torch.cuda.synchronize(self.device)
-            _lib.check(_lib.load().llmops_fc_chain_status(_ptr(self.workspace), ctypes.byref(st)))
-        if st.value != 0:
-            self.workspace[:256].zero_()
-            raise RuntimeError(f"fc chain ended with status {st.value} "
-                               "(1: a grid barrier timed out, 2: plan built for another grid)")
-        return 0
-
-
 def fc_Q4A_partials(xq, weiq, use_mfma=False):
     """The exact int32 core of fc_Q4A: int8 [..,Kg*G] x packed -> int32 [.., Ng*32, Kg]."""
     _dev(xq, torch.int8, None, "xq")

@@ -11,13 +11,7 @@ c_f32 = ctypes.c_float
 c_ptr = ctypes.c_void_p
 c_size = ctypes.c_size_t
 
-class ChainOp(ctypes.Structure):
-    """struct llmops_chain_op of include/llmops_hip.h"""
-    _fields_ = [("weiq", c_ptr), ("Ng", c_i64), ("Kg", c_i64), ("N_out", c_i64), ("x", c_ptr), ("norm_w", c_ptr),
-                ("residual", c_ptr), ("y", c_ptr), ("eps", c_f32), ("glu", ctypes.c_int32)]
-
-
-# name -> (restype, argtypes); kept in the order of include/llmops_hip.h
+# name -> (restype, argtypes); kept in the order of include/llmops_hip.h, then include/llmops_hip_test.h
 SIGNATURES = {
     "llmops_last_error": (ctypes.c_char_p, []),
     "llmops_abi_version": (c_int, []),
@@ -50,20 +44,13 @@ SIGNATURES = {
     "llmops_embedding_q8c_quant_w": (c_int, [c_ptr, c_i64, c_i64, c_ptr, c_ptr, c_ptr]),
     "llmops_embedding_q8c": (c_int, [c_ptr, c_ptr, c_i64, c_ptr, c_ptr, c_i64, c_i64, c_ptr]),
     "llmops_embedding": (c_int, [c_ptr, c_ptr, c_i64, c_ptr, c_i64, c_i64, c_ptr]),
-    "llmops_fc_chain_plan_bytes": (c_size, [c_int]),
-    "llmops_fc_chain_workspace_bytes": (c_int, [c_ptr, c_int, c_int, c_ptr]),
-    "llmops_fc_chain_build": (c_int, [c_ptr, c_int, c_int, c_ptr, c_size, c_ptr, c_size]),
-    "llmops_fc_chain_run": (c_int, [c_ptr, c_int, c_int, c_ptr, c_ptr]),
-    "llmops_fc_chain_status": (c_int, [c_ptr, c_ptr]),
-    "llmops_fc_chain_set_tuning": (None, [c_int, c_int, ctypes.c_longlong]),
-    "llmops_fc_chain_set_trace": (None, [c_ptr]),
-    "llmops_calib_read": (c_int, [c_ptr, c_i64, c_int, c_ptr, c_ptr]),
-    "llmops_calib_copy": (c_int, [c_ptr, c_ptr, c_i64, c_int, c_ptr]),
-    "llmops_fc_set_tuning": (None, [c_int, c_int]),
-    "llmops_gemm_set_tuning": (None, [c_int]),
-    "llmops_gemm_set_reduce": (None, [c_int]),
-    "llmops_fc_set_row_routing": (None, [c_int, c_int]),
-    "llmops_fc_rows_set_split": (None, [c_int]),
+    "llmops_test_calib_read": (c_int, [c_ptr, c_i64, c_int, c_ptr, c_ptr]),
+    "llmops_test_calib_copy": (c_int, [c_ptr, c_ptr, c_i64, c_int, c_ptr]),
+    "llmops_test_fc_set_tuning": (None, [c_int, c_int]),
+    "llmops_test_gemm_set_tuning": (None, [c_int]),
+    "llmops_test_gemm_set_reduce": (None, [c_int]),
+    "llmops_test_fc_set_row_routing": (None, [c_int, c_int]),
+    "llmops_test_fc_rows_set_split": (None, [c_int]),
 }
 
 _lib = None

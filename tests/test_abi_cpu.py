@@ -8,12 +8,12 @@ import pytest
 
 from conftest import ROOT
 
-HEADER = os.path.join(ROOT, "include", "llmops_hip.h")
+HEADERS = [os.path.join(ROOT, "include", n) for n in ("llmops_hip.h", "llmops_hip_test.h")]
 LIB = os.path.join(ROOT, "llama.cl_amd", "llmops", "libllmops_hip.so")
 
 
 def declared_symbols():
-    src = open(HEADER).read()
+    src = "".join(open(h).read() for h in HEADERS)
     src = re.sub(r"/\*.*?\*/", "", src, flags=re.S)
     return sorted(set(re.findall(r"\b(llmops_[A-Za-z0-9_]+)\s*\(", src)))
 

@@ -353,7 +353,7 @@ def test_fc_two_k_splits_both_handoffs(ops, orc, rows, N, K):
     got = {}
     try:
         for knob in (-2, -3, -2):
-            lib.llmops_fc_set_tuning(knob, -1)
+            lib.llmops_test_fc_set_tuning(knob, -1)
             a = ops.fc_Q4A(dev(x), pw, N)
             b = ops.fc_Q4A(dev(x), pw, N)
             c = ops.fc_Q4A_decode(dev(x), pw, N, residual=dev(res))
@@ -364,7 +364,7 @@ def test_fc_two_k_splits_both_handoffs(ops, orc, rows, N, K):
                 assert torch.equal(a, got["a"]) and torch.equal(c, got["c"])
             got = {"a": a, "c": c}
     finally:
-        lib.llmops_fc_set_tuning(-2, -1)
+        lib.llmops_test_fc_set_tuning(-2, -1)
 
 
 @pytest.mark.parametrize("rows", [3, 5, 8, 9, 13, 16, 17, 24, 32])
@@ -384,7 +384,7 @@ def test_fc_rows_kernel_two_k_halves(ops, orc, rows, N, K):
     want = orc.fc(x, host(pw), N)
     try:
         for on in (1, 0, 1):
-            lib.llmops_fc_rows_set_split(on)
+            lib.llmops_test_fc_rows_set_split(on)
             a = ops.fc_Q4A(dev(x), pw, N)
             b = ops.fc_Q4A(dev(x), pw, N)
             c = ops.fc_Q4A(dev(x), pw, N, residual=dev(res))
@@ -392,7 +392,7 @@ def test_fc_rows_kernel_two_k_halves(ops, orc, rows, N, K):
             assert max_rel_err(host(a), want) <= 1e-5
             assert max_rel_err(host(c), want + res) <= 1e-5
     finally:
-        lib.llmops_fc_rows_set_split(1)
+        lib.llmops_test_fc_rows_set_split(1)
 
 
 @pytest.mark.parametrize("rows", [2, 3, 4, 6, 8])
@@ -412,13 +412,13 @@ def test_fc_few_rows_either_kernel(ops, orc, rows, N, K):
     want = orc.fc(x, host(pw), N)
     try:
         for first in (9, 2, 0):  # streaming kernel for all of 2..8 rows; MFMA kernel from 2 rows; defaults
-            lib.llmops_fc_set_row_routing(first, first)
+            lib.llmops_test_fc_set_row_routing(first, first)
             a = ops.fc_Q4A(dev(x), pw, N)
             c = ops.fc_Q4A(dev(x), pw, N, residual=dev(res))
             assert max_rel_err(host(a), want) <= 1e-5
             assert max_rel_err(host(c), want + res) <= 1e-5
     finally:
-        lib.llmops_fc_set_row_routing(0, 0)
+        lib.llmops_test_fc_set_row_routing(0, 0)
 
 
 @pytest.mark.parametrize("rows", [17, 48, 100, 128, 129, 200, 256])
@@ -456,13 +456,13 @@ def test_fc_prefill_every_tiling_vs_oracle(ops, orc, tiling, rows, N, K):
     pw = orc.quant_w(w, 128)
     want = orc.fc(x, pw, N)
     xe, we = oracle.closed_form_fc_inputs(rows, N, K, seed=rows)
-    lib.llmops_gemm_set_tuning(tiling)
+    lib.llmops_test_gemm_set_tuning(tiling)
     try:
         got = host(ops.fc_Q4A(dev(x), dev(pw), N))
         got_res = host(ops.fc_Q4A(dev(x), dev(pw), N, residual=dev(res)))
         ye = host(ops.fc_Q4A(dev(xe.reshape(1, rows, K)), ops.offline_FC_quant_Q4A(dev(we), 128), N))
     finally:
-        lib.llmops_gemm_set_tuning(0)
+        lib.llmops_test_gemm_set_tuning(0)
     assert max_rel_err(got, want) <= 1e-5
     assert max_rel_err(got_res, want + res) <= 1e-5
     assert np.array_equal(ye, (xe.astype(np.float64) @ we.astype(np.float64).T).astype(np.float32).reshape(1, rows, N))
@@ -518,10 +518,10 @@ def test_gemm_split_k_reduced_in_kernel_equals_second_launch(ops, M, N, K):
     x = dev(rng.standard_normal((1, M, K)).astype(np.float32))
     res = dev(rng.standard_normal((1, M, N)).astype(np.float32))
     try:
-        lib.llmops_gemm_set_reduce(0)
+        lib.llmops_test_gemm_set_reduce(0)
         want, want_res = ops.fc_Q4A(x, wq, N), ops.fc_Q4A(x, wq, N, residual=res)
         for mode in (1, 100):                                     # default rule; every split count (several load batches)
-            lib.llmops_gemm_set_reduce(mode)
+            lib.llmops_test_gemm_set_reduce(mode)
             # The planner prices the two ways of adding differently, so the tile size and split count, and with
             # them the order of the fp32 additions, may differ from the second-launch run: equal to rounding.
             # Within a mode the result must not depend on which split arrives last: bit-identical repeats.
@@ -532,7 +532,7 @@ def test_gemm_split_k_reduced_in_kernel_equals_second_launch(ops, M, N, K):
                 assert torch.equal(ops.fc_Q4A(x, wq, N), first)
                 assert torch.equal(ops.fc_Q4A(x, wq, N, residual=res), first_res)
     finally:
-        lib.llmops_gemm_set_reduce(1)
+        lib.llmops_test_gemm_set_reduce(1)
     # and the decode kernels, which share the counters, still find them at zero
     y1 = ops.fc_Q4A(x[:, :1].contiguous(), wq, N)
     assert torch.equal(y1, ops.fc_Q4A(x[:, :1].contiguous(), wq, N))
