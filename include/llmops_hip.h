@@ -102,6 +102,20 @@ int llmops_fc_Q4A(const float* x, int64_t rows, int64_t K, const int8_t* weiq, i
                   int group_k, int64_t N, float* y, void* workspace, size_t workspace_bytes,
                   llmops_stream_t stream);
 
+/* fc_Q4A for callers that cannot allocate device memory or carry a workspace around: code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the
+ * reference.  Same arguments, kernels and results as llmops_fc_Q4A, but the workspace is a fixed array of
+ * LLMOPS_FC_NOALLOC_SCRATCH_BYTES inside the library's device image (every device the library runs on
+ * holds its own copy until the process ends).  The call allocates and frees nothing.  Sizes whose
+ * workspace (llmops_fc_Q4A_workspace_bytes) exceeds the array are refused with LLMOPS_EWORKSPACE.
+ * Every call on a device shares that device's array: calls that can overlap on one device (two streams,
+ * two host threads) race and must use llmops_fc_Q4A with a workspace each instead.  The first call on a
+ * device looks the array's address up (hipGetSymbolAddress); make that call outside stream capture. */
+#define LLMOPS_FC_NOALLOC_SCRATCH_BYTES (32u << 20)
+size_t llmops_fc_Q4A_noalloc_scratch_bytes(void);
+int llmops_fc_Q4A_noalloc(const float* x, int64_t rows, int64_t K, const int8_t* weiq, int64_t Ng, int64_t Kg,
+                          int group_k, int64_t N, float* y, llmops_stream_t stream);
+
 /* fc_Q4A followed by iadd(y, residual) (ops/op_misc.hpp:55-79) in one launch for rows <= 8:
  * y = fc_Q4A(x) + residual, residual fp32 [rows,N].  The decode step uses it for the o and down
  * projections (chatllama/main.py:355-357,372-375). */

@@ -2,6 +2,8 @@
 // between the dot4 streaming kernel (few rows) and the int8 MFMA kernel (many rows).
 #include "common.h"
 
+#include <mutex>
+
 namespace llmops {
 
 constexpr int kMaxGemvRows = 8;
@@ -196,4 +198,65 @@ extern "C" int llmops_fc_Q4A_partials(const int8_t* xq, int64_t rows, const int8
 extern "C" void llmops_test_fc_set_row_routing(int rows_from_small, int rows_from_large) {
     g_rows_from_small = rows_from_small >= 2 ? rows_from_small : 4;
     g_rows_from_large = rows_from_large >= 2 ? rows_from_large : 3;
+}
+
+// ---- fc_Q4A for callers that cannot allocate ---------------------------------------------------
+// The workspace of llmops_fc_Q4A (arrival counters and exchange slots, activation codes and scales,
+// split-K partial sums) lives in a fixed array in the library's device image instead of coming from
+// the caller.  Each device holds its own copy of the array at its own address; the address is looked
+// up once per device and only that pointer is ever handed to kernels (the array's name is a host-side
+// handle, not a device address).
+namespace llmops {
+
+static __device__ __align__(256) unsigned char scratch[LLMOPS_FC_NOALLOC_SCRATCH_BYTES];
+
+constexpr int kMaxDevices = 64;
+static void* g_scratch_ptr[kMaxDevices];
+static std::mutex g_scratch_mutex;
+
+// device pointer of this device's copy of `scratch`, resolved on first use with that device current
+static int scratch_of_current_device(void** out) {
+    int dev = -1;
+    LLMOPS_HIP_CHECK(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices) return fail(LLMOPS_EINVAL, "device ordinal %d out of range", dev);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_scratch_ptr[dev] == nullptr) {
+        void* ptr = nullptr;
+        LLMOPS_HIP_CHECK(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+        if (ptr == nullptr) return fail(LLMOPS_EHIP, "hipGetSymbolAddress returned no address for the scratch array");
+        g_scratch_ptr[dev] = ptr;
+    }
+    *out = g_scratch_ptr[dev];
+    return LLMOPS_OK;
+}
+
+// zero fill with plain vector stores (a kernel rather than a memset node: callers may be capturing a graph)
+__global__ __launch_bounds__(256) void zero16_kernel(uint4* p, int64_t n16) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n16) p[i] = make_uint4(0, 0, 0, 0);
+}
+
+}  // namespace llmops
+
+extern "C" size_t llmops_fc_Q4A_noalloc_scratch_bytes(void) { return LLMOPS_FC_NOALLOC_SCRATCH_BYTES; }
+
+extern "C" int llmops_fc_Q4A_noalloc(const float* x, int64_t rows, int64_t K, const int8_t* weiq, int64_t Ng, int64_t Kg,
+                                     int group_k, int64_t N, float* y, llmops_stream_t stream) {
+    LLMOPS_REQUIRE(valid_group(group_k));
+    LLMOPS_REQUIRE(rows > 0 && K > 0 && Ng > 0 && Kg > 0);
+    const size_t need = fc_layout(rows, Ng, Kg, group_k).total;
+    if (need > (size_t)LLMOPS_FC_NOALLOC_SCRATCH_BYTES)
+        return fail(LLMOPS_EWORKSPACE,
+                    "llmops_fc_Q4A_noalloc: rows=%lld, strips=%lld, k-groups=%lld need %zu scratch bytes, the built-in "
+                    "scratch holds %zu; use llmops_fc_Q4A with a caller-provided workspace",
+                    (long long)rows, (long long)Ng, (long long)Kg, need, (size_t)LLMOPS_FC_NOALLOC_SCRATCH_BYTES);
+    void* ws = nullptr;
+    const int rc = scratch_of_current_device(&ws);
+    if (rc) return rc;
+    // The array keeps whatever the last call on this device left in it.  Counters and exchange slots must
+    // start at zero; the kernels leave them so, but a launch that failed half-way would not.
+    const int64_t n16 = LLMOPS_FC_COUNTER_BYTES / 16;
+    zero16_kernel<<<(unsigned)((n16 + 255) / 256), 256, 0, as_stream(stream)>>>(reinterpret_cast<uint4*>(ws), n16);
+    LLMOPS_LAUNCH_CHECK();
+    return fc_impl(x, rows, K, weiq, Ng, Kg, group_k, N, nullptr, y, ws, LLMOPS_FC_NOALLOC_SCRATCH_BYTES, stream);
 }

@@ -21,7 +21,7 @@ import torch
 from . import _lib
 
 __all__ = [
-    "offline_FC_quant_Q4A", "offline_FC_dequant_Q4A", "fc_Q4A", "fc_Q4A_decode", "interleave_gate_up", "FC_dynamic_quantize_x", "fc_Q4A_partials",
+    "offline_FC_quant_Q4A", "offline_FC_dequant_Q4A", "fc_Q4A", "fc_Q4A_noalloc", "fc_Q4A_decode", "interleave_gate_up", "FC_dynamic_quantize_x", "fc_Q4A_partials",
     "attention_rope", "attention_rope2", "rope_embed", "softmax", "rmsnorm", "iadd", "imul", "itrans", "clone",
     "rmsnorm_out", "silu_mul", "empty", "ones", "embedding", "embedding_q8c_quant_w", "embedding_q8c", "tensor_pool", "set_default_group_k",
     "group_k_of",
@@ -150,6 +150,21 @@ def fc_Q4A(input, weiq, N, residual=None):
         _require(tuple(residual.shape) == (B, M, int(N)), "residual.is({B, M, N})")
         _lib.check(lib.llmops_fc_Q4A_residual(_ptr(input), rows, K, _ptr(weiq), Ng, Kg, g, int(N), _ptr(residual), _ptr(out),
                                               _ptr(ws), ws.numel(), _stream(input)))
+    return out
+
+
+def fc_Q4A_noalloc(input, weiq, N, out):
+    """Extension: fc_Q4A into a caller-provided ``out`` (fp32 [B,M,N]) without allocating anything -- the
+    workspace is a fixed array inside the library (``llmops_fc_Q4A_noalloc``).  For callers that cannot
+    allocate (graph capture, serving loops); sizes beyond the array raise.  Calls that overlap on one device race."""
+    _dev(input, torch.float32, 3, "input")
+    _dev(weiq, torch.int8, 3, "wei_quantized")
+    _dev(out, torch.float32, 3, "out")
+    g = group_k_of(weiq)
+    B, M, K = input.shape
+    Ng, Kg, _ = weiq.shape
+    _require(tuple(out.shape) == (B, M, int(N)), "out.is({B, M, N})")
+    _lib.check(_lib.load().llmops_fc_Q4A_noalloc(_ptr(input), B * M, K, _ptr(weiq), Ng, Kg, g, int(N), _ptr(out), _stream(input)))
     return out
 
 

@@ -22,6 +22,8 @@ SIGNATURES = {
     "llmops_FC_dynamic_quantize_x_rows": (c_int, [c_ptr, c_i64, c_i64, c_int, c_ptr, c_ptr, c_ptr, c_ptr]),
     "llmops_fc_Q4A_workspace_bytes": (c_size, [c_i64, c_i64, c_i64, c_i64, c_int]),
     "llmops_fc_Q4A": (c_int, [c_ptr, c_i64, c_i64, c_ptr, c_i64, c_i64, c_int, c_i64, c_ptr, c_ptr, c_size, c_ptr]),
+    "llmops_fc_Q4A_noalloc_scratch_bytes": (c_size, []),
+    "llmops_fc_Q4A_noalloc": (c_int, [c_ptr, c_i64, c_i64, c_ptr, c_i64, c_i64, c_int, c_i64, c_ptr, c_ptr]),
     "llmops_fc_Q4A_residual": (c_int, [c_ptr, c_i64, c_i64, c_ptr, c_i64, c_i64, c_int, c_i64, c_ptr, c_ptr, c_ptr, c_size,
                                        c_ptr]),
     "llmops_fc_Q4A_decode": (c_int, [c_ptr, c_i64, c_i64, c_ptr, c_i64, c_i64, c_int, c_i64, c_ptr, c_f32, c_ptr, c_int, c_ptr,
