@@ -153,7 +153,8 @@ int llmops_fc_Q4A_prequantized(const int8_t* xq, const float* xd, const float* g
 /* The integer core of fc_Q4A on its own (ops/op_fc.hpp:337-363): acc int32 [rows, Ng*32, Kg].
  * `use_mfma` selects which of the production inner loops computes it (0 = dot4 streaming kernel,
  * 1 = int8 MFMA kernel, 2 = the 256-row int8 MFMA kernel with two wave groups in alternating phases,
- * group 128 only) so that each can be checked bit-for-bit. */
+ * 3 = the weight-streaming int8 MFMA kernel of 3..32 rows; 2 and 3 group 128 only) so that each can be
+ * checked bit-for-bit. */
 int llmops_fc_Q4A_partials(const int8_t* xq, int64_t rows, const int8_t* weiq, int64_t Ng, int64_t Kg,
                            int group_k, int32_t* acc, int use_mfma, llmops_stream_t stream);
 

@@ -41,6 +41,11 @@ void llmops_test_gemm_set_tuning(int row_tile_factor);
  * always with 0, a second launch adds them.  Default 1.  Same result either way; kept for comparisons and tests. */
 void llmops_test_gemm_set_reduce(int in_kernel);
 
+/* prefill GEMM: force the split-K factor (clamped to the number of k-groups); 0 = choose per shape.  Together
+ * with a forced row-tile factor it pins the tiling, so that the two ways of adding the partial sums can be
+ * compared bit for bit. */
+void llmops_test_gemm_set_split(int splits);
+
 /* weight-streaming MFMA kernel (3..16 rows, 17..32 for tensors of fewer than 256 strips): two workgroups per strip with half of K each for tensors of
  * fewer than 256 strips (default on; 0 switches it off, for comparisons and tests) */
 void llmops_test_fc_rows_set_split(int on);
@@ -49,6 +54,15 @@ void llmops_test_fc_rows_set_split(int on);
  * quantization launch) replaces the streaming kernel that quantizes on the fly, for tensors of up to
  * 256 strips and for larger ones (defaults 4 and 3; values below 2 restore them) */
 void llmops_test_fc_set_row_routing(int rows_from_small, int rows_from_large);
+
+/* The decode kernel of llmops_fc_Q4A (rows <= 8, the one that quantizes the activations on the fly) in its
+ * dump build: y as llmops_fc_Q4A computes it, plus what the kernel itself quantized -- xq int8 [rows,Kg*G],
+ * xd and gsum fp32 [rows,Kg] (FC_dynamic_quantize_x, ops/op_fc.hpp:221-272; gsum is a tree sum here) -- and
+ * its int32 dot products acc [rows,Ng*32,Kg] (ops/op_fc.hpp:337-363), so that the production loop can be
+ * compared bit for bit.  Every workgroup stores the activations it quantized (they must all agree). */
+int llmops_test_fc_decode_dump(const float* x, int64_t rows, int64_t K, const int8_t* weiq, int64_t Ng, int64_t Kg,
+                               int group_k, int64_t N, float* y, int8_t* xq, float* xd, float* gsum, int32_t* acc,
+                               void* workspace, size_t workspace_bytes, llmops_stream_t stream);
 
 #ifdef __cplusplus
 }

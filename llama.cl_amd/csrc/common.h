@@ -22,6 +22,14 @@ constexpr int kTicketBytes = 65536;
 
 __host__ __device__ constexpr int64_t block_bytes(int G) { return (int64_t)(G / 8) * kRowBytes + 64 + 64; }
 
+// where the dump build of the decode FC kernel stores what it quantized and its int32 sums
+struct DumpBufs {
+    int8_t* xq;    // [rows][Kg*G]
+    float* xd;     // [rows][Kg]
+    float* gs;     // [rows][Kg]
+    int32_t* acc;  // [rows][Ng*32][Kg]
+};
+
 // ---- error reporting ------------------------------------------------------------------------
 std::string& last_error();
 int fail(int code, const char* fmt, ...);

@@ -15,7 +15,7 @@ int launch_gemv(const uint8_t* w, const int8_t* xq, const float* xd, const float
                 unsigned* counters, int64_t rows, int64_t Ng, int64_t Kg, int G, int64_t N, hipStream_t st);
 int launch_gemv_fused(const uint8_t* w, const float* x, float* y, float* part, unsigned* counters, int64_t rows, int64_t Ng,
                       int64_t Kg, int G, int64_t N, const float* residual, const float* norm_w, float eps, int glu,
-                      const float* sumsq_in, int sumsq_parts, float* sumsq_out, hipStream_t st);
+                      const float* sumsq_in, int sumsq_parts, float* sumsq_out, hipStream_t st, const DumpBufs* dump = nullptr);
 int launch_add(float* a, const float* b, int64_t total, hipStream_t st);
 int launch_gemv_partials(const uint8_t* w, const int8_t* xq, int32_t* acc, int64_t rows, int64_t Ng, int64_t Kg, int G,
                          hipStream_t st);
@@ -27,6 +27,8 @@ int launch_gemm_partials(const uint8_t* w, const int8_t* xq, int32_t* acc, int64
                          bool two_groups, hipStream_t st);
 int launch_fc_rows(const uint8_t* w, const int8_t* xq, const float2* xsT, float* y, int64_t rows, int64_t Ng, int64_t Kg,
                    int64_t N, const float* residual, unsigned long long* slots, size_t slot_bytes, hipStream_t st);
+int launch_fc_rows_partials(const uint8_t* w, const int8_t* xq, int32_t* acc, int64_t rows, int64_t Ng, int64_t Kg,
+                            hipStream_t st);
 bool gemm_rows_kernel_enabled();
 
 static inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
@@ -190,7 +192,11 @@ extern "C" int llmops_fc_Q4A_partials(const int8_t* xq, int64_t rows, const int8
     LLMOPS_REQUIRE(aligned(weiq, 16) && aligned(xq, 16));
     LLMOPS_REQUIRE(Ng * Kg < ((int64_t)1 << 31));
     const uint8_t* w = reinterpret_cast<const uint8_t*>(weiq);
-    LLMOPS_REQUIRE(use_mfma >= 0 && use_mfma <= 2 && (use_mfma != 2 || group_k == 128));
+    LLMOPS_REQUIRE(use_mfma >= 0 && use_mfma <= 3 && (use_mfma < 2 || group_k == 128));
+    if (use_mfma == 3) {
+        LLMOPS_REQUIRE(rows <= 32);
+        return launch_fc_rows_partials(w, xq, acc, rows, Ng, Kg, as_stream(stream));
+    }
     if (use_mfma) return launch_gemm_partials(w, xq, acc, rows, Ng, Kg, group_k, use_mfma == 2, as_stream(stream));
     return launch_gemv_partials(w, xq, acc, rows, Ng, Kg, group_k, as_stream(stream));
 }
@@ -259,4 +265,26 @@ extern "C" int llmops_fc_Q4A_noalloc(const float* x, int64_t rows, int64_t K, co
     zero16_kernel<<<(unsigned)((n16 + 255) / 256), 256, 0, as_stream(stream)>>>(reinterpret_cast<uint4*>(ws), n16);
     LLMOPS_LAUNCH_CHECK();
     return fc_impl(x, rows, K, weiq, Ng, Kg, group_k, N, nullptr, y, ws, LLMOPS_FC_NOALLOC_SCRATCH_BYTES, stream);
+}
+
+// The production decode kernel in its dump build: y as llmops_fc_Q4A computes it for rows <= 8 with the kernel
+// that quantizes on the fly, plus what that kernel quantized and its int32 sums.
+extern "C" int llmops_test_fc_decode_dump(const float* x, int64_t rows, int64_t K, const int8_t* weiq, int64_t Ng, int64_t Kg,
+                                          int group_k, int64_t N, float* y, int8_t* xq, float* xd, float* gsum, int32_t* acc,
+                                          void* workspace, size_t workspace_bytes, llmops_stream_t stream) {
+    LLMOPS_REQUIRE(valid_group(group_k));
+    LLMOPS_REQUIRE(x != nullptr && weiq != nullptr && y != nullptr && workspace != nullptr);
+    LLMOPS_REQUIRE(xq != nullptr && xd != nullptr && gsum != nullptr && acc != nullptr);
+    LLMOPS_REQUIRE(rows > 0 && rows <= kMaxGemvRows && K > 0 && Ng > 0 && Kg > 0 && K == Kg * group_k);
+    LLMOPS_REQUIRE(N > (Ng - 1) * kGroupN && N <= Ng * kGroupN);
+    LLMOPS_REQUIRE(Ng <= kTicketBytes / 4 && Ng * Kg * kGroupN * rows < ((int64_t)1 << 31));
+    LLMOPS_REQUIRE(aligned(weiq, 16) && aligned(workspace, 256) && aligned(x, 8) && aligned(xq, 4));
+    const FcWorkspace lay = fc_layout(rows, Ng, Kg, group_k);
+    if (workspace_bytes < lay.total)
+        return fail(LLMOPS_EWORKSPACE, "fc_Q4A needs %zu workspace bytes, got %zu", lay.total, workspace_bytes);
+    uint8_t* ws = reinterpret_cast<uint8_t*>(workspace);
+    const DumpBufs dump{xq, xd, gsum, acc};
+    return launch_gemv_fused(reinterpret_cast<const uint8_t*>(weiq), x, y, reinterpret_cast<float*>(ws + lay.off_part),
+                             reinterpret_cast<unsigned*>(ws), rows, Ng, Kg, group_k, N, nullptr, nullptr, 0.0f, 0, nullptr, 0,
+                             nullptr, as_stream(stream), &dump);
 }

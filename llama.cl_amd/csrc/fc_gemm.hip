@@ -976,6 +976,7 @@ struct GemmPlan {
 static int g_gemm_pp_min_rows = 256;
 static int g_gemm_rt = 0;  // 0 = choose per shape; -1 = also keep 9..32 rows on the tiled kernel
 static int g_gemm_fused_reduce = 1;  // split-K partial sums added by the product kernel itself (0: by a second launch)
+static int g_gemm_force_split = 0;   // > 0: the split-K factor to use whatever the estimate says (tests)
 bool gemm_rows_kernel_enabled() { return g_gemm_rt >= 0; }
 
 // Split-K factor for `tiles` output tiles on a machine with `slots` resident workgroups.
@@ -1023,6 +1024,7 @@ static GemmPlan plan_gemm(int64_t rows, int64_t Ng, int64_t Kg, int G) {
             GemmPlan q = p;
             q.RT = kRT[i];
             int64_t S = s_try < 1 ? 1 : (s_try > Kg ? Kg : s_try);
+            if (g_gemm_force_split > 0) S = g_gemm_force_split > Kg ? Kg : g_gemm_force_split;
             q.kb_per_split = (int)((Kg + S - 1) / S);
             q.S = (int)((Kg + q.kb_per_split - 1) / q.kb_per_split);
             const int64_t rounds = (tiles * q.S + slots - 1) / slots;
@@ -1183,4 +1185,5 @@ int launch_gemm_partials(const uint8_t* w, const int8_t* xq, int32_t* acc, int64
 }  // namespace llmops
 
 extern "C" void llmops_test_gemm_set_tuning(int rows_per_wave_tile) { llmops::g_gemm_rt = rows_per_wave_tile; }
+extern "C" void llmops_test_gemm_set_split(int splits) { llmops::g_gemm_force_split = splits < 0 ? 0 : splits; }
 extern "C" void llmops_test_gemm_set_reduce(int in_kernel) { llmops::g_gemm_fused_reduce = in_kernel < 0 ? 0 : in_kernel; }

@@ -206,7 +206,13 @@ __global__ __launch_bounds__(NW * 64) void fc_gemv_kernel(const uint8_t* __restr
 //          FC's input is silu(gate)*up, formed as the two halves are loaded.  The FC that produces
 //          the row then keeps one strip per workgroup (no pairing of gate and up strips), which
 //          spreads its strips more evenly over the compute units.
-constexpr int kNorm = 1, kGlu = 2, kSums = 4, kGluIn = 8;
+//   kDump: test build of the loop: besides the outputs it stores what it quantized (codes, scales, raw
+//          group sums of every pass) and the int32 dot product of every (row, column, k-group), so that the
+//          kernel's own quantizer and integer core can be compared bit for bit with the reference's
+//          (llmops_test_fc_decode_dump).  Every workgroup stores the activations it quantized: all of them
+//          must agree.
+constexpr int kNorm = 1, kGlu = 2, kSums = 4, kGluIn = 8, kDump = 16;
+
 
 // One activation row needs few registers; asking for eight waves per SIMD (two workgroups of 16 waves
 // per CU) keeps every variant at or below 64 registers, so that grids of 257..512 workgroups are
@@ -224,9 +230,9 @@ __global__ __launch_bounds__(NW * 64, (MT == 1 ? NW / 2 : 1)) void fc_gemv_fused
                                                                  int steps_per_split, const float* __restrict__ residual,
                                                                  const float* __restrict__ norm_w, float eps,
                                                                  const float* __restrict__ sumsq_in, int sumsq_parts,
-                                                                 float* __restrict__ sumsq_out, int exchange) {
+                                                                 float* __restrict__ sumsq_out, int exchange, const DumpBufs dump) {
     constexpr bool NORM = (MODE & kNorm) != 0, GLU = (MODE & kGlu) != 0, SUMS = (MODE & kSums) != 0;
-    constexpr bool GLUIN = (MODE & kGluIn) != 0;
+    constexpr bool GLUIN = (MODE & kGluIn) != 0, DUMP = (MODE & kDump) != 0;
     static_assert(!(GLUIN && NORM), "the gate|up input has no rmsnorm");
     const int64_t xstride = GLUIN ? 2 * K : K;  // floats between activation rows
     constexpr int NWS = GLU ? NW / 2 : NW;  // waves per strip
@@ -397,9 +403,21 @@ __global__ __launch_bounds__(NW * 64, (MT == 1 ? NW / 2 : 1)) void fc_gemv_fused
         dot_step<G>(ST, slot->codes + (J) * Step<G>::kK, lane, acc);                                  \
         const float2 sc = slot->scale[(G == 128) ? (J) : (J) * 2 + (rs >> 2)];                        \
         fold(f[r], acc, ST.dh, ST.mh, sc.x, first_row ? sc.y : 0.0f);                                 \
+        if constexpr (DUMP) { /* the block's sums over its k8-rows (lane bits 3.. of the block) */    \
+            const int kb_ = (G == 128) ? tp_ + (J) : (tp_ + (J)) * 2 + (rs >> 2);                     \
+            _Pragma("unroll") for (int j = 0; j < 4; j++) {                                           \
+                int v_ = acc[j];                                                                      \
+                v_ += __shfl_xor(v_, 8, 64);                                                          \
+                v_ += __shfl_xor(v_, 16, 64);                                                         \
+                if (G == 128) v_ += __shfl_xor(v_, 32, 64);                                           \
+                if (first_row && kb_ < Kg)                                                            \
+                    dump.acc[((int64_t)r * ((int64_t)gridDim.x / S * kGroupN) + tr.nb * kGroupN + (lane & 7) * 4 + j) * Kg + kb_] = v_; \
+            }                                                                                         \
+        }                                                                                             \
     }
 #define LLMOPS_PAIR(P, TP)                                                                            \
     do {                                                                                              \
+        const int tp_ = (TP);                                                                         \
         _Pragma("unroll") for (int r = 0; r < MT; r++) if (r < rows) {                                \
             float4 v = P.xv[r];                                                                       \
             if (NORM) {                                                                               \
@@ -419,6 +437,21 @@ __global__ __launch_bounds__(NW * 64, (MT == 1 ? NW / 2 : 1)) void fc_gemv_fused
             else quantize_pass32(v, &xs[wave][r], lane);                                              \
         }                                                                                             \
         __builtin_amdgcn_wave_barrier(); /* LDS writes stay ahead of the reads below */               \
+        if constexpr (DUMP) {                                                                         \
+            _Pragma("unroll") for (int r = 0; r < MT; r++) if (r < rows) {                            \
+                const Slot* slot = &xs[wave][r];                                                      \
+                const int64_t k_ = (int64_t)tp_ * Step<G>::kK + lane * 4;                             \
+                if (tp_ + lane_step < tr.t1 && k_ < K)                                                \
+                    *reinterpret_cast<uint32_t*>(dump.xq + (int64_t)r * Kg * G + k_) =                \
+                        *reinterpret_cast<const uint32_t*>(&slot->codes[lane * 4]);                   \
+                constexpr int kBlocksPerPass = 256 / G;                                               \
+                const int kb_ = tp_ * Step<G>::kBlocksPerStep + lane;                                 \
+                if (lane < kBlocksPerPass && tp_ + lane / Step<G>::kBlocksPerStep < tr.t1 && kb_ < Kg) { \
+                    dump.xd[(int64_t)r * Kg + kb_] = slot->scale[lane].x;                             \
+                    dump.gs[(int64_t)r * Kg + kb_] = slot->scale[lane].y;                             \
+                }                                                                                     \
+            }                                                                                         \
+        }                                                                                             \
         LLMOPS_BLOCK(P.s[0], 0)                                                                       \
         _Pragma("unroll") for (int i_ = 1; i_ < SPP; i_++) {                                          \
             if ((TP) + i_ < tr.t1) {                                                                  \
@@ -566,7 +599,8 @@ struct FusedOps {
 
 template <int G, int MT, int NW>
 static void launch_fused_t(const uint8_t* w, const float* x, float* y, float* part, unsigned* counters, int64_t Ng,
-                           int64_t Kg, int64_t N, int rows, GemvPlan p, const FusedOps& o, hipStream_t st) {
+                           int64_t Kg, int64_t N, int rows, GemvPlan p, const FusedOps& o, hipStream_t st,
+                           const DumpBufs* dump = nullptr) {
     const int64_t K = Kg * G;
     // Two k-splits and no sums of squares wanted: the splits meet through one 64-bit exchange per output, in
     // slots behind the arrival counters in the zeroed head of the workspace (if they fit there).
@@ -577,10 +611,12 @@ static void launch_fused_t(const uint8_t* w, const float* x, float* y, float* pa
 #define LLMOPS_FUSED(MODE, GRID)                                                                                      \
     fc_gemv_fused_kernel<G, MT, NW, MODE><<<(unsigned)(GRID), NW * 64, 0, st>>>(                                      \
         w, x, y, part, counters, (int)Kg, K, N, rows, p.S, p.steps_per_split, o.residual, o.norm_w, o.eps, o.sumsq_in, \
-        o.sumsq_parts, o.sumsq_out, exchange)
+        o.sumsq_parts, o.sumsq_out, exchange, dump ? *dump : DumpBufs{nullptr, nullptr, nullptr, nullptr})
     // (the kernel reads up to 256 handed-over partial sums per row; with more, the statistic is recomputed)
     const bool sums = o.norm_w != nullptr && o.sumsq_in != nullptr && o.sumsq_parts <= 256;
-    if (o.glu_in) {
+    if (dump != nullptr) {  // plain fc_Q4A only (the launcher refuses the fused options)
+        LLMOPS_FUSED(kDump, Ng * p.S);
+    } else if (o.glu_in) {
         LLMOPS_FUSED(kGluIn, Ng * p.S);
     } else if (o.glu) {
         if (sums) LLMOPS_FUSED(kNorm | kGlu | kSums, Ng / 2);
@@ -597,11 +633,12 @@ static void launch_fused_t(const uint8_t* w, const float* x, float* y, float* pa
 // raw fp32 activations, quantized inside the kernel (+ optional rmsnorm / residual / gate-up epilogue)
 int launch_gemv_fused(const uint8_t* w, const float* x, float* y, float* part, unsigned* counters, int64_t rows, int64_t Ng,
                       int64_t Kg, int G, int64_t N, const float* residual, const float* norm_w, float eps, int glu,
-                      const float* sumsq_in, int sumsq_parts, float* sumsq_out, hipStream_t st) {
+                      const float* sumsq_in, int sumsq_parts, float* sumsq_out, hipStream_t st, const DumpBufs* dump) {
     GemvPlan p = plan_gemv(rows, Ng, Kg, G, true);
     if (glu == 1) p.S = 1;
+    if (dump != nullptr && (norm_w != nullptr || glu != 0)) return fail(LLMOPS_EINVAL, "the dump build runs the plain FC only");
     const FusedOps o{residual, norm_w, eps, glu == 1, glu == 2, sumsq_in, sumsq_parts, sumsq_out};
-#define LLMOPS_CASE(GG, MT, NWW) launch_fused_t<GG, MT, NWW>(w, x, y, part, counters, Ng, Kg, N, (int)rows, p, o, st)
+#define LLMOPS_CASE(GG, MT, NWW) launch_fused_t<GG, MT, NWW>(w, x, y, part, counters, Ng, Kg, N, (int)rows, p, o, st, dump)
     if (G == 128) {
         if (rows == 1) LLMOPS_CASE(128, 1, 16);
         else if (rows == 2) LLMOPS_CASE(128, 2, 16);

@@ -84,14 +84,17 @@ __device__ __forceinline__ void rows_load(RowsStage<RT>& st, const RowsBufs& bf,
     }
 }
 
-template <int RT, int NW>
+// DUMP: test build that stores the int32 sums of every (row, column, k-group) into `dump`
+// ([rows][Ng*32][Kg]) instead of the outputs (llmops_fc_Q4A_partials with use_mfma = 3).
+template <int RT, int NW, bool DUMP = false>
 __global__ __launch_bounds__(NW * 64, RT == 2 ? 3 : 4) void fc_rows_mfma_kernel(const uint8_t* __restrict__ weiq,
                                                                          const int8_t* __restrict__ xq,
                                                                          const float2* __restrict__ xsT,
                                                                          float* __restrict__ y, int Kg, int64_t N, int rows,
                                                                          const float* __restrict__ residual,
-                                                                         unsigned long long* slots) {
-    __shared__ float red[NW][16 * RT][kGroupN];
+                                                                         unsigned long long* slots,
+                                                                         int32_t* dump = nullptr) {
+    __shared__ float red[DUMP ? 1 : NW][16 * RT][kGroupN];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // uniform: block offsets stay scalar
     const int g = lane >> 4, jj = lane & 15;
@@ -112,7 +115,7 @@ __global__ __launch_bounds__(NW * 64, RT == 2 ? 3 : 4) void fc_rows_mfma_kernel(
     RowsBufs bf;
     bf.w_base = strip, bf.w_bytes = (uint32_t)Kg * (uint32_t)kRowsBlk;
     bf.xq_base = xq, bf.xq_bytes = (uint32_t)rows * (uint32_t)Kp;
-    bf.xs_base = xsT, bf.xs_bytes = (uint32_t)Kg * (uint32_t)rows * 8u;
+    bf.xs_base = xsT, bf.xs_bytes = DUMP ? 0u : (uint32_t)Kg * (uint32_t)rows * 8u;
     bf.lane_w = (uint32_t)(2 * g * kRowBytes + jj * 4);
     bf.lane_s = (uint32_t)((jj >> 1) * 4);  // the dword with this column's fp16 scale; half_sh picks the half
     const int half_sh = (jj & 1) * 16;
@@ -124,7 +127,7 @@ __global__ __launch_bounds__(NW * 64, RT == 2 ? 3 : 4) void fc_rows_mfma_kernel(
 
     // Two stages used alternately (no register copies: a copy would have to wait for the loads it copies):
     // the k-group being multiplied waits for exactly its own loads while the next one's are in flight.
-#define LLMOPS_ROWS_COMPUTE(ST)                                                                              \
+#define LLMOPS_ROWS_COMPUTE(ST, KB)                                                                          \
     do {                                                                                                     \
         v4i_r b[2][2];                                                                                       \
         _Pragma("unroll") for (int h = 0; h < 2; h++) _Pragma("unroll") for (int tau = 0; tau < 2; tau++) {  \
@@ -139,6 +142,14 @@ __global__ __launch_bounds__(NW * 64, RT == 2 ? 3 : 4) void fc_rows_mfma_kernel(
                 v4i_r acc = v4i_r{0, 0, 0, 0};                                                               \
                 acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(ST.a[t][0], b[0][tau], acc, 0, 0, 0);            \
                 acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(ST.a[t][1], b[1][tau], acc, 0, 0, 0);            \
+                if constexpr (DUMP) {                                                                        \
+                    const int64_t Np_ = (int64_t)(slots ? gridDim.x / 2 : gridDim.x) * kGroupN;              \
+                    _Pragma("unroll") for (int v = 0; v < 4; v++) {                                          \
+                        const int row_ = 16 * t + 4 * g + v;                                                 \
+                        if (row_ < rows && (KB) < t1)                                                        \
+                            dump[((int64_t)row_ * Np_ + nb * kGroupN + 16 * tau + jj) * Kg + (KB)] = acc[v]; \
+                    }                                                                                        \
+                }                                                                                            \
                 _Pragma("unroll") for (int v = 0; v < 4; v++) {                                              \
                     f[t][tau][v] = fmaf(d * ST.xs[t][v].x, (float)acc[v], f[t][tau][v]);                     \
                     f[t][tau][v] = fmaf(m, ST.xs[t][v].y, f[t][tau][v]);                                     \
@@ -154,24 +165,25 @@ __global__ __launch_bounds__(NW * 64, RT == 2 ? 3 : 4) void fc_rows_mfma_kernel(
         rows_load<RT>(sa, bf, kb, rows, true);
         rows_load<RT>(sb, bf, kb + 1, rows, kb + 1 < t1);
         __builtin_amdgcn_sched_barrier(0);
-        LLMOPS_ROWS_COMPUTE(sa);
+        LLMOPS_ROWS_COMPUTE(sa, kb);
         __builtin_amdgcn_sched_barrier(0);
         rows_load<RT>(sa, bf, kb + 2, rows, kb + 2 < t1);
         __builtin_amdgcn_sched_barrier(0);
-        LLMOPS_ROWS_COMPUTE(sb);  // (a stage that was not wanted holds zeros and adds nothing)
+        LLMOPS_ROWS_COMPUTE(sb, kb + 1);  // (a stage that was not wanted holds zeros and adds nothing)
         __builtin_amdgcn_sched_barrier(0);
         rows_load<RT>(sb, bf, kb + 3, rows, kb + 3 < t1);
         __builtin_amdgcn_sched_barrier(0);
         // (the loads above are issued whatever the run's length; only the arithmetic on zeros is skipped)
         if (kb + 2 < t1) {
-            LLMOPS_ROWS_COMPUTE(sa);
+            LLMOPS_ROWS_COMPUTE(sa, kb + 2);
         }
         __builtin_amdgcn_sched_barrier(0);
         if (kb + 3 < t1) {
-            LLMOPS_ROWS_COMPUTE(sb);
+            LLMOPS_ROWS_COMPUTE(sb, kb + 3);
         }
     }
 #undef LLMOPS_ROWS_COMPUTE
+    if constexpr (DUMP) return;
 
     // the waves' sums meet in LDS; one thread finishes each output
 #pragma unroll
@@ -226,6 +238,25 @@ int launch_fc_rows(const uint8_t* w, const int8_t* xq, const float2* xsT, float*
         fc_rows_mfma_kernel<1, 16><<<grid, 1024, 0, st>>>(w, xq, xsT, y, (int)Kg, N, (int)rows, residual, sl);
     else
         fc_rows_mfma_kernel<1, 8><<<grid, 512, 0, st>>>(w, xq, xsT, y, (int)Kg, N, (int)rows, residual, sl);
+    LLMOPS_LAUNCH_CHECK();
+    return LLMOPS_OK;
+}
+
+// The same loop in its dump build, launched with the workgroup shape and K split that launch_fc_rows picks for
+// these sizes.  The (scale, sum) pairs are not needed for the integer sums: their descriptor has size 0.
+int launch_fc_rows_partials(const uint8_t* w, const int8_t* xq, int32_t* acc, int64_t rows, int64_t Ng, int64_t Kg,
+                            hipStream_t st) {
+    const bool split = g_rows_split && Ng < 256 && Kg >= 16;
+    const unsigned grid = (unsigned)(split ? 2 * Ng : Ng);
+    // only tested against nullptr in the dump build, never dereferenced
+    unsigned long long* sl = split ? reinterpret_cast<unsigned long long*>(acc) : nullptr;
+    const int64_t k_per_wg = split ? (Kg + 1) / 2 : Kg;
+    if (rows > 16)
+        fc_rows_mfma_kernel<2, 8, true><<<grid, 512, 0, st>>>(w, xq, nullptr, nullptr, (int)Kg, 0, (int)rows, nullptr, sl, acc);
+    else if (k_per_wg > 32)
+        fc_rows_mfma_kernel<1, 16, true><<<grid, 1024, 0, st>>>(w, xq, nullptr, nullptr, (int)Kg, 0, (int)rows, nullptr, sl, acc);
+    else
+        fc_rows_mfma_kernel<1, 8, true><<<grid, 512, 0, st>>>(w, xq, nullptr, nullptr, (int)Kg, 0, (int)rows, nullptr, sl, acc);
     LLMOPS_LAUNCH_CHECK();
     return LLMOPS_OK;
 }

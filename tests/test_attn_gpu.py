@@ -301,3 +301,37 @@ def test_mm_qk_rejects_what_the_reference_asserts(ops):
         ops.mm_qk(torch.zeros(1, 4, 32, device="cuda"), torch.zeros(2, 2, 5, 16, device="cuda"))
     with pytest.raises(RuntimeError):
         ops.mm_qk(torch.zeros(1, 4, 32), torch.zeros(1, 2, 5, 16))  # host tensors: there is no CPU path
+
+
+def _prefill_case(ops, orc, rng, past, qL, maxlen, half, heads, H=32, S=128):
+    """attention over H heads on the device; the oracle on the sampled `heads` (heads are independent)"""
+    B = 1
+    inv_freq = (1.0 / (10000.0 ** (np.arange(0, 2 * half, 2, dtype=np.float32) / np.float32(2 * half)))).astype(np.float32)
+    cache = rng.standard_normal((2, B, H, maxlen, S)).astype(np.float32)
+    q, k, v = (rng.standard_normal((B, qL, H * S)).astype(np.float32) for _ in range(3))
+    slots = ((past + np.arange(qL)) % maxlen).astype(np.int32)
+    g = dict(q=q, k=k, v=v, cache=cache, inv_freq=inv_freq, slots=slots, position_id=past, layer_id=0)
+    out, k_rot, cache_after = run_attention(ops, g)
+    pick = lambda t: np.ascontiguousarray(t.reshape(B, qL, H, S)[:, :, heads].reshape(B, qL, len(heads) * S))
+    want, k_ref, cache_ref = orc.attention(pick(q), pick(k), pick(v), inv_freq, np.ascontiguousarray(cache[:, :, heads]),
+                                           slots, past, 0)
+    assert max_rel_err(pick(out), want) <= 1e-4, (past, qL, half)
+    assert np.abs(pick(k_rot) - k_ref).max() <= 1e-5
+    assert np.abs(cache_after[:, :, heads] - cache_ref).max() <= 1e-5
+    assert np.isfinite(out).all()
+
+
+@pytest.mark.parametrize("past,qL,half", [(0, 1022, 32), (0, 1023, 32), (0, 1024, 32), (0, 1025, 32), (0, 1026, 32),
+                                          (0, 1024, 64), (0, 2048, 32), (0, 2048, 64), (0, 128, 64), (0, 512, 64)])
+def test_attention_prefill_at_the_reference_sweep_sizes(ops, orc, past, qL, half):
+    """The accuracy sweep of the reference's perf script (ops/perf_ops.py:83-100,284-292: 32 heads, head size 128,
+    rotary_dims 64, first chunk of 1022..1026 tokens) and the chunk lengths the benchmark publishes (128, 512,
+    2048 tokens, full rotary), against the oracle on sampled heads."""
+    rng = np.random.default_rng(qL + half)
+    _prefill_case(ops, orc, rng, past, qL, 2048, half, heads=[0, 13, 31])
+
+
+def test_attention_prefill_long_chunk_wrapping_the_ring(ops, orc):
+    """a 1024-token chunk whose slots wrap around a cache of 2048 rows that is already full"""
+    rng = np.random.default_rng(77)
+    _prefill_case(ops, orc, rng, 1500, 1024, 2048, 32, heads=[5, 30])
