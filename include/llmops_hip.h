@@ -186,6 +186,16 @@ int llmops_attention_rope(float* q, float* k, const float* v, int64_t B, int64_t
                           int64_t planes, int64_t maxlen, const int32_t* slots, int position_id,
                           int layer_id, void* workspace, size_t workspace_bytes, llmops_stream_t stream);
 
+/* attention_rope2 (ops/op_attn.hpp:721-1029) for one query token per sequence (qL = 1) with the token's position
+ * in device memory: `slot` and `position_id` are int32 [1] on the device and are read by the kernels, so a HIP
+ * graph that captured the call can be replayed for every following token after the two values have been
+ * updated (the reference passes position_id by value, chatllama/main.py:353).  kvLen = min(position_id + 1,
+ * maxlen).  The launch is sized for a full cache.  Needs half % 4 == 0.  Otherwise as llmops_attention_rope. */
+int llmops_attention_rope_decode(float* q, float* k, const float* v, int64_t B, int64_t H, int64_t S,
+                                 const float* inv_freq, int64_t half, void* kv_cache, int cache_dtype, int64_t planes,
+                                 int64_t maxlen, const int32_t* slot, const int32_t* position_id, int layer_id,
+                                 void* workspace, size_t workspace_bytes, llmops_stream_t stream);
+
 /* softmax (ops/op_misc.hpp:183-194, ops/utils.hpp:484-490): in place over rows of length K */
 int llmops_softmax(float* x, int64_t rows, int64_t K, llmops_stream_t stream);
 

@@ -55,6 +55,10 @@ void llmops_test_fc_rows_set_split(int on);
  * 256 strips and for larger ones (defaults 4 and 3; values below 2 restore them) */
 void llmops_test_fc_set_row_routing(int rows_from_small, int rows_from_large);
 
+/* decode attention (one query token): force the cache rows per wavefront (fp32 cache 4, 8, 16; fp16 cache 8, 16,
+ * 32; a chunk is 4 times that); 0 = choose */
+void llmops_test_attn_set_decode_plan(int rows_per_wave);
+
 /* The decode kernel of llmops_fc_Q4A (rows <= 8, the one that quantizes the activations on the fly) in its
  * dump build: y as llmops_fc_Q4A computes it, plus what the kernel itself quantized -- xq int8 [rows,Kg*G],
  * xd and gsum fp32 [rows,Kg] (FC_dynamic_quantize_x, ops/op_fc.hpp:221-272; gsum is a tree sum here) -- and

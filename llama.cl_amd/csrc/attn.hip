@@ -233,13 +233,17 @@ __device__ __forceinline__ float merge_chunks(const float* rec, int nchunks, int
     return num * (1.0f / den);
 }
 
+// `nchunks` records per query are laid out; with pos_dev (decode graphs) only the first
+// ceil(min(pos_dev[0] + 1, maxlen) / chunk_rows) of them were written by this call.
 __global__ __launch_bounds__(128) void attn_merge_kernel(float* __restrict__ q, const float* __restrict__ part, int64_t qL,
-                                                          int64_t H, int nchunks) {
+                                                          int64_t H, int nchunks, const int32_t* __restrict__ pos_dev = nullptr,
+                                                          int64_t maxlen = 0, int chunk_rows = 1) {
     constexpr int S = 128;
     __shared__ float wsh[2][64];
     const int64_t bhq = blockIdx.x;
     const int64_t pq = bhq % qL, h = (bhq / qL) % H, b = bhq / (qL * H);
     const float* rec = part + (int64_t)bhq * nchunks * (S + 2);
+    if (pos_dev != nullptr) nchunks = (int)((min((int64_t)pos_dev[0] + 1, maxlen) + chunk_rows - 1) / chunk_rows);
     float r;
     if (nchunks <= 64) {
         // The chunk weights exp(m_c - M) / sum are the same for all 128 output elements: each wave computes
@@ -279,15 +283,24 @@ __global__ __launch_bounds__(128) void attn_merge_kernel(float* __restrict__ q, 
 }
 
 // ---- decode attention (one query token) ------------------------------------------------------
-// attention_rope2 for qL == 1 in two launches instead of three: every workgroup rotates q itself
-// (cos/sin of the position computed once per workgroup, one angle per lane), the workgroup whose
-// chunk holds the new token's cache row rotates k, writes the rotated k back in place and k, v
-// into the cache, and attends to the new row from registers; attn_merge_kernel then combines the
-// chunk records into q.  (Merging inside this kernel through an arrival ticket was measured
-// slower, also with all of the last workgroup's record loads in flight at once: kv 2048 21.5 against
-// 18.4 us, kv 4096 39.9 against 30.9 us.  Every workgroup then waits for the acknowledgement of its
-// device-scope stores and for its ticket, 3-4 us during which it holds its place on the CU, and the
-// workgroups of the next round start that much later; a launch costs less.)
+// attention_rope2 for qL == 1: every workgroup rotates q itself (cos/sin of the position computed once
+// per workgroup, one angle per lane), the workgroup whose chunk holds the new token's cache row rotates
+// k, writes the rotated k back in place and k, v into the cache, and attends to the new row from
+// registers.  The chunk records (max, sum, weighted V sum) are merged by attn_merge_kernel, a second
+// launch.  (Merging inside this kernel, by whichever workgroup of a head takes the last arrival ticket, was
+// measured slower at every size: the record stores must be acknowledged before the ticket is taken and the
+// last workgroup then fetches the records, three round trips to memory against one launch -- kv 256: 9.2
+// against 8.2 us, kv 2048: 25.4 against 19.0 us.  One workgroup of 16 wavefronts per head, which needs no
+// merge, is bound by what one compute unit can fetch: kv 256 9.1 against 8.2 us, kv 512 with an fp16 cache 20.4
+// against 9.4 us.)  A head with a single chunk (nchunks == 1) is finished here and written straight into q.
+//
+// A lane always fetches 16 bytes of a cache row: 4 floats or 8 halves.  A 128-element row is therefore
+// LPR = 32 (fp32) or 16 (fp16) lanes wide and one wave-wide load covers RPW = 2 or 4 rows; a wave owns PW
+// rows of the chunk, NL = PW / RPW loads per lane for K and as many for V.
+//
+// The position may come from device memory (pos_dev != nullptr): a HIP graph of a decode step captures the
+// launch once, for the largest kv length (the grid and the record layout are sized by `nchunks`), and every
+// replay reads the current position; workgroups whose chunk lies beyond the current kv length leave at once.
 template <typename T>
 __device__ __forceinline__ float cache_round(float v);
 template <>
@@ -344,21 +357,63 @@ __device__ __forceinline__ int rope_partner(int e4, int half) {
     return e4 >= 2 * half ? e4 : (e4 < half ? e4 + half : e4 - half);
 }
 
+// 16 bytes of a cache row as they come from memory, and their widening to floats
+template <typename T>
+struct RowPiece;
+template <>
+struct RowPiece<float> {
+    static constexpr int EPL = 4;  // elements per lane
+    static __device__ __forceinline__ void widen(const uint4& r, float out[4]) {
+        out[0] = __uint_as_float(r.x), out[1] = __uint_as_float(r.y), out[2] = __uint_as_float(r.z), out[3] = __uint_as_float(r.w);
+    }
+    // the 16 bytes as the cache stores them
+    static __device__ __forceinline__ uint4 pack(const float4* v) {
+        return make_uint4(__float_as_uint(v[0].x), __float_as_uint(v[0].y), __float_as_uint(v[0].z), __float_as_uint(v[0].w));
+    }
+};
+template <>
+struct RowPiece<__half> {
+    static constexpr int EPL = 8;
+    static __device__ __forceinline__ float lo(uint32_t w) { return __half2float(__ushort_as_half((unsigned short)(w & 0xFFFFu))); }
+    static __device__ __forceinline__ float hi(uint32_t w) { return __half2float(__ushort_as_half((unsigned short)(w >> 16))); }
+    static __device__ __forceinline__ void widen(const uint4& r, float out[8]) {
+        out[0] = lo(r.x), out[1] = hi(r.x), out[2] = lo(r.y), out[3] = hi(r.y);
+        out[4] = lo(r.z), out[5] = hi(r.z), out[6] = lo(r.w), out[7] = hi(r.w);
+    }
+    static __device__ __forceinline__ uint32_t pack2(float a, float b) {
+        return (uint32_t)__half_as_ushort(__float2half_rn(a)) | ((uint32_t)__half_as_ushort(__float2half_rn(b)) << 16);
+    }
+    static __device__ __forceinline__ uint4 pack(const float4* v) {
+        return make_uint4(pack2(v[0].x, v[0].y), pack2(v[0].z, v[0].w), pack2(v[1].x, v[1].y), pack2(v[1].z, v[1].w));
+    }
+};
+// cache rows are read exactly once per call: non-temporal, so that they do not displace the records and the
+// activations that are reused out of the caches
+__device__ __forceinline__ uint4 load_row16(const void* p) {
+    return *reinterpret_cast<const uint4*>(p);
+}
+
 template <typename T, int PW>
 __global__ __launch_bounds__(256) void attn_decode_kernel(float* q, float* k, const float* __restrict__ v,
                                                            const float* __restrict__ inv_freq, int half, T* kc, T* vc,
-                                                           int64_t H, int64_t maxlen, int64_t kvLen,
-                                                           const int32_t* __restrict__ slots, int position_id, float* part,
+                                                           int64_t H, int64_t maxlen, const int32_t* __restrict__ slots,
+                                                           int position_id, const int32_t* __restrict__ pos_dev, float* part,
                                                            int nchunks) {
-    constexpr int S = 128, C = 4 * PW, NL = PW / 2;
+    constexpr int S = 128, NWV = 4, C = NWV * PW;  // 4 wavefronts per workgroup
+    constexpr int EPL = RowPiece<T>::EPL, LPR = S / EPL, RPW = 64 / LPR, NL = PW / RPW;
+    static_assert(NL >= 1 && NL <= LPR, "rows per lane");
     __shared__ float sc[C];
-    __shared__ float osh[4][2][S];
+    __shared__ float osh[NWV][RPW][S];
     __shared__ float stat[2];
     __shared__ float cs_sh[64], sn_sh[64];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int hf = lane >> 5, e = lane & 31;
+    const int rsel = lane / LPR, e = lane % LPR;  // which of the RPW rows of a wave-wide load, which 16 bytes of it
     const int chunk = blockIdx.x % nchunks;
     const int64_t bh = blockIdx.x / nchunks;
+    if (pos_dev != nullptr) position_id = pos_dev[0];
+    const int64_t kvLen = min((int64_t)position_id + 1, maxlen);
+    const int nact = (int)((kvLen + C - 1) / C);  // chunks that hold rows at this position
+    if (chunk >= nact) return;
     const int64_t p0 = (int64_t)chunk * C;
     T* kbase = kc + bh * maxlen * S;
     T* vbase = vc + bh * maxlen * S;
@@ -370,31 +425,40 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(float* q, float* k, co
     const int slot = slots[0];
     const bool slot_ok = slot >= 0 && slot < maxlen;
     // the workgroup that owns the new token's row (or the last chunk, if the row lies beyond kvLen)
-    const int owner = (slot_ok && slot / C < nchunks) ? slot / C : nchunks - 1;
-    const int e4 = e * 4, ep = rope_partner(e4, half);
+    const int owner = (slot_ok && slot / C < nact) ? slot / C : nact - 1;
+    const int e0 = e * EPL;  // the lane's first element of the row
     const float freq = inv_freq[min((int)threadIdx.x, half - 1)];
-    const float4 q_own = *reinterpret_cast<const float4*>(q + bh * S + e4);
-    const float4 q_oth = *reinterpret_cast<const float4*>(q + bh * S + ep);
-    float4 kn = make_float4(0.f, 0.f, 0.f, 0.f), k_oth = kn, vn = kn;
+    float4 q_own[EPL / 4], q_oth[EPL / 4];
+#pragma unroll
+    for (int u = 0; u < EPL / 4; u++) {
+        q_own[u] = *reinterpret_cast<const float4*>(q + bh * S + e0 + 4 * u);
+        q_oth[u] = *reinterpret_cast<const float4*>(q + bh * S + rope_partner(e0 + 4 * u, half));
+    }
+    float4 kn[EPL / 4], k_oth[EPL / 4], vn[EPL / 4];
+#pragma unroll
+    for (int u = 0; u < EPL / 4; u++) kn[u] = k_oth[u] = vn[u] = make_float4(0.f, 0.f, 0.f, 0.f);
     if (chunk == owner) {  // (uniform; older than the cache rows, so it does not blur the waits for them)
-        kn = *reinterpret_cast<const float4*>(k + bh * S + e4);
-        k_oth = *reinterpret_cast<const float4*>(k + bh * S + ep);
-        vn = *reinterpret_cast<const float4*>(v + bh * S + e4);
+#pragma unroll
+        for (int u = 0; u < EPL / 4; u++) {
+            kn[u] = *reinterpret_cast<const float4*>(k + bh * S + e0 + 4 * u);
+            k_oth[u] = *reinterpret_cast<const float4*>(k + bh * S + rope_partner(e0 + 4 * u, half));
+            vn[u] = *reinterpret_cast<const float4*>(v + bh * S + e0 + 4 * u);
+        }
     }
     __builtin_amdgcn_sched_barrier(0);
-    float4 kv[NL], vv[NL];
+    uint4 kraw[NL], vraw[NL];
 #pragma unroll
     for (int i = 0; i < NL; i++) {
-        const int64_t p = p0 + wave * PW + i * 2 + hf;
+        const int64_t p = p0 + wave * PW + i * RPW + rsel;
         const int64_t pc = p < kvLen ? p : kvLen - 1;
-        kv[i] = load4(kbase + pc * S + e4);
+        kraw[i] = load_row16(kbase + pc * S + e0);
     }
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int i = 0; i < NL; i++) {
-        const int64_t p = p0 + wave * PW + i * 2 + hf;
+        const int64_t p = p0 + wave * PW + i * RPW + rsel;
         const int64_t pc = p < kvLen ? p : kvLen - 1;
-        vv[i] = load4(vbase + pc * S + e4);
+        vraw[i] = load_row16(vbase + pc * S + e0);
     }
     __builtin_amdgcn_sched_barrier(0);
     if (threadIdx.x < half) {
@@ -403,41 +467,50 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(float* q, float* k, co
         sn_sh[threadIdx.x] = sinf(xita);
     }
     __syncthreads();
-    const float4 qv = rope4_regs(q_own, q_oth, e4, cs_sh, sn_sh, half);
+    float qv[EPL];
+#pragma unroll
+    for (int u = 0; u < EPL / 4; u++) {
+        const float4 r = rope4_regs(q_own[u], q_oth[u], e0 + 4 * u, cs_sh, sn_sh, half);
+        qv[4 * u] = r.x, qv[4 * u + 1] = r.y, qv[4 * u + 2] = r.z, qv[4 * u + 3] = r.w;
+    }
+    // the new token's row as the cache holds it (rounded to T): it is attended to from registers
+    uint4 knraw = make_uint4(0, 0, 0, 0), vnraw = knraw;
     if (chunk == owner) {
-        kn = rope4_regs(kn, k_oth, e4, cs_sh, sn_sh, half);
+#pragma unroll
+        for (int u = 0; u < EPL / 4; u++) kn[u] = rope4_regs(kn[u], k_oth[u], e0 + 4 * u, cs_sh, sn_sh, half);
+        knraw = RowPiece<T>::pack(kn);
+        vnraw = RowPiece<T>::pack(vn);
         __syncthreads();  // every wave has read the raw k before it is overwritten
-        if (wave == 0 && hf == 0) {
-            *reinterpret_cast<float4*>(k + bh * S + e4) = kn;
+        if (wave == 0 && rsel == 0) {
+#pragma unroll
+            for (int u = 0; u < EPL / 4; u++) *reinterpret_cast<float4*>(k + bh * S + e0 + 4 * u) = kn[u];
             if (slot_ok) {
-                store4<T>(kbase + (int64_t)slot * S + e4, kn);
-                store4<T>(vbase + (int64_t)slot * S + e4, vn);
+                *reinterpret_cast<uint4*>(kbase + (int64_t)slot * S + e0) = knraw;
+                *reinterpret_cast<uint4*>(vbase + (int64_t)slot * S + e0) = vnraw;
             }
         }
-        kn = make_float4(cache_round<T>(kn.x), cache_round<T>(kn.y), cache_round<T>(kn.z), cache_round<T>(kn.w));
-        vn = make_float4(cache_round<T>(vn.x), cache_round<T>(vn.y), cache_round<T>(vn.z), cache_round<T>(vn.w));
-    }
-    const float d_scale = 1.0f / sqrtf((float)S);
-    // NL partial dot products per lane, each to be summed over the 32 lanes of a half-wave.  Summing
-    // them one by one takes 5 lane exchanges each; instead the lanes split the rows between them while
-    // they add: at every exchange a lane keeps one half of its rows and hands the other half to its
-    // partner, so NL rows cost NL/2 + NL/4 + .. + 1 exchanges plus one per remaining lane bit.
-    float sp[NL];
-    if (chunk == owner) {  // the new token's row comes from registers (K here, V where the V rows are used)
 #pragma unroll
         for (int i = 0; i < NL; i++)
-            if (p0 + wave * PW + i * 2 + hf == slot) kv[i] = kn;
+            if (p0 + wave * PW + i * RPW + rsel == slot) kraw[i] = knraw;
     }
+    const float d_scale = 1.0f / sqrtf((float)S);
+    // NL partial dot products per lane, each to be summed over the LPR lanes of a row.  Summing them one
+    // by one takes log2(LPR) lane exchanges each; instead the lanes split the rows between them while they
+    // add: at every exchange a lane keeps one half of its rows and hands the other half to its partner,
+    // so NL rows cost NL/2 + NL/4 + .. + 1 exchanges plus one per remaining lane bit.
+    float sp[NL];
 #pragma unroll
     for (int i = 0; i < NL; i++) {
-        float s = qv.x * kv[i].x;
-        s = fmaf(qv.y, kv[i].y, s);
-        s = fmaf(qv.z, kv[i].z, s);
-        sp[i] = fmaf(qv.w, kv[i].w, s);
+        float kf[EPL];
+        RowPiece<T>::widen(kraw[i], kf);
+        float s = 0.0f;
+#pragma unroll
+        for (int c = 0; c < EPL; c++) s = fmaf(qv[c], kf[c], s);
+        sp[i] = s;
     }
     int row_of_lane = 0;  // which of the NL rows this lane ends up holding
     {
-        int n = NL, off = 16;
+        int n = NL, off = LPR / 2;
 #pragma unroll
         for (; n > 1; n >>= 1, off >>= 1) {
             const bool up = (e & off) != 0;
@@ -456,17 +529,28 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(float* q, float* k, co
     }
     {
         // lanes whose remaining (low) bits are zero write the row they hold
-        constexpr int kLowMask = (NL >= 8) ? 3 : (NL == 4 ? 7 : 15);
-        const int r = wave * PW + row_of_lane * 2 + hf;
+        constexpr int kLowMask = LPR / NL - 1;
+        const int r = wave * PW + row_of_lane * RPW + rsel;
         if ((e & kLowMask) == 0) sc[r] = (p0 + r < kvLen) ? sp[0] * d_scale : -FLT_MAX;
     }
     __syncthreads();
     if (wave == 0) {
-        const float x = lane < C ? sc[lane] : -FLT_MAX;
-        const float mx = wave_max(x);
-        const float ex = (lane < C && x != -FLT_MAX) ? expf(x - mx) : 0.0f;
-        if (lane < C) sc[lane] = ex;
-        const float sum = wave_sum(ex);
+        float mx = -FLT_MAX;
+#pragma unroll
+        for (int u = 0; u < (C + 63) / 64; u++) mx = fmaxf(mx, lane + 64 * u < C ? sc[lane + 64 * u] : -FLT_MAX);
+        mx = wave_max(mx);
+        float sum = 0.0f;
+#pragma unroll
+        for (int u = 0; u < (C + 63) / 64; u++) {
+            const int r = lane + 64 * u;
+            if (r < C) {
+                const float x = sc[r];
+                const float ex = (x != -FLT_MAX) ? expf(x - mx) : 0.0f;
+                sc[r] = ex;
+                sum += ex;
+            }
+        }
+        sum = wave_sum(sum);
         if (lane == 0) {
             stat[0] = mx;
             stat[1] = sum;
@@ -476,27 +560,37 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(float* q, float* k, co
     if (chunk == owner) {
 #pragma unroll
         for (int i = 0; i < NL; i++)
-            if (p0 + wave * PW + i * 2 + hf == slot) vv[i] = vn;
+            if (p0 + wave * PW + i * RPW + rsel == slot) vraw[i] = vnraw;
     }
-    float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
+    float o[EPL];
+#pragma unroll
+    for (int c = 0; c < EPL; c++) o[c] = 0.0f;
 #pragma unroll
     for (int i = 0; i < NL; i++) {
-        const float w = sc[wave * PW + i * 2 + hf];
-        o.x = fmaf(w, vv[i].x, o.x);
-        o.y = fmaf(w, vv[i].y, o.y);
-        o.z = fmaf(w, vv[i].z, o.z);
-        o.w = fmaf(w, vv[i].w, o.w);
+        float vf[EPL];
+        RowPiece<T>::widen(vraw[i], vf);
+        const float w = sc[wave * PW + i * RPW + rsel];
+#pragma unroll
+        for (int c = 0; c < EPL; c++) o[c] = fmaf(w, vf[c], o[c]);
     }
-    *reinterpret_cast<float4*>(&osh[wave][hf][e * 4]) = o;
+#pragma unroll
+    for (int u = 0; u < EPL / 4; u++)
+        *reinterpret_cast<float4*>(&osh[wave][rsel][e0 + 4 * u]) = make_float4(o[4 * u], o[4 * u + 1], o[4 * u + 2], o[4 * u + 3]);
     __syncthreads();
     float* rec0 = part + bh * nchunks * (S + 2);
     float* rec = rec0 + (int64_t)chunk * (S + 2);
+    float mine = 0.0f;  // this thread's element of the chunk's weighted V sum (threads 0..127)
     if (threadIdx.x < S) {
-        float a = 0.0f;
 #pragma unroll
-        for (int w = 0; w < 4; w++) a += osh[w][0][threadIdx.x] + osh[w][1][threadIdx.x];
-        rec[2 + threadIdx.x] = a;
+        for (int w = 0; w < NWV; w++)
+#pragma unroll
+            for (int r = 0; r < RPW; r++) mine += osh[w][r][threadIdx.x];
     }
+    if (nchunks == 1) {  // the workgroup saw every row of the head
+        if (threadIdx.x < S) q[bh * S + threadIdx.x] = mine * (1.0f / stat[1]);
+        return;
+    }
+    if (threadIdx.x < S) rec[2 + threadIdx.x] = mine;
     if (threadIdx.x == 0) {
         rec[0] = stat[0];
         rec[1] = stat[1];
@@ -694,6 +788,30 @@ static int pick_pw(int64_t bhq, int64_t kvLen) {
     return 4;
 }
 
+// Decode (one query token): cache rows per wavefront (a chunk is 4 times that).  g_decode_pw forces it (tests,
+// measurements); 0 = choose.
+static int g_decode_pw = 0;
+struct DecodePlan {
+    int pw;
+};
+static DecodePlan plan_decode(int64_t bh, int64_t kv, bool half_cache, int64_t max_records) {
+    // fp32 rows are 32 lanes wide (2 rows per wave-wide load), fp16 rows 16 lanes (4 rows): 2..8 loads per lane
+    const int lo = half_cache ? 8 : 4, hi = half_cache ? 32 : 16;
+    auto chunks = [&](int pw) { return (kv + 4 * pw - 1) / (4 * pw); };
+    // Chunks of 4 wavefronts, merged by a second launch: the largest chunk that still gives 256
+    // workgroups, and 512 for the two larger chunk sizes (measured, us, fp32: kv 256 -- 16/32/64-row chunks 8.6 / 8.2 /
+    // 9.3; kv 512 -- 11.1 / 10.1 / 10.3; kv 1024 -- 15.1 / 13.3 / 13.1; kv 2048 -- 30.7 / 19.7 / 19.0)
+    DecodePlan p{lo};
+    for (int pw = hi; pw >= lo; pw >>= 1)
+        if (bh * chunks(pw) >= (pw > 2 * lo ? 512 : 256)) {
+            p.pw = pw;
+            break;
+        }
+    if (g_decode_pw >= lo && g_decode_pw <= hi && (g_decode_pw & (g_decode_pw - 1)) == 0) p.pw = g_decode_pw;
+    while (p.pw < hi && bh * chunks(p.pw) > max_records) p.pw <<= 1;  // the records must fit the workspace
+    return p;
+}
+
 }  // namespace llmops
 
 using namespace llmops;
@@ -710,8 +828,8 @@ extern "C" int llmops_rope_embed(float* x, int64_t B, int64_t H, int64_t L, int6
 
 extern "C" size_t llmops_attention_workspace_bytes(int64_t B, int64_t qL, int64_t H, int64_t S, int64_t maxlen) {
     if (B <= 0 || qL <= 0 || H <= 0 || S <= 0 || maxlen <= 0) return 0;
-    // pick_pw() uses 64-row chunks unless that gives fewer than 1024 workgroups, and the finer
-    // chunkings it then falls back to stay below 2048 workgroups
+    // the planners use 64-row chunks (128 with an fp16 cache) unless that gives fewer than 1024 workgroups, and the
+    // finer chunkings they then fall back to stay below 2048 workgroups; a plan that does not fit is coarsened
     const int64_t bhq = B * H * qL;
     int64_t records = bhq * ((maxlen + 63) / 64);
     if (records < 2048) records = 2048;
@@ -722,34 +840,50 @@ extern "C" size_t llmops_attention_workspace_bytes(int64_t B, int64_t qL, int64_
 template <typename T>
 static int attention_impl(float* q, float* k, const float* v, int64_t B, int64_t qL, int64_t H, int64_t S,
                           const float* inv_freq, int64_t half, T* cache, int64_t maxlen, const int32_t* slots,
-                          int position_id, int layer_id, void* workspace, hipStream_t st) {
+                          int position_id, const int32_t* pos_dev, int layer_id, void* workspace, size_t workspace_bytes,
+                          hipStream_t st) {
+    constexpr bool kHalfCache = sizeof(T) == 2;
     T* kc = cache + (int64_t)(2 * layer_id + 0) * B * H * maxlen * S;
     T* vc = cache + (int64_t)(2 * layer_id + 1) * B * H * maxlen * S;
     uint8_t* wsb = reinterpret_cast<uint8_t*>(workspace);
     int32_t* row_token = reinterpret_cast<int32_t*>(wsb + LLMOPS_ATTN_COUNTER_BYTES);
-    float* part = reinterpret_cast<float*>(wsb + LLMOPS_ATTN_COUNTER_BYTES + align_up((size_t)maxlen * 4, 256));
+    const size_t part_off = LLMOPS_ATTN_COUNTER_BYTES + align_up((size_t)maxlen * 4, 256);
+    float* part = reinterpret_cast<float*>(wsb + part_off);
+    const int64_t max_records = (int64_t)((workspace_bytes - part_off) / ((S + 2) * sizeof(float)));
     int64_t kvLen = (int64_t)position_id + qL;
     if (kvLen > maxlen) kvLen = maxlen;
     const int64_t bhq = B * H * qL;
+    if (qL == 1 && (half % 4) == 0) {
+        // decode: rope, cache update and split-KV attention in one launch, then the merge of the chunk records
+        // (none when a head has a single chunk).  With the position in device memory the launch is sized for a
+        // full cache.
+        const int64_t kv_plan = pos_dev ? maxlen : kvLen;
+        const DecodePlan p = plan_decode(bhq, kv_plan, kHalfCache, max_records);
+        const int nchunks = (int)((kv_plan + 4 * p.pw - 1) / (4 * p.pw));
+        if ((int64_t)bhq * nchunks > max_records)
+            return fail(LLMOPS_EWORKSPACE, "attention workspace too small for %lld chunk records", (long long)bhq * nchunks);
+        const unsigned grid = (unsigned)(bhq * nchunks);
+#define LLMOPS_DECODE(PWV)                                                                                         \
+    attn_decode_kernel<T, PWV><<<grid, 256, 0, st>>>(q, k, v, inv_freq, (int)half, kc, vc, H, maxlen, slots, position_id, \
+                                                     pos_dev, part, nchunks)
+        switch (p.pw) {
+            case 4: if constexpr (!kHalfCache) LLMOPS_DECODE(4); break;
+            case 8: LLMOPS_DECODE(8); break;
+            case 16: LLMOPS_DECODE(16); break;
+            case 32: if constexpr (kHalfCache) LLMOPS_DECODE(32); break;
+        }
+#undef LLMOPS_DECODE
+        LLMOPS_LAUNCH_CHECK();
+        if (nchunks > 1) {
+            attn_merge_kernel<<<(unsigned)bhq, 128, 0, st>>>(q, part, qL, H, nchunks, pos_dev, maxlen, 4 * p.pw);
+            LLMOPS_LAUNCH_CHECK();
+        }
+        return LLMOPS_OK;
+    }
+    if (pos_dev != nullptr) return fail(LLMOPS_EINVAL, "a position in device memory needs one query token and half %% 4 == 0");
     const int pw = pick_pw(bhq, kvLen);
     const int nchunks = (int)((kvLen + 4 * pw - 1) / (4 * pw));
     const unsigned grid = (unsigned)(bhq * nchunks);
-    if (qL == 1 && (half % 4) == 0) {
-        // decode: rope, cache update and split-KV attention in one launch, then the merge
-        if (pw == 16)
-            attn_decode_kernel<T, 16><<<grid, 256, 0, st>>>(q, k, v, inv_freq, (int)half, kc, vc, H, maxlen, kvLen, slots,
-                                                          position_id, part, nchunks);
-        else if (pw == 8)
-            attn_decode_kernel<T, 8><<<grid, 256, 0, st>>>(q, k, v, inv_freq, (int)half, kc, vc, H, maxlen, kvLen, slots,
-                                                         position_id, part, nchunks);
-        else
-            attn_decode_kernel<T, 4><<<grid, 256, 0, st>>>(q, k, v, inv_freq, (int)half, kc, vc, H, maxlen, kvLen, slots,
-                                                         position_id, part, nchunks);
-        LLMOPS_LAUNCH_CHECK();
-        attn_merge_kernel<<<(unsigned)bhq, 128, 0, st>>>(q, part, qL, H, nchunks);
-        LLMOPS_LAUNCH_CHECK();
-        return LLMOPS_OK;
-    }
     if (qL > 1) {
         fill_i32_kernel<<<(unsigned)((maxlen + 255) / 256), 256, 0, st>>>(row_token, maxlen, -1);
         LLMOPS_LAUNCH_CHECK();
@@ -764,6 +898,7 @@ static int attention_impl(float* q, float* k, const float* v, int64_t B, int64_t
         LLMOPS_LAUNCH_CHECK();
         return LLMOPS_OK;
     }
+    if ((int64_t)bhq * nchunks > max_records) return fail(LLMOPS_EWORKSPACE, "attention workspace too small for %lld chunk records", (long long)bhq * nchunks);
     if (pw == 16)
         attn_split_kernel<T, 16><<<grid, 256, 0, st>>>(q, kc, vc, qL, H, maxlen, kvLen, row_token, part, nchunks);
     else if (pw == 8)
@@ -776,10 +911,10 @@ static int attention_impl(float* q, float* k, const float* v, int64_t B, int64_t
     return LLMOPS_OK;
 }
 
-extern "C" int llmops_attention_rope(float* q, float* k, const float* v, int64_t B, int64_t qL, int64_t H, int64_t S,
-                                     const float* inv_freq, int64_t half, void* kv_cache, int cache_dtype,
-                                     int64_t planes, int64_t maxlen, const int32_t* slots, int position_id,
-                                     int layer_id, void* workspace, size_t workspace_bytes, llmops_stream_t stream) {
+static int attention_entry(float* q, float* k, const float* v, int64_t B, int64_t qL, int64_t H, int64_t S,
+                           const float* inv_freq, int64_t half, void* kv_cache, int cache_dtype, int64_t planes,
+                           int64_t maxlen, const int32_t* slots, int position_id, const int32_t* pos_dev, int layer_id,
+                           void* workspace, size_t workspace_bytes, llmops_stream_t stream) {
     LLMOPS_REQUIRE(q != nullptr && k != nullptr && v != nullptr && inv_freq != nullptr && kv_cache != nullptr);
     LLMOPS_REQUIRE(slots != nullptr && workspace != nullptr);
     LLMOPS_REQUIRE(B > 0 && qL > 0 && H > 0 && maxlen > 0);
@@ -788,7 +923,7 @@ extern "C" int llmops_attention_rope(float* q, float* k, const float* v, int64_t
     LLMOPS_REQUIRE(layer_id >= 0 && 2 * (int64_t)layer_id + 1 < planes);
     LLMOPS_REQUIRE(position_id >= 0);
     LLMOPS_REQUIRE(cache_dtype == LLMOPS_CACHE_F32 || cache_dtype == LLMOPS_CACHE_F16);
-    LLMOPS_REQUIRE(aligned(q, 16) && aligned(kv_cache, 16) && aligned(workspace, 256));
+    LLMOPS_REQUIRE(aligned(q, 16) && aligned(k, 16) && aligned(v, 16) && aligned(kv_cache, 16) && aligned(workspace, 256));
     LLMOPS_REQUIRE(B * H * qL * ((maxlen + 63) / 64) < ((int64_t)1 << 31));
     const size_t need = llmops_attention_workspace_bytes(B, qL, H, S, maxlen);
     if (workspace_bytes < need)
@@ -796,10 +931,30 @@ extern "C" int llmops_attention_rope(float* q, float* k, const float* v, int64_t
     hipStream_t st = as_stream(stream);
     if (cache_dtype == LLMOPS_CACHE_F32)
         return attention_impl<float>(q, k, v, B, qL, H, S, inv_freq, half, reinterpret_cast<float*>(kv_cache), maxlen, slots,
-                                     position_id, layer_id, workspace, st);
+                                     position_id, pos_dev, layer_id, workspace, workspace_bytes, st);
     return attention_impl<__half>(q, k, v, B, qL, H, S, inv_freq, half, reinterpret_cast<__half*>(kv_cache), maxlen, slots,
-                                  position_id, layer_id, workspace, st);
+                                  position_id, pos_dev, layer_id, workspace, workspace_bytes, st);
 }
+
+extern "C" int llmops_attention_rope(float* q, float* k, const float* v, int64_t B, int64_t qL, int64_t H, int64_t S,
+                                     const float* inv_freq, int64_t half, void* kv_cache, int cache_dtype,
+                                     int64_t planes, int64_t maxlen, const int32_t* slots, int position_id,
+                                     int layer_id, void* workspace, size_t workspace_bytes, llmops_stream_t stream) {
+    return attention_entry(q, k, v, B, qL, H, S, inv_freq, half, kv_cache, cache_dtype, planes, maxlen, slots, position_id,
+                           nullptr, layer_id, workspace, workspace_bytes, stream);
+}
+
+extern "C" int llmops_attention_rope_decode(float* q, float* k, const float* v, int64_t B, int64_t H, int64_t S,
+                                            const float* inv_freq, int64_t half, void* kv_cache, int cache_dtype,
+                                            int64_t planes, int64_t maxlen, const int32_t* slot,
+                                            const int32_t* position_id, int layer_id, void* workspace,
+                                            size_t workspace_bytes, llmops_stream_t stream) {
+    LLMOPS_REQUIRE(position_id != nullptr && (half % 4) == 0);
+    return attention_entry(q, k, v, B, 1, H, S, inv_freq, half, kv_cache, cache_dtype, planes, maxlen, slot, 0, position_id,
+                           layer_id, workspace, workspace_bytes, stream);
+}
+
+extern "C" void llmops_test_attn_set_decode_plan(int rows_per_wave) { llmops::g_decode_pw = rows_per_wave; }
 
 extern "C" int llmops_softmax(float* x, int64_t rows, int64_t K, llmops_stream_t stream) {
     LLMOPS_REQUIRE(x != nullptr && rows > 0 && K > 0 && rows < ((int64_t)1 << 31));

@@ -23,12 +23,19 @@ from . import _lib
 __all__ = [
     "offline_FC_quant_Q4A", "offline_FC_dequant_Q4A", "fc_Q4A", "fc_Q4A_noalloc", "fc_Q4A_decode", "interleave_gate_up", "FC_dynamic_quantize_x", "fc_Q4A_partials",
     "attention_rope", "attention_rope2", "rope_embed", "softmax", "rmsnorm", "iadd", "imul", "itrans", "clone",
-    "rmsnorm_out", "silu_mul", "empty", "ones", "embedding", "embedding_q8c_quant_w", "embedding_q8c", "tensor_pool", "set_default_group_k",
+    "rmsnorm_out", "silu_mul", "empty", "ones", "embedding", "embedding_q8c_quant_w", "embedding_q8c", "tensor_pool", "set_default_group_k", "reserve_workspace",
     "group_k_of",
 ]
 
+# Callers of the reference read ``tensor.item_size`` (chatllama/main.py:171-173, ops/perf_ops.py:242; bound at
+# ops/main.cpp:95-142).  torch spells it ``itemsize`` / ``element_size()``; the reference's spelling is added as
+# a read-only property so that such callers run unchanged on the tensors this module hands out.
+if not hasattr(torch.Tensor, "item_size"):
+    torch.Tensor.item_size = property(lambda self: self.element_size())
+
 _default_group_k = 32  # the reference's compiled-in default (ops/op_fc.hpp:109)
 _workspaces = {}
+_retired = []  # superseded workspaces, kept alive for graphs that recorded their addresses
 
 
 def set_default_group_k(g):
@@ -67,15 +74,40 @@ def _dev(t, dtype, rank=None, name="tensor"):
 def _workspace(device, nbytes, kind="fc"):
     """Persistent scratch, one per op family, device and stream: ops enqueued on different streams may run
     at the same time and must not share counters or partial sums.  Its first bytes hold arrival counters,
-    which must start at zero and which the kernels leave at zero."""
+    which must start at zero and which the kernels leave at zero.
+
+    A HIP graph that captured an op replays the raw address of the workspace the op was given, so a
+    workspace is never freed: when a later call needs more, the old tensor is kept (``_retired``) and a
+    larger one takes its place for the calls that follow.  While the stream is capturing nothing may be
+    allocated or zero-filled (the fill would be recorded into the graph, and the first replay could find
+    counters that were never zeroed): an op that would need a new or larger workspace then raises.  Run the
+    op once, at the largest size, on the stream that will capture -- or call ``reserve_workspace`` -- first."""
     index = device.index if device.index is not None else torch.cuda.current_device()
     key = (kind, device.type, index, torch._C._cuda_getCurrentRawStream(index))
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
+        if torch.cuda.is_current_stream_capturing():
+            raise RuntimeError(
+                f"llmops: the {kind} workspace of this stream would have to be "
+                f"{'created' if ws is None else 'enlarged'} ({int(nbytes)} bytes) while the stream is capturing a graph; "
+                "run the op once on this stream before the capture, or call llmops.reserve_workspace")
+        if ws is not None:
+            _retired.append(ws)  # a graph captured earlier may still replay its address
         size = max(int(nbytes), 16 << 20)
         ws = torch.zeros(size, dtype=torch.uint8, device=device)
         _workspaces[key] = ws
     return ws
+
+
+def reserve_workspace(device=None, fc_bytes=0, attn_bytes=0):
+    """Make sure the current stream's FC / attention workspaces on ``device`` hold at least this many bytes
+    (``llmops_fc_Q4A_workspace_bytes`` / ``llmops_attention_workspace_bytes`` give the figures), so that a graph
+    capture on this stream finds them in place."""
+    device = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
+    if fc_bytes:
+        _workspace(device, fc_bytes, "fc")
+    if attn_bytes:
+        _workspace(device, attn_bytes, "attn")
 
 
 def group_k_of(weiq):
@@ -262,7 +294,9 @@ def rope_embed(x, inv_freq, position_id):
 
 def attention_rope2(q, k, v, inv_freq, kv_cache, kvc_slots, position_id, layer_id):
     """q,k,v fp32 [B,qL,H*S]; kv_cache [2*layers,B,H,maxlen,S]; kvc_slots int32 [qL].
-    In place: q <- attention output, k <- rotated k, cache rows updated (ops/op_attn.hpp:721-1029)."""
+    In place: q <- attention output, k <- rotated k, cache rows updated (ops/op_attn.hpp:721-1029).
+    Extension: with qL == 1, ``position_id`` may be an int32 tensor [1] on the device; the kernels then read the
+    position (and the slot) from memory, so a HIP graph that captured the call serves every following token."""
     _dev(q, torch.float32, 3, "q")
     _dev(k, torch.float32, 3, "k")
     _dev(v, torch.float32, 3, "v")
@@ -281,6 +315,13 @@ def attention_rope2(q, k, v, inv_freq, kv_cache, kvc_slots, position_id, layer_i
     need = lib.llmops_attention_workspace_bytes(B, qL, H, S, maxlen)
     ws = _workspace(q.device, need, kind="attn")
     dt = 0 if kv_cache.dtype == torch.float32 else 1
+    if isinstance(position_id, torch.Tensor):
+        _dev(position_id, torch.int32, 1, "position_id")
+        _require(qL == 1 and position_id.numel() == 1, "position_id tensor: one query token, one value")
+        _lib.check(lib.llmops_attention_rope_decode(_ptr(q), _ptr(k), _ptr(v), B, H, S, _ptr(inv_freq), inv_freq.shape[0],
+                                                    _ptr(kv_cache), dt, planes, maxlen, _ptr(kvc_slots), _ptr(position_id),
+                                                    int(layer_id), _ptr(ws), ws.numel(), _stream(q)))
+        return
     _lib.check(lib.llmops_attention_rope(_ptr(q), _ptr(k), _ptr(v), B, qL, H, S, _ptr(inv_freq), inv_freq.shape[0],
                                          _ptr(kv_cache), dt, planes, maxlen, _ptr(kvc_slots), int(position_id),
                                          int(layer_id), _ptr(ws), ws.numel(), _stream(q)))

@@ -35,6 +35,8 @@ SIGNATURES = {
     "llmops_attention_workspace_bytes": (c_size, [c_i64, c_i64, c_i64, c_i64, c_i64]),
     "llmops_attention_rope": (c_int, [c_ptr, c_ptr, c_ptr, c_i64, c_i64, c_i64, c_i64, c_ptr, c_i64, c_ptr, c_int,
                                       c_i64, c_i64, c_ptr, c_int, c_int, c_ptr, c_size, c_ptr]),
+    "llmops_attention_rope_decode": (c_int, [c_ptr, c_ptr, c_ptr, c_i64, c_i64, c_i64, c_ptr, c_i64, c_ptr, c_int, c_i64, c_i64,
+                                             c_ptr, c_ptr, c_int, c_ptr, c_size, c_ptr]),
     "llmops_softmax": (c_int, [c_ptr, c_i64, c_i64, c_ptr]),
     "llmops_mm_qk": (c_int, [c_ptr, c_i64, c_i64, c_i64, c_ptr, c_i64, c_ptr, c_i64, c_i64, c_i64, c_i64, c_i64, c_ptr]),
     "llmops_rmsnorm": (c_int, [c_ptr, c_i64, c_i64, c_ptr, c_f32, c_ptr]),
@@ -54,6 +56,7 @@ SIGNATURES = {
     "llmops_test_gemm_set_split": (None, [c_int]),
     "llmops_test_fc_set_row_routing": (None, [c_int, c_int]),
     "llmops_test_fc_rows_set_split": (None, [c_int]),
+    "llmops_test_attn_set_decode_plan": (None, [c_int]),
     "llmops_test_fc_decode_dump": (c_int, [c_ptr, c_i64, c_i64, c_ptr, c_i64, c_i64, c_int, c_i64, c_ptr, c_ptr, c_ptr, c_ptr,
                                            c_ptr, c_ptr, c_size, c_ptr]),
 }

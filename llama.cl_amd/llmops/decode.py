@@ -203,30 +203,53 @@ class LlamaDecoder:
         return llmops.fc_Q4A_decode(act, ops["down_proj"].weight, H, residual=attn_output, want_sumsq=True)
 
     def capture_decode(self, kv_cache, slot, position_id, stream=None):
-        """Capture one decode step (batch 1, one token, fixed slot/position) as a HIP graph.
-        Returns a DecodeGraph: write the token into ``.input_ids``, call ``.replay()``, read ``.logits``."""
+        """Capture one decode step (batch 1, one token) as a HIP graph that serves every position: the token id,
+        the cache slot and the position live in device memory and are read by the kernels at replay time.
+        Returns a DecodeGraph: ``step(token, slot, position_id)`` (or write ``.input_ids``, ``set_position`` and
+        ``replay()``), then read ``.logits``."""
         stream = stream or torch.cuda.Stream()
         input_ids = torch.zeros(1, 1, dtype=torch.int64, device=self.device)
         slots = torch.tensor([slot], dtype=torch.int32, device=self.device)
+        position = torch.tensor([position_id], dtype=torch.int32, device=self.device)
         with torch.cuda.stream(stream):
             stream.wait_stream(torch.cuda.default_stream(self.device))
-            self.forward(input_ids, kv_cache, slots, position_id)  # warm-up: code objects, workspace size
+            self.forward(input_ids, kv_cache, slots, position)  # warm-up: code objects, workspaces of this stream
             torch.cuda.synchronize()
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph, stream=stream):
-                logits = self.forward(input_ids, kv_cache, slots, position_id)
-        # the per-device workspaces are captured by address too; pin the ones in use
+                logits = self.forward(input_ids, kv_cache, slots, position)
+        # the workspaces are captured by address too (the module never frees one; the graph object also holds them)
         workspace = [w for key, w in llmops._workspaces.items() if key[1] == self.device.type]
-        return DecodeGraph(graph, input_ids, slots, kv_cache, logits, stream, workspace)
+        return DecodeGraph(graph, input_ids, slots, position, kv_cache, logits, stream, workspace)
 
 
 class DecodeGraph:
     """A captured decode step together with every tensor whose address the graph has recorded.
-    The graph replays raw device pointers, so these tensors must live as long as the graph does."""
+    The graph replays raw device pointers, so these tensors must live as long as the graph does.
+    Token, slot and position are device values the kernels read at replay time: one graph serves a
+    whole generation loop."""
 
-    def __init__(self, graph, input_ids, slots, kv_cache, logits, stream, workspace):
-        self.graph, self.input_ids, self.slots, self.kv_cache, self.logits, self.stream, self.workspace = \
-            graph, input_ids, slots, kv_cache, logits, stream, workspace
+    def __init__(self, graph, input_ids, slots, position, kv_cache, logits, stream, workspace):
+        self.graph, self.input_ids, self.slots, self.position, self.kv_cache, self.logits, self.stream, self.workspace = \
+            graph, input_ids, slots, position, kv_cache, logits, stream, workspace
+        self._host = torch.empty(2, dtype=torch.int32).pin_memory()
+
+    def set_position(self, slot, position_id):
+        """cache row the next token goes to and its position (kv length = position + 1, up to the cache size)"""
+        if not (0 <= int(slot) < self.kv_cache.shape[3]) or int(position_id) < 0:
+            raise ValueError("slot outside the cache or negative position")
+        self._host[0], self._host[1] = int(slot), int(position_id)
+        with torch.cuda.stream(self.stream):
+            self.slots.copy_(self._host[0:1], non_blocking=True)
+            self.position.copy_(self._host[1:2], non_blocking=True)
 
     def replay(self):
-        self.graph.replay()
+        with torch.cuda.stream(self.stream):
+            self.graph.replay()
+
+    def step(self, token, slot, position_id):
+        with torch.cuda.stream(self.stream):
+            self.input_ids.fill_(int(token))
+        self.set_position(slot, position_id)
+        self.replay()
+        return self.logits

@@ -94,3 +94,12 @@ def test_kvcache_slot_manager():
     # sentence 2 holds the instruction: asked to fail rather than overwrite it
     assert not kv.prepare(1, 4, 2)
     assert kv.cur_kv_len == 8 and kv.slots.dtype == torch.int32
+
+
+def test_tensor_attributes_the_reference_callers_use():
+    """``weight.numel() * weight.item_size`` (chatllama/main.py:171-173) must work on what the ops return."""
+    import torch
+    import llmops  # noqa: F401  (adds the reference's spelling of the element size)
+    t = torch.zeros(3, 5, dtype=torch.int8)
+    assert t.item_size == 1 and torch.zeros(2, dtype=torch.float32).item_size == 4
+    assert t.numel() * t.item_size == 15 and tuple(t.shape) == (3, 5) and t.clone().numpy().shape == (3, 5)

@@ -335,3 +335,43 @@ def test_attention_prefill_long_chunk_wrapping_the_ring(ops, orc):
     """a 1024-token chunk whose slots wrap around a cache of 2048 rows that is already full"""
     rng = np.random.default_rng(77)
     _prefill_case(ops, orc, rng, 1500, 1024, 2048, 32, heads=[5, 30])
+
+
+@pytest.mark.parametrize("cache_dtype", [torch.float32, torch.float16])
+def test_decode_attention_every_chunking_and_device_position(ops, orc, cache_dtype):
+    """Decode attention (one query token) with every chunk size forced in turn and with the position read from
+    device memory (the launch is then sized for the whole cache
+    and chunks beyond the current length leave at once): all against the oracle, at kv lengths around the
+    chunk and tile edges.  The new row's slot lies inside, at the end of, and beyond the attended rows."""
+    from llmops import _lib
+    lib = _lib.load()
+    rng = np.random.default_rng(12)
+    B, H, S, maxlen = 1, 5, 128, 1100
+    inv_freq = (1.0 / (10000.0 ** (np.arange(0, 64, 2, dtype=np.float32) / np.float32(64)))).astype(np.float32)
+    cache0 = rng.standard_normal((2, B, H, maxlen, S)).astype(np.float32)
+    if cache_dtype == torch.float16:
+        cache0 = cache0.astype(np.float16).astype(np.float32)
+    plans = [0] + list((4, 8, 16) if cache_dtype == torch.float32 else (8, 16, 32))
+    tol = 1e-5 if cache_dtype == torch.float32 else 3e-3   # fp16: rounding of the one new row (extension, no reference)
+    try:
+        for kv in (1, 2, 17, 64, 65, 255, 256, 257, 511, 512, 513, 1025, 1100):
+            q, k, v = (rng.standard_normal((B, 1, H * S)).astype(np.float32) for _ in range(3))
+            pos = kv - 1
+            slot = pos if kv % 2 else (pos * 7) % kv          # odd lengths: the last row; even: somewhere inside
+            slots = np.array([slot], np.int32)
+            want, k_ref, cache_ref = orc.attention(q, k, v, inv_freq, cache0, slots, pos, 0)
+            if cache_dtype == torch.float16:
+                c16 = cache_ref.astype(np.float16).astype(np.float32)
+                want = _attend_cache(orc, q, inv_freq, c16, slots, pos, maxlen)
+            for pw in plans:
+                lib.llmops_test_attn_set_decode_plan(pw)
+                for dev_pos in (False, True):
+                    tq, tk, tc = dev(q), dev(k), dev(cache0).to(cache_dtype)
+                    p = torch.tensor([pos], dtype=torch.int32, device="cuda") if dev_pos else pos
+                    ops.attention_rope2(tq, tk, dev(v), dev(inv_freq), tc, dev(slots), p, 0)
+                    assert max_rel_err(host(tq), want) <= tol, (kv, pw, dev_pos)
+                    if cache_dtype == torch.float32:
+                        assert np.abs(host(tk) - k_ref).max() <= 1e-5
+                        assert np.abs(host(tc) - cache_ref).max() <= 1e-5
+    finally:
+        lib.llmops_test_attn_set_decode_plan(0)

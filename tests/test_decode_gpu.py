@@ -211,3 +211,88 @@ def test_decoder_from_reference_format_file(tmp_path, plan):
         assert max_rel_err(got.cpu().numpy(), want.cpu().numpy()) <= 5e-2  # fused vs unfused: re-quantized activations drift
         direct = LlamaDecoder(CFG, group_k=128, seed=9, plan="fused")       # same seed -> same tensors, stacked directly
         assert torch.equal(got, run(direct))
+
+
+def test_graph_keeps_its_workspace_when_a_later_call_needs_a_larger_one():
+    """A captured one-row FC replays the address of the workspace it was given.  A 2048-row FC on the same stream
+    then needs a much larger workspace: the module must not free the old one (the replay would write its
+    partial sums and arrival counters into memory that now belongs to someone else).  And an op that would have
+    to create or enlarge a workspace while its stream is capturing must raise instead of allocating."""
+    import llmops
+    dev = torch.device("cuda:0")
+    rng = np.random.default_rng(21)
+    N, K = 4096, 11008        # a one-row FC on this shape meets its two k-splits in the workspace
+    wq = llmops.offline_FC_quant_Q4A(torch.from_numpy((rng.standard_normal((N, K)) * 0.02).astype(np.float32)).to(dev), 128)
+    x1 = torch.from_numpy(rng.standard_normal((1, 1, K)).astype(np.float32)).to(dev)
+    xb = torch.from_numpy(rng.standard_normal((1, 2048, K)).astype(np.float32)).to(dev)
+    s = torch.cuda.Stream()
+    with torch.cuda.stream(s):
+        want = llmops.fc_Q4A(x1, wq, N)            # warm-up on the capture stream: creates its workspace
+        torch.cuda.synchronize()
+        ws_before = [w.data_ptr() for k, w in llmops._workspaces.items() if k[0] == "fc"]
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=s):
+            y = llmops.fc_Q4A(x1, wq, N)
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y, want)
+        big = llmops.fc_Q4A(xb, wq, N)             # needs a larger workspace on the same stream
+        # fill freshly allocated memory with garbage: if the old workspace had been freed, this is where it would land
+        junk = [torch.full((4 << 20,), 0x7F, dtype=torch.uint8, device=dev) for _ in range(8)]
+        torch.cuda.synchronize()
+        assert any(w.data_ptr() not in ws_before for k, w in llmops._workspaces.items() if k[0] == "fc")
+        for _ in range(3):
+            y.zero_()
+            g.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(y, want)
+        assert torch.equal(llmops.fc_Q4A(xb[:, :1].contiguous(), wq, N), llmops.fc_Q4A(xb[:, :1].contiguous(), wq, N))
+        del junk, big
+    # a stream that has never run an FC: capturing one must be refused, not allocate inside the capture
+    s2 = torch.cuda.Stream()
+    g2 = torch.cuda.CUDAGraph()
+    with pytest.raises(RuntimeError, match="capturing"):
+        with torch.cuda.graph(g2, stream=s2):
+            llmops.fc_Q4A(x1, wq, N)
+
+
+def test_one_decode_graph_serves_successive_positions(orc):
+    """The captured step reads token, slot and position from device memory: ONE graph is replayed over a run
+    of successive positions (crossing a chunk boundary of the attention kernel and wrapping the ring buffer of
+    cache slots) and must give, at every position, exactly what the eager step with the same device-side
+    position gives, the eager step with the position passed by value to rounding, and the oracle's logits to
+    the end-to-end tolerance."""
+    from llmops.decode import LlamaDecoder
+    from llmops.opset import KVCache
+    model = LlamaDecoder(CFG, group_k=128, seed=6)
+    maxlen = 40
+    kv = KVCache(CFG, 1, maxlen)
+    rng = np.random.default_rng(8)
+    ids0 = rng.integers(0, CFG["vocab_size"], (1, 13)).astype(np.int64)
+    assert kv.prepare(13, 1, 0)
+    model.forward(torch.from_numpy(ids0).cuda(), kv.cache, kv.slots, kv.position_id)   # 13 tokens of context
+    eager_cache = kv.cache.clone()
+    cache_h = kv.cache.cpu().numpy()
+    dg = model.capture_decode(kv.cache, 0, 0)          # captured at an unrelated position
+    kv.cache.copy_(eager_cache)                        # (the capture's warm-up wrote slot 0)
+    pos_t = torch.zeros(1, dtype=torch.int32, device="cuda")
+    for step in range(34):                             # positions 13 .. 46: kv length saturates at 40, slots wrap
+        assert kv.prepare(1, 1, 0)
+        slot, pos = int(kv.slots[0]), kv.position_id
+        tok = int(rng.integers(0, CFG["vocab_size"]))
+        ids = torch.tensor([[tok]], dtype=torch.int64, device="cuda")
+        # eager, position by value and position on the device, each on its own copy of the cache
+        c_val, c_dev = eager_cache.clone(), eager_cache.clone()
+        by_value = model.forward(ids, c_val, kv.slots, pos)
+        pos_t.fill_(pos)
+        on_device = model.forward(ids, c_dev, kv.slots, pos_t)
+        logits = dg.step(tok, slot, pos)
+        torch.cuda.synchronize()
+        assert torch.equal(logits, on_device), (step, pos)
+        assert torch.equal(kv.cache, c_dev), (step, pos)
+        assert max_rel_err(logits.cpu().numpy(), by_value.cpu().numpy()) <= 1e-4, (step, pos)
+        if step % 8 == 0 or step == 33:
+            want, _ = oracle_forward(orc, model, np.array([[tok]], np.int64), eager_cache.cpu().numpy(), np.array([slot], np.int32), pos)
+            assert max_rel_err(logits.cpu().numpy(), want) <= 5e-2, (step, pos)
+        eager_cache.copy_(c_dev)
+    assert kv.position_id == 46 and kv.cur_kv_len == maxlen
