@@ -143,6 +143,14 @@ int llmops_fc_Q4A_decode(const float* x, int64_t rows, int64_t K, const int8_t* 
                          const float* sumsq_in, int64_t sumsq_parts, float* sumsq_out, float* y, void* workspace,
                          size_t workspace_bytes, llmops_stream_t stream);
 
+/* fc_Q4A (one row, group 128) on the output of llmops_attention_rope_decode_records: the o projection of a decode
+ * step (chatllama/main.py:353-355) with the merge of the attention chunks (ops/op_attn.hpp:1012-1025 computes the
+ * same softmax-weighted sum in one piece) folded into the FC's input side.  K = H*128 = Kg*128; residual and
+ * sumsq_out as in llmops_fc_Q4A_decode. */
+int llmops_fc_Q4A_decode_attn(const float* rec_stats, const float* rec_outs, int64_t chunks, int64_t H, const int8_t* weiq,
+                              int64_t Ng, int64_t Kg, int64_t N_out, const float* residual, float* sumsq_out, float* y,
+                              void* workspace, size_t workspace_bytes, llmops_stream_t stream);
+
 /* The second half of fc_Q4A on its own (ops/op_fc.hpp:318-423): the product for activations that
  * llmops_FC_dynamic_quantize_x has already quantized (xq int8 [rows,Kg*G], xd and gsum fp32
  * [rows,Kg]).  llmops_fc_Q4A == llmops_FC_dynamic_quantize_x into the workspace + this. */
@@ -195,6 +203,20 @@ int llmops_attention_rope_decode(float* q, float* k, const float* v, int64_t B, 
                                  const float* inv_freq, int64_t half, void* kv_cache, int cache_dtype, int64_t planes,
                                  int64_t maxlen, const int32_t* slot, const int32_t* position_id, int layer_id,
                                  void* workspace, size_t workspace_bytes, llmops_stream_t stream);
+
+/* attention_rope2 for one query token (B sequences of one token) that leaves the merge of its split-KV chunks to
+ * the consumer: instead of overwriting q with softmax(qK^T)V (ops/op_attn.hpp:1012-1025) it writes, per head,
+ * up to 8 chunk records -- rec_stats fp32 [B*H][8][2] (max score, sum of exp) and rec_outs fp32 [B*H][8][128]
+ * (sum of exp-weighted V rows) -- which llmops_fc_Q4A_decode_attn merges while it loads its input.  q is left as
+ * it came in; k is rotated in place and the cache updated as usual.  The position is `position_id`, or, when
+ * position_id_dev is not NULL, the int32 it points at in device memory.  llmops_attention_records_chunks returns 8
+ * when a cache of `maxlen` rows can be served this way (fp32: up to 2048 rows, fp16: up to 4096), else 0. */
+int64_t llmops_attention_records_chunks(int64_t maxlen, int cache_dtype);
+int llmops_attention_rope_decode_records(float* q, float* k, const float* v, int64_t B, int64_t H, int64_t S,
+                                         const float* inv_freq, int64_t half, void* kv_cache, int cache_dtype,
+                                         int64_t planes, int64_t maxlen, const int32_t* slot, int position_id,
+                                         const int32_t* position_id_dev, int layer_id, float* rec_stats, float* rec_outs,
+                                         void* workspace, size_t workspace_bytes, llmops_stream_t stream);
 
 /* softmax (ops/op_misc.hpp:183-194, ops/utils.hpp:484-490): in place over rows of length K */
 int llmops_softmax(float* x, int64_t rows, int64_t K, llmops_stream_t stream);

@@ -68,6 +68,12 @@ int llmops_test_fc_decode_dump(const float* x, int64_t rows, int64_t K, const in
                                int group_k, int64_t N, float* y, int8_t* xq, float* xd, float* gsum, int32_t* acc,
                                void* workspace, size_t workspace_bytes, llmops_stream_t stream);
 
+/* llmops_fc_Q4A_decode_attn in the same dump build: the codes and scales of the attention output the kernel merged
+ * from the chunk records, and its int32 sums */
+int llmops_test_fc_decode_attn_dump(const float* rec_stats, const float* rec_outs, int64_t chunks, int64_t H,
+                                    const int8_t* weiq, int64_t Ng, int64_t Kg, int64_t N_out, float* y, int8_t* xq, float* xd,
+                                    float* gsum, int32_t* acc, void* workspace, size_t workspace_bytes, llmops_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

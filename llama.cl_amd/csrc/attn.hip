@@ -390,16 +390,26 @@ struct RowPiece<__half> {
 // cache rows are read exactly once per call: non-temporal, so that they do not displace the records and the
 // activations that are reused out of the caches
 __device__ __forceinline__ uint4 load_row16(const void* p) {
-    return *reinterpret_cast<const uint4*>(p);
+    typedef unsigned int u32x4_a __attribute__((ext_vector_type(4)));
+    const u32x4_a v = __builtin_nontemporal_load(reinterpret_cast<const u32x4_a*>(p));
+    return make_uint4(v.x, v.y, v.z, v.w);
 }
 
-template <typename T, int PW>
-__global__ __launch_bounds__(256) void attn_decode_kernel(float* q, float* k, const float* __restrict__ v,
+//
+// RECS: the chunk records are not merged here at all but handed to the FC that consumes the attention output
+// (the o projection merges them as it loads its input, llmops_fc_Q4A_decode_attn): workgroups of NWV = 16
+// wavefronts take 256 or 512 cache rows each, so that a head has at most kAttnRecChunks records, laid out as
+// stats [B*H][kAttnRecChunks][2] (max, sum) and outs [B*H][kAttnRecChunks][128]; a chunk beyond the current kv
+// length leaves an empty record (sum 0, zeros).  q is then left as it came in.
+constexpr int kAttnRecChunks = 8;
+
+template <typename T, int PW, int NWV = 4, bool RECS = false>
+__global__ __launch_bounds__(NWV * 64) void attn_decode_kernel(float* q, float* k, const float* __restrict__ v,
                                                            const float* __restrict__ inv_freq, int half, T* kc, T* vc,
                                                            int64_t H, int64_t maxlen, const int32_t* __restrict__ slots,
                                                            int position_id, const int32_t* __restrict__ pos_dev, float* part,
-                                                           int nchunks) {
-    constexpr int S = 128, NWV = 4, C = NWV * PW;  // 4 wavefronts per workgroup
+                                                           int nchunks, float* rec_stats = nullptr, float* rec_outs = nullptr) {
+    constexpr int S = 128, C = NWV * PW;
     constexpr int EPL = RowPiece<T>::EPL, LPR = S / EPL, RPW = 64 / LPR, NL = PW / RPW;
     static_assert(NL >= 1 && NL <= LPR, "rows per lane");
     __shared__ float sc[C];
@@ -413,7 +423,16 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(float* q, float* k, co
     if (pos_dev != nullptr) position_id = pos_dev[0];
     const int64_t kvLen = min((int64_t)position_id + 1, maxlen);
     const int nact = (int)((kvLen + C - 1) / C);  // chunks that hold rows at this position
-    if (chunk >= nact) return;
+    if (chunk >= nact) {
+        if (RECS) {  // an empty record: weight 0 whatever the others hold
+            if (threadIdx.x < S) rec_outs[(bh * kAttnRecChunks + chunk) * S + threadIdx.x] = 0.0f;
+            if (threadIdx.x == 0) {
+                rec_stats[(bh * kAttnRecChunks + chunk) * 2] = -FLT_MAX;
+                rec_stats[(bh * kAttnRecChunks + chunk) * 2 + 1] = 0.0f;
+            }
+        }
+        return;
+    }
     const int64_t p0 = (int64_t)chunk * C;
     T* kbase = kc + bh * maxlen * S;
     T* vbase = vc + bh * maxlen * S;
@@ -585,6 +604,14 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(float* q, float* k, co
         for (int w = 0; w < NWV; w++)
 #pragma unroll
             for (int r = 0; r < RPW; r++) mine += osh[w][r][threadIdx.x];
+    }
+    if (RECS) {
+        if (threadIdx.x < S) rec_outs[(bh * kAttnRecChunks + chunk) * S + threadIdx.x] = mine;
+        if (threadIdx.x == 0) {
+            rec_stats[(bh * kAttnRecChunks + chunk) * 2] = stat[0];
+            rec_stats[(bh * kAttnRecChunks + chunk) * 2 + 1] = stat[1];
+        }
+        return;
     }
     if (nchunks == 1) {  // the workgroup saw every row of the head
         if (threadIdx.x < S) q[bh * S + threadIdx.x] = mine * (1.0f / stat[1]);
@@ -788,6 +815,14 @@ static int pick_pw(int64_t bhq, int64_t kvLen) {
     return 4;
 }
 
+// cache rows per chunk when the chunk records go to the consumer FC (at most kAttnRecChunks chunks per head): 0 = the
+// cache is too long for that
+static int records_chunk_rows(int64_t maxlen, bool half_cache) {
+    if (maxlen <= kAttnRecChunks * 256) return 256;
+    if (half_cache && maxlen <= kAttnRecChunks * 512) return 512;
+    return 0;
+}
+
 // Decode (one query token): cache rows per wavefront (a chunk is 4 times that).  g_decode_pw forces it (tests,
 // measurements); 0 = choose.
 static int g_decode_pw = 0;
@@ -841,7 +876,7 @@ template <typename T>
 static int attention_impl(float* q, float* k, const float* v, int64_t B, int64_t qL, int64_t H, int64_t S,
                           const float* inv_freq, int64_t half, T* cache, int64_t maxlen, const int32_t* slots,
                           int position_id, const int32_t* pos_dev, int layer_id, void* workspace, size_t workspace_bytes,
-                          hipStream_t st) {
+                          hipStream_t st, float* rec_stats = nullptr, float* rec_outs = nullptr) {
     constexpr bool kHalfCache = sizeof(T) == 2;
     T* kc = cache + (int64_t)(2 * layer_id + 0) * B * H * maxlen * S;
     T* vc = cache + (int64_t)(2 * layer_id + 1) * B * H * maxlen * S;
@@ -853,6 +888,23 @@ static int attention_impl(float* q, float* k, const float* v, int64_t B, int64_t
     int64_t kvLen = (int64_t)position_id + qL;
     if (kvLen > maxlen) kvLen = maxlen;
     const int64_t bhq = B * H * qL;
+    if (rec_stats != nullptr) {
+        // decode with the merge left to the consumer: 16 wavefronts x 16 rows per chunk, or x 32 with an fp16 cache
+        // longer than 2048 rows
+        const int64_t kv_plan = pos_dev ? maxlen : kvLen;
+        const int rows = records_chunk_rows(maxlen, kHalfCache);
+        if (qL != 1 || (half % 4) != 0 || rows == 0) return fail(LLMOPS_EINVAL, "chunk records need one query token, half %% 4 == 0 and a cache of at most %d rows", kAttnRecChunks * (kHalfCache ? 512 : 256));
+        const int nchunks = (int)((kv_plan + rows - 1) / rows);
+        const unsigned grid = (unsigned)(bhq * nchunks);
+        if (rows == 256)
+            attn_decode_kernel<T, 16, 16, true><<<grid, 1024, 0, st>>>(q, k, v, inv_freq, (int)half, kc, vc, H, maxlen, slots, position_id,
+                                                                       pos_dev, nullptr, nchunks, rec_stats, rec_outs);
+        else if constexpr (kHalfCache)
+            attn_decode_kernel<T, 32, 16, true><<<grid, 1024, 0, st>>>(q, k, v, inv_freq, (int)half, kc, vc, H, maxlen, slots, position_id,
+                                                                       pos_dev, nullptr, nchunks, rec_stats, rec_outs);
+        LLMOPS_LAUNCH_CHECK();
+        return LLMOPS_OK;
+    }
     if (qL == 1 && (half % 4) == 0) {
         // decode: rope, cache update and split-KV attention in one launch, then the merge of the chunk records
         // (none when a head has a single chunk).  With the position in device memory the launch is sized for a
@@ -914,7 +966,8 @@ static int attention_impl(float* q, float* k, const float* v, int64_t B, int64_t
 static int attention_entry(float* q, float* k, const float* v, int64_t B, int64_t qL, int64_t H, int64_t S,
                            const float* inv_freq, int64_t half, void* kv_cache, int cache_dtype, int64_t planes,
                            int64_t maxlen, const int32_t* slots, int position_id, const int32_t* pos_dev, int layer_id,
-                           void* workspace, size_t workspace_bytes, llmops_stream_t stream) {
+                           void* workspace, size_t workspace_bytes, llmops_stream_t stream, float* rec_stats = nullptr,
+                           float* rec_outs = nullptr) {
     LLMOPS_REQUIRE(q != nullptr && k != nullptr && v != nullptr && inv_freq != nullptr && kv_cache != nullptr);
     LLMOPS_REQUIRE(slots != nullptr && workspace != nullptr);
     LLMOPS_REQUIRE(B > 0 && qL > 0 && H > 0 && maxlen > 0);
@@ -931,9 +984,9 @@ static int attention_entry(float* q, float* k, const float* v, int64_t B, int64_
     hipStream_t st = as_stream(stream);
     if (cache_dtype == LLMOPS_CACHE_F32)
         return attention_impl<float>(q, k, v, B, qL, H, S, inv_freq, half, reinterpret_cast<float*>(kv_cache), maxlen, slots,
-                                     position_id, pos_dev, layer_id, workspace, workspace_bytes, st);
+                                     position_id, pos_dev, layer_id, workspace, workspace_bytes, st, rec_stats, rec_outs);
     return attention_impl<__half>(q, k, v, B, qL, H, S, inv_freq, half, reinterpret_cast<__half*>(kv_cache), maxlen, slots,
-                                  position_id, pos_dev, layer_id, workspace, workspace_bytes, st);
+                                  position_id, pos_dev, layer_id, workspace, workspace_bytes, st, rec_stats, rec_outs);
 }
 
 extern "C" int llmops_attention_rope(float* q, float* k, const float* v, int64_t B, int64_t qL, int64_t H, int64_t S,
@@ -952,6 +1005,21 @@ extern "C" int llmops_attention_rope_decode(float* q, float* k, const float* v, 
     LLMOPS_REQUIRE(position_id != nullptr && (half % 4) == 0);
     return attention_entry(q, k, v, B, 1, H, S, inv_freq, half, kv_cache, cache_dtype, planes, maxlen, slot, 0, position_id,
                            layer_id, workspace, workspace_bytes, stream);
+}
+
+extern "C" int64_t llmops_attention_records_chunks(int64_t maxlen, int cache_dtype) {
+    return records_chunk_rows(maxlen, cache_dtype == LLMOPS_CACHE_F16) ? kAttnRecChunks : 0;
+}
+
+extern "C" int llmops_attention_rope_decode_records(float* q, float* k, const float* v, int64_t B, int64_t H, int64_t S,
+                                                    const float* inv_freq, int64_t half, void* kv_cache, int cache_dtype,
+                                                    int64_t planes, int64_t maxlen, const int32_t* slot, int position_id,
+                                                    const int32_t* position_id_dev, int layer_id, float* rec_stats,
+                                                    float* rec_outs, void* workspace, size_t workspace_bytes,
+                                                    llmops_stream_t stream) {
+    LLMOPS_REQUIRE(rec_stats != nullptr && rec_outs != nullptr && aligned(rec_stats, 16) && aligned(rec_outs, 16));
+    return attention_entry(q, k, v, B, 1, H, S, inv_freq, half, kv_cache, cache_dtype, planes, maxlen, slot, position_id,
+                           position_id_dev, layer_id, workspace, workspace_bytes, stream, rec_stats, rec_outs);
 }
 
 extern "C" void llmops_test_attn_set_decode_plan(int rows_per_wave) { llmops::g_decode_pw = rows_per_wave; }

@@ -15,7 +15,8 @@ int launch_gemv(const uint8_t* w, const int8_t* xq, const float* xd, const float
                 unsigned* counters, int64_t rows, int64_t Ng, int64_t Kg, int G, int64_t N, hipStream_t st);
 int launch_gemv_fused(const uint8_t* w, const float* x, float* y, float* part, unsigned* counters, int64_t rows, int64_t Ng,
                       int64_t Kg, int G, int64_t N, const float* residual, const float* norm_w, float eps, int glu,
-                      const float* sumsq_in, int sumsq_parts, float* sumsq_out, hipStream_t st, const DumpBufs* dump = nullptr);
+                      const float* sumsq_in, int sumsq_parts, float* sumsq_out, hipStream_t st, const DumpBufs* dump = nullptr,
+                      const float* rec_stats = nullptr, const float* rec_outs = nullptr, int rec_chunks = 0);
 int launch_add(float* a, const float* b, int64_t total, hipStream_t st);
 int launch_gemv_partials(const uint8_t* w, const int8_t* xq, int32_t* acc, int64_t rows, int64_t Ng, int64_t Kg, int G,
                          hipStream_t st);
@@ -160,6 +161,42 @@ extern "C" int llmops_fc_Q4A_decode(const float* x, int64_t rows, int64_t K, con
     return launch_gemv_fused(reinterpret_cast<const uint8_t*>(weiq), x, y, reinterpret_cast<float*>(ws + lay.off_part),
                              reinterpret_cast<unsigned*>(ws), rows, Ng, Kg, group_k, N_out, residual, norm_w, eps, glu,
                              sumsq_in, (int)sumsq_parts, sumsq_out, as_stream(stream));
+}
+
+static int fc_decode_attn(const float* rec_stats, const float* rec_outs, int64_t chunks, int64_t H, const int8_t* weiq,
+                          int64_t Ng, int64_t Kg, int64_t N_out, const float* residual, float* sumsq_out, float* y,
+                          void* workspace, size_t workspace_bytes, llmops_stream_t stream, const DumpBufs* dump) {
+    LLMOPS_REQUIRE(rec_stats != nullptr && rec_outs != nullptr && weiq != nullptr && y != nullptr && workspace != nullptr);
+    LLMOPS_REQUIRE(chunks > 0 && chunks <= 8 && H > 0 && Ng > 0 && Kg > 0 && Kg == H);  // K = H * 128, group 128
+    LLMOPS_REQUIRE(N_out > (Ng - 1) * kGroupN && N_out <= Ng * kGroupN);
+    LLMOPS_REQUIRE(Ng <= kTicketBytes / 4 && Ng * 64 < ((int64_t)1 << 31));
+    LLMOPS_REQUIRE(aligned(weiq, 16) && aligned(workspace, 256) && aligned(rec_stats, 16) && aligned(rec_outs, 16));
+    const FcWorkspace lay = fc_layout(1, Ng, Kg, 128);
+    if (workspace_bytes < lay.total)
+        return fail(LLMOPS_EWORKSPACE, "fc_Q4A needs %zu workspace bytes, got %zu", lay.total, workspace_bytes);
+    uint8_t* ws = reinterpret_cast<uint8_t*>(workspace);
+    return launch_gemv_fused(reinterpret_cast<const uint8_t*>(weiq), rec_outs, y, reinterpret_cast<float*>(ws + lay.off_part),
+                             reinterpret_cast<unsigned*>(ws), 1, Ng, Kg, 128, N_out, residual, nullptr, 0.0f, 0, nullptr, 0,
+                             sumsq_out, as_stream(stream), dump, rec_stats, rec_outs, (int)chunks);
+}
+
+extern "C" int llmops_fc_Q4A_decode_attn(const float* rec_stats, const float* rec_outs, int64_t chunks, int64_t H,
+                                         const int8_t* weiq, int64_t Ng, int64_t Kg, int64_t N_out, const float* residual,
+                                         float* sumsq_out, float* y, void* workspace, size_t workspace_bytes,
+                                         llmops_stream_t stream) {
+    return fc_decode_attn(rec_stats, rec_outs, chunks, H, weiq, Ng, Kg, N_out, residual, sumsq_out, y, workspace, workspace_bytes,
+                          stream, nullptr);
+}
+
+// the same kernel in its dump build (what it merged and quantized, and its int32 sums)
+extern "C" int llmops_test_fc_decode_attn_dump(const float* rec_stats, const float* rec_outs, int64_t chunks, int64_t H,
+                                               const int8_t* weiq, int64_t Ng, int64_t Kg, int64_t N_out, float* y, int8_t* xq,
+                                               float* xd, float* gsum, int32_t* acc, void* workspace, size_t workspace_bytes,
+                                               llmops_stream_t stream) {
+    LLMOPS_REQUIRE(xq != nullptr && xd != nullptr && gsum != nullptr && acc != nullptr && aligned(xq, 4));
+    const DumpBufs dump{xq, xd, gsum, acc};
+    return fc_decode_attn(rec_stats, rec_outs, chunks, H, weiq, Ng, Kg, N_out, nullptr, nullptr, y, workspace, workspace_bytes,
+                          stream, &dump);
 }
 
 extern "C" int llmops_fc_Q4A_prequantized(const int8_t* xq, const float* xd, const float* gsum, int64_t rows,

@@ -211,8 +211,49 @@ __global__ __launch_bounds__(NW * 64) void fc_gemv_kernel(const uint8_t* __restr
 //          kernel's own quantizer and integer core can be compared bit for bit with the reference's
 //          (llmops_test_fc_decode_dump).  Every workgroup stores the activations it quantized: all of them
 //          must agree.
-constexpr int kNorm = 1, kGlu = 2, kSums = 4, kGluIn = 8, kDump = 16;
+//   kAttnIn: the activation row is the output of decode attention, not yet merged: per head up to
+//          kAttnRecChunks chunk records (max, sum, weighted V sum over the chunk's cache rows) as
+//          llmops_attention_rope_decode_records leaves them.  A lane needs four consecutive elements of one head:
+//          it fetches the head's statistics and its 16 bytes of every record, forms the chunk weights
+//          exp(m_c - M) and the merged, normalised output -- the work of attn_merge_kernel -- and quantizes that.
+//          One row only (group 128).  Saves the merge launch between attention and the o projection.
+constexpr int kNorm = 1, kGlu = 2, kSums = 4, kGluIn = 8, kDump = 16, kAttnIn = 32;
+constexpr int kAttnRecChunks = 8;  // as in attn.hip
+struct AttnRecs {
+    const float* stats;  // [rows*H][kAttnRecChunks][2]
+    const float* outs;   // [rows*H][kAttnRecChunks][128]
+    int chunks;          // records per head that were written (<= kAttnRecChunks)
+};
 
+
+// The lane's four elements of the attention output from the chunk records of its head: weights exp(m_c - M)
+// over the chunks that hold rows (sum > 0), out = sum_c w_c o_c / sum_c w_c s_c (the arithmetic of
+// attn_merge_kernel).  st[c/2] holds (m, s) of chunks c and c+1; a record that was not asked for reads as zeros.
+__device__ __forceinline__ float4 merge_attn_records(const float4 (&ro)[kAttnRecChunks], const float4 (&st)[kAttnRecChunks / 2],
+                                                     int chunks) {
+    float m[kAttnRecChunks], sm[kAttnRecChunks];
+#pragma unroll
+    for (int c = 0; c < kAttnRecChunks / 2; c++) {  // (the statistics come in pairs: the second of the last pair may not exist)
+        m[2 * c] = st[c].x, sm[2 * c] = st[c].y;
+        m[2 * c + 1] = st[c].z, sm[2 * c + 1] = (2 * c + 1 < chunks) ? st[c].w : 0.0f;
+    }
+    float M = -3.402823466e+38f;
+#pragma unroll
+    for (int c = 0; c < kAttnRecChunks; c++) M = fmaxf(M, sm[c] == 0.0f ? -3.402823466e+38f : m[c]);
+    float den = 0.0f;
+    float4 num = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+    for (int c = 0; c < kAttnRecChunks; c++) {
+        const float w = (sm[c] == 0.0f) ? 0.0f : expf(m[c] - M);
+        den = fmaf(w, sm[c], den);
+        num.x = fmaf(w, ro[c].x, num.x);
+        num.y = fmaf(w, ro[c].y, num.y);
+        num.z = fmaf(w, ro[c].z, num.z);
+        num.w = fmaf(w, ro[c].w, num.w);
+    }
+    const float inv = 1.0f / den;
+    return make_float4(num.x * inv, num.y * inv, num.z * inv, num.w * inv);
+}
 
 // One activation row needs few registers; asking for eight waves per SIMD (two workgroups of 16 waves
 // per CU) keeps every variant at or below 64 registers, so that grids of 257..512 workgroups are
@@ -224,15 +265,17 @@ constexpr int kNorm = 1, kGlu = 2, kSums = 4, kGluIn = 8, kDump = 16;
 // 0-31 the first block's group, lanes 32-63 the second's; group 32: eight groups of 8 lanes) and uses the
 // weight buffers of the pass in place, without register copies.
 template <int G, int MT, int NW, int MODE>
-__global__ __launch_bounds__(NW * 64, (MT == 1 ? NW / 2 : 1)) void fc_gemv_fused_kernel(const uint8_t* __restrict__ weiq, const float* __restrict__ x,
+__global__ __launch_bounds__(NW * 64, (MT == 1 ? ((MODE & kAttnIn) ? NW / 4 : NW / 2) : 1)) void fc_gemv_fused_kernel(const uint8_t* __restrict__ weiq, const float* __restrict__ x,
                                                                  float* __restrict__ y, float* part, unsigned* counters,
                                                                  int Kg, int64_t K, int64_t N, int rows, int S,
                                                                  int steps_per_split, const float* __restrict__ residual,
                                                                  const float* __restrict__ norm_w, float eps,
                                                                  const float* __restrict__ sumsq_in, int sumsq_parts,
-                                                                 float* __restrict__ sumsq_out, int exchange, const DumpBufs dump) {
+                                                                 float* __restrict__ sumsq_out, int exchange, const DumpBufs dump,
+                                                                 const AttnRecs recs) {
     constexpr bool NORM = (MODE & kNorm) != 0, GLU = (MODE & kGlu) != 0, SUMS = (MODE & kSums) != 0;
-    constexpr bool GLUIN = (MODE & kGluIn) != 0, DUMP = (MODE & kDump) != 0;
+    constexpr bool GLUIN = (MODE & kGluIn) != 0, DUMP = (MODE & kDump) != 0, ATTN = (MODE & kAttnIn) != 0;
+    static_assert(!ATTN || (G == 128 && MT == 1 && !NORM && !GLU && !GLUIN), "chunk records: one row, group 128, plain input");
     static_assert(!(GLUIN && NORM), "the gate|up input has no rmsnorm");
     const int64_t xstride = GLUIN ? 2 * K : K;  // floats between activation rows
     constexpr int NWS = GLU ? NW / 2 : NW;  // waves per strip
@@ -303,6 +346,7 @@ __global__ __launch_bounds__(NW * 64, (MT == 1 ? NW / 2 : 1)) void fc_gemv_fused
     struct PairBuf {
         Step<G> s[SPP];
         float4 xv[MT], uv[GLUIN ? MT : 1], wv;
+        float4 ro[ATTN ? kAttnRecChunks : 1], rs[ATTN ? kAttnRecChunks / 2 : 1];  // chunk records: outputs, (max, sum) pairs
     };
     PairBuf P0;
     const int lane_step = lane / (64 / SPP);  // which step of the pass this lane's four activations belong to
@@ -312,6 +356,9 @@ __global__ __launch_bounds__(NW * 64, (MT == 1 ? NW / 2 : 1)) void fc_gemv_fused
     const buffer_rsrc strip_rs = make_rsrc(strip, (uint32_t)Kg * (uint32_t)block_bytes(G));
     const buffer_rsrc x_rs = make_rsrc(x, (uint32_t)rows * (uint32_t)xstride * 4u);
     const buffer_rsrc nw_rs = make_rsrc(NORM ? norm_w : x, NORM ? (uint32_t)K * 4u : 0u);
+    // chunk records: K / 128 heads; a pass of 256 k-values covers two heads (lanes 0-31 the first, 32-63 the second)
+    const buffer_rsrc ro_rs = make_rsrc(ATTN ? recs.outs : x, ATTN ? (uint32_t)(K / 128) * (uint32_t)(kAttnRecChunks * 128 * 4) : 0u);
+    const buffer_rsrc rt_rs = make_rsrc(ATTN ? recs.stats : x, ATTN ? (uint32_t)(K / 128) * (uint32_t)(kAttnRecChunks * 2 * 4) : 0u);
     if constexpr (NORM && !SUMS) {
         // the row for the statistic, four floats per thread and slice of NW*256: asked for unconditionally (a
         // slice beyond K at an offset that returns 0) and first, so that the statistic waits for these only
@@ -329,11 +376,20 @@ __global__ __launch_bounds__(NW * 64, (MT == 1 ? NW / 2 : 1)) void fc_gemv_fused
     do { /* branch-free: what is not wanted is asked for at an offset that returns 0 (see kNoLoad) */            \
         const bool ok_ = (WANT) && (TP) + lane_step < tr.t1 && (int64_t)(TP) * Step<G>::kK + lane * 4 < K;       \
         const uint32_t so_ = (uint32_t)(TP) * (uint32_t)(Step<G>::kK * 4);                                       \
+        if constexpr (ATTN) { /* head = (TP) + (lane >> 5): statistics first (the weights need them), then the outputs */ \
+            const uint32_t hs_ = (uint32_t)(TP) * (uint32_t)(kAttnRecChunks * 2 * 4);                            \
+            const uint32_t ho_ = (uint32_t)(TP) * (uint32_t)(kAttnRecChunks * 128 * 4);                          \
+            _Pragma("unroll") for (int c_ = 0; c_ < kAttnRecChunks / 2; c_++)                                    \
+                P.rs[ATTN ? c_ : 0] = buf_ldf4(rt_rs, (ok_ && 2 * c_ < recs.chunks) ? (uint32_t)(lane >> 5) * (uint32_t)(kAttnRecChunks * 8) + (uint32_t)c_ * 16u : kNoLoad, hs_); \
+            _Pragma("unroll") for (int c_ = 0; c_ < kAttnRecChunks; c_++)                                        \
+                P.ro[ATTN ? c_ : 0] = buf_ldf4(ro_rs, (ok_ && c_ < recs.chunks) ? (uint32_t)(lane >> 5) * (uint32_t)(kAttnRecChunks * 512) + (uint32_t)(lane & 31) * 16u + (uint32_t)c_ * 512u : kNoLoad, ho_); \
+        } else {                                                                                                 \
         _Pragma("unroll") for (int r = 0; r < MT; r++) {                                                         \
             const uint32_t ro_ = so_ + (uint32_t)r * (uint32_t)xstride * 4u;                                     \
             const uint32_t lo_ = (ok_ && r < rows) ? (uint32_t)lane * 16u : kNoLoad;                             \
             P.xv[r] = buf_ldf4(x_rs, lo_, ro_);                                                                  \
             if (GLUIN) P.uv[GLUIN ? r : 0] = buf_ldf4(x_rs, lo_, ro_ + (uint32_t)K * 4u);                        \
+        }                                                                                                        \
         }                                                                                                        \
         if (NORM) P.wv = buf_ldf4(nw_rs, ok_ ? (uint32_t)lane * 16u : kNoLoad, so_);                             \
         __builtin_amdgcn_sched_barrier(0); /* the compiler's scheduler must not move the weights ahead */       \
@@ -420,6 +476,7 @@ __global__ __launch_bounds__(NW * 64, (MT == 1 ? NW / 2 : 1)) void fc_gemv_fused
         const int tp_ = (TP);                                                                         \
         _Pragma("unroll") for (int r = 0; r < MT; r++) if (r < rows) {                                \
             float4 v = P.xv[r];                                                                       \
+            if constexpr (ATTN) v = merge_attn_records(P.ro, P.rs, recs.chunks);                      \
             if (NORM) {                                                                               \
                 v.x = v.x * rsn[r] * P.wv.x;                                                          \
                 v.y = v.y * rsn[r] * P.wv.y;                                                          \
@@ -595,6 +652,7 @@ struct FusedOps {
     const float* sumsq_in;  // per-part sums of squares of x (instead of reading the row for the rmsnorm)
     int sumsq_parts;
     float* sumsq_out;       // per-strip sums of squares of y [rows, Ng]
+    AttnRecs recs;          // stats != nullptr: the input is the chunk records of decode attention
 };
 
 template <int G, int MT, int NW>
@@ -611,11 +669,14 @@ static void launch_fused_t(const uint8_t* w, const float* x, float* y, float* pa
 #define LLMOPS_FUSED(MODE, GRID)                                                                                      \
     fc_gemv_fused_kernel<G, MT, NW, MODE><<<(unsigned)(GRID), NW * 64, 0, st>>>(                                      \
         w, x, y, part, counters, (int)Kg, K, N, rows, p.S, p.steps_per_split, o.residual, o.norm_w, o.eps, o.sumsq_in, \
-        o.sumsq_parts, o.sumsq_out, exchange, dump ? *dump : DumpBufs{nullptr, nullptr, nullptr, nullptr})
+        o.sumsq_parts, o.sumsq_out, exchange, dump ? *dump : DumpBufs{nullptr, nullptr, nullptr, nullptr}, o.recs)
     // (the kernel reads up to 256 handed-over partial sums per row; with more, the statistic is recomputed)
     const bool sums = o.norm_w != nullptr && o.sumsq_in != nullptr && o.sumsq_parts <= 256;
-    if (dump != nullptr) {  // plain fc_Q4A only (the launcher refuses the fused options)
-        LLMOPS_FUSED(kDump, Ng * p.S);
+    if (dump != nullptr) {  // plain fc_Q4A, or the chunk records of attention as input
+        if (o.recs.stats == nullptr) LLMOPS_FUSED(kDump, Ng * p.S);
+        else if constexpr (G == 128 && MT == 1) LLMOPS_FUSED(kDump | kAttnIn, Ng * p.S);
+    } else if (o.recs.stats != nullptr) {
+        if constexpr (G == 128 && MT == 1) LLMOPS_FUSED(kAttnIn, Ng * p.S);
     } else if (o.glu_in) {
         LLMOPS_FUSED(kGluIn, Ng * p.S);
     } else if (o.glu) {
@@ -633,11 +694,14 @@ static void launch_fused_t(const uint8_t* w, const float* x, float* y, float* pa
 // raw fp32 activations, quantized inside the kernel (+ optional rmsnorm / residual / gate-up epilogue)
 int launch_gemv_fused(const uint8_t* w, const float* x, float* y, float* part, unsigned* counters, int64_t rows, int64_t Ng,
                       int64_t Kg, int G, int64_t N, const float* residual, const float* norm_w, float eps, int glu,
-                      const float* sumsq_in, int sumsq_parts, float* sumsq_out, hipStream_t st, const DumpBufs* dump) {
+                      const float* sumsq_in, int sumsq_parts, float* sumsq_out, hipStream_t st, const DumpBufs* dump,
+                      const float* rec_stats, const float* rec_outs, int rec_chunks) {
     GemvPlan p = plan_gemv(rows, Ng, Kg, G, true);
     if (glu == 1) p.S = 1;
     if (dump != nullptr && (norm_w != nullptr || glu != 0)) return fail(LLMOPS_EINVAL, "the dump build runs the plain FC only");
-    const FusedOps o{residual, norm_w, eps, glu == 1, glu == 2, sumsq_in, sumsq_parts, sumsq_out};
+    if (rec_stats != nullptr && (rows != 1 || G != 128 || norm_w != nullptr || glu != 0))
+        return fail(LLMOPS_EINVAL, "chunk records as input: one row, group 128, no rmsnorm, no gate/up forms");
+    const FusedOps o{residual, norm_w, eps, glu == 1, glu == 2, sumsq_in, sumsq_parts, sumsq_out, AttnRecs{rec_stats, rec_outs, rec_chunks}};
 #define LLMOPS_CASE(GG, MT, NWW) launch_fused_t<GG, MT, NWW>(w, x, y, part, counters, Ng, Kg, N, (int)rows, p, o, st, dump)
     if (G == 128) {
         if (rows == 1) LLMOPS_CASE(128, 1, 16);

@@ -22,7 +22,7 @@ from . import _lib
 
 __all__ = [
     "offline_FC_quant_Q4A", "offline_FC_dequant_Q4A", "fc_Q4A", "fc_Q4A_noalloc", "fc_Q4A_decode", "interleave_gate_up", "FC_dynamic_quantize_x", "fc_Q4A_partials",
-    "attention_rope", "attention_rope2", "rope_embed", "softmax", "rmsnorm", "iadd", "imul", "itrans", "clone",
+    "attention_rope", "attention_rope2", "attention_rope2_records", "attention_records_supported", "AttentionRecords", "rope_embed", "softmax", "rmsnorm", "iadd", "imul", "itrans", "clone",
     "rmsnorm_out", "silu_mul", "empty", "ones", "embedding", "embedding_q8c_quant_w", "embedding_q8c", "tensor_pool", "set_default_group_k", "reserve_workspace",
     "group_k_of",
 ]
@@ -208,17 +208,39 @@ def interleave_gate_up(gate_packed, up_packed):
 
 
 def fc_Q4A_decode(input, weiq, N_out, norm=None, residual=None, glu=False, sumsq_in=None, want_sumsq=False,
-                  glu_in=False):
+                  glu_in=False, attn_records=None):
     """Extension: fc_Q4A with its neighbours of the decode step folded in (one launch for B*M <= 8).
 
     norm=(weight, eps): input is rmsnorm'ed first;  residual: added to the result;
     glu=True: ``weiq`` holds interleaved gate/up strips (``interleave_gate_up``) and the result is
     silu(gate)*up with N_out = F columns.  glu_in=True: ``input`` is a gate|up row [B, M, 2K] (what an FC
     over the gate and up weights stacked along N leaves behind) and the FC runs on silu(gate)*up.
+    attn_records=...: ``input`` is None and the FC's input is the output of decode attention still in chunk records
+    (``attention_rope2_records``), merged as it is loaded.
     want_sumsq=True returns ``(out, sumsq)`` where ``sumsq``
     [B*M, strips] holds the sum of squares of every 32 outputs; passed as ``sumsq_in`` to the FC that
     rmsnorms ``out`` it saves that FC the pass over the row.  With more than 8 rows the same
     arithmetic is composed from the separate ops."""
+    if attn_records is not None:
+        # input = the attention output still in chunk records (attention_rope2_records); merged on the way in
+        r = attn_records
+        _dev(weiq, torch.int8, 3, "wei_quantized")
+        _require(input is None and norm is None and not glu and not glu_in and sumsq_in is None, "attn_records: plain FC")
+        _require(r.B == 1 and group_k_of(weiq) == 128 and weiq.shape[1] == r.H, "attn_records: one row, group 128, K = H*128")
+        Ng, Kg, _ = weiq.shape
+        N_out = int(N_out)
+        if residual is not None:
+            _dev(residual, torch.float32, 3, "residual")
+            _require(tuple(residual.shape) == (1, 1, N_out), "residual.is({B, M, N})")
+        lib = _lib.load()
+        ws = _workspace(weiq.device, lib.llmops_fc_Q4A_workspace_bytes(1, Kg * 128, Ng, Kg, 128))
+        out = torch.empty((1, 1, N_out), dtype=torch.float32, device=weiq.device)
+        sumsq = torch.empty((1, Ng), dtype=torch.float32, device=weiq.device) if want_sumsq else None
+        _lib.check(lib.llmops_fc_Q4A_decode_attn(_ptr(r.stats), _ptr(r.outs), r.chunks, r.H, _ptr(weiq), Ng, Kg, N_out,
+                                                 _ptr(residual) if residual is not None else None,
+                                                 _ptr(sumsq) if sumsq is not None else None, _ptr(out), _ptr(ws), ws.numel(),
+                                                 _stream(weiq)))
+        return (out, sumsq) if want_sumsq else out
     _dev(input, torch.float32, 3, "input")
     _dev(weiq, torch.int8, 3, "wei_quantized")
     g = group_k_of(weiq)
@@ -329,6 +351,64 @@ def attention_rope2(q, k, v, inv_freq, kv_cache, kvc_slots, position_id, layer_i
 
 # the reference exports two kernels with one contract (ops/main.cpp:154-155)
 attention_rope = attention_rope2
+
+
+class AttentionRecords:
+    """What ``attention_rope2_records`` leaves behind: per head up to 8 split-KV chunk records (max, sum of exp;
+    exp-weighted V sum) that ``fc_Q4A_decode(..., attn_records=...)`` merges on its input side."""
+
+    def __init__(self, stats, outs, chunks, B, H):
+        self.stats, self.outs, self.chunks, self.B, self.H = stats, outs, chunks, B, H
+
+
+def attention_records_supported(kv_cache):
+    """True if decode attention over this cache can hand its chunk records to the o projection
+    (fp32 cache of up to 2048 rows, fp16 of up to 4096)."""
+    dt = 0 if kv_cache.dtype == torch.float32 else 1
+    return _lib.load().llmops_attention_records_chunks(kv_cache.shape[3], dt) > 0
+
+
+def attention_rope2_records(q, k, v, inv_freq, kv_cache, kvc_slots, position_id, layer_id, records=None):
+    """Extension: ``attention_rope2`` for ONE query token that does not overwrite q with the attention output but
+    returns the split-KV chunk records for the FC that consumes the output (``fc_Q4A_decode(attn_records=...)``
+    merges them as it loads its input: one launch fewer per decoder layer).  k is rotated in place and the cache
+    updated as usual; ``position_id`` is an int or an int32 device tensor [1].  ``records`` reuses an earlier
+    result's buffers."""
+    _dev(q, torch.float32, 3, "q")
+    _dev(k, torch.float32, 3, "k")
+    _dev(v, torch.float32, 3, "v")
+    _require(isinstance(kv_cache, torch.Tensor) and kv_cache.is_cuda and kv_cache.dim() == 5 and kv_cache.is_contiguous(),
+             "kv_cache.is<float>(5)")
+    _require(kv_cache.dtype in (torch.float32, torch.float16), "kv_cache.is<float>(5)")
+    _dev(kvc_slots, torch.int32, 1, "kvc_slots")
+    _dev(inv_freq, torch.float32, 1, "inv_freq")
+    B, qL, _ = q.shape
+    planes, Bc, H, maxlen, S = kv_cache.shape
+    _require(qL == 1 and Bc == B, "one query token; kv_cache.size(1) == B")
+    for t, n in ((q, "q"), (k, "k"), (v, "v")):
+        _require(tuple(t.shape) == (B, 1, H * S), f"{n}.is({{B, 1, H * S}})")
+    lib = _lib.load()
+    dt = 0 if kv_cache.dtype == torch.float32 else 1
+    chunks = lib.llmops_attention_records_chunks(maxlen, dt)
+    _require(chunks > 0, "cache short enough for chunk records (attention_records_supported)")
+    if records is None:
+        records = AttentionRecords(torch.empty((B * H, chunks, 2), dtype=torch.float32, device=q.device),
+                                   torch.empty((B * H, chunks, S), dtype=torch.float32, device=q.device), 0, B, H)
+    ws = _workspace(q.device, lib.llmops_attention_workspace_bytes(B, 1, H, S, maxlen), kind="attn")
+    on_dev = isinstance(position_id, torch.Tensor)
+    if on_dev:
+        _dev(position_id, torch.int32, 1, "position_id")
+        kv_plan = maxlen
+    else:
+        kv_plan = min(int(position_id) + 1, maxlen)
+    rows = 256 if maxlen <= 2048 else 512
+    records.chunks = -(-kv_plan // rows)
+    _lib.check(lib.llmops_attention_rope_decode_records(_ptr(q), _ptr(k), _ptr(v), B, H, S, _ptr(inv_freq), inv_freq.shape[0],
+                                                        _ptr(kv_cache), dt, planes, maxlen, _ptr(kvc_slots),
+                                                        0 if on_dev else int(position_id), _ptr(position_id) if on_dev else None,
+                                                        int(layer_id), _ptr(records.stats), _ptr(records.outs), _ptr(ws),
+                                                        ws.numel(), _stream(q)))
+    return records
 
 
 def softmax(x):

@@ -28,6 +28,8 @@ SIGNATURES = {
                                        c_ptr]),
     "llmops_fc_Q4A_decode": (c_int, [c_ptr, c_i64, c_i64, c_ptr, c_i64, c_i64, c_int, c_i64, c_ptr, c_f32, c_ptr, c_int, c_ptr,
                                      c_i64, c_ptr, c_ptr, c_ptr, c_size, c_ptr]),
+    "llmops_fc_Q4A_decode_attn": (c_int, [c_ptr, c_ptr, c_i64, c_i64, c_ptr, c_i64, c_i64, c_i64, c_ptr, c_ptr, c_ptr, c_ptr,
+                                          c_size, c_ptr]),
     "llmops_fc_Q4A_prequantized": (c_int, [c_ptr, c_ptr, c_ptr, c_i64, c_ptr, c_i64, c_i64, c_int, c_i64, c_ptr, c_ptr,
                                            c_size, c_ptr]),
     "llmops_fc_Q4A_partials": (c_int, [c_ptr, c_i64, c_ptr, c_i64, c_i64, c_int, c_ptr, c_int, c_ptr]),
@@ -37,6 +39,9 @@ SIGNATURES = {
                                       c_i64, c_i64, c_ptr, c_int, c_int, c_ptr, c_size, c_ptr]),
     "llmops_attention_rope_decode": (c_int, [c_ptr, c_ptr, c_ptr, c_i64, c_i64, c_i64, c_ptr, c_i64, c_ptr, c_int, c_i64, c_i64,
                                              c_ptr, c_ptr, c_int, c_ptr, c_size, c_ptr]),
+    "llmops_attention_records_chunks": (c_i64, [c_i64, c_int]),
+    "llmops_attention_rope_decode_records": (c_int, [c_ptr, c_ptr, c_ptr, c_i64, c_i64, c_i64, c_ptr, c_i64, c_ptr, c_int, c_i64,
+                                                     c_i64, c_ptr, c_int, c_ptr, c_int, c_ptr, c_ptr, c_ptr, c_size, c_ptr]),
     "llmops_softmax": (c_int, [c_ptr, c_i64, c_i64, c_ptr]),
     "llmops_mm_qk": (c_int, [c_ptr, c_i64, c_i64, c_i64, c_ptr, c_i64, c_ptr, c_i64, c_i64, c_i64, c_i64, c_i64, c_ptr]),
     "llmops_rmsnorm": (c_int, [c_ptr, c_i64, c_i64, c_ptr, c_f32, c_ptr]),
@@ -57,6 +62,8 @@ SIGNATURES = {
     "llmops_test_fc_set_row_routing": (None, [c_int, c_int]),
     "llmops_test_fc_rows_set_split": (None, [c_int]),
     "llmops_test_attn_set_decode_plan": (None, [c_int]),
+    "llmops_test_fc_decode_attn_dump": (c_int, [c_ptr, c_ptr, c_i64, c_i64, c_ptr, c_i64, c_i64, c_i64, c_ptr, c_ptr, c_ptr, c_ptr,
+                                                c_ptr, c_ptr, c_size, c_ptr]),
     "llmops_test_fc_decode_dump": (c_int, [c_ptr, c_i64, c_i64, c_ptr, c_i64, c_i64, c_int, c_i64, c_ptr, c_ptr, c_ptr, c_ptr,
                                            c_ptr, c_ptr, c_size, c_ptr]),
 }

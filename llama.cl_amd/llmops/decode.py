@@ -29,6 +29,7 @@ class LlamaDecoder:
         cfg.update(configs or {})
         self.configs = cfg
         self.plan = plan
+        self.merge_in_o_proj = True  # fused plan, one token: the o projection merges the attention chunks
         self.device = torch.device(device)
         gen = torch.Generator(device="cpu").manual_seed(seed)
         H, F, V = cfg["hidden_size"], cfg["intermediate_size"], cfg["vocab_size"]
@@ -85,6 +86,7 @@ class LlamaDecoder:
         self = cls.__new__(cls)
         self.device = torch.device(device)
         self.plan = plan
+        self.merge_in_o_proj = True
 
         def dev(a):
             return torch.from_numpy(a).to(self.device)
@@ -191,8 +193,15 @@ class LlamaDecoder:
         q, k, v = qkv[..., :H], qkv[..., H:2 * H], qkv[..., 2 * H:]
         if not q.is_contiguous():  # more than one token: the op needs dense [B,qL,H*S] tensors
             q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
-        llmops.attention_rope2(q, k, v, self.inv_freq, kv_cache, kv_cache_slots, position_id, i)
-        attn_output, ss = llmops.fc_Q4A_decode(q, ops["o_proj"].weight, H, residual=hidden_states, want_sumsq=True)
+        if qkv.shape[0] * qkv.shape[1] == 1 and self.merge_in_o_proj and llmops.attention_records_supported(kv_cache) \
+                and llmops.group_k_of(ops["o_proj"].weight) == 128 and self.inv_freq.shape[0] % 4 == 0:
+            # one token: attention leaves its split-KV chunk records and the o projection merges them on its way in
+            recs = llmops.attention_rope2_records(q, k, v, self.inv_freq, kv_cache, kv_cache_slots, position_id, i)
+            attn_output, ss = llmops.fc_Q4A_decode(None, ops["o_proj"].weight, H, residual=hidden_states, want_sumsq=True,
+                                                   attn_records=recs)
+        else:
+            llmops.attention_rope2(q, k, v, self.inv_freq, kv_cache, kv_cache_slots, position_id, i)
+            attn_output, ss = llmops.fc_Q4A_decode(q, ops["o_proj"].weight, H, residual=hidden_states, want_sumsq=True)
         if self.stacked_gate_up:
             gate_up = llmops.fc_Q4A_decode(attn_output, ops["gate_up_proj"].weight, 2 * F, norm=(n2.weight, n2.eps),
                                            sumsq_in=ss)

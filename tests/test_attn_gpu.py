@@ -375,3 +375,73 @@ def test_decode_attention_every_chunking_and_device_position(ops, orc, cache_dty
                         assert np.abs(host(tc) - cache_ref).max() <= 1e-5
     finally:
         lib.llmops_test_attn_set_decode_plan(0)
+
+
+@pytest.mark.parametrize("cache_dtype,maxlen", [(torch.float32, 2048), (torch.float32, 700), (torch.float16, 2048), (torch.float16, 4096)])
+def test_attention_records_merged_by_the_o_projection(ops, orc, cache_dtype, maxlen):
+    """Decode attention that hands its split-KV chunk records to the o projection (the merge runs on the FC's input
+    side): attention_rope2_records + fc_Q4A_decode(attn_records=...) against attention_rope2 + fc_Q4A_decode on
+    the same inputs.  Three layers of checks, because two evaluations of the attention output that differ in the
+    last bit may quantize an activation on a rounding boundary to neighbouring codes:
+    (1) the records, merged on the host in fp64, equal the unfused attention output to 1e-5;
+    (2) what the FC kernel itself merged and quantized (its dump build): scales equal to rounding, codes equal but
+        for a handful of +-1 boundary cases, and its int32 sums exactly the integer product of ITS codes;
+    (3) the outputs agree to 1e-2 and, at selected lengths, with the oracle's attention + FC to the same bar."""
+    import ctypes
+    from llmops import _lib
+    lib = _lib.load()
+    rng = np.random.default_rng(31)
+    B, H, S, G = 1, 32, 128, 128
+    N = K = H * S
+    inv_freq = (1.0 / (10000.0 ** (np.arange(0, S, 2, dtype=np.float32) / np.float32(S)))).astype(np.float32)
+    w = (rng.standard_normal((N, K)) * 0.02).astype(np.float32)
+    wq = ops.offline_FC_quant_Q4A(dev(w), G)
+    pw = host(wq)
+    Ng, Kg, _ = pw.shape
+    cache0 = rng.standard_normal((2, B, H, maxlen, S)).astype(np.float32)
+    if cache_dtype == torch.float16:
+        cache0 = cache0.astype(np.float16).astype(np.float32)
+    res = rng.standard_normal((1, 1, N)).astype(np.float32)
+    kvs = [k_ for k_ in (1, 100, 256, 257, 512, 700, 1024, 2047, 2048, 3000, 4096) if k_ <= maxlen]
+    P = lambda t: ctypes.c_void_p(t.data_ptr())
+    for kv in kvs:
+        q, k, v = (rng.standard_normal((B, 1, H * S)).astype(np.float32) for _ in range(3))
+        pos, slots = kv - 1, np.array([kv - 1], np.int32)
+        tq, tk, tc = dev(q), dev(k), dev(cache0).to(cache_dtype)
+        ops.attention_rope2(tq, tk, dev(v), dev(inv_freq), tc, dev(slots), pos, 0)       # unfused
+        att = host(tq)
+        want_y, want_ss = ops.fc_Q4A_decode(tq, wq, N, residual=dev(res), want_sumsq=True)
+        for dev_pos in (False, True):
+            fq, fk, fc = dev(q), dev(k), dev(cache0).to(cache_dtype)
+            p = torch.tensor([pos], dtype=torch.int32, device="cuda") if dev_pos else pos
+            recs = ops.attention_rope2_records(fq, fk, dev(v), dev(inv_freq), fc, dev(slots), p, 0)
+            assert torch.equal(fk, tk) and torch.equal(fc, tc)              # k rotated, cache updated alike
+            assert np.array_equal(host(fq), q)                              # q is left as it came in
+            # (1) the records themselves (every one of recs.chunks was written; empty ones have sum 0)
+            st, ou = host(recs.stats)[:, :recs.chunks].astype(np.float64), host(recs.outs)[:, :recs.chunks].astype(np.float64)
+            m, sm = st[..., 0], st[..., 1]
+            wgt = np.where(sm > 0, np.exp(m - np.where(sm > 0, m, -np.inf).max(1, keepdims=True)), 0.0)
+            merged = ((wgt[..., None] * ou).sum(1) / (wgt * sm).sum(1, keepdims=True)).reshape(1, K)
+            assert max_rel_err(merged, att.reshape(1, K)) <= (1e-5 if cache_dtype == torch.float32 else 3e-3), (kv, dev_pos)
+            # (2) the FC kernel's own merge + quantization + integer core
+            y = torch.empty((1, N), dtype=torch.float32, device="cuda")
+            xq = torch.empty((1, K), dtype=torch.int8, device="cuda")
+            xd, gs = torch.empty((1, Kg), dtype=torch.float32, device="cuda"), torch.empty((1, Kg), dtype=torch.float32, device="cuda")
+            acc = torch.empty((1, Ng * 32, Kg), dtype=torch.int32, device="cuda")
+            ws = ops._workspace(y.device, lib.llmops_fc_Q4A_workspace_bytes(1, K, Ng, Kg, G))
+            _lib.check(lib.llmops_test_fc_decode_attn_dump(P(recs.stats), P(recs.outs), recs.chunks, H, P(wq), Ng, Kg, N, P(y), P(xq),
+                                                           P(xd), P(gs), P(acc), P(ws), ws.numel(),
+                                                           ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)))
+            oq, od, og = orc.quant_x(merged.astype(np.float32), G)
+            assert np.abs(host(xd) / od - 1.0).max() <= 1e-6
+            diff = host(xq).astype(np.int32) - oq.astype(np.int32)
+            assert np.abs(diff).max() <= 1 and np.count_nonzero(diff) <= 8, (kv, np.count_nonzero(diff))
+            assert np.array_equal(host(acc), orc.fc_partials(host(xq), pw))
+            # (3) outputs
+            yf, ss = ops.fc_Q4A_decode(None, wq, N, residual=dev(res), want_sumsq=True, attn_records=recs)
+            assert np.array_equal(host(yf)[0], host(y) + res[0])            # production build == dump build (+ residual)
+            assert max_rel_err(host(yf), host(want_y)) <= 1e-2, (kv, dev_pos)
+            assert max_rel_err(host(ss), host(want_ss)) <= 2e-2
+        if cache_dtype == torch.float32 and kv in (257, 2048):              # and the oracle's two ops
+            oatt, _, _ = orc.attention(q, k, v, inv_freq, cache0, slots, pos, 0)
+            assert max_rel_err(host(yf), orc.fc(oatt, pw, N) + res) <= 1e-2
