@@ -31,11 +31,35 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 # the per-shape figures is profiles/fc_gemv_fused_kernel__hbm_traffic_pmc.md.  Counters cannot be read from inside
 # this process, so the figure is the recorded one and only holds for the fused plan at group 128, M=1.
 MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 27188727
+MEASURED_TRAFFIC_PROFILE = "profiles/fc_gemv_fused_kernel__hbm_traffic_pmc.md"
+# sha256 (first 16 hex digits) of the kernel's sources (csrc/fc_gemv.hip + csrc/gemv_device.h) when the counters were
+# read: the bench line says whether the sources have changed since, i.e. whether the recorded figure is stale
+MEASURED_TRAFFIC_KERNEL_SHA16 = "unrecorded"
 G = 128
 LAYERS = 32
 # (name, N, K) of one layer's FCs, in the order the model calls them (chatllama/main.py:344-375)
 LAYER_FCS = [("q", 4096, 4096), ("k", 4096, 4096), ("v", 4096, 4096), ("o", 4096, 4096),
              ("gate", 11008, 4096), ("up", 11008, 4096), ("down", 4096, 11008)]
+
+
+def kernel_source_sha16():
+    import hashlib
+    h = hashlib.sha256()
+    for f in ("fc_gemv.hip", "gemv_device.h"):
+        with open(os.path.join(ROOT, "llama.cl_amd", "csrc", f), "rb") as fh:
+            h.update(fh.read())
+    return h.hexdigest()[:16]
+
+
+def host_cpu_model():
+    try:
+        with open("/proc/cpuinfo") as fh:
+            for line in fh:
+                if line.lower().startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
 
 
 def blk_bytes(g):
@@ -150,7 +174,10 @@ def main():
     achieved = step_bytes / (main_r["event_ms_per_step"] * 1e-3) / 1e9
     roof = {"bound": "hbm", "kernel": "fc_gemv_fused_kernel<128,1,16,0>", "achieved": round(achieved, 1),
             "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH,
-            "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a 1 GiB copy kernel (recorded run)",
+            "traffic_source": {"how": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a 1 GiB copy kernel (recorded run)",
+                               "profile": MEASURED_TRAFFIC_PROFILE, "kernel_sources_sha16_when_measured": MEASURED_TRAFFIC_KERNEL_SHA16,
+                               "kernel_sources_sha16_now": kernel_source_sha16(),
+                               "stale": kernel_source_sha16() != MEASURED_TRAFFIC_KERNEL_SHA16},
             "avg_launch_us": round(avg_us, 3), "launches_per_step": main_r["launches"],
             "bytes_per_launch_avg": int(step_bytes / main_r["launches"]), "per_shape": per_shape,
             "dispatch_floor_us": round(floor_us, 3),
@@ -520,8 +547,25 @@ def cpu_baseline(budget_s=12.0):
         done += 1
     dt = time.perf_counter() - t0
     layer_bytes = sum(fc_bytes(N, K) for _, N, K in LAYER_FCS)
-    res = {"value": round(done * layer_bytes / dt / 1e9, 2), "unit": "GB/s", "cores": eng.max_threads(), "kind": kind,
-           "isa": eng.isa,
+    all_cores = eng.max_threads()
+    # the same sample on 8 threads, the thread count of the reference's published CPU figures (README.md:54-57,
+    # doc/fc-perf.md:22-26), for about a third of the budget
+    eight = None
+    if all_cores > 8:
+        eng.set_threads(8)
+        for (name, N, K), wq in zip(LAYER_FCS, layers[0]):
+            eng.fc(xs[K], wq, N)
+        n8, t8 = 0, time.perf_counter()
+        while time.perf_counter() - t8 < budget_s / 3:
+            for (name, N, K), wq in zip(LAYER_FCS, layers[n8 % copies]):
+                eng.fc(xs[K], wq, N)
+            n8 += 1
+        d8 = time.perf_counter() - t8
+        eight = {"value": round(n8 * sum(fc_bytes(N, K) for _, N, K in LAYER_FCS) / d8 / 1e9, 2), "unit": "GB/s", "cores": 8,
+                 "sample": f"{n8} passes, {d8:.1f} s"}
+        eng.set_threads(0)
+    res = {"value": round(done * layer_bytes / dt / 1e9, 2), "unit": "GB/s", "cores": all_cores, "kind": kind,
+           "isa": eng.isa, "cpu_model": host_cpu_model(), "eight_threads": eight,
            "sample": f"{done} passes over one layer's 7 decode FCs (Q4_1 g128, M=1), cycling {copies} distinct "
                      f"layer weight sets, {dt:.1f} s", "ms_per_layer": round(dt / done * 1e3, 3),
            "ms_per_32_layers": round(dt / done * 32e3, 2)}

@@ -96,8 +96,9 @@ size_t llmops_fc_Q4A_workspace_bytes(int64_t rows, int64_t K, int64_t Ng, int64_
  *   y[r,n] = sum_kb  fp32(d[n,kb])*dx[r,kb] * float(acc[r,n,kb]) + fp32(m[n,kb])*gsum[r,kb]
  * with acc the exact int32 dot product of 4-bit codes and int8 activation codes.  One or two rows (at
  * group 32 up to 8; at group 128 three rows of tensors of up to 256 strips as well) run the
- * HBM-streaming dot4 kernel, larger row counts the int8 MFMA kernels.  Requires K == Kg*G
- * (every shape the reference is used with); N may be any value in (Ng*32-32, Ng*32]. */
+ * HBM-streaming dot4 kernel, larger row counts the int8 MFMA kernels.  K may be any value in (Kg*G-G, Kg*G]: a short
+ * last k-group is zero padded as the reference does (ops/op_fc.hpp:259-261; a separate quantization launch then,
+ * not the tuned path: no shape the reference is used with has such a K); N any value in (Ng*32-32, Ng*32]. */
 int llmops_fc_Q4A(const float* x, int64_t rows, int64_t K, const int8_t* weiq, int64_t Ng, int64_t Kg,
                   int group_k, int64_t N, float* y, void* workspace, size_t workspace_bytes,
                   llmops_stream_t stream);
@@ -243,6 +244,13 @@ int llmops_rmsnorm_out(const float* x, float* out, int64_t rows, int64_t hidden,
 /* itrans(gate,"silu") + imul(up,gate) (chatllama/main.py:363-367) on a row that holds gate and up
  * side by side: out[r,i] = silu(gate_up[r,i]) * gate_up[r,F+i] */
 int llmops_silu_mul(const float* gate_up, float* out, int64_t rows, int64_t F, llmops_stream_t stream);
+/* the same two ops on a row whose strips of 32 columns alternate gate, up, gate, up ... (what an FC over interleaved
+ * gate/up strips leaves): out[r,i] = silu(gate_up[r,(i/32)*64 + i%32]) * gate_up[r,(i/32)*64 + 32 + i%32]; F % 32 == 0 */
+int llmops_silu_mul_interleaved(const float* gate_up, float* out, int64_t rows, int64_t F, llmops_stream_t stream);
+/* sum of squares of every strip of 32 columns of y fp32 [rows,N] -> out fp32 [rows, ceil(N/32)]: the partial sums of
+ * the rmsnorm statistic (ops/op_misc.hpp:158-166) in the form llmops_fc_Q4A_decode's sumsq_out / sumsq_in exchange,
+ * for more rows than that entry takes */
+int llmops_strip_sumsq(const float* y, int64_t rows, int64_t N, float* out, llmops_stream_t stream);
 /* iadd / imul (ops/op_misc.hpp:55-107): a (+|*)= b; b is [rows,inner] or, if b_is_row, [inner] */
 int llmops_iadd(float* a, const float* b, int64_t rows, int64_t inner, int b_is_row, llmops_stream_t stream);
 int llmops_imul(float* a, const float* b, int64_t rows, int64_t inner, int b_is_row, llmops_stream_t stream);

@@ -76,11 +76,12 @@ static int fc_impl(const float* x, int64_t rows, int64_t K, const int8_t* weiq, 
     LLMOPS_REQUIRE(valid_group(group_k));
     LLMOPS_REQUIRE(x != nullptr && weiq != nullptr && y != nullptr && workspace != nullptr);
     LLMOPS_REQUIRE(rows > 0 && K > 0 && Ng > 0 && Kg > 0);
-    LLMOPS_REQUIRE(K == Kg * group_k);  // the reference reads past K otherwise (ops/op_fc.hpp:184)
+    LLMOPS_REQUIRE(K > (Kg - 1) * group_k && K <= Kg * group_k);  // a short last k-group is zero padded (ops/op_fc.hpp:259-261)
     LLMOPS_REQUIRE(N > (Ng - 1) * kGroupN && N <= Ng * kGroupN);
     LLMOPS_REQUIRE(Ng <= kTicketBytes / 4);
     LLMOPS_REQUIRE(Ng * 64 < ((int64_t)1 << 31));
-    LLMOPS_REQUIRE(aligned(weiq, 16) && aligned(workspace, 256) && aligned(x, 8));
+    const bool k_tail = K != Kg * group_k;
+    LLMOPS_REQUIRE(aligned(weiq, 16) && aligned(workspace, 256) && aligned(x, k_tail ? 4 : 8));
     const FcWorkspace lay = fc_layout(rows, Ng, Kg, group_k);
     if (workspace_bytes < lay.total)
         return fail(LLMOPS_EWORKSPACE, "fc_Q4A needs %zu workspace bytes, got %zu", lay.total, workspace_bytes);
@@ -101,6 +102,17 @@ static int fc_impl(const float* x, int64_t rows, int64_t K, const int8_t* weiq, 
     //   8192x4096 (256 strips):    2 rows  6.7 /  8.9, 3 rows  8.1 /  8.6, 4 rows  8.8 /  8.6, 8 rows 14.5 /  8.9
     //   12288x4096 (384 strips):   2 rows  9.3 / 12.0, 3 rows 13.4 / 11.6, 4 rows 15.6 / 11.7, 8 rows 22.4 / 12.2
     //   22016x4096 (688 strips):   2 rows 12.8 / 16.1, 3 rows 20.1 / 16.0, 4 rows 22.2 / 15.3, 8 rows 31.0 / 16.1
+    if (k_tail) {
+        // K is not a whole number of k-groups (no shape the reference is used with): the general quantization kernel
+        // pads the last group's codes with zeros, as FC_dynamic_quantize_x does, and the product runs on the codes
+        float2* xst_t = reinterpret_cast<float2*>(ws + lay.off_xst);
+        int rc_t = launch_quant_x(x, rows, K, group_k, xq, xd, gs, xst_t, false, st);
+        if (rc_t) return rc_t;
+        if (rows > kMaxGemvRows) return launch_gemm(w, xq, xd, gs, xst_t, y, part, counters, rows, Ng, Kg, group_k, N, residual, st);
+        rc_t = launch_gemv(w, xq, xd, gs, y, part, counters, rows, Ng, Kg, group_k, N, st);
+        if (rc_t == 0 && residual != nullptr) rc_t = launch_add(y, residual, rows * N, st);
+        return rc_t;
+    }
     const bool rows_kernel = group_k == 128 && Ng >= 64 && gemm_rows_kernel_enabled();
     const bool gemv = rows <= kMaxGemvRows && !(rows_kernel && rows >= (Ng > 256 ? g_rows_from_large : g_rows_from_small));
     if (gemv)

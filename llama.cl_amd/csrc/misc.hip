@@ -71,6 +71,32 @@ __global__ void silu_mul_kernel(const float* __restrict__ gu, float* __restrict_
     out[i] = silu_times(g, u);
 }
 
+// the same for a row whose strips of 32 columns alternate gate, up, gate, up ... (the layout a gate|up FC over
+// interleaved strips leaves behind): out[r, i] = silu(gu[r, (i/32)*64 + i%32]) * gu[r, (i/32)*64 + 32 + i%32]
+__global__ void silu_mul_interleaved_kernel(const float* __restrict__ gu, float* __restrict__ out, int64_t rows, int64_t F) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= rows * F) return;
+    const int64_t r = i / F, c = i % F;
+    const int64_t base = r * 2 * F + (c >> 5) * 64 + (c & 31);
+    out[i] = silu_times(gu[base], gu[base + 32]);
+}
+
+// sum of squares of every strip of 32 columns of y [rows, N] (columns beyond N count as 0): out [rows, Ng].
+// One half-wave per (row, strip).  What the decode FC's epilogue hands to the next rmsnorm, for many rows.
+__global__ __launch_bounds__(256) void strip_sumsq_kernel(const float* __restrict__ y, int64_t rows, int64_t N, int64_t Ng,
+                                                           float* __restrict__ out) {
+    const int64_t item = ((int64_t)blockIdx.x * 256 + threadIdx.x) >> 5;
+    const int c = threadIdx.x & 31;
+    const bool live = item < rows * Ng;
+    const int64_t r = live ? item / Ng : 0, nb = live ? item % Ng : 0;
+    const int64_t n = nb * 32 + c;
+    const float v = (live && n < N) ? y[r * N + n] : 0.0f;
+    float sq = v * v;
+#pragma unroll
+    for (int o = 16; o > 0; o >>= 1) sq += __shfl_xor(sq, o, 64);
+    if (live && c == 0) out[r * Ng + nb] = sq;
+}
+
 template <bool MUL>
 __global__ void ibinary_kernel(float* __restrict__ a, const float* __restrict__ b, int64_t total, int64_t inner,
                                int b_is_row) {
@@ -179,6 +205,24 @@ extern "C" int llmops_silu_mul(const float* gate_up, float* out, int64_t rows, i
     const int64_t total = rows * F;
     LLMOPS_REQUIRE((total + 255) / 256 < ((int64_t)1 << 31));
     silu_mul_kernel<<<(unsigned)((total + 255) / 256), 256, 0, as_stream(stream)>>>(gate_up, out, rows, F);
+    LLMOPS_LAUNCH_CHECK();
+    return LLMOPS_OK;
+}
+
+extern "C" int llmops_silu_mul_interleaved(const float* gate_up, float* out, int64_t rows, int64_t F, llmops_stream_t stream) {
+    LLMOPS_REQUIRE(gate_up != nullptr && out != nullptr && rows > 0 && F > 0 && (F % 32) == 0);
+    const int64_t total = rows * F;
+    LLMOPS_REQUIRE((total + 255) / 256 < ((int64_t)1 << 31));
+    silu_mul_interleaved_kernel<<<(unsigned)((total + 255) / 256), 256, 0, as_stream(stream)>>>(gate_up, out, rows, F);
+    LLMOPS_LAUNCH_CHECK();
+    return LLMOPS_OK;
+}
+
+extern "C" int llmops_strip_sumsq(const float* y, int64_t rows, int64_t N, float* out, llmops_stream_t stream) {
+    LLMOPS_REQUIRE(y != nullptr && out != nullptr && rows > 0 && N > 0);
+    const int64_t Ng = (N + 31) / 32, threads = rows * Ng * 32;
+    LLMOPS_REQUIRE((threads + 255) / 256 < ((int64_t)1 << 31));
+    strip_sumsq_kernel<<<(unsigned)((threads + 255) / 256), 256, 0, as_stream(stream)>>>(y, rows, N, Ng, out);
     LLMOPS_LAUNCH_CHECK();
     return LLMOPS_OK;
 }

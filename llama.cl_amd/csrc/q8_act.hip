@@ -19,6 +19,9 @@ __device__ __forceinline__ int q8_code(float v, float id) {
     if (t != t) return -128;  // cvtps2dq(NaN) = INT_MIN, which the saturating packs turn into -128
     return (int)fminf(127.0f, fmaxf(-128.0f, rintf(t)));
 }
+// the last len % 8 values of a short group go through the reference's scalar tail, which rounds half away from
+// zero (std::round, ops/utils.hpp:217-219) instead of half to even
+__device__ __forceinline__ int q8_code_tail(float v, float id) { return (int)(int8_t)roundf(v * id); }
 
 // EXACT_SUM: raw group sum accumulated left to right (bit-equal to the reference); otherwise a
 // tree sum, which is what the prefill FC uses (the sum only feeds its fp32 output).
@@ -37,6 +40,7 @@ __global__ __launch_bounds__(256) void quant_x_kernel(const float* __restrict__ 
     const int64_t left = K - kb * G;
     const int len = (int)(left < G ? left : G);
 
+    const int vec = len & ~7;  // values the reference quantizes eight at a time; the rest take its scalar tail
     float v[E];
 #pragma unroll
     for (int j = 0; j < E; j++) {
@@ -53,13 +57,13 @@ __global__ __launch_bounds__(256) void quant_x_kernel(const float* __restrict__ 
     if (lane < LANES) {
         int8_t* q = xq + (r * Kg + kb) * G + lane * E;
         if (E == 2) {
-            const uint32_t c0 = (uint32_t)q8_code(v[0], id) & 0xFFu;
-            const uint32_t c1 = (uint32_t)q8_code(v[E - 1], id) & 0xFFu;
             const int e = lane * E;
+            const uint32_t c0 = (uint32_t)(e < vec ? q8_code(v[0], id) : q8_code_tail(v[0], id)) & 0xFFu;
+            const uint32_t c1 = (uint32_t)(e + 1 < vec ? q8_code(v[E - 1], id) : q8_code_tail(v[E - 1], id)) & 0xFFu;
             // padding beyond len is zero (ops/op_fc.hpp:259-261)
             *reinterpret_cast<uint16_t*>(q) = (uint16_t)((e < len ? c0 : 0u) | ((e + 1 < len ? c1 : 0u) << 8));
         } else {
-            q[0] = (lane < len) ? (int8_t)q8_code(v[0], id) : (int8_t)0;
+            q[0] = (lane < len) ? (int8_t)(lane < vec ? q8_code(v[0], id) : q8_code_tail(v[0], id)) : (int8_t)0;
         }
     }
 
@@ -169,7 +173,7 @@ extern "C" int llmops_FC_dynamic_quantize_x(const float* x, int64_t rows, int64_
                                             float* xd, float* gsum, llmops_stream_t stream) {
     LLMOPS_REQUIRE(valid_group(group_k));
     LLMOPS_REQUIRE(x != nullptr && xq != nullptr && xd != nullptr && gsum != nullptr);
-    LLMOPS_REQUIRE(rows > 0 && K > 0 && (K % 8) == 0);
+    LLMOPS_REQUIRE(rows > 0 && K > 0);
     LLMOPS_REQUIRE(aligned(xq, 2));
     const int64_t Kg = (K + group_k - 1) / group_k;
     LLMOPS_REQUIRE(rows * Kg < ((int64_t)1 << 33));

@@ -265,15 +265,18 @@ def fc_Q4A_decode(input, weiq, N_out, norm=None, residual=None, glu=False, sumsq
         x = input if norm is None else rmsnorm_out(input, norm[0], norm[1])
         if glu_in:
             x = silu_mul(input)
+        lib = _lib.load()
         if glu:
             _require(N_out % 32 == 0, "F % 32 == 0")
-            y = fc_Q4A(x, weiq, 2 * N_out).view(B, M, N_out // 32, 2, 32)
-            gu = torch.cat((y[..., 0, :].reshape(B, M, N_out), y[..., 1, :].reshape(B, M, N_out)), dim=-1)
-            return silu_mul(gu)
+            y = fc_Q4A(x, weiq, 2 * N_out)  # strips alternate gate, up
+            act = torch.empty((B, M, N_out), dtype=torch.float32, device=input.device)
+            _lib.check(lib.llmops_silu_mul_interleaved(_ptr(y), _ptr(act), rows, N_out, _stream(y)))
+            return act
         out = fc_Q4A(x, weiq, N_out, residual=residual)
         if want_sumsq:
-            pad = torch.nn.functional.pad(out.reshape(rows, N_out), (0, Ng * 32 - N_out))
-            return out, pad.view(rows, Ng, 32).square().sum(-1)
+            sumsq = torch.empty((rows, Ng), dtype=torch.float32, device=input.device)
+            _lib.check(lib.llmops_strip_sumsq(_ptr(out), rows, N_out, _ptr(sumsq), _stream(out)))
+            return out, sumsq
         return out
     lib = _lib.load()
     ws = _workspace(input.device, lib.llmops_fc_Q4A_workspace_bytes(rows, K, Ng, Kg, g))

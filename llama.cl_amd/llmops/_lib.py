@@ -47,6 +47,8 @@ SIGNATURES = {
     "llmops_rmsnorm": (c_int, [c_ptr, c_i64, c_i64, c_ptr, c_f32, c_ptr]),
     "llmops_rmsnorm_out": (c_int, [c_ptr, c_ptr, c_i64, c_i64, c_ptr, c_f32, c_ptr]),
     "llmops_silu_mul": (c_int, [c_ptr, c_ptr, c_i64, c_i64, c_ptr]),
+    "llmops_silu_mul_interleaved": (c_int, [c_ptr, c_ptr, c_i64, c_i64, c_ptr]),
+    "llmops_strip_sumsq": (c_int, [c_ptr, c_i64, c_i64, c_ptr, c_ptr]),
     "llmops_iadd": (c_int, [c_ptr, c_ptr, c_i64, c_i64, c_int, c_ptr]),
     "llmops_imul": (c_int, [c_ptr, c_ptr, c_i64, c_i64, c_int, c_ptr]),
     "llmops_itrans_silu": (c_int, [c_ptr, c_i64, c_ptr]),

@@ -76,6 +76,10 @@ class Oracle:
     def max_threads(self):
         return self.lib.orc_max_threads()
 
+    def set_threads(self, n):
+        """OpenMP threads of the calls that follow (0 = one per processor)"""
+        self.lib.orc_set_threads(int(n))
+
     def fp32_to_fp16_bits(self, a):
         a = _c32(a).ravel()
         return np.array([self.lib.orc_fp32_to_fp16(float(v)) for v in a], dtype=np.uint16)
@@ -268,6 +272,10 @@ class Reference:
 
     def max_threads(self):
         return self.lib.ref_max_threads()
+
+    def set_threads(self, n):
+        """OpenMP threads of the calls that follow (0 = one per processor)"""
+        self.lib.ref_set_threads(int(n))
 
     def _chk(self, rc):
         if rc != 0:

@@ -500,3 +500,4 @@ void orc_embedding_q8c(float* out, const int64_t* ids, int64_t n, const int8_t* 
 }
 
 int orc_max_threads(void) { return omp_get_max_threads(); }
+void orc_set_threads(int n) { omp_set_num_threads(n > 0 ? n : omp_get_num_procs()); }

@@ -68,6 +68,7 @@ int ref_has_avxvnni() {
 #endif
 }
 int ref_max_threads() { return omp_get_max_threads(); }
+void ref_set_threads(int n) { omp_set_num_threads(n > 0 ? n : omp_get_num_procs()); }
 
 // wei fp32 [N,K] -> out int8 [ceil(N/32), ceil(K/G), sizeof(q4_block)]
 int ref_offline_FC_quant_Q4A(const float* wei, int64_t N, int64_t K, int8_t* out) {

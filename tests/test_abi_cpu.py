@@ -56,9 +56,9 @@ def test_argument_validation_without_device(lib):
     i64, vp = ctypes.c_int64, ctypes.c_void_p
     rc = lib.llmops_offline_FC_quant_Q4A(vp(16), i64(32), i64(64), i64(64), 64, vp(16), vp(0))
     assert rc == 1 and b"valid_group" in lib.llmops_last_error()
-    rc = lib.llmops_fc_Q4A(vp(256), i64(1), i64(100), vp(256), i64(1), i64(1), 128, i64(32), vp(256), vp(256),
-                           ctypes.c_size_t(1 << 20), vp(0))
-    assert rc == 1 and b"K == Kg * group_k" in lib.llmops_last_error()
+    rc = lib.llmops_fc_Q4A(vp(256), i64(1), i64(300), vp(256), i64(1), i64(1), 128, i64(32), vp(256), vp(256),
+                           ctypes.c_size_t(1 << 20), vp(0))      # 300 activations cannot belong to one k-group of 128
+    assert rc == 1 and b"K <= Kg * group_k" in lib.llmops_last_error()
     lib.llmops_fc_Q4A_workspace_bytes.restype = ctypes.c_size_t
     need = lib.llmops_fc_Q4A_workspace_bytes(i64(1), i64(4096), i64(128), i64(32), 128)
     assert need > 65536

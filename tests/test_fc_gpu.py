@@ -537,3 +537,40 @@ def test_gemm_split_k_reduced_in_kernel_equals_second_launch(ops, M, N, K):
     y1 = ops.fc_Q4A(x[:, :1].contiguous(), wq, N)
     assert torch.equal(y1, ops.fc_Q4A(x[:, :1].contiguous(), wq, N))
     assert max_rel_err(host(y1)[0, 0], host(want)[0, 0]) <= TOL
+
+
+# ---- K that is not a whole number of k-groups (nor of eights) ---------------------------------------------------
+@pytest.mark.parametrize("G", [32, 128])
+@pytest.mark.parametrize("rows,K", [(1, 5), (3, 100), (2, 333), (17, 1001), (5, 4100)])
+def test_quant_x_short_last_group(ops, orc, G, rows, K):
+    """codes (zero padded; the last K % 8 values rounded half away from zero like the reference's scalar tail),
+    scales and left-to-right sums bit for bit"""
+    rng = np.random.default_rng(K + G + rows)
+    x = rng.standard_normal((rows, K)).astype(np.float32)
+    last = (K - 1) // G * G
+    x[0, last:] = 0
+    x[0, last] = 127.0
+    ties = np.array([2.5, 3.5, -2.5, -0.5, 0.5, 1.5, -3.5], np.float32)
+    n = min(len(ties), K - last - 1)
+    x[0, K - n:] = ties[:n]
+    xq, xd, gs = ops.FC_dynamic_quantize_x(dev(x), G)
+    wq, wd, wg = orc.quant_x(x, G)
+    assert np.array_equal(host(xq), wq)
+    assert np.array_equal(host(xd).view(np.uint32), wd.view(np.uint32))
+    assert np.array_equal(host(gs).view(np.uint32), wg.view(np.uint32))
+
+
+@pytest.mark.parametrize("G", [32, 128])
+@pytest.mark.parametrize("rows,N,K", [(1, 4096, 4100), (2, 100, 1001), (8, 352, 333), (17, 96, 1001), (300, 160, 700)])
+def test_fc_short_last_group(ops, orc, G, rows, N, K):
+    """fc_Q4A with K not a multiple of the group size, on the kernels of few and of many rows, with and without
+    the residual epilogue, against the oracle (whose tail handling is pinned by the reference build)."""
+    rng = np.random.default_rng(rows + N + K + G)
+    w = (rng.standard_normal((N, K)) * 0.02).astype(np.float32)
+    pw = orc.quant_w(w, G)
+    assert np.array_equal(host(ops.offline_FC_quant_Q4A(dev(w), G)), pw)
+    x = rng.standard_normal((1, rows, K)).astype(np.float32)
+    res = rng.standard_normal((1, rows, N)).astype(np.float32)
+    want = orc.fc(x, pw, N)
+    assert max_rel_err(host(ops.fc_Q4A(dev(x), dev(pw), N)), want) <= 1e-5
+    assert max_rel_err(host(ops.fc_Q4A(dev(x), dev(pw), N, residual=dev(res))), want + res) <= 1e-5

@@ -368,3 +368,40 @@ def test_mm_qk_oracle_against_reference_build(orc, variant):
         mine = orc.mm_qk(q, kc)
     assert got.shape == mine.shape
     assert np.abs(got - mine).max() <= 1e-5 * np.abs(mine).max()
+
+
+@pytest.mark.parametrize("G", [32, 128])
+@pytest.mark.parametrize("K", [5, 100, 333, 1001, 4100])
+def test_quant_x_short_last_group_vs_reference_build(orc, G, K):
+    """A K that is not a whole number of groups, nor of eights: the reference zero-pads the last group's codes
+    (ops/op_fc.hpp:259-261) and its last K % 8 values round half away from zero (ops/utils.hpp:217-219).  The
+    restatement against the reference build, bit for bit, ties included."""
+    R = _ref(G)
+    rng = np.random.default_rng(K + G)
+    x = rng.standard_normal((3, K)).astype(np.float32)
+    last = (K - 1) // G * G                      # first element of the short group
+    x[0, last:] = 0
+    x[0, last] = 127.0                            # amax 127 -> d = 1: the products are the values themselves
+    ties = np.array([2.5, 3.5, -2.5, -0.5, 0.5, 1.5, -3.5], np.float32)
+    n = min(len(ties), K - last - 1)
+    x[0, K - n:] = ties[:n]                       # the tail values: where the two roundings differ
+    oq, od, og = orc.quant_x(x, G)
+    rq, rd, rg = R.quant_x(x)
+    assert np.array_equal(oq, rq)
+    assert np.array_equal(od.view(np.uint32), rd.view(np.uint32))
+    assert np.array_equal(og.view(np.uint32), rg.view(np.uint32))
+    assert np.all(oq[:, K:] == 0)
+
+
+@pytest.mark.parametrize("G", [32, 128])
+@pytest.mark.parametrize("rows,N,K", [(1, 64, 100), (3, 96, 1001), (17, 32, 4100)])
+def test_fc_short_last_group_vs_reference_build(orc, G, rows, N, K):
+    """fc_Q4A with a K that is not a whole number of k-groups: the reference pads the activation codes of the last
+    group with zeros, so whatever codes the weights hold beyond K do not matter.  (The weights are packed by the
+    restatement, which clips the min/max scan to K; the reference's own packing reads past the row there,
+    ops/op_fc.hpp:184.)  Output of the restatement against the reference build's fc_Q4A, bit for bit."""
+    R = _ref(G)
+    rng = np.random.default_rng(rows + N + K + G)
+    wq = orc.quant_w((rng.standard_normal((N, K)) * 0.02).astype(np.float32), G)
+    x = rng.standard_normal((1, rows, K)).astype(np.float32)
+    assert np.array_equal(orc.fc(x, wq, N).view(np.uint32), R.fc(x, wq, N).view(np.uint32))
