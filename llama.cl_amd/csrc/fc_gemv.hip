@@ -104,21 +104,41 @@ __device__ __forceinline__ void finish_strip(float f[MT][4], float (*red)[MT][kG
         if (sumsq_out != nullptr) strip_sumsq(out, mine, tr, nb, (int)(gridDim.x / S), sumsq_out);
         return;
     }
-    // Two k-splits and nobody waiting for the strip's sum of squares: the hand-off is one 64-bit exchange
-    // per output.  A slot is empty (0) or holds (1 << 32 | value bits); whoever finds the other split's
+    // Two k-splits: the hand-off is one 64-bit exchange per output.  A slot is empty (0) or holds (1 << 32 | value bits); whoever finds the other split's
     // value there adds the two (a + b: the same bits whichever came first), stores the output and empties
     // the slot for the next launch; whoever finds it empty has parked its own value and is done.  The value
     // travels inside the atomic, so there is nothing to order, and the cost is one round trip to memory
     // instead of three (store and acknowledgement, ticket, loads).
     if (slots != nullptr) {
-        if (!(mine && n < N)) return;
-        unsigned long long* slot = slots + ((int64_t)tr * Np + n);
-        const unsigned long long parked = (1ull << 32) | (unsigned long long)__float_as_uint(v);
-        const unsigned long long old = __hip_atomic_exchange(slot, parked, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        if ((old >> 32) == 0ull) return;
-        const float both = v + __uint_as_float((unsigned)(old & 0xFFFFFFFFull));
-        y[(int64_t)tr * N + n] = has_residual ? both + residual_value : both;
-        __hip_atomic_store(slot, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        float done = 0.0f;  // the finished output if this thread is the one that finished it, else 0
+        if (mine && n < N) {
+            unsigned long long* slot = slots + ((int64_t)tr * Np + n);
+            const unsigned long long parked = (1ull << 32) | (unsigned long long)__float_as_uint(v);
+            const unsigned long long old = __hip_atomic_exchange(slot, parked, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if ((old >> 32) != 0ull) {
+                const float both = v + __uint_as_float((unsigned)(old & 0xFFFFFFFFull));
+                done = has_residual ? both + residual_value : both;
+                y[(int64_t)tr * N + n] = done;
+                __hip_atomic_store(slot, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
+        if (sumsq_out == nullptr) return;
+        // The strip's sum of squares: each of the two workgroups knows the squares of the outputs it finished;
+        // the two partial sums meet through one more exchange per (row, strip), in slots behind the outputs'
+        // (p0 + p1: the same bits whichever came first).
+        float sq = done * done;
+#pragma unroll
+        for (int o = 16; o > 0; o >>= 1) sq += __shfl_xor(sq, o, 64);
+        if (mine && (lane_id_now() & 31) == 0) {
+            const int64_t strips = (int64_t)gridDim.x / S;
+            unsigned long long* slot = slots + (int64_t)rows * Np + ((int64_t)tr * strips + nb);
+            const unsigned long long parked = (1ull << 32) | (unsigned long long)__float_as_uint(sq);
+            const unsigned long long old = __hip_atomic_exchange(slot, parked, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if ((old >> 32) != 0ull) {
+                sumsq_out[(int64_t)tr * strips + nb] = sq + __uint_as_float((unsigned)(old & 0xFFFFFFFFull));
+                __hip_atomic_store(slot, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
         return;
     }
     // Cross-workgroup hand-off without cache-wide fences: partial sums are written and read with
@@ -660,11 +680,11 @@ static void launch_fused_t(const uint8_t* w, const float* x, float* y, float* pa
                            int64_t Kg, int64_t N, int rows, GemvPlan p, const FusedOps& o, hipStream_t st,
                            const DumpBufs* dump = nullptr) {
     const int64_t K = Kg * G;
-    // Two k-splits and no sums of squares wanted: the splits meet through one 64-bit exchange per output, in
-    // slots behind the arrival counters in the zeroed head of the workspace (if they fit there).
-    const int64_t slot_bytes = (int64_t)rows * Ng * kGroupN * 8;
-    const int exchange = g_exchange_handoff && p.S == 2 && !o.glu && o.sumsq_out == nullptr &&
-                         slot_bytes <= LLMOPS_FC_COUNTER_BYTES - kTicketBytes;
+    // Two k-splits: the splits meet through one 64-bit exchange per output, in slots behind the arrival
+    // counters in the zeroed head of the workspace (if they fit there).
+    // (outputs' slots, then one slot per (row, strip) for the partial sums of squares)
+    const int64_t slot_bytes = (int64_t)rows * Ng * kGroupN * 8 + (int64_t)rows * Ng * 8;
+    const int exchange = g_exchange_handoff && p.S == 2 && !o.glu && slot_bytes <= LLMOPS_FC_COUNTER_BYTES - kTicketBytes;
     if (exchange) part = reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(counters) + kTicketBytes);
 #define LLMOPS_FUSED(MODE, GRID)                                                                                      \
     fc_gemv_fused_kernel<G, MT, NW, MODE><<<(unsigned)(GRID), NW * 64, 0, st>>>(                                      \
