@@ -23,7 +23,7 @@ from . import _lib
 __all__ = [
     "offline_FC_quant_Q4A", "offline_FC_dequant_Q4A", "fc_Q4A", "fc_Q4A_noalloc", "fc_Q4A_decode", "interleave_gate_up", "FC_dynamic_quantize_x", "fc_Q4A_partials",
     "attention_rope", "attention_rope2", "attention_rope2_records", "attention_records_supported", "AttentionRecords", "rope_embed", "softmax", "rmsnorm", "iadd", "imul", "itrans", "clone",
-    "rmsnorm_out", "silu_mul", "empty", "ones", "embedding", "embedding_q8c_quant_w", "embedding_q8c", "tensor_pool", "set_default_group_k", "reserve_workspace",
+    "rmsnorm_out", "silu_mul", "empty", "ones", "embedding", "embedding_q8c_quant_w", "embedding_q8c", "tensor_pool", "set_default_group_k", "reserve_workspace", "reset_workspaces",
     "group_k_of",
 ]
 
@@ -108,6 +108,16 @@ def reserve_workspace(device=None, fc_bytes=0, attn_bytes=0):
         _workspace(device, fc_bytes, "fc")
     if attn_bytes:
         _workspace(device, attn_bytes, "attn")
+
+
+def reset_workspaces():
+    """Zero the hand-off areas (arrival counters, exchange slots) of every workspace this module holds.  The
+    kernels leave them zero after every call that runs to its end; after a launch that did not (a device error in
+    the middle of an op) call this once, with no op in flight, before using the module again."""
+    torch.cuda.synchronize()
+    for ws in list(_workspaces.values()) + _retired:
+        ws[:min(ws.numel(), 4 << 20)].zero_()
+    torch.cuda.synchronize()
 
 
 def group_k_of(weiq):
