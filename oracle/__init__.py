@@ -41,12 +41,13 @@ def _isa():
     return "vnni" if " avx_vnni" in flags else "avx2"
 
 
-def build(ref=True):
+def build(ref=True, force=False):
     """Compile the checkers (gcc/g++ only).  ``ref`` also builds oracle/_ref when the reference
-    sources are present on this machine."""
-    subprocess.check_call(["make", "-s", "-C", _HERE, "oracle"])
+    sources are present on this machine.  ``force`` recompiles what is already built."""
+    flags = ["-B"] if force else []
+    subprocess.check_call(["make", "-s"] + flags + ["-C", _HERE, "oracle"])
     if ref and os.path.isdir("/root/reference/ops"):
-        subprocess.check_call(["make", "-s", "-C", _HERE, "ref"])
+        subprocess.check_call(["make", "-s"] + flags + ["-C", _HERE, "ref"])
 
 
 def block_bytes(G):
