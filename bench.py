@@ -167,7 +167,7 @@ def main():
                 per_shape = measure_shapes(torch, llmops, plan, dims, weights, xs, stream)
                 overlapped = concurrent_streams(torch, llmops, dims, weights, xs, stream, step_bytes) if args.concurrent else \
                     {"skipped": "opt-in (--concurrent): replaying a multi-branch graph has crashed inside the HIP runtime "
-                                "on some boxes; figures of recorded runs are in the design notes"}
+                                "on some boxes (sporadic host-side segmentation fault under hipGraphLaunch)"}
             del weights, graph
         floor_us = dispatch_floor(torch, stream)
     ceiling_gbs = read_ceiling(torch, llmops)
