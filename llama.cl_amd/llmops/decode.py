@@ -241,16 +241,14 @@ class DecodeGraph:
     def __init__(self, graph, input_ids, slots, position, kv_cache, logits, stream, workspace):
         self.graph, self.input_ids, self.slots, self.position, self.kv_cache, self.logits, self.stream, self.workspace = \
             graph, input_ids, slots, position, kv_cache, logits, stream, workspace
-        self._host = torch.empty(2, dtype=torch.int32).pin_memory()
 
     def set_position(self, slot, position_id):
         """cache row the next token goes to and its position (kv length = position + 1, up to the cache size)"""
         if not (0 <= int(slot) < self.kv_cache.shape[3]) or int(position_id) < 0:
             raise ValueError("slot outside the cache or negative position")
-        self._host[0], self._host[1] = int(slot), int(position_id)
-        with torch.cuda.stream(self.stream):
-            self.slots.copy_(self._host[0:1], non_blocking=True)
-            self.position.copy_(self._host[1:2], non_blocking=True)
+        with torch.cuda.stream(self.stream):  # (scalar fills: no host buffer that a later call could overwrite too early)
+            self.slots.fill_(int(slot))
+            self.position.fill_(int(position_id))
 
     def replay(self):
         with torch.cuda.stream(self.stream):
