@@ -70,7 +70,9 @@ int llmops_offline_FC_dequant_Q4A(const int8_t* weiq, int64_t Ng, int64_t Kg, in
 /* FC_dynamic_quantize_x (ops/op_fc.hpp:221-272; get_amax ops/utils.hpp:177-197, quant_row_q8_0
  * ops/utils.hpp:200-220).  x fp32 [rows,K] -> xq int8 [rows,Kg*G] (round half to even, zero
  * padded), xd fp32 [rows,Kg] = amax/127, gsum fp32 [rows,Kg] = left-to-right fp32 sum of the raw
- * group.  All three outputs are bit-exact with the reference.  Requires K % 8 == 0. */
+ * group.  All three outputs are bit-exact with the reference.  K is any positive value: the last K % 8
+ * values of a short last group take the reference's scalar tail, which rounds half away from zero
+ * (ops/utils.hpp:217-219). */
 int llmops_FC_dynamic_quantize_x(const float* x, int64_t rows, int64_t K, int group_k, int8_t* xq,
                                  float* xd, float* gsum, llmops_stream_t stream);
 
@@ -119,7 +121,9 @@ int llmops_fc_Q4A_noalloc(const float* x, int64_t rows, int64_t K, const int8_t*
 
 /* fc_Q4A followed by iadd(y, residual) (ops/op_misc.hpp:55-79) in one launch for rows <= 8:
  * y = fc_Q4A(x) + residual, residual fp32 [rows,N].  The decode step uses it for the o and down
- * projections (chatllama/main.py:355-357,372-375). */
+ * projections (chatllama/main.py:355-357,372-375).  residual may be y itself (the add in place the
+ * reference does), except when K is not a multiple of group_k and rows <= 8: that combination adds
+ * the residual in a second launch and is refused with LLMOPS_EINVAL if the two alias. */
 int llmops_fc_Q4A_residual(const float* x, int64_t rows, int64_t K, const int8_t* weiq, int64_t Ng, int64_t Kg,
                            int group_k, int64_t N, const float* residual, float* y, void* workspace,
                            size_t workspace_bytes, llmops_stream_t stream);

@@ -109,6 +109,7 @@ static int fc_impl(const float* x, int64_t rows, int64_t K, const int8_t* weiq, 
         int rc_t = launch_quant_x(x, rows, K, group_k, xq, xd, gs, xst_t, false, st);
         if (rc_t) return rc_t;
         if (rows > kMaxGemvRows) return launch_gemm(w, xq, xd, gs, xst_t, y, part, counters, rows, Ng, Kg, group_k, N, residual, st);
+        if (residual == y) return fail(LLMOPS_EINVAL, "fc_Q4A with a short last k-group and up to 8 rows: residual must not be y");
         rc_t = launch_gemv(w, xq, xd, gs, y, part, counters, rows, Ng, Kg, group_k, N, st);
         if (rc_t == 0 && residual != nullptr) rc_t = launch_add(y, residual, rows * N, st);
         return rc_t;

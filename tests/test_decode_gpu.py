@@ -296,3 +296,26 @@ def test_one_decode_graph_serves_successive_positions(orc):
             assert max_rel_err(logits.cpu().numpy(), want) <= 5e-2, (step, pos)
         eager_cache.copy_(c_dev)
     assert kv.position_id == 46 and kv.cur_kv_len == maxlen
+
+
+def test_reset_workspaces_restores_a_dirty_hand_off_area():
+    """What a launch that did not run to its end may leave behind: non-zero arrival counters and exchange slots.
+    The two k-splits of a 4096x11008 FC then never meet (a parked value is taken for the partner's): the output is
+    wrong until the hand-off areas are zeroed again."""
+    import llmops
+    dev = torch.device("cuda:0")
+    rng = np.random.default_rng(3)
+    N, K = 4096, 11008
+    wq = llmops.offline_FC_quant_Q4A(torch.from_numpy((rng.standard_normal((N, K)) * 0.02).astype(np.float32)).to(dev), 128)
+    x = torch.from_numpy(rng.standard_normal((1, 1, K)).astype(np.float32)).to(dev)
+    want = llmops.fc_Q4A(x, wq, N)
+    torch.cuda.synchronize()
+    for key, ws in llmops._workspaces.items():
+        if key[0] == "fc":
+            ws[65536:65536 + 8 * N].fill_(0x11)          # garbage in the exchange slots of this shape
+    torch.cuda.synchronize()
+    dirty = llmops.fc_Q4A(x, wq, N)
+    assert not torch.equal(dirty, want)
+    llmops.reset_workspaces()
+    assert torch.equal(llmops.fc_Q4A(x, wq, N), want)
+    assert torch.equal(llmops.fc_Q4A(x, wq, N), want)

@@ -574,3 +574,33 @@ def test_fc_short_last_group(ops, orc, G, rows, N, K):
     want = orc.fc(x, pw, N)
     assert max_rel_err(host(ops.fc_Q4A(dev(x), dev(pw), N)), want) <= 1e-5
     assert max_rel_err(host(ops.fc_Q4A(dev(x), dev(pw), N, residual=dev(res))), want + res) <= 1e-5
+
+
+@pytest.mark.parametrize("rows,N,K", [(1, 4096, 4096), (2, 4096, 11008), (1, 1000, 2048), (5, 352, 512), (40, 4096, 4096)])
+def test_fc_residual_in_place(ops, rows, N, K):
+    """y = fc_Q4A(x) + y, the add in place the reference's iadd does (ops/op_misc.hpp:55-79): residual and y one
+    buffer, on the one-launch kernels of few rows (with and without k-splits) and on the MFMA kernel: bit-equal to
+    the call with a separate residual.  With a short last k-group and few rows the add is a second launch: refused."""
+    rng = np.random.default_rng(rows * 7 + N + K)
+    G = 128
+    wq = ops.offline_FC_quant_Q4A(dev((rng.standard_normal((N, K)) * 0.02).astype(np.float32)), G)
+    x = dev(rng.standard_normal((1, rows, K)).astype(np.float32))
+    res = dev(rng.standard_normal((1, rows, N)).astype(np.float32))
+    want = ops.fc_Q4A(x, wq, N, residual=res)
+    lib = ops._lib.load()
+    Ng, Kg, _ = wq.shape
+
+    def in_place(xx, kk):
+        y = res.clone()
+        ws = ops._workspace(xx.device, lib.llmops_fc_Q4A_workspace_bytes(rows, kk, Ng, Kg, G))
+        rc = lib.llmops_fc_Q4A_residual(ops._ptr(xx), rows, kk, ops._ptr(wq), Ng, Kg, G, N, ops._ptr(y), ops._ptr(y),
+                                        ops._ptr(ws), ws.numel(), ops._stream(xx))
+        return rc, y
+
+    for _ in range(3):
+        rc, y = in_place(x, K)
+        assert rc == 0 and torch.equal(y, want)
+    if rows <= 8:
+        rc, y = in_place(x[:, :, :K - 3].contiguous(), K - 3)
+        assert rc == 1 and b"residual must not be y" in lib.llmops_last_error()        # LLMOPS_EINVAL
+        assert torch.equal(y, res)                                                     # nothing was launched
