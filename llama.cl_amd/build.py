@@ -22,6 +22,7 @@ FLAGS = [
     "-fhip-fp32-correctly-rounded-divide-sqrt",  # quantization divides must be IEEE-exact
     "-ffp-contract=on",  # contract only within a statement; never across statements
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-mllvm", "-amdgpu-kernarg-preload-count=16",
     "-Wall", "-Wno-unused-function", "-Wno-unknown-attributes", "-Wno-inline-asm",
 ]
 

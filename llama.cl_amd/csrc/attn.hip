@@ -404,11 +404,13 @@ __device__ __forceinline__ uint4 load_row16(const void* p) {
 constexpr int kAttnRecChunks = 8;
 
 template <typename T, int PW, int NWV = 4, bool RECS = false>
-__global__ __launch_bounds__(NWV * 64) void attn_decode_kernel(float* q, float* k, const float* __restrict__ v,
-                                                           const float* __restrict__ inv_freq, int half, T* kc, T* vc,
-                                                           int64_t H, int64_t maxlen, const int32_t* __restrict__ slots,
-                                                           int position_id, const int32_t* __restrict__ pos_dev, float* part,
-                                                           int nchunks, float* rec_stats = nullptr, float* rec_outs = nullptr) {
+__global__ __launch_bounds__(NWV * 64) void attn_decode_kernel(const int32_t* __restrict__ pos_dev, int position_id, int nchunks,
+                                                           int64_t maxlen, T* kc, T* vc, const int32_t* __restrict__ slots,
+                                                           float* q, float* k, const float* __restrict__ v,
+                                                           const float* __restrict__ inv_freq, int half, float* part,
+                                                           float* rec_stats = nullptr, float* rec_outs = nullptr) {
+    // (argument order: the first 14 dwords arrive in scalar registers with the wave (kernel-argument preload);
+    // they are what the position, the slot and the cache rows' addresses need)
     constexpr int S = 128, C = NWV * PW;
     constexpr int EPL = RowPiece<T>::EPL, LPR = S / EPL, RPW = 64 / LPR, NL = PW / RPW;
     static_assert(NL >= 1 && NL <= LPR, "rows per lane");
@@ -897,11 +899,11 @@ static int attention_impl(float* q, float* k, const float* v, int64_t B, int64_t
         const int nchunks = (int)((kv_plan + rows - 1) / rows);
         const unsigned grid = (unsigned)(bhq * nchunks);
         if (rows == 256)
-            attn_decode_kernel<T, 16, 16, true><<<grid, 1024, 0, st>>>(q, k, v, inv_freq, (int)half, kc, vc, H, maxlen, slots, position_id,
-                                                                       pos_dev, nullptr, nchunks, rec_stats, rec_outs);
+            attn_decode_kernel<T, 16, 16, true><<<grid, 1024, 0, st>>>(pos_dev, position_id, nchunks, maxlen, kc, vc, slots, q, k, v,
+                                                                       inv_freq, (int)half, nullptr, rec_stats, rec_outs);
         else if constexpr (kHalfCache)
-            attn_decode_kernel<T, 32, 16, true><<<grid, 1024, 0, st>>>(q, k, v, inv_freq, (int)half, kc, vc, H, maxlen, slots, position_id,
-                                                                       pos_dev, nullptr, nchunks, rec_stats, rec_outs);
+            attn_decode_kernel<T, 32, 16, true><<<grid, 1024, 0, st>>>(pos_dev, position_id, nchunks, maxlen, kc, vc, slots, q, k, v,
+                                                                       inv_freq, (int)half, nullptr, rec_stats, rec_outs);
         LLMOPS_LAUNCH_CHECK();
         return LLMOPS_OK;
     }
@@ -916,8 +918,8 @@ static int attention_impl(float* q, float* k, const float* v, int64_t B, int64_t
             return fail(LLMOPS_EWORKSPACE, "attention workspace too small for %lld chunk records", (long long)bhq * nchunks);
         const unsigned grid = (unsigned)(bhq * nchunks);
 #define LLMOPS_DECODE(PWV)                                                                                         \
-    attn_decode_kernel<T, PWV><<<grid, 256, 0, st>>>(q, k, v, inv_freq, (int)half, kc, vc, H, maxlen, slots, position_id, \
-                                                     pos_dev, part, nchunks)
+    attn_decode_kernel<T, PWV><<<grid, 256, 0, st>>>(pos_dev, position_id, nchunks, maxlen, kc, vc, slots, q, k, v, inv_freq, \
+                                                     (int)half, part)
         switch (p.pw) {
             case 4: if constexpr (!kHalfCache) LLMOPS_DECODE(4); break;
             case 8: LLMOPS_DECODE(8); break;

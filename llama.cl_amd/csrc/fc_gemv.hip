@@ -286,17 +286,22 @@ __device__ __forceinline__ float4 merge_attn_records(const float4 (&ro)[kAttnRec
 // weight buffers of the pass in place, without register copies.
 template <int G, int MT, int NW, int MODE>
 __global__ __launch_bounds__(NW * 64, (MT == 1 ? ((MODE & kAttnIn) ? NW / 4 : NW / 2) : 1)) void fc_gemv_fused_kernel(const uint8_t* __restrict__ weiq, const float* __restrict__ x,
-                                                                 float* __restrict__ y, float* part, unsigned* counters,
-                                                                 int Kg, int64_t K, int64_t N, int rows, int S,
-                                                                 int steps_per_split, const float* __restrict__ residual,
+                                                                 int Kg, int S, int steps_per_split, int rows, int N, int sumsq_parts,
+                                                                 const float* __restrict__ residual,
+                                                                 const float* __restrict__ sumsq_in,
                                                                  const float* __restrict__ norm_w, float eps,
-                                                                 const float* __restrict__ sumsq_in, int sumsq_parts,
+                                                                 float* __restrict__ y, float* part, unsigned* counters,
                                                                  float* __restrict__ sumsq_out, int exchange, const DumpBufs dump,
                                                                  const AttnRecs recs) {
     constexpr bool NORM = (MODE & kNorm) != 0, GLU = (MODE & kGlu) != 0, SUMS = (MODE & kSums) != 0;
     constexpr bool GLUIN = (MODE & kGluIn) != 0, DUMP = (MODE & kDump) != 0, ATTN = (MODE & kAttnIn) != 0;
     static_assert(!ATTN || (G == 128 && MT == 1 && !NORM && !GLU && !GLUIN), "chunk records: one row, group 128, plain input");
     static_assert(!(GLUIN && NORM), "the gate|up input has no rmsnorm");
+    // (argument order: the first 14 dwords of a kernel's arguments arrive in scalar registers together with the
+    // wave (the library is built with kernel-argument preload), so everything the first loads need -- tensor,
+    // activations, the plan, the residual and the handed-over sums -- comes first: a wave then asks for its
+    // data without a round trip to the argument buffer in front of it)
+    const int64_t K = (int64_t)Kg * G;
     const int64_t xstride = GLUIN ? 2 * K : K;  // floats between activation rows
     constexpr int NWS = GLU ? NW / 2 : NW;  // waves per strip
     __shared__ float red[NW][MT][kGroupN];
@@ -679,7 +684,6 @@ template <int G, int MT, int NW>
 static void launch_fused_t(const uint8_t* w, const float* x, float* y, float* part, unsigned* counters, int64_t Ng,
                            int64_t Kg, int64_t N, int rows, GemvPlan p, const FusedOps& o, hipStream_t st,
                            const DumpBufs* dump = nullptr) {
-    const int64_t K = Kg * G;
     // Two k-splits: the splits meet through one 64-bit exchange per output, in slots behind the arrival
     // counters in the zeroed head of the workspace (if they fit there).
     // (outputs' slots, then one slot per (row, strip) for the partial sums of squares)
@@ -688,8 +692,8 @@ static void launch_fused_t(const uint8_t* w, const float* x, float* y, float* pa
     if (exchange) part = reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(counters) + kTicketBytes);
 #define LLMOPS_FUSED(MODE, GRID)                                                                                      \
     fc_gemv_fused_kernel<G, MT, NW, MODE><<<(unsigned)(GRID), NW * 64, 0, st>>>(                                      \
-        w, x, y, part, counters, (int)Kg, K, N, rows, p.S, p.steps_per_split, o.residual, o.norm_w, o.eps, o.sumsq_in, \
-        o.sumsq_parts, o.sumsq_out, exchange, dump ? *dump : DumpBufs{nullptr, nullptr, nullptr, nullptr}, o.recs)
+        w, x, (int)Kg, p.S, p.steps_per_split, rows, (int)N, o.sumsq_parts, o.residual, o.sumsq_in, o.norm_w, o.eps, y,   \
+        part, counters, o.sumsq_out, exchange, dump ? *dump : DumpBufs{nullptr, nullptr, nullptr, nullptr}, o.recs)
     // (the kernel reads up to 256 handed-over partial sums per row; with more, the statistic is recomputed)
     const bool sums = o.norm_w != nullptr && o.sumsq_in != nullptr && o.sumsq_parts <= 256;
     if (dump != nullptr) {  // plain fc_Q4A, or the chunk records of attention as input
@@ -718,6 +722,7 @@ int launch_gemv_fused(const uint8_t* w, const float* x, float* y, float* part, u
                       const float* rec_stats, const float* rec_outs, int rec_chunks) {
     GemvPlan p = plan_gemv(rows, Ng, Kg, G, true);
     if (glu == 1) p.S = 1;
+    if (N > INT32_MAX || Kg * G > INT32_MAX) return fail(LLMOPS_EINVAL, "fc_Q4A for up to 8 rows: N and K must fit 31 bits");
     if (dump != nullptr && (norm_w != nullptr || glu != 0)) return fail(LLMOPS_EINVAL, "the dump build runs the plain FC only");
     if (rec_stats != nullptr && (rows != 1 || G != 128 || norm_w != nullptr || glu != 0))
         return fail(LLMOPS_EINVAL, "chunk records as input: one row, group 128, no rmsnorm, no gate/up forms");
