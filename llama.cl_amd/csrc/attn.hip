@@ -236,8 +236,8 @@ __device__ __forceinline__ float merge_chunks(const float* rec, int nchunks, int
 // `nchunks` records per query are laid out; with pos_dev (decode graphs) only the first
 // ceil(min(pos_dev[0] + 1, maxlen) / chunk_rows) of them were written by this call.
 __global__ __launch_bounds__(128) void attn_merge_kernel(float* __restrict__ q, const float* __restrict__ part, int64_t qL,
-                                                          int64_t H, int nchunks, const int32_t* __restrict__ pos_dev = nullptr,
-                                                          int64_t maxlen = 0, int chunk_rows = 1) {
+                                                          int64_t H, int nchunks, int chunk_rows = 1,
+                                                          const int32_t* __restrict__ pos_dev = nullptr, int64_t maxlen = 0) {
     constexpr int S = 128;
     __shared__ float wsh[2][64];
     const int64_t bhq = blockIdx.x;
@@ -422,7 +422,13 @@ __global__ __launch_bounds__(NWV * 64) void attn_decode_kernel(const int32_t* __
     const int rsel = lane / LPR, e = lane % LPR;  // which of the RPW rows of a wave-wide load, which 16 bytes of it
     const int chunk = blockIdx.x % nchunks;
     const int64_t bh = blockIdx.x / nchunks;
-    if (pos_dev != nullptr) position_id = pos_dev[0];
+    // One round trip for everything that did not come with the wave: the slot, the position (read through a
+    // pointer that is always valid, so that there is no branch around the load) and the remaining arguments,
+    // which the compiler would otherwise fetch one by one where the code first uses them.
+    const int slot = slots[0];
+    const int pos_loaded = (pos_dev != nullptr ? pos_dev : slots)[0];
+    asm volatile("" ::"s"(slot), "s"(pos_loaded), "s"(k), "s"(v), "s"(inv_freq), "s"(half), "s"(rec_stats), "s"(rec_outs), "s"(part));
+    if (pos_dev != nullptr) position_id = pos_loaded;
     const int64_t kvLen = min((int64_t)position_id + 1, maxlen);
     const int nact = (int)((kvLen + C - 1) / C);  // chunks that hold rows at this position
     if (chunk >= nact) {
@@ -443,7 +449,6 @@ __global__ __launch_bounds__(NWV * 64) void attn_decode_kernel(const int32_t* __
     // loads whose data the rotation needs go first, then the K rows, then the V rows: the cos/sin table,
     // the rotation of q (and k) and the scores are then computed while the rows behind them are still in
     // flight, instead of after the last V row has landed.
-    const int slot = slots[0];
     const bool slot_ok = slot >= 0 && slot < maxlen;
     // the workgroup that owns the new token's row (or the last chunk, if the row lies beyond kvLen)
     const int owner = (slot_ok && slot / C < nact) ? slot / C : nact - 1;
@@ -929,7 +934,7 @@ static int attention_impl(float* q, float* k, const float* v, int64_t B, int64_t
 #undef LLMOPS_DECODE
         LLMOPS_LAUNCH_CHECK();
         if (nchunks > 1) {
-            attn_merge_kernel<<<(unsigned)bhq, 128, 0, st>>>(q, part, qL, H, nchunks, pos_dev, maxlen, 4 * p.pw);
+            attn_merge_kernel<<<(unsigned)bhq, 128, 0, st>>>(q, part, qL, H, nchunks, 4 * p.pw, pos_dev, maxlen);
             LLMOPS_LAUNCH_CHECK();
         }
         return LLMOPS_OK;

@@ -90,10 +90,12 @@ template <int RT, int NW, bool DUMP = false>
 __global__ __launch_bounds__(NW * 64, RT == 2 ? 3 : 4) void fc_rows_mfma_kernel(const uint8_t* __restrict__ weiq,
                                                                          const int8_t* __restrict__ xq,
                                                                          const float2* __restrict__ xsT,
-                                                                         float* __restrict__ y, int Kg, int64_t N, int rows,
+                                                                         unsigned long long* slots, int Kg, int rows,
+                                                                         int64_t N, float* __restrict__ y,
                                                                          const float* __restrict__ residual,
-                                                                         unsigned long long* slots,
                                                                          int32_t* dump = nullptr) {
+    // (argument order: what the first loads need comes in the first 14 dwords, which arrive in scalar registers
+    // with the wave)
     __shared__ float red[DUMP ? 1 : NW][16 * RT][kGroupN];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // uniform: block offsets stay scalar
@@ -233,11 +235,11 @@ int launch_fc_rows(const uint8_t* w, const int8_t* xq, const float2* xsT, float*
     // 17..32 rows: two row tiles per wave, 8 waves (16 would not have the registers).
     const int64_t k_per_wg = split ? (Kg + 1) / 2 : Kg;
     if (rows > 16)
-        fc_rows_mfma_kernel<2, 8><<<grid, 512, 0, st>>>(w, xq, xsT, y, (int)Kg, N, (int)rows, residual, sl);
+        fc_rows_mfma_kernel<2, 8><<<grid, 512, 0, st>>>(w, xq, xsT, sl, (int)Kg, (int)rows, N, y, residual);
     else if (k_per_wg > 32)
-        fc_rows_mfma_kernel<1, 16><<<grid, 1024, 0, st>>>(w, xq, xsT, y, (int)Kg, N, (int)rows, residual, sl);
+        fc_rows_mfma_kernel<1, 16><<<grid, 1024, 0, st>>>(w, xq, xsT, sl, (int)Kg, (int)rows, N, y, residual);
     else
-        fc_rows_mfma_kernel<1, 8><<<grid, 512, 0, st>>>(w, xq, xsT, y, (int)Kg, N, (int)rows, residual, sl);
+        fc_rows_mfma_kernel<1, 8><<<grid, 512, 0, st>>>(w, xq, xsT, sl, (int)Kg, (int)rows, N, y, residual);
     LLMOPS_LAUNCH_CHECK();
     return LLMOPS_OK;
 }
@@ -252,11 +254,11 @@ int launch_fc_rows_partials(const uint8_t* w, const int8_t* xq, int32_t* acc, in
     unsigned long long* sl = split ? reinterpret_cast<unsigned long long*>(acc) : nullptr;
     const int64_t k_per_wg = split ? (Kg + 1) / 2 : Kg;
     if (rows > 16)
-        fc_rows_mfma_kernel<2, 8, true><<<grid, 512, 0, st>>>(w, xq, nullptr, nullptr, (int)Kg, 0, (int)rows, nullptr, sl, acc);
+        fc_rows_mfma_kernel<2, 8, true><<<grid, 512, 0, st>>>(w, xq, nullptr, sl, (int)Kg, (int)rows, 0, nullptr, nullptr, acc);
     else if (k_per_wg > 32)
-        fc_rows_mfma_kernel<1, 16, true><<<grid, 1024, 0, st>>>(w, xq, nullptr, nullptr, (int)Kg, 0, (int)rows, nullptr, sl, acc);
+        fc_rows_mfma_kernel<1, 16, true><<<grid, 1024, 0, st>>>(w, xq, nullptr, sl, (int)Kg, (int)rows, 0, nullptr, nullptr, acc);
     else
-        fc_rows_mfma_kernel<1, 8, true><<<grid, 512, 0, st>>>(w, xq, nullptr, nullptr, (int)Kg, 0, (int)rows, nullptr, sl, acc);
+        fc_rows_mfma_kernel<1, 8, true><<<grid, 512, 0, st>>>(w, xq, nullptr, sl, (int)Kg, (int)rows, 0, nullptr, nullptr, acc);
     LLMOPS_LAUNCH_CHECK();
     return LLMOPS_OK;
 }
