@@ -51,10 +51,12 @@ __device__ __forceinline__ TileRange tile_range(int Kg, int S, int steps_per_spl
         r.nb = blockIdx.x / S;
         r.s = blockIdx.x % S;
     }
-    const int T = (Kg + BPS - 1) / BPS;  // steps in a strip
+    const int T = (int)((unsigned)(Kg + BPS - 1) / BPS);  // steps in a strip
     const int t_lo = r.s * steps_per_split;
     const int t_hi = min(T, t_lo + steps_per_split);
-    const int per_wave = (t_hi - t_lo + NW - 1) / NW;
+    // (unsigned: every wave runs this before it can ask for its first byte, and a signed division by NW costs
+    // three scalar instructions more)
+    const int per_wave = (int)((unsigned)(t_hi - t_lo + NW - 1) / NW);
     r.t0 = min(t_hi, t_lo + wave * per_wave);
     r.t1 = min(t_hi, r.t0 + per_wave);
     return r;
@@ -324,7 +326,8 @@ __global__ __launch_bounds__(NW * 64, (MT == 1 ? ((MODE & kAttnIn) ? NW / 4 : NW
     } else {
         tr = tile_range<G, NW>(Kg, S, steps_per_split, wave);
     }
-    const uint8_t* strip = weiq + (int64_t)tr.nb * Kg * block_bytes(G);
+    // (a tensor has fewer than 2^32 blocks: one 32-bit product, then one widening multiplication)
+    const uint8_t* strip = weiq + (uint64_t)((uint32_t)tr.nb * (uint32_t)Kg) * (uint32_t)block_bytes(G);
     const bool first_row = (G == 128) ? (rs == 0) : ((rs & 3) == 0);
     // The residual element this thread will add at the very end (thread = (row, column) of the strip) is
     // asked for now: at the end it would put a memory round trip behind the last barrier.  (With the
@@ -399,7 +402,7 @@ __global__ __launch_bounds__(NW * 64, (MT == 1 ? ((MODE & kAttnIn) ? NW / 4 : NW
     }
 #define LLMOPS_LOAD_PAIR(P, TP, WANT)                                                                            \
     do { /* branch-free: what is not wanted is asked for at an offset that returns 0 (see kNoLoad) */            \
-        const bool ok_ = (WANT) && (TP) + lane_step < tr.t1 && (int64_t)(TP) * Step<G>::kK + lane * 4 < K;       \
+        const bool ok_ = (WANT) && (TP) + lane_step < tr.t1 && (uint32_t)(TP) * Step<G>::kK + lane * 4 < (uint32_t)K; \
         const uint32_t so_ = (uint32_t)(TP) * (uint32_t)(Step<G>::kK * 4);                                       \
         if constexpr (ATTN) { /* head = (TP) + (lane >> 5): statistics first (the weights need them), then the outputs */ \
             const uint32_t hs_ = (uint32_t)(TP) * (uint32_t)(kAttnRecChunks * 2 * 4);                            \
@@ -411,7 +414,7 @@ __global__ __launch_bounds__(NW * 64, (MT == 1 ? ((MODE & kAttnIn) ? NW / 4 : NW
         } else {                                                                                                 \
         _Pragma("unroll") for (int r = 0; r < MT; r++) {                                                         \
             const uint32_t ro_ = so_ + (uint32_t)r * (uint32_t)xstride * 4u;                                     \
-            const uint32_t lo_ = (ok_ && r < rows) ? (uint32_t)lane * 16u : kNoLoad;                             \
+            const uint32_t lo_ = (ok_ && (MT == 1 || r < rows)) ? (uint32_t)lane * 16u : kNoLoad; /* MT == 1: one row */ \
             P.xv[r] = buf_ldf4(x_rs, lo_, ro_);                                                                  \
             if (GLUIN) P.uv[GLUIN ? r : 0] = buf_ldf4(x_rs, lo_, ro_ + (uint32_t)K * 4u);                        \
         }                                                                                                        \
