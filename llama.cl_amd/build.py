@@ -22,6 +22,8 @@ FLAGS = [
     "-fhip-fp32-correctly-rounded-divide-sqrt",  # quantization divides must be IEEE-exact
     "-ffp-contract=on",  # contract only within a statement; never across statements
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # the first 14 dwords of a kernel's arguments arrive in scalar registers with the wave instead of being
+    # fetched by its first instructions: the short decode kernels take what their first loads need there
     "-mllvm", "-amdgpu-kernarg-preload-count=16",
     "-Wall", "-Wno-unused-function", "-Wno-unknown-attributes", "-Wno-inline-asm",
 ]
