@@ -405,7 +405,7 @@ constexpr int kAttnRecChunks = 8;
 
 template <typename T, int PW, int NWV = 4, bool RECS = false>
 __global__ __launch_bounds__(NWV * 64) void attn_decode_kernel(const int32_t* __restrict__ pos_dev, int position_id, int nchunks,
-                                                           int64_t maxlen, T* kc, T* vc, const int32_t* __restrict__ slots,
+                                                           int maxlen, T* kc, T* vc, const int32_t* __restrict__ slots,
                                                            float* q, float* k, const float* __restrict__ v,
                                                            const float* __restrict__ inv_freq, int half, float* part,
                                                            float* rec_stats = nullptr, float* rec_outs = nullptr) {
@@ -420,8 +420,10 @@ __global__ __launch_bounds__(NWV * 64) void attn_decode_kernel(const int32_t* __
     __shared__ float cs_sh[64], sn_sh[64];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int rsel = lane / LPR, e = lane % LPR;  // which of the RPW rows of a wave-wide load, which 16 bytes of it
-    const int chunk = blockIdx.x % nchunks;
-    const int64_t bh = blockIdx.x / nchunks;
+    // grid = (chunks, heads): no division, and 32-bit row arithmetic throughout -- every instruction in front of
+    // the first cache row is paid once per wave before the memory system has anything to do
+    const int chunk = blockIdx.x;
+    const uint32_t bh = blockIdx.y;
     // One round trip for everything that did not come with the wave: the slot, the position (read through a
     // pointer that is always valid, so that there is no branch around the load) and the remaining arguments,
     // which the compiler would otherwise fetch one by one where the code first uses them.
@@ -429,21 +431,25 @@ __global__ __launch_bounds__(NWV * 64) void attn_decode_kernel(const int32_t* __
     const int pos_loaded = (pos_dev != nullptr ? pos_dev : slots)[0];
     asm volatile("" ::"s"(slot), "s"(pos_loaded), "s"(k), "s"(v), "s"(inv_freq), "s"(half), "s"(rec_stats), "s"(rec_outs), "s"(part));
     if (pos_dev != nullptr) position_id = pos_loaded;
-    const int64_t kvLen = min((int64_t)position_id + 1, maxlen);
-    const int nact = (int)((kvLen + C - 1) / C);  // chunks that hold rows at this position
-    if (chunk >= nact) {
+    const int kvLen = position_id < maxlen ? position_id + 1 : maxlen;
+    const int nact = (int)((unsigned)(kvLen + C - 1) / C);  // chunks that hold rows at this position (none if kvLen <= 0)
+    if (chunk >= nact || kvLen <= 0) {
         if (RECS) {  // an empty record: weight 0 whatever the others hold
-            if (threadIdx.x < S) rec_outs[(bh * kAttnRecChunks + chunk) * S + threadIdx.x] = 0.0f;
+            if (threadIdx.x < S) rec_outs[((size_t)bh * kAttnRecChunks + chunk) * S + threadIdx.x] = 0.0f;
             if (threadIdx.x == 0) {
-                rec_stats[(bh * kAttnRecChunks + chunk) * 2] = -FLT_MAX;
-                rec_stats[(bh * kAttnRecChunks + chunk) * 2 + 1] = 0.0f;
+                rec_stats[((size_t)bh * kAttnRecChunks + chunk) * 2] = -FLT_MAX;
+                rec_stats[((size_t)bh * kAttnRecChunks + chunk) * 2 + 1] = 0.0f;
             }
         }
         return;
     }
-    const int64_t p0 = (int64_t)chunk * C;
-    T* kbase = kc + bh * maxlen * S;
-    T* vbase = vc + bh * maxlen * S;
+    const int p0 = chunk * C;
+    // a head's plane of the cache is below 4 GiB (checked by the launcher): uniform 64-bit base, 32-bit lane offsets
+    T* kbase = kc + (size_t)bh * ((uint32_t)maxlen * (uint32_t)S);
+    T* vbase = vc + (size_t)bh * ((uint32_t)maxlen * (uint32_t)S);
+    const float* qrow = q + (size_t)bh * S;
+    float* krow = k + (size_t)bh * S;
+    const float* vrow = v + (size_t)bh * S;
 
     // Loads return in issue order and a wave can only wait for "all but the youngest n".  So the small
     // loads whose data the rotation needs go first, then the K rows, then the V rows: the cos/sin table,
@@ -457,34 +463,31 @@ __global__ __launch_bounds__(NWV * 64) void attn_decode_kernel(const int32_t* __
     float4 q_own[EPL / 4], q_oth[EPL / 4];
 #pragma unroll
     for (int u = 0; u < EPL / 4; u++) {
-        q_own[u] = *reinterpret_cast<const float4*>(q + bh * S + e0 + 4 * u);
-        q_oth[u] = *reinterpret_cast<const float4*>(q + bh * S + rope_partner(e0 + 4 * u, half));
+        q_own[u] = *reinterpret_cast<const float4*>(qrow + (uint32_t)(e0 + 4 * u));
+        q_oth[u] = *reinterpret_cast<const float4*>(qrow + (uint32_t)rope_partner(e0 + 4 * u, half));
     }
+    // The new token's k and v rows: only the owner uses them, but every workgroup asks for them (48-96 bytes per
+    // lane out of L2): a branch around these loads would leave the registers with two definitions, and the copies
+    // that merge them wait for the loads -- one memory round trip in front of the owner's first cache row.
     float4 kn[EPL / 4], k_oth[EPL / 4], vn[EPL / 4];
 #pragma unroll
-    for (int u = 0; u < EPL / 4; u++) kn[u] = k_oth[u] = vn[u] = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (chunk == owner) {  // (uniform; older than the cache rows, so it does not blur the waits for them)
-#pragma unroll
-        for (int u = 0; u < EPL / 4; u++) {
-            kn[u] = *reinterpret_cast<const float4*>(k + bh * S + e0 + 4 * u);
-            k_oth[u] = *reinterpret_cast<const float4*>(k + bh * S + rope_partner(e0 + 4 * u, half));
-            vn[u] = *reinterpret_cast<const float4*>(v + bh * S + e0 + 4 * u);
-        }
+    for (int u = 0; u < EPL / 4; u++) {
+        kn[u] = *reinterpret_cast<const float4*>(krow + (uint32_t)(e0 + 4 * u));
+        k_oth[u] = *reinterpret_cast<const float4*>(krow + (uint32_t)rope_partner(e0 + 4 * u, half));
+        vn[u] = *reinterpret_cast<const float4*>(vrow + (uint32_t)(e0 + 4 * u));
     }
     __builtin_amdgcn_sched_barrier(0);
     uint4 kraw[NL], vraw[NL];
 #pragma unroll
     for (int i = 0; i < NL; i++) {
-        const int64_t p = p0 + wave * PW + i * RPW + rsel;
-        const int64_t pc = p < kvLen ? p : kvLen - 1;
-        kraw[i] = load_row16(kbase + pc * S + e0);
+        const int pc = min(p0 + wave * PW + i * RPW + rsel, kvLen - 1);
+        kraw[i] = load_row16(kbase + (uint32_t)(pc * S + e0));
     }
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int i = 0; i < NL; i++) {
-        const int64_t p = p0 + wave * PW + i * RPW + rsel;
-        const int64_t pc = p < kvLen ? p : kvLen - 1;
-        vraw[i] = load_row16(vbase + pc * S + e0);
+        const int pc = min(p0 + wave * PW + i * RPW + rsel, kvLen - 1);
+        vraw[i] = load_row16(vbase + (uint32_t)(pc * S + e0));
     }
     __builtin_amdgcn_sched_barrier(0);
     if (threadIdx.x < half) {
@@ -502,6 +505,14 @@ __global__ __launch_bounds__(NWV * 64) void attn_decode_kernel(const int32_t* __
     // the new token's row as the cache holds it (rounded to T): it is attended to from registers
     uint4 knraw = make_uint4(0, 0, 0, 0), vnraw = knraw;
     if (chunk == owner) {
+        // The new v row is only needed here, and its conversion to the cache's type must stay here: the compiler
+        // otherwise moves it up into the block that loads the row, in front of the cache rows' loads, and the
+        // owner workgroup then waits for one round trip before it asks for its first cache row.  Tying the values
+        // to something read after the barrier keeps the conversion below it.
+        const float after_barrier = cs_sh[0];
+#pragma unroll
+        for (int u = 0; u < EPL / 4; u++)
+            asm volatile("" : "+v"(vn[u].x), "+v"(vn[u].y), "+v"(vn[u].z), "+v"(vn[u].w) : "v"(after_barrier));
 #pragma unroll
         for (int u = 0; u < EPL / 4; u++) kn[u] = rope4_regs(kn[u], k_oth[u], e0 + 4 * u, cs_sh, sn_sh, half);
         knraw = RowPiece<T>::pack(kn);
@@ -509,10 +520,10 @@ __global__ __launch_bounds__(NWV * 64) void attn_decode_kernel(const int32_t* __
         __syncthreads();  // every wave has read the raw k before it is overwritten
         if (wave == 0 && rsel == 0) {
 #pragma unroll
-            for (int u = 0; u < EPL / 4; u++) *reinterpret_cast<float4*>(k + bh * S + e0 + 4 * u) = kn[u];
+            for (int u = 0; u < EPL / 4; u++) *reinterpret_cast<float4*>(krow + (uint32_t)(e0 + 4 * u)) = kn[u];
             if (slot_ok) {
-                *reinterpret_cast<uint4*>(kbase + (int64_t)slot * S + e0) = knraw;
-                *reinterpret_cast<uint4*>(vbase + (int64_t)slot * S + e0) = vnraw;
+                *reinterpret_cast<uint4*>(kbase + (uint32_t)(slot * S + e0)) = knraw;
+                *reinterpret_cast<uint4*>(vbase + (uint32_t)(slot * S + e0)) = vnraw;
             }
         }
 #pragma unroll
@@ -603,8 +614,7 @@ __global__ __launch_bounds__(NWV * 64) void attn_decode_kernel(const int32_t* __
     for (int u = 0; u < EPL / 4; u++)
         *reinterpret_cast<float4*>(&osh[wave][rsel][e0 + 4 * u]) = make_float4(o[4 * u], o[4 * u + 1], o[4 * u + 2], o[4 * u + 3]);
     __syncthreads();
-    float* rec0 = part + bh * nchunks * (S + 2);
-    float* rec = rec0 + (int64_t)chunk * (S + 2);
+    float* rec = part + ((size_t)bh * nchunks + chunk) * (S + 2);
     float mine = 0.0f;  // this thread's element of the chunk's weighted V sum (threads 0..127)
     if (threadIdx.x < S) {
 #pragma unroll
@@ -613,15 +623,15 @@ __global__ __launch_bounds__(NWV * 64) void attn_decode_kernel(const int32_t* __
             for (int r = 0; r < RPW; r++) mine += osh[w][r][threadIdx.x];
     }
     if (RECS) {
-        if (threadIdx.x < S) rec_outs[(bh * kAttnRecChunks + chunk) * S + threadIdx.x] = mine;
+        if (threadIdx.x < S) rec_outs[((size_t)bh * kAttnRecChunks + chunk) * S + threadIdx.x] = mine;
         if (threadIdx.x == 0) {
-            rec_stats[(bh * kAttnRecChunks + chunk) * 2] = stat[0];
-            rec_stats[(bh * kAttnRecChunks + chunk) * 2 + 1] = stat[1];
+            rec_stats[((size_t)bh * kAttnRecChunks + chunk) * 2] = stat[0];
+            rec_stats[((size_t)bh * kAttnRecChunks + chunk) * 2 + 1] = stat[1];
         }
         return;
     }
     if (nchunks == 1) {  // the workgroup saw every row of the head
-        if (threadIdx.x < S) q[bh * S + threadIdx.x] = mine * (1.0f / stat[1]);
+        if (threadIdx.x < S) q[(size_t)bh * S + threadIdx.x] = mine * (1.0f / stat[1]);
         return;
     }
     if (threadIdx.x < S) rec[2 + threadIdx.x] = mine;
@@ -902,12 +912,14 @@ static int attention_impl(float* q, float* k, const float* v, int64_t B, int64_t
         const int rows = records_chunk_rows(maxlen, kHalfCache);
         if (qL != 1 || (half % 4) != 0 || rows == 0) return fail(LLMOPS_EINVAL, "chunk records need one query token, half %% 4 == 0 and a cache of at most %d rows", kAttnRecChunks * (kHalfCache ? 512 : 256));
         const int nchunks = (int)((kv_plan + rows - 1) / rows);
-        const unsigned grid = (unsigned)(bhq * nchunks);
+        if (bhq > 65535 || maxlen * S * (int64_t)sizeof(T) >= ((int64_t)1 << 32))
+            return fail(LLMOPS_EINVAL, "decode attention: at most 65535 heads in all and a cache plane per head below 4 GiB");
+        const dim3 grid((unsigned)nchunks, (unsigned)bhq);
         if (rows == 256)
-            attn_decode_kernel<T, 16, 16, true><<<grid, 1024, 0, st>>>(pos_dev, position_id, nchunks, maxlen, kc, vc, slots, q, k, v,
+            attn_decode_kernel<T, 16, 16, true><<<grid, 1024, 0, st>>>(pos_dev, position_id, nchunks, (int)maxlen, kc, vc, slots, q, k, v,
                                                                        inv_freq, (int)half, nullptr, rec_stats, rec_outs);
         else if constexpr (kHalfCache)
-            attn_decode_kernel<T, 32, 16, true><<<grid, 1024, 0, st>>>(pos_dev, position_id, nchunks, maxlen, kc, vc, slots, q, k, v,
+            attn_decode_kernel<T, 32, 16, true><<<grid, 1024, 0, st>>>(pos_dev, position_id, nchunks, (int)maxlen, kc, vc, slots, q, k, v,
                                                                        inv_freq, (int)half, nullptr, rec_stats, rec_outs);
         LLMOPS_LAUNCH_CHECK();
         return LLMOPS_OK;
@@ -921,9 +933,11 @@ static int attention_impl(float* q, float* k, const float* v, int64_t B, int64_t
         const int nchunks = (int)((kv_plan + 4 * p.pw - 1) / (4 * p.pw));
         if ((int64_t)bhq * nchunks > max_records)
             return fail(LLMOPS_EWORKSPACE, "attention workspace too small for %lld chunk records", (long long)bhq * nchunks);
-        const unsigned grid = (unsigned)(bhq * nchunks);
+        if (bhq > 65535 || maxlen * S * (int64_t)sizeof(T) >= ((int64_t)1 << 32))
+            return fail(LLMOPS_EINVAL, "decode attention: at most 65535 heads in all and a cache plane per head below 4 GiB");
+        const dim3 grid((unsigned)nchunks, (unsigned)bhq);
 #define LLMOPS_DECODE(PWV)                                                                                         \
-    attn_decode_kernel<T, PWV><<<grid, 256, 0, st>>>(pos_dev, position_id, nchunks, maxlen, kc, vc, slots, q, k, v, inv_freq, \
+    attn_decode_kernel<T, PWV><<<grid, 256, 0, st>>>(pos_dev, position_id, nchunks, (int)maxlen, kc, vc, slots, q, k, v, inv_freq, \
                                                      (int)half, part)
         switch (p.pw) {
             case 4: if constexpr (!kHalfCache) LLMOPS_DECODE(4); break;

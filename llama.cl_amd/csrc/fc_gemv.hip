@@ -44,9 +44,12 @@ template <int G, int NW>
 __device__ __forceinline__ TileRange tile_range(int Kg, int S, int steps_per_split, int wave) {
     constexpr int BPS = Step<G>::kBlocksPerStep;
     TileRange r;
-    if (S == 1) {  // no division for the common case
+    if (S == 1) {  // no division for the common cases (a division is ~25 instructions in front of the first load)
         r.nb = blockIdx.x;
         r.s = 0;
+    } else if (S == 2) {
+        r.nb = blockIdx.x >> 1;
+        r.s = blockIdx.x & 1;
     } else {
         r.nb = blockIdx.x / S;
         r.s = blockIdx.x % S;
