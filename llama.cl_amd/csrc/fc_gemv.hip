@@ -40,7 +40,7 @@ struct TileRange {
     int nb, s, t0, t1;
 };
 
-template <int G, int NW>
+template <int G, int NW, int PASS = 1>
 __device__ __forceinline__ TileRange tile_range(int Kg, int S, int steps_per_split, int wave) {
     constexpr int BPS = Step<G>::kBlocksPerStep;
     TileRange r;
@@ -59,9 +59,22 @@ __device__ __forceinline__ TileRange tile_range(int Kg, int S, int steps_per_spl
     const int t_hi = min(T, t_lo + steps_per_split);
     // (unsigned: every wave runs this before it can ask for its first byte, and a signed division by NW costs
     // three scalar instructions more)
-    const int per_wave = (int)((unsigned)(t_hi - t_lo + NW - 1) / NW);
-    r.t0 = min(t_hi, t_lo + wave * per_wave);
-    r.t1 = min(t_hi, r.t0 + per_wave);
+    if constexpr (PASS == 1) {
+        const int per_wave = (int)((unsigned)(t_hi - t_lo + NW - 1) / NW);
+        r.t0 = min(t_hi, t_lo + wave * per_wave);
+        r.t1 = min(t_hi, r.t0 + per_wave);
+    } else {
+        // The kernel that quantizes on the fly works in passes of PASS steps, and a pass costs its quantization
+        // whether all of its steps are wanted or one: whole passes are dealt out, the first `rem` waves one more
+        // than the others (43 blocks of a split: 22 passes = 6 waves with two and 10 with one, instead of 14 waves
+        // with a full and a half-empty pass each).
+        const unsigned np = (unsigned)(t_hi - t_lo + PASS - 1) / PASS;
+        const unsigned q = np / NW, rem = np % NW;
+        const unsigned first = (unsigned)wave * q + min((unsigned)wave, rem);
+        const unsigned count = q + ((unsigned)wave < rem ? 1u : 0u);
+        r.t0 = min(t_hi, t_lo + (int)(first * PASS));
+        r.t1 = min(t_hi, r.t0 + (int)(count * PASS));
+    }
     return r;
 }
 
@@ -327,7 +340,7 @@ __global__ __launch_bounds__(NW * 64, (MT == 1 ? ((MODE & kAttnIn) ? NW / 4 : NW
         tr.t0 = min(T, (wave % NWS) * per_wave);
         tr.t1 = min(T, tr.t0 + per_wave);
     } else {
-        tr = tile_range<G, NW>(Kg, S, steps_per_split, wave);
+        tr = tile_range<G, NW, (G == 128) ? 2 : 4>(Kg, S, steps_per_split, wave);  // passes of 256 k-values
     }
     // (a tensor has fewer than 2^32 blocks: one 32-bit product, then one widening multiplication)
     const uint8_t* strip = weiq + (uint64_t)((uint32_t)tr.nb * (uint32_t)Kg) * (uint32_t)block_bytes(G);
