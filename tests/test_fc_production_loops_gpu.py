@@ -113,6 +113,25 @@ def test_decode_kernel_config_shapes(orc, G, N, K):
     check_dump(orc, x, wq, N, G)
 
 
+@pytest.mark.parametrize("G,N,kgs", [(128, 64, [1, 2, 3, 5, 15, 16, 17, 31, 33, 43, 86, 87, 129]),     # many k-splits
+                                     (128, 4096, [33, 43, 47, 80, 86, 87]),                            # two k-splits
+                                     (128, 8192, [33, 43, 86, 87]),                                    # none
+                                     (32, 64, [1, 3, 4, 5, 8, 9, 63, 65, 127, 344]), (32, 4096, [129, 131, 344])])
+def test_decode_kernel_pass_distribution(orc, G, N, kgs):
+    """The waves of a workgroup are dealt whole passes of 256 k-values (two blocks at group 128, eight at group
+    32), the first few one more than the rest, and the last pass of a split may be partly empty: block counts on
+    either side of every boundary of that split, with one, two and many k-splits, one and two rows."""
+    rng = np.random.default_rng(G + N)
+    for Kg in kgs:
+        K = Kg * G
+        wq = orc.quant_w((rng.standard_normal((N, K)) * 0.02).astype(np.float32), G)
+        for rows in (1, 2):
+            x = rng.standard_normal((rows, K)).astype(np.float32)
+            x[0, :8] = TIE
+            x[0, 8:G] = 0
+            check_dump(orc, x, wq, N, G)
+
+
 @pytest.mark.parametrize("rows", [3, 9, 16, 17, 32])
 @pytest.mark.parametrize("N,K", [(4096, 4096), (4096, 11008), (12288, 4096), (2080, 1024)])
 def test_streaming_mfma_kernel_int32_sums(orc, rows, N, K):
