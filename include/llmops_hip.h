@@ -193,7 +193,8 @@ size_t llmops_attention_workspace_bytes(int64_t B, int64_t qL, int64_t H, int64_
  * on fp16-rounded K/V); slots int32 [qL] (device).  Effects: q,k rotated in place (k stays
  * rotated), k,v rows written to cache[2*layer_id+{0,1}, b, h, slots[p], :], and q overwritten by
  * softmax((q.K^T)/sqrt(S) with in-chunk causal mask via slots) . V over
- * kvLen = min(position_id+qL, maxlen) cache rows. */
+ * kvLen = min(position_id+qL, maxlen) cache rows.  One query token (qL == 1, the decode form): B*H <= 65535
+ * and maxlen*S*sizeof(cache element) < 4 GiB (LLMOPS_EINVAL otherwise). */
 int llmops_attention_rope(float* q, float* k, const float* v, int64_t B, int64_t qL, int64_t H, int64_t S,
                           const float* inv_freq, int64_t half, void* kv_cache, int cache_dtype,
                           int64_t planes, int64_t maxlen, const int32_t* slots, int position_id,
