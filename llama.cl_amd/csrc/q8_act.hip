@@ -132,6 +132,44 @@ __global__ __launch_bounds__(256) void quant_x_rows_kernel(const float* __restri
     }
 }
 
+// The form the group-128 prefill FC runs: only the codes and the transposed (scale, sum) pairs [Kg][rows] that
+// its kernels read are written.  A workgroup takes 8 consecutive rows x U consecutive k-groups (a team of 32
+// threads per row): a team reads U*512 contiguous bytes and writes U*128 contiguous bytes of codes, and the 8
+// teams' pairs of one k-group are 64 contiguous bytes -- with one row per workgroup every pair was an 8-byte
+// store into a line of its own, 16 KB from the next.  Codes and scales as in quant_x_rows_kernel.
+template <int U>
+__global__ __launch_bounds__(256) void quant_x_tile128_kernel(const float* __restrict__ x, int rows, int Kg, int kparts,
+                                                               int8_t* __restrict__ xq, float2* __restrict__ xsT) {
+    constexpr int G = 128;
+    const int sub = threadIdx.x & 31, team = threadIdx.x >> 5;
+    const int rb = blockIdx.x / kparts, kp = blockIdx.x - rb * kparts;
+    const int row = rb * 8 + team, kb0 = kp * U;
+    const bool row_ok = row < rows;
+    const int64_t rbase = (int64_t)(row_ok ? row : rows - 1) * Kg;
+    float4 v[U];
+#pragma unroll
+    for (int u = 0; u < U; u++) v[u] = *reinterpret_cast<const float4*>(x + (rbase + min(kb0 + u, Kg - 1)) * G + sub * 4);
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+        float amax = fmaxf(fmaxf(fabsf(v[u].x), fabsf(v[u].y)), fmaxf(fabsf(v[u].z), fabsf(v[u].w)));
+        float s = (v[u].x + v[u].y) + (v[u].z + v[u].w);
+#pragma unroll
+        for (int o = 16; o > 0; o >>= 1) {
+            amax = fmaxf(amax, __shfl_xor(amax, o, 64));
+            s += __shfl_xor(s, o, 64);
+        }
+        const float d = amax / 127.0f;
+        const float id = (d != 0.0f) ? (1.0f / d) : 0.0f;
+        const uint32_t c = ((uint32_t)q8_code(v[u].x, id) & 0xFFu) | (((uint32_t)q8_code(v[u].y, id) & 0xFFu) << 8) |
+                           (((uint32_t)q8_code(v[u].z, id) & 0xFFu) << 16) | (((uint32_t)q8_code(v[u].w, id) & 0xFFu) << 24);
+        const int kb = kb0 + u;
+        if (row_ok && kb < Kg) {
+            *reinterpret_cast<uint32_t*>(xq + (rbase + kb) * G + sub * 4) = c;
+            if (sub == 0) xsT[(int64_t)kb * rows + row] = make_float2(d, s);
+        }
+    }
+}
+
 }  // namespace llmops
 
 using namespace llmops;
@@ -142,6 +180,19 @@ int launch_quant_x(const float* x, int64_t rows, int64_t K, int group_k, int8_t*
                    bool exact_sum, hipStream_t stream) {
     const int64_t Kg = (K + group_k - 1) / group_k;
     const int64_t items = rows * Kg;
+    if (!exact_sum && xsT != nullptr && group_k == 128 && K == Kg * group_k && aligned(x, 16) && aligned(xq, 4) &&
+        rows < ((int64_t)1 << 28) && Kg < ((int64_t)1 << 20)) {
+        // the group-128 prefill kernels read only the codes and the transposed pairs: xd and gsum stay unwritten
+        const int64_t rblocks = (rows + 7) / 8;
+        if (rblocks * ((Kg + 3) / 4) >= 1024) {  // enough workgroups with four k-groups per team
+            const int kparts = (int)((Kg + 3) / 4);
+            quant_x_tile128_kernel<4><<<(unsigned)(rblocks * kparts), 256, 0, stream>>>(x, (int)rows, (int)Kg, kparts, xq, xsT);
+        } else {
+            quant_x_tile128_kernel<1><<<(unsigned)(rblocks * Kg), 256, 0, stream>>>(x, (int)rows, (int)Kg, (int)Kg, xq, xsT);
+        }
+        LLMOPS_LAUNCH_CHECK();
+        return LLMOPS_OK;
+    }
     if (!exact_sum && K == Kg * group_k && aligned(x, 16) && aligned(xq, 4)) {  // whole groups only: vector loads
         const int64_t teams = (group_k == 32) ? 32 : 8;  // per workgroup
         if (items >= 32768) {  // enough groups to fill the chip with four per team
