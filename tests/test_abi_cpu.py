@@ -68,6 +68,10 @@ def test_argument_validation_without_device(lib):
     rc = lib.llmops_attention_rope(vp(256), vp(256), vp(256), i64(1), i64(1), i64(32), i64(64), vp(256), i64(32), vp(256), 0,
                                    i64(2), i64(16), vp(256), 0, 0, vp(256), ctypes.c_size_t(1 << 30), vp(0))
     assert rc == 1 and b"S == 128" in lib.llmops_last_error()
+    # the one-token form runs on a (chunk, head) grid: more than 65535 heads in all are refused before any launch
+    rc = lib.llmops_attention_rope(vp(256), vp(256), vp(256), i64(2200), i64(1), i64(32), i64(128), vp(256), i64(64), vp(256), 0,
+                                   i64(2), i64(16), vp(256), 3, 0, vp(256), ctypes.c_size_t(1 << 40), vp(0))
+    assert rc == 1 and b"65535 heads" in lib.llmops_last_error()
 
 
 def test_python_ops_refuse_host_tensors():
