@@ -125,7 +125,9 @@ def test_decode_kernel_pass_distribution(orc, G, N, kgs):
     for Kg in kgs:
         K = Kg * G
         wq = orc.quant_w((rng.standard_normal((N, K)) * 0.02).astype(np.float32), G)
-        for rows in (1, 2):
+        # (3..8 rows run 8-wave workgroups; with 64 strips or more and group 128 fc_Q4A sends them to the MFMA kernel,
+        # whose output check_dump could not compare bit for bit)
+        for rows in ((1, 2, 3, 5, 8) if (N < 2048 or G == 32) else (1, 2)):
             x = rng.standard_normal((rows, K)).astype(np.float32)
             x[0, :8] = TIE
             x[0, 8:G] = 0
