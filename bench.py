@@ -170,6 +170,8 @@ def main():
                                 "on some boxes (sporadic host-side segmentation fault under hipGraphLaunch)"}
             del weights, graph
         floor_us = dispatch_floor(torch, stream)
+        read_chain = read_only_chain(torch, llmops, stream,
+                                     [(sum(SHAPE[p][0] for p in parts), SHAPE[parts[0]][1]) for _, parts in FUSED_PLAN])
     ceiling_gbs = read_ceiling(torch, llmops)
     setup_s = time.time() - t0
 
@@ -185,10 +187,10 @@ def main():
                                "stale": kernel_source_sha16() != MEASURED_TRAFFIC_KERNEL_SHA16},
             "avg_launch_us": round(avg_us, 3), "launches_per_step": main_r["launches"],
             "bytes_per_launch_avg": int(step_bytes / main_r["launches"]), "per_shape": per_shape,
-            "dispatch_floor_us": round(floor_us, 3),
+            "dispatch_floor_us": round(floor_us, 3), "read_only_chain": read_chain,
             "read_ceiling": {"GB/s": round(ceiling_gbs, 1), "frac_of_it": round(achieved / ceiling_gbs, 4),
-                             "what": "plain read kernel (16-byte loads) over 2 GiB, one launch: what this part's HBM "
-                                     "delivers to a kernel that does nothing else"},
+                             "what": "plain read kernel (16-byte non-temporal loads, contiguous slab per workgroup) over "
+                                     "2 GiB, one launch: what this part's HBM delivers to a kernel that does nothing else"},
             "timing": "HIP events on the launch stream around the timed graph replays; every node of the graph is this "
                       "kernel, so the average includes the dispatch gap between dependent launches (dispatch_floor_us)"}
     out = {
@@ -317,6 +319,45 @@ def dispatch_floor(torch, stream, n=64, reps=10):
     e1.record(stream)
     torch.cuda.synchronize()
     return e0.elapsed_time(e1) * 1e3 / (n * reps)
+
+
+def read_only_chain(torch, llmops, stream, dims, layers=32, reps=10):
+    """The plain read kernel (non-temporal 16-byte loads, a slab per workgroup) in the launch structure of `value`:
+    a graph of dependent launches over `layers` distinct buffers of each FC tensor's size.  What a kernel that only
+    reads reaches in this chain; the FC kernel's quantization, products, reduction and stores come on top."""
+    import ctypes
+    lib = llmops._lib.load()
+    out4 = torch.zeros(4, dtype=torch.int32, device="cuda")
+    sizes = [fc_bytes(N, K) // 16 * 16 for (N, K) in dims]
+    stride = (max(sizes) + 4095) // 4096 * 4096
+    pool = torch.zeros(layers * stride, dtype=torch.uint8, device="cuda")
+    st = ctypes.c_void_p(stream.cuda_stream)
+    per_shape, total = {}, 0.0
+    for (N, K), nbytes in zip(dims, sizes):
+        best = None
+        for wgs in (512, 1024, 2048):
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g, stream=stream):
+                for l in range(layers):
+                    llmops._lib.check(lib.llmops_test_calib_read(pool.data_ptr() + l * stride, nbytes, wgs, out4.data_ptr(), st))
+            for _ in range(3):
+                g.replay()
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(stream)
+            for _ in range(reps):
+                g.replay()
+            e1.record(stream)
+            torch.cuda.synchronize()
+            us = e0.elapsed_time(e1) * 1e3 / (reps * layers)
+            best = us if best is None else min(best, us)
+            del g
+        per_shape[f"{N}x{K}"] = round(best, 3)
+        total += best
+    layer_bytes = sum(fc_bytes(N, K) for (N, K) in dims)
+    return {"us_per_layer": round(total, 2), "GB/s": round(layer_bytes / total / 1e3, 1), "us_per_shape": per_shape,
+            "what": "plain read kernel over buffers of the FC tensors' sizes, same graph of dependent launches (best of "
+                    "512/1024/2048 workgroups per size)"}
 
 
 def decode_step(torch, stream, kv_len=2048, reps=20):

@@ -6,19 +6,23 @@
 
 namespace llmops {
 
-// each workgroup streams a contiguous slab; 16-byte accesses, UNROLL loads in flight per lane
+// each workgroup streams a contiguous slab; 16-byte non-temporal accesses (what the FC and attention kernels use for
+// bytes they read once; on 2 GiB: 7.0 TB/s against 6.0-6.2 TB/s with plain loads and 5.2-6.1 TB/s with a grid-stride
+// pattern instead of slabs), UNROLL loads in flight per lane
+typedef unsigned int calib_u32x4 __attribute__((ext_vector_type(4)));
 template <int UNROLL>
-__global__ __launch_bounds__(256) void calib_read_kernel(const uint4* __restrict__ src, int64_t n16, uint32_t* out) {
+__global__ __launch_bounds__(256) void calib_read_kernel(const calib_u32x4* __restrict__ src, int64_t n16, uint32_t* out) {
     const int64_t per_wg = (n16 + gridDim.x - 1) / gridDim.x;
     const int64_t lo = (int64_t)blockIdx.x * per_wg;
     const int64_t hi = lo + per_wg < n16 ? lo + per_wg : n16;
     uint32_t acc = 0;
     for (int64_t i = lo + threadIdx.x; i < hi; i += 256 * UNROLL) {
-        uint4 v[UNROLL];
+        calib_u32x4 v[UNROLL];
 #pragma unroll
         for (int u = 0; u < UNROLL; u++) {
             const int64_t j = i + (int64_t)u * 256;
-            v[u] = j < hi ? src[j] : make_uint4(0, 0, 0, 0);
+            if (j < hi) v[u] = __builtin_nontemporal_load(src + j);
+            else v[u] = calib_u32x4{0, 0, 0, 0};
         }
 #pragma unroll
         for (int u = 0; u < UNROLL; u++) acc ^= v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
@@ -40,7 +44,7 @@ using namespace llmops;
 extern "C" int llmops_test_calib_read(const void* src, int64_t bytes, int workgroups, void* out4, llmops_stream_t stream) {
     LLMOPS_REQUIRE(src != nullptr && out4 != nullptr && bytes > 0 && (bytes % 16) == 0 && workgroups > 0);
     LLMOPS_REQUIRE(aligned(src, 16));
-    calib_read_kernel<4><<<(unsigned)workgroups, 256, 0, as_stream(stream)>>>(reinterpret_cast<const uint4*>(src), bytes / 16,
+    calib_read_kernel<4><<<(unsigned)workgroups, 256, 0, as_stream(stream)>>>(reinterpret_cast<const calib_u32x4*>(src), bytes / 16,
                                                                               reinterpret_cast<uint32_t*>(out4));
     LLMOPS_LAUNCH_CHECK();
     return LLMOPS_OK;
