@@ -30,7 +30,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 # of `--calib` (one FETCH_SIZE count = 2.000 KiB, one WRITE_SIZE count = 1.000 KiB on this part); the summary with
 # the per-shape figures is profiles/fc_gemv_fused_kernel__hbm_traffic_pmc.md.  Counters cannot be read from inside
 # this process, so the figure is the recorded one and only holds for the fused plan at group 128, M=1.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 27191817
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 27191830
 MEASURED_TRAFFIC_PROFILE = "profiles/fc_gemv_fused_kernel__hbm_traffic_pmc.md"
 # sha256 (first 16 hex digits) of the kernel's sources (csrc/fc_gemv.hip + csrc/gemv_device.h) when the counters were
 # read: the bench line says whether the sources have changed since, i.e. whether the recorded figure is stale
