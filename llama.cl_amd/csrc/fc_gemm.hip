@@ -268,6 +268,12 @@ __device__ __forceinline__ void splitk_finish(const v4f (&f)[RT][4], float* __re
 constexpr int kAStride = 144;
 constexpr int kBlk128 = 2176;
 
+__device__ __forceinline__ v2f buf_ld_pair(buffer_rsrc r, uint32_t voff, uint32_t soff) {
+    typedef unsigned int u32x2_g __attribute__((ext_vector_type(2)));
+    const u32x2_g t = __builtin_amdgcn_raw_buffer_load_b64(r, voff, soff, 0);
+    return v2f{__uint_as_float(t.x), __uint_as_float(t.y)};
+}
+
 template <int RT>
 struct GemmSmem {
     static constexpr int BM = RT * 32;
@@ -322,31 +328,40 @@ __global__ __launch_bounds__(256, (RT == 4 ? 2 : (RT == 2 ? 3 : 4))) void fc_gem
     // ---- global -> register staging of one k-group (macros: the arrays must stay in registers) ----
     v4u ra[A_PER_THREAD], rb[B_PER_THREAD];  // native vector types: these must live in registers
     v2f rxs = {0.f, 0.f};
-    // per-thread source addresses that do not depend on kb
-    const int8_t* asrc[A_PER_THREAD];
+    // Source addresses: buffer descriptors whose base is the same for the whole workgroup, a scalar offset that advances
+    // with kb, and a 32-bit offset per thread that does not depend on kb: no 64-bit address arithmetic in the loop,
+    // which is bound by instruction issue (128 rows, 4096 -> 11008: 26.65 -> 26.2 us).
+    const buffer_rsrc a_rs = make_rsrc(xq + (int64_t)row0 * Kp, (uint32_t)min(BM, rows - row0) * (uint32_t)Kp);
+    const buffer_rsrc b_rs = make_rsrc(weiq + (int64_t)strip0 * Kg * kBlk128, (uint32_t)min(4, Ng - strip0) * (uint32_t)Kg * (uint32_t)kBlk128);
+    const buffer_rsrc x_rs = make_rsrc(xsT != nullptr ? xsT : reinterpret_cast<const float2*>(xq), xsT != nullptr ? (uint32_t)Kg * (uint32_t)rows * 8u : 0u);
+    uint32_t aoff[A_PER_THREAD];
     int adst[A_PER_THREAD];
 #pragma unroll
     for (int i = 0; i < A_PER_THREAD; i++) {
         const int c = tid + i * 256, r = c >> 3, part = c & 7;
-        asrc[i] = xq + (int64_t)min(rows - 1, row0 + r) * Kp + part * 16;
+        aoff[i] = (uint32_t)(min(rows - 1, row0 + r) - row0) * (uint32_t)Kp + (uint32_t)(part * 16);
         adst[i] = r * kAStride + part * 16;
     }
-    const uint8_t* bsrc[B_PER_THREAD];
+    uint32_t boff[B_PER_THREAD];
 #pragma unroll
     for (int i = 0; i < B_PER_THREAD; i++) {
         const int c = min(B_CHUNKS - 1, tid + i * 256);
         const int st = c / (kBlk128 / 16), off = c % (kBlk128 / 16);
-        bsrc[i] = weiq + (int64_t)min(Ng - 1, strip0 + st) * Kg * kBlk128 + off * 16;
+        boff[i] = (uint32_t)(min(Ng - 1, strip0 + st) - strip0) * (uint32_t)Kg * (uint32_t)kBlk128 + (uint32_t)(off * 16);
     }
     const int64_t xrow = min(rows - 1, row0 + (tid < BM ? tid : 0));
 #define LLMOPS_FETCH(KB)                                                                                              \
     do {                                                                                                              \
-        _Pragma("unroll") for (int i = 0; i < A_PER_THREAD; i++)                                                      \
-            ra[i] = *reinterpret_cast<const v4u*>(asrc[i] + (int64_t)(KB) * 128);                                     \
-        _Pragma("unroll") for (int i = 0; i < B_PER_THREAD; i++)                                                      \
-            rb[i] = *reinterpret_cast<const v4u*>(bsrc[i] + (int64_t)(KB) * kBlk128); /* clamped address */            \
+        _Pragma("unroll") for (int i = 0; i < A_PER_THREAD; i++) {                                                    \
+            const u32x4 t_ = __builtin_amdgcn_raw_buffer_load_b128(a_rs, aoff[i], (uint32_t)(KB) * 128u, 0);          \
+            ra[i] = v4u{t_.x, t_.y, t_.z, t_.w};                                                                      \
+        }                                                                                                             \
+        _Pragma("unroll") for (int i = 0; i < B_PER_THREAD; i++) { /* clamped offset */                               \
+            const u32x4 t_ = __builtin_amdgcn_raw_buffer_load_b128(b_rs, boff[i], (uint32_t)(KB) * (uint32_t)kBlk128, 0); \
+            rb[i] = v4u{t_.x, t_.y, t_.z, t_.w};                                                                      \
+        }                                                                                                             \
         if (!PARTIALS)                                                                                                \
-            rxs = xsT ? *reinterpret_cast<const v2f*>(&xsT[(int64_t)(KB) * rows + xrow])                             \
+            rxs = xsT ? buf_ld_pair(x_rs, (uint32_t)xrow * 8u, (uint32_t)(KB) * (uint32_t)rows * 8u)                  \
                       : v2f{xd[xrow * Kg + (KB)], gs[xrow * Kg + (KB)]};                                            \
     } while (0)
 #define LLMOPS_STASH(BUF)                                                                                  \
