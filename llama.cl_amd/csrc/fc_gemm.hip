@@ -1090,6 +1090,9 @@ static int launch_gemm_lds_t(const uint8_t* w, const int8_t* xq, const float* xd
                                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(GemmSmem<RT>)));
         configured = true;
     }
+    // (the kernel's staging loads take 32-bit offsets into the scale pairs [Kg][rows] and into a tile's rows)
+    if (rows * Kg * 8 >= ((int64_t)1 << 32) || Kg * 128 * 128 >= ((int64_t)1 << 32))
+        return fail(LLMOPS_EINVAL, "fc_Q4A: rows * Kg must be below 2^29 for the tiled kernel");
     const int64_t tiles = ((Ng + 3) / 4) * ((rows + RT * 32 - 1) / (RT * 32));
     dim3 grid((unsigned)(8 * ((tiles + 7) / 8)), 1, (unsigned)p.S);  // one run of tiles per XCD
     fc_gemm_lds_kernel<RT, false><<<grid, 256, sizeof(GemmSmem<RT>), st>>>(w, xq, xd, gs, xsT, out, nullptr, (int)Ng, (int)Kg,
