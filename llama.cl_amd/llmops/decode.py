@@ -24,21 +24,26 @@ LLAMA_7B = dict(layer_num=32, head_num=32, head_size=128, hidden_size=4096, inte
 
 
 class LlamaDecoder:
-    def __init__(self, configs=None, group_k=128, seed=5, device="cuda", plan="fused", embed_rows=None):
+    def __init__(self, configs=None, group_k=128, seed=5, device="cuda", plan="fused", embed_rows=None, device_rng=False):
+        """``device_rng``: draw the random weights on the device (much faster for the full-size model; the values
+        then differ from the host generator's for the same seed)."""
         cfg = dict(LLAMA_7B)
         cfg.update(configs or {})
         self.configs = cfg
         self.plan = plan
         self.merge_in_o_proj = True  # fused plan, one token: the o projection merges the attention chunks
         self.device = torch.device(device)
-        gen = torch.Generator(device="cpu").manual_seed(seed)
+        gen = torch.Generator(device=self.device if device_rng else "cpu").manual_seed(seed)
         H, F, V = cfg["hidden_size"], cfg["intermediate_size"], cfg["vocab_size"]
+
+        def randn(*shape):
+            return torch.randn(*shape, generator=gen, device=gen.device).to(self.device)
 
         def fc(N, K, parts=1):
             # parts > 1: several projections sharing one input, packed and concatenated along N
             packed = []
             for _ in range(parts):
-                w = (torch.randn(N, K, generator=gen) * 0.02).to(self.device)
+                w = randn(N, K) * 0.02
                 packed.append(llmops.offline_FC_quant_Q4A(w, group_k))
                 del w
             t = torch.cat(packed, dim=0) if parts > 1 else packed[0]
@@ -70,7 +75,7 @@ class LlamaDecoder:
         self.lm_head = fc(V, H)
         # the embedding table is only gathered from (one row per token); a small table suffices for timing
         rows = V if embed_rows is None else embed_rows
-        self.embed_tokens = llmop_embedding_q8c((torch.randn(rows, H, generator=gen)).to(self.device))
+        self.embed_tokens = llmop_embedding_q8c(randn(rows, H))
         rd = cfg["head_size"]
         inv_freq = 1.0 / (cfg["rope_base"] ** (torch.arange(0, rd, 2).float() / rd))  # chatllama/main.py:294-296
         self.inv_freq = inv_freq.to(self.device)
@@ -140,7 +145,8 @@ class LlamaDecoder:
         return self
 
     def fc_weight_size(self):
-        n = 0
+        """bytes of every packed FC tensor a step streams: the layers' projections and the lm_head"""
+        n = self.lm_head.weight_size()
         for layer in self.layers:
             n += sum(op.weight_size() for op in layer.values() if isinstance(op, llmop_fc_q4a))
         return n

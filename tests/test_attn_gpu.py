@@ -437,9 +437,19 @@ def test_attention_records_merged_by_the_o_projection(ops, orc, cache_dtype, max
             diff = host(xq).astype(np.int32) - oq.astype(np.int32)
             assert np.abs(diff).max() <= 1 and np.count_nonzero(diff) <= 8, (kv, np.count_nonzero(diff))
             assert np.array_equal(host(acc), orc.fc_partials(host(xq), pw))
+            # ... and its fold: y = sum over k-groups of (d*dx)*acc + m*gsum (ops/op_fc.hpp:381-412) evaluated in
+            # fp64 on the kernel's OWN scales, group sums and int32 sums
+            blocks = np.ascontiguousarray(pw).view(np.uint8)
+            wd = blocks[:, :, G // 8 * 128:G // 8 * 128 + 64].copy().view(np.float16).astype(np.float64)      # [Ng, Kg, 32]
+            wm = blocks[:, :, G // 8 * 128 + 64:].copy().view(np.float16).astype(np.float64)
+            wd, wm = wd.transpose(0, 2, 1).reshape(Ng * 32, Kg), wm.transpose(0, 2, 1).reshape(Ng * 32, Kg)
+            dx, sums = host(xd).astype(np.float64)[0], host(gs).astype(np.float64)[0]
+            folded = (wd * dx[None, :] * host(acc)[0].astype(np.float64) + wm * sums[None, :]).sum(1)
+            assert max_rel_err(host(y)[0], folded[:N]) <= 1e-5, (kv, dev_pos)
             # (3) outputs
             yf, ss = ops.fc_Q4A_decode(None, wq, N, residual=dev(res), want_sumsq=True, attn_records=recs)
             assert np.array_equal(host(yf)[0], host(y) + res[0])            # production build == dump build (+ residual)
+            print("records-vs-unfused", cache_dtype, maxlen, kv, dev_pos, max_rel_err(host(yf), host(want_y)), max_rel_err(host(ss), host(want_ss)))
             assert max_rel_err(host(yf), host(want_y)) <= 1e-2, (kv, dev_pos)
             assert max_rel_err(host(ss), host(want_ss)) <= 2e-2
         if cache_dtype == torch.float32 and kv in (257, 2048):              # and the oracle's two ops

@@ -12,8 +12,9 @@ CFG = dict(layer_num=2, head_num=2, head_size=128, hidden_size=256, intermediate
            rms_norm_eps=1e-5, rope_base=10000.0)
 
 
-def oracle_forward(orc, model, ids, cache, slots, pos):
+def oracle_forward(orc, model, ids, cache, slots, pos, cfg=None):
     """Same op sequence with oracle ops on host copies of the model's packed weights."""
+    CFG = cfg or globals()["CFG"]
     H, F = CFG["hidden_size"], CFG["intermediate_size"]
 
     def w(op):
