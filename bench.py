@@ -20,6 +20,9 @@ import os
 import sys
 import time
 
+# the plain read / copy kernels behind `read_ceiling`, `read_only_chain` and `--calib` are test hooks of the library
+os.environ.setdefault("LLMOPS_TEST_HOOKS", "1")
+
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 sys.path.insert(0, os.path.join(ROOT, "llama.cl_amd"))
@@ -90,16 +93,23 @@ def main():
     ap.add_argument("--no-decode", action="store_true", help="skip the full decode-step timing (BASELINE config 5)")
     ap.add_argument("--no-extra", action="store_true", help="skip the prefill GEMM (config 3) and attention (config 4) legs")
     ap.add_argument("--concurrent", action="store_true",
-                    help="also run the FC set on 2-4 concurrent streams inside one graph (not `value`).  Opt-in: replaying "
-                         "a graph with several branches has crashed inside the HIP runtime on some boxes (a sporadic "
-                         "host-side segmentation fault under hipGraphLaunch), and a crash would lose the whole line")
-    ap.add_argument("--no-concurrent", action="store_true", help="accepted and ignored (the leg is opt-in, see --concurrent)")
+                    help="refused: the leg that dealt the FC set to 2-4 streams inside one graph is switched off (replaying "
+                         "such a multi-branch graph ended twice in a host-side segmentation fault under hipGraphLaunch and "
+                         "no cause has been shown)")
+    ap.add_argument("--no-concurrent", action="store_true", help="accepted and ignored (that leg no longer exists)")
     ap.add_argument("--calib", action="store_true",
                     help="only run the plain copy/read kernels over 1 GiB (reference points for traffic counters and "
                          "for the attainable HBM rate) and print their rates")
     args = ap.parse_args()
     if args.calib:
         return calib()
+    if args.concurrent:
+        print("bench.py: --concurrent is switched off. The leg replayed one HIP graph with 2-4 branches (the FC set dealt "
+              "to side streams); twice in about twenty runs that replay ended in a host-side segmentation fault under "
+              "hipGraphLaunch (the fault handler named graph.replay() of that leg). During a replay no code of this "
+              "repository runs on the host, no cause has been shown, and the case must not be run again before one is. "
+              "The product captures single-branch graphs only.", file=sys.stderr)
+        sys.exit(2)
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU (the path is data-parallel per GPU; nothing here uses a second "
               "one). Re-run with --gpus 1.", file=sys.stderr)
@@ -165,9 +175,6 @@ def main():
                               "launches": LAYERS * len(plan)}
             if label == "fused":
                 per_shape = measure_shapes(torch, llmops, plan, dims, weights, xs, stream)
-                overlapped = concurrent_streams(torch, llmops, dims, weights, xs, stream, step_bytes) if args.concurrent else \
-                    {"skipped": "opt-in (--concurrent): replaying a multi-branch graph has crashed inside the HIP runtime "
-                                "on some boxes (sporadic host-side segmentation fault under hipGraphLaunch)"}
             del weights, graph
         floor_us = dispatch_floor(torch, stream)
         read_chain = read_only_chain(torch, llmops, stream,
@@ -214,7 +221,6 @@ def main():
         "pct_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
         "unfused_7_launches_per_layer": {"GB/s": round(step_bytes / (results["unfused"]["ms_per_step"] * 1e-3) / 1e9, 2),
                                          "ms_per_step": round(results["unfused"]["ms_per_step"], 4)},
-        "independent_fcs_on_concurrent_streams": overlapped,
         "roofline": roof,
     }
     if not args.no_decode:
@@ -260,47 +266,6 @@ def measure_shapes(torch, llmops, plan, dims, weights, xs, stream, reps=10):
         per_shape[f"{name} {N}x{K}"] = {"us": round(us, 3), "GB/s": round(b / us / 1e3, 1), "bytes": b}
         del g
     return per_shape
-
-
-def concurrent_streams(torch, llmops, dims, weights, xs, stream, step_bytes, reps=10):
-    """The same FC set with the layers dealt to 2-4 streams inside one graph.  The benchmark's FCs have no data
-    dependence on each other (each takes the synthetic x); a decode step has, so this is NOT `value`: it shows what
-    the kernel sustains once one launch's start-up and drain are covered by another launch's stream of weights."""
-    out = {}
-    for n in (2, 3, 4):
-        side = [torch.cuda.Stream() for _ in range(n - 1)]
-        lanes = [stream] + side
-
-        def run_step():
-            for s in side:
-                s.wait_stream(stream)
-            for layer in range(LAYERS):
-                with torch.cuda.stream(lanes[layer % n]):
-                    for (N, K), wq in zip(dims, weights[layer]):
-                        llmops.fc_Q4A(xs[K], wq, N)
-            for s in side:
-                stream.wait_stream(s)
-
-        run_step()  # each stream gets its own workspace before anything is captured
-        torch.cuda.synchronize()
-        g = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(g, stream=stream):
-            run_step()
-        g.replay()
-        torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record(stream)
-        for _ in range(reps):
-            g.replay()
-        e1.record(stream)
-        torch.cuda.synchronize()
-        ms = e0.elapsed_time(e1) / reps
-        out[f"{n}_streams"] = {"ms_per_step": round(ms, 4), "GB/s": round(step_bytes / ms / 1e6, 1),
-                               "pct_hbm_peak": round(100.0 * step_bytes / ms / 1e6 / HBM_PEAK_GBS, 2)}
-        del g
-    out["note"] = ("layers dealt round-robin to n streams in one HIP graph; FCs of different streams overlap. Not the "
-                   "headline value: in a decode step every FC waits for the one before it")
-    return out
 
 
 def dispatch_floor(torch, stream, n=64, reps=10):

@@ -105,6 +105,14 @@ int llmops_fc_Q4A(const float* x, int64_t rows, int64_t K, const int8_t* weiq, i
                   int group_k, int64_t N, float* y, void* workspace, size_t workspace_bytes,
                   llmops_stream_t stream);
 
+/* Zero the hand-off area at the head of an FC or attention workspace (arrival counters, exchange slots: the first
+ * min(workspace_bytes, LLMOPS_FC_COUNTER_BYTES) bytes) with a fill kernel on `stream`.  The kernels leave that area
+ * zero after every call that runs to its end; a launch that did not (a device error in the middle of an op) may
+ * leave parked values behind, after which two k-splits no longer meet and outputs are wrong.  Call this once, with no
+ * op in flight on the workspace, before using it again.  No counterpart in the reference (its scratch is host
+ * memory owned by one call). */
+int llmops_fc_workspace_reset(void* workspace, size_t workspace_bytes, llmops_stream_t stream);
+
 /* fc_Q4A for callers that cannot allocate device memory or carry a workspace around: code under HIP
  * graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the
  * reference.  Same arguments, kernels and results as llmops_fc_Q4A, but the workspace is a fixed array of
@@ -193,8 +201,9 @@ size_t llmops_attention_workspace_bytes(int64_t B, int64_t qL, int64_t H, int64_
  * on fp16-rounded K/V); slots int32 [qL] (device).  Effects: q,k rotated in place (k stays
  * rotated), k,v rows written to cache[2*layer_id+{0,1}, b, h, slots[p], :], and q overwritten by
  * softmax((q.K^T)/sqrt(S) with in-chunk causal mask via slots) . V over
- * kvLen = min(position_id+qL, maxlen) cache rows.  One query token (qL == 1, the decode form): B*H <= 65535
- * and maxlen*S*sizeof(cache element) < 4 GiB (LLMOPS_EINVAL otherwise). */
+ * kvLen = min(position_id+qL, maxlen) cache rows.  One query token (qL == 1, the decode form) needs
+ * maxlen*S*sizeof(cache element) < 4 GiB (LLMOPS_EINVAL otherwise); more than 65535 heads in all (B*H) are served
+ * by the general kernels (three launches instead of two). */
 int llmops_attention_rope(float* q, float* k, const float* v, int64_t B, int64_t qL, int64_t H, int64_t S,
                           const float* inv_freq, int64_t half, void* kv_cache, int cache_dtype,
                           int64_t planes, int64_t maxlen, const int32_t* slots, int position_id,
@@ -218,6 +227,11 @@ int llmops_attention_rope_decode(float* q, float* k, const float* v, int64_t B, 
  * position_id_dev is not NULL, the int32 it points at in device memory.  llmops_attention_records_chunks returns 8
  * when a cache of `maxlen` rows can be served this way (fp32: up to 2048 rows, fp16: up to 4096), else 0. */
 int64_t llmops_attention_records_chunks(int64_t maxlen, int cache_dtype);
+/* cache rows that one chunk record of llmops_attention_rope_decode_records covers for a cache of `maxlen` rows (0: such
+ * a cache cannot be served this way).  A call at kv length L writes ceil(L / rows) records per head -- with the
+ * position in device memory ceil(maxlen / rows), empty ones (sum 0) beyond the current length included -- and that
+ * count is the `chunks` argument of llmops_fc_Q4A_decode_attn. */
+int64_t llmops_attention_records_chunk_rows(int64_t maxlen, int cache_dtype);
 int llmops_attention_rope_decode_records(float* q, float* k, const float* v, int64_t B, int64_t H, int64_t S,
                                          const float* inv_freq, int64_t half, void* kv_cache, int cache_dtype,
                                          int64_t planes, int64_t maxlen, const int32_t* slot, int position_id,

@@ -2,7 +2,9 @@
  *
  * None of these has a counterpart in the reference and none is part of the product ABI
  * (include/llmops_hip.h): they change process-wide planner state or run measurement kernels, so a
- * program that serves requests must not call them.  Tests flip a knob, run one op, and restore the
+ * program that serves requests must not call them -- and cannot by accident: every hook is refused
+ * (LLMOPS_EINVAL; the setters do nothing and say so once on stderr) unless the process was started with
+ * the environment variable LLMOPS_TEST_HOOKS=1, which the tests and bench.py set.  Tests flip a knob, run one op, and restore the
  * default in a finally block; bench.py uses the read/copy kernels for the measured HBM ceiling and
  * to calibrate the traffic counters.
  */
@@ -35,6 +37,10 @@ void llmops_test_fc_set_tuning(int target_workgroups, int waves_per_workgroup);
  * MFMA and fold phases, which the planner takes from 512 rows on); 0 = choose per shape; -1 = choose
  * per shape and send 9..16 rows to the tiled kernel too instead of the weight-streaming MFMA kernel */
 void llmops_test_gemm_set_tuning(int row_tile_factor);
+
+/* prefill GEMM, 256-row tiles: 1 (default) the kernel whose wavefronts interleave the fold with the MFMAs, 0 the
+ * kernel with two wave groups in alternating phases; kept for comparisons */
+void llmops_test_gemm_set_interleaved(int on);
 
 /* prefill GEMM with split-K: the product kernel adds the partial sums itself (the last split of a tile to
  * arrive adds all of them in index order) when the split count is at most 12 x in_kernel; otherwise, and

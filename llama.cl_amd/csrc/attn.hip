@@ -924,7 +924,9 @@ static int attention_impl(float* q, float* k, const float* v, int64_t B, int64_t
         LLMOPS_LAUNCH_CHECK();
         return LLMOPS_OK;
     }
-    if (qL == 1 && (half % 4) == 0) {
+    // (the decode kernels index heads with the grid's y dimension: more than 65535 heads in all take the general
+    // path below, which the position in device memory cannot)
+    if (qL == 1 && (half % 4) == 0 && (bhq <= 65535 || pos_dev != nullptr)) {
         // decode: rope, cache update and split-KV attention in one launch, then the merge of the chunk records
         // (none when a head has a single chunk).  With the position in device memory the launch is sized for a
         // full cache.
@@ -1032,6 +1034,10 @@ extern "C" int64_t llmops_attention_records_chunks(int64_t maxlen, int cache_dty
     return records_chunk_rows(maxlen, cache_dtype == LLMOPS_CACHE_F16) ? kAttnRecChunks : 0;
 }
 
+extern "C" int64_t llmops_attention_records_chunk_rows(int64_t maxlen, int cache_dtype) {
+    return records_chunk_rows(maxlen, cache_dtype == LLMOPS_CACHE_F16);
+}
+
 extern "C" int llmops_attention_rope_decode_records(float* q, float* k, const float* v, int64_t B, int64_t H, int64_t S,
                                                     const float* inv_freq, int64_t half, void* kv_cache, int cache_dtype,
                                                     int64_t planes, int64_t maxlen, const int32_t* slot, int position_id,
@@ -1043,7 +1049,9 @@ extern "C" int llmops_attention_rope_decode_records(float* q, float* k, const fl
                            position_id_dev, layer_id, workspace, workspace_bytes, stream, rec_stats, rec_outs);
 }
 
-extern "C" void llmops_test_attn_set_decode_plan(int rows_per_wave) { llmops::g_decode_pw = rows_per_wave; }
+extern "C" void llmops_test_attn_set_decode_plan(int rows_per_wave) {
+    if (llmops::test_hooks_enabled("llmops_test_attn_set_decode_plan")) llmops::g_decode_pw = rows_per_wave;
+}
 
 extern "C" int llmops_softmax(float* x, int64_t rows, int64_t K, llmops_stream_t stream) {
     LLMOPS_REQUIRE(x != nullptr && rows > 0 && K > 0 && rows < ((int64_t)1 << 31));

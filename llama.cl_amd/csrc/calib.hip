@@ -42,6 +42,7 @@ __global__ __launch_bounds__(256) void calib_copy_kernel(const uint4* __restrict
 using namespace llmops;
 
 extern "C" int llmops_test_calib_read(const void* src, int64_t bytes, int workgroups, void* out4, llmops_stream_t stream) {
+    LLMOPS_TEST_HOOK();
     LLMOPS_REQUIRE(src != nullptr && out4 != nullptr && bytes > 0 && (bytes % 16) == 0 && workgroups > 0);
     LLMOPS_REQUIRE(aligned(src, 16));
     calib_read_kernel<4><<<(unsigned)workgroups, 256, 0, as_stream(stream)>>>(reinterpret_cast<const calib_u32x4*>(src), bytes / 16,
@@ -51,6 +52,7 @@ extern "C" int llmops_test_calib_read(const void* src, int64_t bytes, int workgr
 }
 
 extern "C" int llmops_test_calib_copy(const void* src, void* dst, int64_t bytes, int workgroups, llmops_stream_t stream) {
+    LLMOPS_TEST_HOOK();
     LLMOPS_REQUIRE(src != nullptr && dst != nullptr && bytes > 0 && (bytes % 16) == 0 && workgroups > 0);
     LLMOPS_REQUIRE(aligned(src, 16) && aligned(dst, 16));
     calib_copy_kernel<<<(unsigned)workgroups, 256, 0, as_stream(stream)>>>(reinterpret_cast<const uint4*>(src),

@@ -33,6 +33,13 @@ struct DumpBufs {
 // ---- error reporting ------------------------------------------------------------------------
 std::string& last_error();
 int fail(int code, const char* fmt, ...);
+// true if the process was started with LLMOPS_TEST_HOOKS=1; otherwise records why `hook` was refused (and says so
+// once on stderr) and returns false
+bool test_hooks_enabled(const char* hook);
+#define LLMOPS_TEST_HOOK()                                                                            \
+    do {                                                                                            \
+        if (!::llmops::test_hooks_enabled(__func__)) return LLMOPS_EINVAL;                          \
+    } while (0)
 
 #define LLMOPS_REQUIRE(cond)                                                                        \
     do {                                                                                            \

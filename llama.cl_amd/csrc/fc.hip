@@ -70,18 +70,27 @@ extern "C" size_t llmops_fc_Q4A_workspace_bytes(int64_t rows, int64_t K, int64_t
 // on the fly: tensors of up to 256 strips / of more
 static int g_rows_from_small = 4, g_rows_from_large = 3;
 
-static int fc_impl(const float* x, int64_t rows, int64_t K, const int8_t* weiq, int64_t Ng, int64_t Kg, int group_k,
-                   int64_t N, const float* residual, float* y, void* workspace, size_t workspace_bytes,
-                   llmops_stream_t stream) {
+// argument checks of fc_Q4A that do not involve the workspace
+static int fc_check_args(const float* x, int64_t rows, int64_t K, const int8_t* weiq, int64_t Ng, int64_t Kg, int group_k,
+                         int64_t N, const float* y) {
     LLMOPS_REQUIRE(valid_group(group_k));
-    LLMOPS_REQUIRE(x != nullptr && weiq != nullptr && y != nullptr && workspace != nullptr);
+    LLMOPS_REQUIRE(x != nullptr && weiq != nullptr && y != nullptr);
     LLMOPS_REQUIRE(rows > 0 && K > 0 && Ng > 0 && Kg > 0);
     LLMOPS_REQUIRE(K > (Kg - 1) * group_k && K <= Kg * group_k);  // a short last k-group is zero padded (ops/op_fc.hpp:259-261)
     LLMOPS_REQUIRE(N > (Ng - 1) * kGroupN && N <= Ng * kGroupN);
     LLMOPS_REQUIRE(Ng <= kTicketBytes / 4);
     LLMOPS_REQUIRE(Ng * 64 < ((int64_t)1 << 31));
+    LLMOPS_REQUIRE(aligned(weiq, 16) && aligned(x, K != Kg * group_k ? 4 : 8));
+    return LLMOPS_OK;
+}
+
+static int fc_impl(const float* x, int64_t rows, int64_t K, const int8_t* weiq, int64_t Ng, int64_t Kg, int group_k,
+                   int64_t N, const float* residual, float* y, void* workspace, size_t workspace_bytes,
+                   llmops_stream_t stream) {
+    const int bad = fc_check_args(x, rows, K, weiq, Ng, Kg, group_k, N, y);
+    if (bad) return bad;
+    LLMOPS_REQUIRE(workspace != nullptr && aligned(workspace, 256));
     const bool k_tail = K != Kg * group_k;
-    LLMOPS_REQUIRE(aligned(weiq, 16) && aligned(workspace, 256) && aligned(x, k_tail ? 4 : 8));
     const FcWorkspace lay = fc_layout(rows, Ng, Kg, group_k);
     if (workspace_bytes < lay.total)
         return fail(LLMOPS_EWORKSPACE, "fc_Q4A needs %zu workspace bytes, got %zu", lay.total, workspace_bytes);
@@ -206,6 +215,7 @@ extern "C" int llmops_test_fc_decode_attn_dump(const float* rec_stats, const flo
                                                const int8_t* weiq, int64_t Ng, int64_t Kg, int64_t N_out, float* y, int8_t* xq,
                                                float* xd, float* gsum, int32_t* acc, void* workspace, size_t workspace_bytes,
                                                llmops_stream_t stream) {
+    LLMOPS_TEST_HOOK();
     LLMOPS_REQUIRE(xq != nullptr && xd != nullptr && gsum != nullptr && acc != nullptr && aligned(xq, 4));
     const DumpBufs dump{xq, xd, gsum, acc};
     return fc_decode_attn(rec_stats, rec_outs, chunks, H, weiq, Ng, Kg, N_out, nullptr, nullptr, y, workspace, workspace_bytes,
@@ -252,6 +262,7 @@ extern "C" int llmops_fc_Q4A_partials(const int8_t* xq, int64_t rows, const int8
 }
 
 extern "C" void llmops_test_fc_set_row_routing(int rows_from_small, int rows_from_large) {
+    if (!test_hooks_enabled(__func__)) return;
     g_rows_from_small = rows_from_small >= 2 ? rows_from_small : 4;
     g_rows_from_large = rows_from_large >= 2 ? rows_from_large : 3;
 }
@@ -296,10 +307,20 @@ __global__ __launch_bounds__(256) void zero16_kernel(uint4* p, int64_t n16) {
 
 extern "C" size_t llmops_fc_Q4A_noalloc_scratch_bytes(void) { return LLMOPS_FC_NOALLOC_SCRATCH_BYTES; }
 
+extern "C" int llmops_fc_workspace_reset(void* workspace, size_t workspace_bytes, llmops_stream_t stream) {
+    LLMOPS_REQUIRE(workspace != nullptr && aligned(workspace, 256) && workspace_bytes >= 16);
+    const size_t head = workspace_bytes < (size_t)LLMOPS_FC_COUNTER_BYTES ? workspace_bytes : (size_t)LLMOPS_FC_COUNTER_BYTES;
+    const int64_t n16 = (int64_t)(head / 16);
+    zero16_kernel<<<(unsigned)((n16 + 255) / 256), 256, 0, as_stream(stream)>>>(reinterpret_cast<uint4*>(workspace), n16);
+    LLMOPS_LAUNCH_CHECK();
+    return LLMOPS_OK;
+}
+
 extern "C" int llmops_fc_Q4A_noalloc(const float* x, int64_t rows, int64_t K, const int8_t* weiq, int64_t Ng, int64_t Kg,
                                      int group_k, int64_t N, float* y, llmops_stream_t stream) {
-    LLMOPS_REQUIRE(valid_group(group_k));
-    LLMOPS_REQUIRE(rows > 0 && K > 0 && Ng > 0 && Kg > 0);
+    // everything fc_impl will check is checked here first: a refused call must not enqueue the zero fill either
+    const int bad = fc_check_args(x, rows, K, weiq, Ng, Kg, group_k, N, y);
+    if (bad) return bad;
     const size_t need = fc_layout(rows, Ng, Kg, group_k).total;
     if (need > (size_t)LLMOPS_FC_NOALLOC_SCRATCH_BYTES)
         return fail(LLMOPS_EWORKSPACE,
@@ -322,6 +343,7 @@ extern "C" int llmops_fc_Q4A_noalloc(const float* x, int64_t rows, int64_t K, co
 extern "C" int llmops_test_fc_decode_dump(const float* x, int64_t rows, int64_t K, const int8_t* weiq, int64_t Ng, int64_t Kg,
                                           int group_k, int64_t N, float* y, int8_t* xq, float* xd, float* gsum, int32_t* acc,
                                           void* workspace, size_t workspace_bytes, llmops_stream_t stream) {
+    LLMOPS_TEST_HOOK();
     LLMOPS_REQUIRE(valid_group(group_k));
     LLMOPS_REQUIRE(x != nullptr && weiq != nullptr && y != nullptr && workspace != nullptr);
     LLMOPS_REQUIRE(xq != nullptr && xd != nullptr && gsum != nullptr && acc != nullptr);

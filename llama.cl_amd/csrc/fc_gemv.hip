@@ -817,6 +817,7 @@ int launch_gemv_partials(const uint8_t* w, const int8_t* xq, int32_t* acc, int64
 }  // namespace llmops
 
 extern "C" void llmops_test_fc_set_tuning(int target_workgroups, int waves_per_workgroup) {
+    if (!llmops::test_hooks_enabled(__func__)) return;
     if (target_workgroups == -2 || target_workgroups == -3) {  // hand-off of two k-splits: -2 exchange slots, -3 ticket
         llmops::g_exchange_handoff = target_workgroups == -2;
         return;

@@ -265,4 +265,6 @@ int launch_fc_rows_partials(const uint8_t* w, const int8_t* xq, int32_t* acc, in
 
 }  // namespace llmops
 
-extern "C" void llmops_test_fc_rows_set_split(int on) { llmops::g_rows_split = on != 0; }
+extern "C" void llmops_test_fc_rows_set_split(int on) {
+    if (llmops::test_hooks_enabled(__func__)) llmops::g_rows_split = on != 0;
+}

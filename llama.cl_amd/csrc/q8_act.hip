@@ -181,7 +181,7 @@ int launch_quant_x(const float* x, int64_t rows, int64_t K, int group_k, int8_t*
     const int64_t Kg = (K + group_k - 1) / group_k;
     const int64_t items = rows * Kg;
     if (!exact_sum && xsT != nullptr && group_k == 128 && K == Kg * group_k && aligned(x, 16) && aligned(xq, 4) &&
-        rows < ((int64_t)1 << 28) && Kg < ((int64_t)1 << 20)) {
+        rows < ((int64_t)1 << 28) && Kg < ((int64_t)1 << 20) && ((rows + 7) / 8) * Kg < ((int64_t)1 << 31)) {  // (the grid)
         // the group-128 prefill kernels read only the codes and the transposed pairs: xd and gsum stay unwritten
         const int64_t rblocks = (rows + 7) / 8;
         if (rblocks * ((Kg + 3) / 4) >= 1024) {  // enough workgroups with four k-groups per team

@@ -1,6 +1,8 @@
 // Error reporting shared by every entry point of the C ABI.
 #include "common.h"
 
+#include <cstdlib>
+
 namespace llmops {
 
 std::string& last_error() {
@@ -16,6 +18,21 @@ int fail(int code, const char* fmt, ...) {
     va_end(ap);
     last_error() = buf;
     return code;
+}
+
+bool test_hooks_enabled(const char* hook) {
+    static const bool on = [] {
+        const char* e = std::getenv("LLMOPS_TEST_HOOKS");
+        return e != nullptr && e[0] == '1' && e[1] == '\0';
+    }();
+    if (on) return true;
+    fail(LLMOPS_EINVAL, "%s: test hooks are switched off (start the process with LLMOPS_TEST_HOOKS=1)", hook);
+    static bool said = false;
+    if (!said) {
+        said = true;
+        std::fprintf(stderr, "llmops: %s\n", last_error().c_str());
+    }
+    return false;
 }
 
 }  // namespace llmops

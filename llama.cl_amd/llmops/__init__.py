@@ -35,7 +35,8 @@ if not hasattr(torch.Tensor, "item_size"):
 
 _default_group_k = 32  # the reference's compiled-in default (ops/op_fc.hpp:109)
 _workspaces = {}
-_retired = []  # superseded workspaces, kept alive for graphs that recorded their addresses
+_captured = set()  # keys of workspaces whose address a stream capture has recorded
+_retired = []  # superseded workspaces that a captured graph may still replay into
 
 
 def set_default_group_k(g):
@@ -76,24 +77,36 @@ def _workspace(device, nbytes, kind="fc"):
     at the same time and must not share counters or partial sums.  Its first bytes hold arrival counters,
     which must start at zero and which the kernels leave at zero.
 
-    A HIP graph that captured an op replays the raw address of the workspace the op was given, so a
-    workspace is never freed: when a later call needs more, the old tensor is kept (``_retired``) and a
-    larger one takes its place for the calls that follow.  While the stream is capturing nothing may be
+    A HIP graph that captured an op replays the raw address of the workspace the op was given, so a workspace
+    that a capture has seen is never freed: when a later call needs more, the old tensor is kept (``_retired``)
+    and a larger one takes its place for the calls that follow.  A workspace no capture has seen is simply
+    replaced, and sizes grow geometrically, so a serving loop whose prefill length creeps upward does not keep
+    every intermediate size.  While the stream is capturing nothing may be
     allocated or zero-filled (the fill would be recorded into the graph, and the first replay could find
     counters that were never zeroed): an op that would need a new or larger workspace then raises.  Run the
     op once, at the largest size, on the stream that will capture -- or call ``reserve_workspace`` -- first."""
     index = device.index if device.index is not None else torch.cuda.current_device()
     key = (kind, device.type, index, torch._C._cuda_getCurrentRawStream(index))
     ws = _workspaces.get(key)
+    capturing = torch.cuda.is_current_stream_capturing()
+    if capturing and ws is not None and ws.numel() >= nbytes:
+        _captured.add(key)
     if ws is None or ws.numel() < nbytes:
-        if torch.cuda.is_current_stream_capturing():
+        if capturing:
             raise RuntimeError(
                 f"llmops: the {kind} workspace of this stream would have to be "
                 f"{'created' if ws is None else 'enlarged'} ({int(nbytes)} bytes) while the stream is capturing a graph; "
                 "run the op once on this stream before the capture, or call llmops.reserve_workspace")
-        if ws is not None:
-            _retired.append(ws)  # a graph captured earlier may still replay its address
         size = max(int(nbytes), 16 << 20)
+        if ws is not None:
+            size = max(size, 2 * ws.numel())
+            if key in _captured:
+                _retired.append(ws)  # a graph captured earlier may still replay its address
+                _captured.discard(key)
+            else:
+                # work enqueued earlier on this stream may still use the old tensor; torch's allocator only hands its
+                # memory out again to this same stream, i.e. behind that work
+                del ws
         ws = torch.zeros(size, dtype=torch.uint8, device=device)
         _workspaces[key] = ws
     return ws
@@ -115,8 +128,9 @@ def reset_workspaces():
     kernels leave them zero after every call that runs to its end; after a launch that did not (a device error in
     the middle of an op) call this once, with no op in flight, before using the module again."""
     torch.cuda.synchronize()
+    lib = _lib.load()
     for ws in list(_workspaces.values()) + _retired:
-        ws[:min(ws.numel(), 4 << 20)].zero_()
+        _lib.check(lib.llmops_fc_workspace_reset(_ptr(ws), ws.numel(), _stream(ws)))
     torch.cuda.synchronize()
 
 
@@ -414,8 +428,7 @@ def attention_rope2_records(q, k, v, inv_freq, kv_cache, kvc_slots, position_id,
         kv_plan = maxlen
     else:
         kv_plan = min(int(position_id) + 1, maxlen)
-    rows = 256 if maxlen <= 2048 else 512
-    records.chunks = -(-kv_plan // rows)
+    records.chunks = -(-kv_plan // lib.llmops_attention_records_chunk_rows(maxlen, dt))
     _lib.check(lib.llmops_attention_rope_decode_records(_ptr(q), _ptr(k), _ptr(v), B, H, S, _ptr(inv_freq), inv_freq.shape[0],
                                                         _ptr(kv_cache), dt, planes, maxlen, _ptr(kvc_slots),
                                                         0 if on_dev else int(position_id), _ptr(position_id) if on_dev else None,

@@ -22,6 +22,7 @@ SIGNATURES = {
     "llmops_FC_dynamic_quantize_x_rows": (c_int, [c_ptr, c_i64, c_i64, c_int, c_ptr, c_ptr, c_ptr, c_ptr]),
     "llmops_fc_Q4A_workspace_bytes": (c_size, [c_i64, c_i64, c_i64, c_i64, c_int]),
     "llmops_fc_Q4A": (c_int, [c_ptr, c_i64, c_i64, c_ptr, c_i64, c_i64, c_int, c_i64, c_ptr, c_ptr, c_size, c_ptr]),
+    "llmops_fc_workspace_reset": (c_int, [c_ptr, c_size, c_ptr]),
     "llmops_fc_Q4A_noalloc_scratch_bytes": (c_size, []),
     "llmops_fc_Q4A_noalloc": (c_int, [c_ptr, c_i64, c_i64, c_ptr, c_i64, c_i64, c_int, c_i64, c_ptr, c_ptr]),
     "llmops_fc_Q4A_residual": (c_int, [c_ptr, c_i64, c_i64, c_ptr, c_i64, c_i64, c_int, c_i64, c_ptr, c_ptr, c_ptr, c_size,
@@ -40,6 +41,7 @@ SIGNATURES = {
     "llmops_attention_rope_decode": (c_int, [c_ptr, c_ptr, c_ptr, c_i64, c_i64, c_i64, c_ptr, c_i64, c_ptr, c_int, c_i64, c_i64,
                                              c_ptr, c_ptr, c_int, c_ptr, c_size, c_ptr]),
     "llmops_attention_records_chunks": (c_i64, [c_i64, c_int]),
+    "llmops_attention_records_chunk_rows": (c_i64, [c_i64, c_int]),
     "llmops_attention_rope_decode_records": (c_int, [c_ptr, c_ptr, c_ptr, c_i64, c_i64, c_i64, c_ptr, c_i64, c_ptr, c_int, c_i64,
                                                      c_i64, c_ptr, c_int, c_ptr, c_int, c_ptr, c_ptr, c_ptr, c_size, c_ptr]),
     "llmops_softmax": (c_int, [c_ptr, c_i64, c_i64, c_ptr]),
@@ -59,6 +61,7 @@ SIGNATURES = {
     "llmops_test_calib_copy": (c_int, [c_ptr, c_ptr, c_i64, c_int, c_ptr]),
     "llmops_test_fc_set_tuning": (None, [c_int, c_int]),
     "llmops_test_gemm_set_tuning": (None, [c_int]),
+    "llmops_test_gemm_set_interleaved": (None, [c_int]),
     "llmops_test_gemm_set_reduce": (None, [c_int]),
     "llmops_test_gemm_set_split": (None, [c_int]),
     "llmops_test_fc_set_row_routing": (None, [c_int, c_int]),

@@ -4,6 +4,9 @@ import sys
 import numpy as np
 import pytest
 
+# the library's test hooks (planner knobs, dump builds, calibration kernels) are refused unless the process asks for them
+os.environ.setdefault("LLMOPS_TEST_HOOKS", "1")
+
 ROOT = os.path.abspath(os.path.join(os.path.dirname(__file__), ".."))
 for p in (ROOT, os.path.join(ROOT, "llama.cl_amd")):
     if p not in sys.path:

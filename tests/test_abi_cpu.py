@@ -68,10 +68,39 @@ def test_argument_validation_without_device(lib):
     rc = lib.llmops_attention_rope(vp(256), vp(256), vp(256), i64(1), i64(1), i64(32), i64(64), vp(256), i64(32), vp(256), 0,
                                    i64(2), i64(16), vp(256), 0, 0, vp(256), ctypes.c_size_t(1 << 30), vp(0))
     assert rc == 1 and b"S == 128" in lib.llmops_last_error()
-    # the one-token form runs on a (chunk, head) grid: more than 65535 heads in all are refused before any launch
-    rc = lib.llmops_attention_rope(vp(256), vp(256), vp(256), i64(2200), i64(1), i64(32), i64(128), vp(256), i64(64), vp(256), 0,
-                                   i64(2), i64(16), vp(256), 3, 0, vp(256), ctypes.c_size_t(1 << 40), vp(0))
+    # the one-token kernels run on a (chunk, head) grid.  With the position by value more than 65535 heads in all take
+    # the general kernels (GPU test); with the position in device memory they are refused before any launch
+    rc = lib.llmops_attention_rope_decode(vp(256), vp(256), vp(256), i64(2200), i64(32), i64(128), vp(256), i64(64), vp(256), 0,
+                                          i64(2), i64(16), vp(256), vp(256), 0, vp(256), ctypes.c_size_t(1 << 40), vp(0))
     assert rc == 1 and b"65535 heads" in lib.llmops_last_error()
+    rc = lib.llmops_fc_workspace_reset(vp(0), ctypes.c_size_t(1 << 20), vp(0))
+    assert rc == 1 and b"workspace != nullptr" in lib.llmops_last_error()
+    # the entry point that allocates nothing validates its arguments before it enqueues anything (no device here:
+    # a launch would fail with a HIP error, not with this message)
+    rc = lib.llmops_fc_Q4A_noalloc(vp(0), i64(1), i64(4096), vp(256), i64(128), i64(32), 128, i64(4096), vp(256), vp(0))
+    assert rc == 1 and b"x != nullptr" in lib.llmops_last_error()
+
+
+def test_test_hooks_are_refused_unless_the_process_asks_for_them():
+    """The planner knobs, dump builds and calibration kernels of include/llmops_hip_test.h live in the product
+    library; a process that was not started with LLMOPS_TEST_HOOKS=1 cannot use them."""
+    import subprocess
+    import sys
+    code = (
+        "import ctypes, sys\n"
+        f"lib = ctypes.CDLL({LIB!r})\n"
+        "lib.llmops_last_error.restype = ctypes.c_char_p\n"
+        "vp, i64 = ctypes.c_void_p, ctypes.c_int64\n"
+        "rc = lib.llmops_test_calib_read(vp(256), i64(1024), 4, vp(256), vp(0))\n"
+        "msg = lib.llmops_last_error()\n"
+        "lib.llmops_test_fc_set_tuning(64, 8)\n"
+        "print(rc, msg.decode())\n"
+    )
+    env = {k: v for k, v in os.environ.items() if k != "LLMOPS_TEST_HOOKS"}
+    out = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=120)
+    assert out.returncode == 0, out.stderr
+    assert out.stdout.startswith("1 ") and "LLMOPS_TEST_HOOKS=1" in out.stdout
+    assert "test hooks are switched off" in out.stderr
 
 
 def test_python_ops_refuse_host_tensors():

@@ -455,3 +455,22 @@ def test_attention_records_merged_by_the_o_projection(ops, orc, cache_dtype, max
         if cache_dtype == torch.float32 and kv in (257, 2048):              # and the oracle's two ops
             oatt, _, _ = orc.attention(q, k, v, inv_freq, cache0, slots, pos, 0)
             assert max_rel_err(host(yf), orc.fc(oatt, pw, N) + res) <= 1e-2
+
+
+def test_decode_attention_with_more_than_65535_heads_in_all(ops, orc):
+    """One query token for 2050 sequences of 32 heads: B*H exceeds what the decode kernels' (chunk, head) grid can
+    index, so the call is served by the general kernels (the reference has no such limit, ops/op_attn.hpp:976)."""
+    rng = np.random.default_rng(77)
+    B, H, S, maxlen, kv = 2050, 32, 128, 8, 6
+    inv_freq = (1.0 / (10000.0 ** (np.arange(0, S, 2, dtype=np.float32) / np.float32(S)))).astype(np.float32)
+    q, k, v = (rng.standard_normal((B, 1, H * S)).astype(np.float32) for _ in range(3))
+    cache = rng.standard_normal((2, B, H, maxlen, S)).astype(np.float32)
+    slots = np.array([kv - 1], np.int32)
+    tq, tk, tc = dev(q), dev(k), dev(cache)
+    ops.attention_rope2(tq, tk, dev(v), dev(inv_freq), tc, dev(slots), kv - 1, 0)
+    sel = [0, 1, 1023, 2047, 2048, 2049]                       # the oracle on a few sequences (they are independent)
+    want, k_ref, cache_ref = orc.attention(q[sel], k[sel], v[sel], inv_freq, np.ascontiguousarray(cache[:, sel]), slots, kv - 1, 0)
+    assert max_rel_err(host(tq)[sel], want) <= 1e-5
+    assert np.abs(host(tk)[sel] - k_ref).max() <= 1e-5
+    assert np.abs(host(tc)[:, sel] - cache_ref).max() <= 1e-5
+    assert torch.isfinite(tq).all()

@@ -134,15 +134,20 @@ def test_full_width_fused_plan_vs_reference_plan_and_oracle(orc):
     r_ref, r_fused, r_plans = rms(out["reference"][0], want), rms(out["fused"][0], want), rms(out["fused"][0], out["reference"][0])
     print("logits max: reference plan vs oracle", e_ref, "fused plan vs oracle", e_fused, "fused vs reference plan", e_plans)
     print("logits rms: reference plan vs oracle", r_ref, "fused plan vs oracle", r_fused, "fused vs reference plan", r_plans)
-    # End to end, any two evaluations drift apart up to the noise floor of the 8-bit activation quantization itself:
-    # once an FC's input differs by more than a fraction of a code step, the two runs round to independent codes,
-    # which is worth ~1 % of an output's spread per FC (K = 4096, step = amax/127).  Even the reference's own op
-    # sequence on the GPU against the oracle shows it (observed: max 5e-2 of the largest logit, rms 1-2 %), so this
-    # test only bounds the drift; the per-launch test above carries the 1e-3 contract (observed 1e-6).
-    assert max(e_ref, e_fused, e_plans) <= 1e-1
-    assert max(r_ref, r_fused, r_plans) <= 4e-2
-    assert np.abs(out["reference"][1] - cache_h).max() <= 1e-3
-    assert np.abs(out["fused"][1] - cache_h).max() <= 1e-3
+    # End to end, any two evaluations drift apart up to the noise floor of the 8-bit activation quantization itself.
+    # A 1e-6 difference flips a code now and then (step = amax/127); one flipped code moves an FC output by ~3e-4 of
+    # its spread, which flips ~3 % of the next FC's codes, and after three or four FCs the two runs round to
+    # independent codes: ~1 % of an output's spread per FC from then on.  Even the reference's own op sequence on
+    # the GPU against the oracle shows it (observed over these 9 FCs: rms 2.4-4.9 % of the logits' rms, max 5 % of the
+    # largest logit), so this test only bounds the drift; the per-launch test above carries the 1e-3 contract
+    # (observed 1e-6).
+    assert max(e_ref, e_fused, e_plans) <= 1.5e-1
+    assert max(r_ref, r_fused, r_plans) <= 1e-1
+    for plan in ("reference", "fused"):
+        got = out[plan][1]
+        assert np.abs(got[:2] - cache_h[:2]).max() <= 1e-4        # first layer: the new row's k, v are one FC deep
+        assert np.abs(got[2:] - cache_h[2:]).max() <= 1.5e-1 * np.abs(cache_h[2:, ..., KV - 1, :]).max()   # second: drift as above
+        assert np.array_equal(got[..., :KV - 1, :], cache_h[..., :KV - 1, :])                                # other rows untouched
 
 
 @pytest.mark.parametrize("cache_dtype", [torch.float32, torch.float16])

@@ -24,16 +24,26 @@ def _case(orc, rng, M, N, K, G):
     tx = torch.from_numpy(x).to(dev)
     want = llmops.fc_Q4A(tx, wq, N)
     out = torch.full((1, M, N), float("nan"), dtype=torch.float32, device=dev)
-    torch.cuda.synchronize()
-    before = torch.cuda.memory_stats(dev)["allocation.all.allocated"]
     lib = _lib.load()
     Ng, Kg, _ = wq.shape
-    rc = lib.llmops_fc_Q4A_noalloc(ctypes.c_void_p(tx.data_ptr()), M, K, ctypes.c_void_p(wq.data_ptr()), Ng, Kg, G, N,
-                                   ctypes.c_void_p(out.data_ptr()),
-                                   ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream))
-    assert rc == 0, lib.llmops_last_error()
+
+    def call():
+        rc = lib.llmops_fc_Q4A_noalloc(ctypes.c_void_p(tx.data_ptr()), M, K, ctypes.c_void_p(wq.data_ptr()), Ng, Kg, G, N,
+                                       ctypes.c_void_p(out.data_ptr()),
+                                       ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream))
+        assert rc == 0, lib.llmops_last_error()
+        torch.cuda.synchronize()
+
+    call()  # the first call on a device may load code objects and looks the array's address up
+    out.fill_(float("nan"))
     torch.cuda.synchronize()
+    # torch's statistics only see torch's allocator; the driver's free-memory figure also sees a hipMalloc made
+    # inside the library
+    before = torch.cuda.memory_stats(dev)["allocation.all.allocated"]
+    free_before = torch.cuda.mem_get_info(dev)[0]
+    call()
     assert torch.cuda.memory_stats(dev)["allocation.all.allocated"] == before
+    assert torch.cuda.mem_get_info(dev)[0] == free_before
     assert torch.equal(out, want), (M, N, K, G)
     # the oracle on a few rows (FC rows are independent)
     rows = sorted({0, M // 2, M - 1})
@@ -62,3 +72,7 @@ def test_noalloc_refuses_sizes_beyond_its_array():
     rc = lib.llmops_fc_Q4A_noalloc(ctypes.c_void_p(t.data_ptr()), 4096, 11008, ctypes.c_void_p(t.data_ptr()), 128, 86, 128,
                                    4096, ctypes.c_void_p(t.data_ptr()), ctypes.c_void_p(0))
     assert rc == 2 and b"scratch" in lib.llmops_last_error()
+    # a refused call enqueues nothing: bad arguments are reported before the zero fill of the array's head is launched
+    rc = lib.llmops_fc_Q4A_noalloc(ctypes.c_void_p(0), 1, 4096, ctypes.c_void_p(t.data_ptr()), 128, 32, 128, 4096,
+                                   ctypes.c_void_p(t.data_ptr()), ctypes.c_void_p(0))
+    assert rc == 1 and b"x != nullptr" in lib.llmops_last_error()
