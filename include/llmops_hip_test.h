@@ -38,10 +38,6 @@ void llmops_test_fc_set_tuning(int target_workgroups, int waves_per_workgroup);
  * per shape and send 9..16 rows to the tiled kernel too instead of the weight-streaming MFMA kernel */
 void llmops_test_gemm_set_tuning(int row_tile_factor);
 
-/* prefill GEMM, 256-row tiles: 1 (default) the kernel whose wavefronts interleave the fold with the MFMAs, 0 the
- * kernel with two wave groups in alternating phases; kept for comparisons */
-void llmops_test_gemm_set_interleaved(int on);
-
 /* prefill GEMM with split-K: the product kernel adds the partial sums itself (the last split of a tile to
  * arrive adds all of them in index order) when the split count is at most 12 x in_kernel; otherwise, and
  * always with 0, a second launch adds them.  Default 1.  Same result either way; kept for comparisons and tests. */

@@ -917,315 +917,6 @@ __global__ __launch_bounds__(512, 2) void fc_gemm_pp_kernel(const uint8_t* __res
         }
 }
 
-// ---- 256-row tiles, the fold interleaved with the MFMAs inside every wavefront (group 128, many rows) ---------
-// Same tile (256 rows x 128 columns, 8 wavefronts of 64 x 64), same LDS image and same staging as the kernel above
-// (weights unpacked once per workgroup into MFMA operand order, activations and their scales by asynchronous
-// global->LDS copies, XCD-aware tile order), but no phases: a wavefront walks its 16 sub-tiles of 16 x 16 and in
-// every step issues the two MFMAs of one sub-tile and the fold (convert, scale product, fma per element) of the
-// sub-tile before it.  The MFMAs run in the matrix pipe while the wavefront's own vector instructions issue behind
-// them, and the second wavefront of the SIMD fills what is left; a scheduling fence after every step keeps the
-// compiler from collecting the MFMAs in one place and the folds in another (which is what it does on its own).
-// Only two int32 sub-tiles are ever live (8 registers instead of 64), which is what makes room for this.
-//   operands: the wave's A operands (4 row tiles x 2 k halves) stay in registers for the k-group; the B operands
-//   of one column set (2 k halves) are fetched from LDS one column set ahead; in the last column set of a k-group
-//   the A operands and the first B operands of the NEXT k-group are fetched from the other LDS buffer.
-//   one barrier per k-group, after the third column set: by then every wave has read the last thing it needs from
-//   this k-group's LDS buffer, and the next k-group's buffer (copies issued a whole k-group earlier, weights
-//   fetched into registers a k-group earlier and unpacked just before the barrier) is complete.  Right after the
-//   barrier the copies and the weight fetch for the k-group after next go out into the buffer that just became free.
-template <bool PARTIALS>
-__global__ __launch_bounds__(512, 2) void fc_gemm_il_kernel(const uint8_t* __restrict__ weiq, const int8_t* __restrict__ xq,
-                                                             const float* __restrict__ xd, const float* __restrict__ gs,
-                                                             const float2* __restrict__ xsT, float* __restrict__ out,
-                                                             int32_t* __restrict__ out_i, int Ng, int Kg, int64_t ldo,
-                                                             int64_t N, int rows, int kb_per_split, int64_t split_stride,
-                                                             const float* __restrict__ residual) {
-    constexpr int RT = 4, BM = 256, GM = 128;
-    extern __shared__ __align__(16) uint8_t smem_raw[];
-    GemmPPSmem& sm = *reinterpret_cast<GemmPPSmem*>(smem_raw);
-
-    const int tid = threadIdx.x, lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int grp = wave >> 2, w4 = wave & 3;  // (grp, w4): which rows this wave copies; its tile is rows 64*(wave>>1)
-    const int wr = w4 >> 1, wc = w4 & 1;
-    const int g = lane >> 4, jj = lane & 15, q = jj & 7, sp = jj >> 3;
-    const int nbx = (Ng + 3) / 4, nby = (rows + BM - 1) / BM;
-    int bx, by;
-    {
-        const int total = nbx * nby, per_xcd = (total + 7) / 8;
-        const int i = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-        if ((int)(blockIdx.x >> 3) >= per_xcd || i >= total) return;  // uniform for the workgroup
-        constexpr int kBand = 8;
-        const int band = i / (kBand * nbx), in_band = i % (kBand * nbx);
-        const int first = band * kBand, rows_in_band = min(kBand, nby - first);
-        by = first + in_band % rows_in_band;
-        bx = in_band / rows_in_band;
-    }
-    const int strip0 = bx * 4;
-    const int row0 = by * BM + grp * GM;
-    const int kb0 = blockIdx.z * kb_per_split, kb1 = min(Kg, kb0 + kb_per_split);
-    const int64_t Kp = (int64_t)Kg * 128;
-
-    // ---- what this lane copies per k-group (as in the kernel above) ----
-    uint32_t aoff[4];
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-        const int r = (w4 * 4 + i) * 8 + (lane >> 3);
-        const int key = (r + ((r >> 3) & 1)) & 7;
-        aoff[i] = (uint32_t)(min(rows - 1, row0 + r) * (int)Kp + (((lane & 7) ^ key) * 16));
-    }
-    const int xr = (w4 & 1) * 64 + lane;
-    const int64_t xrow = min(rows - 1, row0 + xr);
-    const uint8_t* xbase = nullptr;
-    uint32_t xoff = 0;
-    int64_t xstep = 0;
-    if (!PARTIALS) {
-        if (xsT) {
-            xbase = reinterpret_cast<const uint8_t*>(xsT);
-            xoff = (uint32_t)((xrow * 2 + (w4 >> 1)) * 4);
-            xstep = (int64_t)rows * 8;
-        } else {
-            xbase = reinterpret_cast<const uint8_t*>((w4 >> 1) ? gs : xd);
-            xoff = (uint32_t)(xrow * Kg * 4);
-            xstep = 4;
-        }
-    }
-    const uint32_t lds_a = lds_off(&sm.a[0][0]);
-    const uint32_t lds_x = (w4 >> 1) ? lds_off(&sm.gs[0][0]) : lds_off(&sm.dx[0][0]);
-#define LLMOPS_COPY(KB, BUF)                                                                                       \
-    do {                                                                                                           \
-        _Pragma("unroll") for (int i = 0; i < 4; i++)                                                              \
-            copy16_to_lds(xq + (int64_t)(KB) * 128, aoff[i], lds_a + (BUF) * (BM * 128) + (grp * GM + (w4 * 4 + i) * 8) * 128); \
-        if (!PARTIALS) copy4_to_lds(xbase + (int64_t)(KB) * xstep, xoff, lds_x + (BUF) * (BM * 4) + (grp * GM + (w4 & 1) * 64) * 4); \
-    } while (0)
-
-    // weights: thread t takes the 16-byte chunk t of the tile's 512 (chunk = strip (2 bits) | k8-row (4 bits) |
-    // column quad (3 bits)); the first 32 threads also the 32 chunks of fp16 scales
-    uint32_t boff;
-    int bdst;
-    {
-        const int st = tid >> 7, r = (tid >> 3) & 15, q4 = tid & 7;
-        boff = (uint32_t)(min(Ng - 1, strip0 + st) * Kg * kBlk128 + r * 128 + q4 * 16);
-        bdst = st * kBuStrip + ((((r >> 3) * 4) * 4 + ((r & 7) >> 1)) * 8 + q4) * 16 + (r & 1) * 8;
-    }
-    const int sst = (tid >> 3) & 3, spart = tid & 7;
-    const uint32_t soff = (uint32_t)(min(Ng - 1, strip0 + sst) * Kg * kBlk128 + 2048 + spart * 16);
-    v4u rb = {0u, 0u, 0u, 0u}, rs = {0u, 0u, 0u, 0u};
-#define LLMOPS_FETCH_B(KB)                                                                                 \
-    do {                                                                                                   \
-        const uint8_t* wkb = weiq + (int64_t)(KB) * kBlk128;                                               \
-        rb = *reinterpret_cast<const v4u*>(wkb + boff);                                                    \
-        if (tid < 32) rs = *reinterpret_cast<const v4u*>(wkb + soff);                                      \
-    } while (0)
-#define LLMOPS_STASH_B(BUF)                                                                                \
-    do {                                                                                                   \
-        _Pragma("unroll") for (int c = 0; c < 4; c++) {                                                    \
-            uint2 u;                                                                                       \
-            u.x = lo4(rb[c]);                                                                              \
-            u.y = hi4(rb[c]);                                                                              \
-            *reinterpret_cast<uint2*>(&sm.bu[BUF][bdst + c * 512]) = u;                                    \
-        }                                                                                                  \
-        if (tid < 32) {                                                                                    \
-            float* dstf = (spart < 4 ? sm.d[BUF] : sm.m[BUF]) + sst * 32 + (spart & 3) * 8;                \
-            float4 lo, hi;                                                                                 \
-            lo.x = f16_bits_to_f32((uint16_t)(rs[0] & 0xFFFFu));                                           \
-            lo.y = f16_bits_to_f32((uint16_t)(rs[0] >> 16));                                               \
-            lo.z = f16_bits_to_f32((uint16_t)(rs[1] & 0xFFFFu));                                           \
-            lo.w = f16_bits_to_f32((uint16_t)(rs[1] >> 16));                                               \
-            hi.x = f16_bits_to_f32((uint16_t)(rs[2] & 0xFFFFu));                                           \
-            hi.y = f16_bits_to_f32((uint16_t)(rs[2] >> 16));                                               \
-            hi.z = f16_bits_to_f32((uint16_t)(rs[3] & 0xFFFFu));                                           \
-            hi.w = f16_bits_to_f32((uint16_t)(rs[3] >> 16));                                               \
-            *reinterpret_cast<float4*>(dstf) = lo;                                                         \
-            *reinterpret_cast<float4*>(dstf + 4) = hi;                                                     \
-        }                                                                                                  \
-    } while (0)
-
-    v4f f[RT][4];
-#pragma unroll
-    for (int t = 0; t < RT; t++)
-#pragma unroll
-        for (int c = 0; c < 4; c++) f[t][c] = v4f{0.f, 0.f, 0.f, 0.f};
-    float gk[RT], mk[4];  // min term, four k-groups at a time by fp32 MFMA
-#pragma unroll
-    for (int t = 0; t < RT; t++) gk[t] = 0.0f;
-#pragma unroll
-    for (int c = 0; c < 4; c++) mk[c] = 0.0f;
-
-    if (kb0 < kb1) {
-        LLMOPS_COPY(kb0, 0);
-        LLMOPS_FETCH_B(kb0);
-        LLMOPS_STASH_B(0);
-    }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-    if (kb0 + 1 < kb1) {
-        LLMOPS_COPY(kb0 + 1, 1);
-        LLMOPS_FETCH_B(kb0 + 1);
-    }
-
-    const int strip_l = wc * 2 + sp;      // strip (0..3) of the tile this lane's B operands come from
-    const int lrow = grp * GM + wr * 64;  // first tile row of this wave
-    const int akey = (jj + (jj >> 3)) & 7;
-    // A operand of row tile t, k half h: row lrow + 16t + jj, chunk 4h + g, swizzled by the row's low bits
-    const int a_rd0 = (lrow + jj) * 128 + (((0 + g) ^ akey) * 16);
-    const int a_rd1 = (lrow + jj) * 128 + (((4 + g) ^ akey) * 16);
-    const int b_rd = strip_l * kBuStrip + (g * 8 + q) * 16;  // + (4h + c) * 512
-    v4i a[RT][2], bc[2][2];
-#define LLMOPS_LOAD_A(T, BUF)                                                                              \
-    do {                                                                                                   \
-        a[T][0] = *reinterpret_cast<const v4i*>(&sm.a[BUF][a_rd0 + (T) * 2048]);                           \
-        a[T][1] = *reinterpret_cast<const v4i*>(&sm.a[BUF][a_rd1 + (T) * 2048]);                           \
-    } while (0)
-#define LLMOPS_LOAD_B(SLOT, BUF, C)                                                                        \
-    do {                                                                                                   \
-        bc[SLOT][0] = *reinterpret_cast<const v4i*>(&sm.bu[BUF][b_rd + (0 * 4 + (C)) * 512]);              \
-        bc[SLOT][1] = *reinterpret_cast<const v4i*>(&sm.bu[BUF][b_rd + (1 * 4 + (C)) * 512]);              \
-    } while (0)
-    if (kb0 < kb1) {
-#pragma unroll
-        for (int t = 0; t < RT; t++) LLMOPS_LOAD_A(t, 0);
-        LLMOPS_LOAD_B(0, 0, 0);
-    }
-    // The int32 sums start from the bit pattern of 1.5 * 2^23 instead of 0: read as a float the result is then
-    // 12582912 + sum exactly (|sum| <= 128 * 15 * 128 < 2^22 stays inside that binade, whose ulp is 1), and one
-    // subtraction gives float(sum) -- the same value v_cvt_f32_i32 would, from an instruction that issues at full rate.
-    constexpr int kMagicBits = 0x4B400000;
-    constexpr float kMagic = 12582912.0f;
-    const v4i zero4 = v4i{kMagicBits, kMagicBits, kMagicBits, kMagicBits};
-    for (int kb = kb0; kb < kb1; kb++) {
-        const int buf = (kb - kb0) & 1;
-        const bool more = kb + 1 < kb1;
-        const int nbuf = more ? buf ^ 1 : buf;
-        const float4 d4 = *reinterpret_cast<const float4*>(&sm.d[buf][strip_l * 32 + q * 4]);
-        const float d[4] = {d4.x, d4.y, d4.z, d4.w};
-        float dxv[RT][4];
-        float gsr[RT];
-        float4 m4 = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (!PARTIALS) {
-#pragma unroll
-            for (int t = 0; t < RT; t++) {
-                const float4 x4 = *reinterpret_cast<const float4*>(&sm.dx[buf][lrow + t * 16 + g * 4]);
-                dxv[t][0] = x4.x, dxv[t][1] = x4.y, dxv[t][2] = x4.z, dxv[t][3] = x4.w;
-                gsr[t] = sm.gs[buf][lrow + t * 16 + jj];
-            }
-            m4 = *reinterpret_cast<const float4*>(&sm.m[buf][strip_l * 32 + q * 4]);
-        }
-        // (three sub-tiles in rotation: the one being multiplied, the one whose MFMAs were issued a step ago and are
-        // still in the pipe, and the one being folded -- with two the fold would wait for the pipe in every step)
-        v4i acc[3];
-        // what happens to a finished int32 sub-tile: folded into the fp32 accumulators, or (test build) stored
-#define LLMOPS_FOLD(T, C, P)                                                                               \
-    do {                                                                                                   \
-        if (PARTIALS) {                                                                                    \
-            const int strip = strip0 + strip_l;                                                            \
-            if (strip < Ng) {                                                                              \
-                _Pragma("unroll") for (int v = 0; v < 4; v++) {                                            \
-                    const int row = row0 + wr * 64 + (T) * 16 + g * 4 + v;                                 \
-                    if (row < rows)                                                                        \
-                        out_i[((int64_t)row * ((int64_t)Ng * kGroupN) + strip * kGroupN + q * 4 + (C)) * Kg + kb] = acc[P][v] - kMagicBits; \
-                }                                                                                          \
-            }                                                                                              \
-        } else {                                                                                           \
-            _Pragma("unroll") for (int v = 0; v < 4; v++)                                                  \
-                f[T][C][v] = fmaf(d[C] * dxv[T][v], __int_as_float(acc[P][v]) - kMagic, f[T][C][v]);       \
-        }                                                                                                  \
-    } while (0)
-#pragma unroll
-        for (int c = 0; c < 4; c++) {
-            // the B operands of the next column set (of the next k-group's first one, from the other buffer)
-            // (without a next k-group the same buffer is read again: the values are not used, and no branch
-            // splits the steps)
-            if (c < 3) LLMOPS_LOAD_B((c + 1) & 1, buf, c + 1);
-            else LLMOPS_LOAD_B(0, nbuf, 0);
-#pragma unroll
-            for (int t = 0; t < RT; t++) {
-                const int step = c * 4 + t, p = step % 3;
-                acc[p] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[t][0], bc[c & 1][0], zero4, 0, 0, 0);
-                acc[p] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[t][1], bc[c & 1][1], acc[p], 0, 0, 0);
-                if (step > 1) LLMOPS_FOLD((step - 2) & 3, (step - 2) >> 2, (step - 2) % 3);
-                if (c == 3) LLMOPS_LOAD_A(t, nbuf);  // this row tile's operands are done for this k-group
-                // Register arithmetic has no place in the program's order of side effects, and left to itself the
-                // compiler gathers all MFMAs of a k-group in one place and all folds in another.  An empty
-                // statement that names this step's results pins them to the step; the fence keeps the
-                // instruction scheduler from moving anything across the step's end.
-                if (!PARTIALS && step > 1)
-                    asm volatile("" : "+v"(acc[p]), "+v"(f[(step - 2) & 3][(step - 2) >> 2]));
-                else
-                    asm volatile("" : "+v"(acc[p]));
-                __builtin_amdgcn_sched_barrier(0);
-            }
-            if (c == 2 && more) {
-                LLMOPS_STASH_B(buf ^ 1);                          // weights of the next k-group, fetched a k-group ago
-                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's copies for the next k-group have landed
-                __syncthreads();
-                if (kb + 2 < kb1) {
-                    LLMOPS_COPY(kb + 2, buf);
-                    LLMOPS_FETCH_B(kb + 2);
-                }
-                __builtin_amdgcn_sched_barrier(0);
-            }
-        }
-        LLMOPS_FOLD(2, 3, 14 % 3);
-        LLMOPS_FOLD(3, 3, 15 % 3);
-        if (!PARTIALS) asm volatile("" : "+v"(f[2][3]), "+v"(f[3][3]));
-        if (!PARTIALS) {
-            const float m[4] = {m4.x, m4.y, m4.z, m4.w};
-            const int slot4 = (kb - kb0) & 3;
-            const bool mine4 = slot4 == g;
-#pragma unroll
-            for (int c = 0; c < 4; c++) mk[c] = mine4 ? m[c] : mk[c];
-#pragma unroll
-            for (int t = 0; t < RT; t++) gk[t] = mine4 ? gsr[t] : gk[t];
-            if (slot4 == 3 || kb + 1 == kb1) {
-#pragma unroll
-                for (int t = 0; t < RT; t++) {
-#pragma unroll
-                    for (int c = 0; c < 4; c++) f[t][c] = __builtin_amdgcn_mfma_f32_16x16x4f32(gk[t], mk[c], f[t][c], 0, 0, 0);
-                    gk[t] = 0.0f;
-                }
-#pragma unroll
-                for (int c = 0; c < 4; c++) mk[c] = 0.0f;
-            }
-        }
-        __builtin_amdgcn_sched_barrier(0);
-#undef LLMOPS_FOLD
-    }
-#undef LLMOPS_COPY
-#undef LLMOPS_FETCH_B
-#undef LLMOPS_STASH_B
-#undef LLMOPS_LOAD_A
-#undef LLMOPS_LOAD_B
-
-    if (PARTIALS) return;
-    const int strip = strip0 + strip_l;
-    if (strip >= Ng) return;
-    float* o = out + (int64_t)blockIdx.z * split_stride;
-    const int64_t n0 = (int64_t)strip * kGroupN + q * 4;
-#pragma unroll
-    for (int t = 0; t < RT; t++)
-#pragma unroll
-        for (int v = 0; v < 4; v++) {
-            const int row = row0 + wr * 64 + t * 16 + g * 4 + v;
-            if (row >= rows) continue;
-            float* dst = o + (int64_t)row * ldo + n0;
-            // residual != nullptr only without split-K: then o is the result itself, row stride ldo
-            const float* res = residual ? residual + (int64_t)row * ldo + n0 : nullptr;
-            if (n0 + 3 < N && (ldo & 3) == 0) {
-                float4 val = make_float4(f[t][0][v], f[t][1][v], f[t][2][v], f[t][3][v]);
-                if (res) {
-                    const float4 r4 = *reinterpret_cast<const float4*>(res);
-                    val.x += r4.x, val.y += r4.y, val.z += r4.z, val.w += r4.w;
-                }
-                *reinterpret_cast<float4*>(dst) = val;
-            } else {
-#pragma unroll
-                for (int c = 0; c < 4; c++)
-                    if (n0 + c < N) dst[c] = res ? f[t][c][v] + res[c] : f[t][c][v];
-            }
-        }
-}
-
 // y[row][n] = sum over splits (index order) of part[s][row][n] (+ residual[row][n]); four columns per
 // thread (the partial sums' row stride ldp is a multiple of 32 floats, so their 16-byte loads are aligned)
 __global__ void gemm_reduce_kernel(const float* __restrict__ part, float* __restrict__ y, int64_t rows, int64_t N,
@@ -1301,7 +992,6 @@ static int g_gemm_pp_min_rows = 256;
 static int g_gemm_rt = 0;  // 0 = choose per shape; -1 = also keep 9..32 rows on the tiled kernel
 static int g_gemm_fused_reduce = 1;  // split-K partial sums added by the product kernel itself (0: by a second launch)
 static int g_gemm_force_split = 0;   // > 0: the split-K factor to use whatever the estimate says (tests)
-static int g_gemm_interleaved = 1;   // 256-row tiles: the kernel whose waves interleave fold and MFMAs (0: two wave groups in phases)
 bool gemm_rows_kernel_enabled() { return g_gemm_rt >= 0; }
 
 // Split-K factor for `tiles` output tiles on a machine with `slots` resident workgroups.
@@ -1418,18 +1108,12 @@ static int launch_gemm_pp(const uint8_t* w, const int8_t* xq, const float* xd, c
     if (!configured) {
         LLMOPS_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&fc_gemm_pp_kernel<false>),
                                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(GemmPPSmem)));
-        LLMOPS_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&fc_gemm_il_kernel<false>),
-                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(GemmPPSmem)));
         configured = true;
     }
     const int64_t tiles = ((Ng + 3) / 4) * ((rows + 255) / 256);
     dim3 grid((unsigned)(8 * ((tiles + 7) / 8)), 1, (unsigned)p.S);
-    if (g_gemm_interleaved)
-        fc_gemm_il_kernel<false><<<grid, 512, sizeof(GemmPPSmem), st>>>(w, xq, xd, gs, xsT, out, nullptr, (int)Ng, (int)Kg, ldo, N,
-                                                                       (int)rows, p.kb_per_split, split_stride, residual);
-    else
-        fc_gemm_pp_kernel<false><<<grid, 512, sizeof(GemmPPSmem), st>>>(w, xq, xd, gs, xsT, out, nullptr, (int)Ng, (int)Kg, ldo, N,
-                                                                       (int)rows, p.kb_per_split, split_stride, residual);
+    fc_gemm_pp_kernel<false><<<grid, 512, sizeof(GemmPPSmem), st>>>(w, xq, xd, gs, xsT, out, nullptr, (int)Ng, (int)Kg, ldo, N,
+                                                                   (int)rows, p.kb_per_split, split_stride, residual);
     return LLMOPS_OK;
 }
 
@@ -1491,18 +1175,12 @@ int launch_gemm_partials(const uint8_t* w, const int8_t* xq, int32_t* acc, int64
         if (!configured) {
             LLMOPS_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&fc_gemm_pp_kernel<true>),
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(GemmPPSmem)));
-            LLMOPS_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&fc_gemm_il_kernel<true>),
-                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(GemmPPSmem)));
             configured = true;
         }
         const int64_t tiles = ((Ng + 3) / 4) * ((rows + 255) / 256);
         dim3 grid((unsigned)(8 * ((tiles + 7) / 8)), 1, 1);
-        if (g_gemm_interleaved)
-            fc_gemm_il_kernel<true><<<grid, 512, sizeof(GemmPPSmem), st>>>(w, xq, nullptr, nullptr, nullptr, nullptr, acc, (int)Ng,
-                                                                          (int)Kg, 0, 0, (int)rows, (int)Kg, 0, nullptr);
-        else
-            fc_gemm_pp_kernel<true><<<grid, 512, sizeof(GemmPPSmem), st>>>(w, xq, nullptr, nullptr, nullptr, nullptr, acc, (int)Ng,
-                                                                          (int)Kg, 0, 0, (int)rows, (int)Kg, 0, nullptr);
+        fc_gemm_pp_kernel<true><<<grid, 512, sizeof(GemmPPSmem), st>>>(w, xq, nullptr, nullptr, nullptr, nullptr, acc, (int)Ng,
+                                                                      (int)Kg, 0, 0, (int)rows, (int)Kg, 0, nullptr);
     } else if (G == 128) {  // the production LDS-tiled loop, writing its int32 tiles instead of folding them
         static bool configured = false;
         if (!configured) {
@@ -1526,9 +1204,6 @@ int launch_gemm_partials(const uint8_t* w, const int8_t* xq, int32_t* acc, int64
 
 extern "C" void llmops_test_gemm_set_tuning(int rows_per_wave_tile) {
     if (llmops::test_hooks_enabled(__func__)) llmops::g_gemm_rt = rows_per_wave_tile;
-}
-extern "C" void llmops_test_gemm_set_interleaved(int on) {
-    if (llmops::test_hooks_enabled(__func__)) llmops::g_gemm_interleaved = on != 0;
 }
 extern "C" void llmops_test_gemm_set_split(int splits) {
     if (llmops::test_hooks_enabled(__func__)) llmops::g_gemm_force_split = splits < 0 ? 0 : splits;

@@ -61,7 +61,6 @@ SIGNATURES = {
     "llmops_test_calib_copy": (c_int, [c_ptr, c_ptr, c_i64, c_int, c_ptr]),
     "llmops_test_fc_set_tuning": (None, [c_int, c_int]),
     "llmops_test_gemm_set_tuning": (None, [c_int]),
-    "llmops_test_gemm_set_interleaved": (None, [c_int]),
     "llmops_test_gemm_set_reduce": (None, [c_int]),
     "llmops_test_gemm_set_split": (None, [c_int]),
     "llmops_test_fc_set_row_routing": (None, [c_int, c_int]),
