@@ -35,9 +35,15 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 # this process, so the figure is the recorded one and only holds for the fused plan at group 128, M=1.
 MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 27191830
 MEASURED_TRAFFIC_PROFILE = "profiles/fc_gemv_fused_kernel__hbm_traffic_pmc.md"
-# sha256 (first 16 hex digits) of the kernel's sources (csrc/fc_gemv.hip + csrc/gemv_device.h) when the counters were
-# read: the bench line says whether the sources have changed since, i.e. whether the recorded figure is stale
-MEASURED_TRAFFIC_KERNEL_SHA16 = "e1bc5639bf7d1534"
+# Counter summaries under profiles/ and the kernel sources each was taken from: sha256 (first 16 hex digits) of the
+# sources when the counters were read.  The bench line says for each whether the sources have changed since, i.e.
+# whether the recorded figures are stale.
+PROFILE_SOURCES = {
+    "profiles/fc_gemv_fused_kernel__hbm_traffic_pmc.md": (("fc_gemv.hip", "gemv_device.h"), "e1bc5639bf7d1534"),
+    "profiles/fc_gemv_fused_kernel__vector_alu_pmc.md": (("fc_gemv.hip", "gemv_device.h"), "e1bc5639bf7d1534"),
+    "profiles/fc_gemm_kernels__prefill_g128_pmc.md": (("fc_gemm.hip", "fc_rows.hip", "q8_act.hip"), "0000000000000000"),
+}
+MEASURED_TRAFFIC_KERNEL_SHA16 = PROFILE_SOURCES[MEASURED_TRAFFIC_PROFILE][1]
 G = 128
 LAYERS = 32
 # (name, N, K) of one layer's FCs, in the order the model calls them (chatllama/main.py:344-375)
@@ -45,13 +51,19 @@ LAYER_FCS = [("q", 4096, 4096), ("k", 4096, 4096), ("v", 4096, 4096), ("o", 4096
              ("gate", 11008, 4096), ("up", 11008, 4096), ("down", 4096, 11008)]
 
 
-def kernel_source_sha16():
+def kernel_source_sha16(files=("fc_gemv.hip", "gemv_device.h")):
     import hashlib
     h = hashlib.sha256()
-    for f in ("fc_gemv.hip", "gemv_device.h"):
+    for f in files:
         with open(os.path.join(ROOT, "llama.cl_amd", "csrc", f), "rb") as fh:
             h.update(fh.read())
     return h.hexdigest()[:16]
+
+
+def profiles_staleness():
+    """for every counter summary under profiles/: have the kernel sources it was taken from changed since?"""
+    return {prof: {"sources": list(files), "sha16_when_measured": sha, "sha16_now": kernel_source_sha16(files),
+                   "stale": kernel_source_sha16(files) != sha} for prof, (files, sha) in PROFILE_SOURCES.items()}
 
 
 def host_cpu_model():
@@ -222,6 +234,7 @@ def main():
         "unfused_7_launches_per_layer": {"GB/s": round(step_bytes / (results["unfused"]["ms_per_step"] * 1e-3) / 1e9, 2),
                                          "ms_per_step": round(results["unfused"]["ms_per_step"], 4)},
         "roofline": roof,
+        "profiles": profiles_staleness(),
     }
     if not args.no_decode:
         out["decode_step"] = decode_step(torch, stream)
@@ -325,7 +338,7 @@ def read_only_chain(torch, llmops, stream, dims, layers=32, reps=10):
                     "512/1024/2048 workgroups per size)"}
 
 
-def decode_step(torch, stream, kv_len=2048, reps=20):
+def decode_step(torch, stream, kv_len=2048, reps=50, warm=10):
     """BASELINE config 5: one token through a random-init Llama-2-7B-shape model (32 layers, hidden 4096, FFN 11008,
     32 heads, vocab 55296 lm_head, all FC Q4_1 group 128), fp32 KV cache filled to kv_len-1, batch 1; the step is
     captured once as a HIP graph and replayed."""
@@ -339,7 +352,8 @@ def decode_step(torch, stream, kv_len=2048, reps=20):
         kv.cache.normal_()
         dg = model.capture_decode(kv.cache, kv_len - 1, kv_len - 1, stream=stream)
         with torch.cuda.stream(stream):
-            dg.replay()
+            for _ in range(warm):  # the first replays of a fresh graph run 3-4 % slower than the steady state
+                dg.replay()
             torch.cuda.synchronize()
             t0 = time.perf_counter()
             for _ in range(reps):
