@@ -33,15 +33,15 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 # of `--calib` (one FETCH_SIZE count = 2.000 KiB, one WRITE_SIZE count = 1.000 KiB on this part); the summary with
 # the per-shape figures is profiles/fc_gemv_fused_kernel__hbm_traffic_pmc.md.  Counters cannot be read from inside
 # this process, so the figure is the recorded one and only holds for the fused plan at group 128, M=1.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 27191830
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 27191835
 MEASURED_TRAFFIC_PROFILE = "profiles/fc_gemv_fused_kernel__hbm_traffic_pmc.md"
 # Counter summaries under profiles/ and the kernel sources each was taken from: sha256 (first 16 hex digits) of the
 # sources when the counters were read.  The bench line says for each whether the sources have changed since, i.e.
 # whether the recorded figures are stale.
 PROFILE_SOURCES = {
-    "profiles/fc_gemv_fused_kernel__hbm_traffic_pmc.md": (("fc_gemv.hip", "gemv_device.h"), "e1bc5639bf7d1534"),
-    "profiles/fc_gemv_fused_kernel__vector_alu_pmc.md": (("fc_gemv.hip", "gemv_device.h"), "e1bc5639bf7d1534"),
-    "profiles/fc_gemm_kernels__prefill_g128_pmc.md": (("fc_gemm.hip", "fc_rows.hip", "q8_act.hip"), "0000000000000000"),
+    "profiles/fc_gemv_fused_kernel__hbm_traffic_pmc.md": (("fc_gemv.hip", "gemv_device.h"), "13290cb794320013"),
+    "profiles/fc_gemv_fused_kernel__vector_alu_pmc.md": (("fc_gemv.hip", "gemv_device.h"), "13290cb794320013"),
+    "profiles/fc_gemm_kernels__prefill_g128_pmc.md": (("fc_gemm.hip", "fc_rows.hip", "q8_act.hip"), "750904eb0dc879db"),
 }
 MEASURED_TRAFFIC_KERNEL_SHA16 = PROFILE_SOURCES[MEASURED_TRAFFIC_PROFILE][1]
 G = 128
