@@ -136,8 +136,14 @@ int llmops_fc_Q4A_residual(const float* x, int64_t rows, int64_t K, const int8_t
                            int group_k, int64_t N, const float* residual, float* y, void* workspace,
                            size_t workspace_bytes, llmops_stream_t stream);
 
-/* Decode-step form of fc_Q4A (rows <= 8) with the neighbouring ops of chatllama/main.py:344-375
- * folded into the one launch.  Each option may be left out (NULL / 0):
+/* fc_Q4A with the neighbouring ops of chatllama/main.py:344-375 folded in.  Up to 8 rows (a decode step) it is
+ * one launch.  With more rows (a batch of decode steps, a prompt) the producer of the input -- rmsnorm, or
+ * silu(gate)*up -- runs inside the quantization launch, so that its fp32 result never passes through memory,
+ * the residual is added in the product's stores and the sums of squares take a launch of their own; the codes,
+ * scales and results are those of the separate ops (llmops_rmsnorm_out / llmops_silu_mul, then llmops_fc_Q4A).
+ * More than 8 rows need whole 16-byte aligned rows, take glu 0 or 2 (2 with group 128 only), hidden sizes up to
+ * 16384 with norm_w, and compute the rmsnorm's statistic from the row (sumsq_in is accepted and not read).
+ * Each option may be left out (NULL / 0):
  *   norm_w, eps : x is rmsnorm'ed first (clone + rmsnorm, ops/op_misc.hpp:142-181); needs K % 4 == 0
  *   residual    : y += residual (iadd, ops/op_misc.hpp:55-79), fp32 [rows,N_out]
  *   glu == 1    : weiq holds gate and up strips interleaved (strip 2i = gate strip i, 2i+1 = up strip i,

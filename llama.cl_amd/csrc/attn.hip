@@ -647,34 +647,47 @@ __global__ __launch_bounds__(NWV * 64) void attn_decode_kernel(const int32_t* __
 // (4 waves x 32 queries, ONE QUERY PER LANE PAIR) and walks the cache in tiles of 32 rows that are
 // staged once in LDS:
 //
-//   S^T = K_tile * Q^T     v_mfma_f32_32x32x2_f32: A = K[kv = lane%32][k = lane/32 + 2i] from LDS,
-//                          B = the lane's own query row, kept in 64 registers.  The result puts
-//                          query lane%32 into the lane, 16 cache rows 8j + 4*(lane/32) + v each.
+//   S^T = K_tile * Q^T     v_mfma_f32_32x32x2_f32, 64 steps: in step i the lanes of half hf = lane/32
+//                          cover k = 64*hf + i (which k-values a step sums is free, as long as A and B
+//                          agree).  A = K[kv = lane%32][64*hf + i]: a lane's 64 operands are contiguous
+//                          in the LDS row, so one 16-byte read feeds four steps.  B = the lane's own
+//                          query row, elements 64*hf .. 64*hf+63, kept in 64 registers.  The result puts
+//                          query lane%32 into the lane, 16 cache rows 8j + 4*hf + v each.  Two
+//                          accumulators take alternate steps, so that no MFMA waits for the one before it.
 //   mask, online softmax   per lane, plus one exchange with lane^32 (the other 16 rows of the tile)
-//   O^T += V_tile^T * P^T  B = the lane's 16 probabilities exactly as they sit in registers (the k
-//                          index of this product is just a summation index, so the cache rows are
-//                          taken in the order 8j + 4*(lane/32) + v), A = V[that row][column] from LDS.
+//   O^T += V_tile^T * P^T  16 steps of 4 MFMAs.  B = the lane's 16 probabilities exactly as they sit in
+//                          registers (step i takes cache row 8*(i/4) + 4*hf + i%4).  MFMA c of a step
+//                          owns the output columns 4*m + c, m = 0..31, so A = V[row][4*(lane%32) + c]:
+//                          the four MFMAs' operands are one 16-byte read.
 //
-// Everything a lane holds (running max, sum, 4 x 16 output values) belongs to its own query, so
-// the rescaling needs no cross-lane traffic, and no probability ever goes through LDS.  Tiles that
-// no query of a wave may see (in-chunk causal mask, ops/op_attn.hpp:1007-1011) are skipped.
-// K rows are padded to 130 floats and V rows to 136 so that both operand reads are free of bank
-// conflicts.  Arithmetic is fp32 throughout (fp16 caches are widened when a tile is staged).
+// The operand reads run two reads (eight MFMAs) ahead of their use; scheduling fences keep them there
+// (left alone, the compiler issues every read right in front of its first use and the matrix pipe waits
+// out the LDS latency 48 times per tile).  Everything a lane holds (running max, sum, 4 x 16 output
+// values) belongs to its own query, so the rescaling needs no cross-lane traffic, and no probability
+// ever goes through LDS.  Tiles that no query of a wave may see (in-chunk causal mask,
+// ops/op_attn.hpp:1007-1011) are skipped.  K rows are padded to 132 floats: the 16 lanes that one phase
+// of a 16-byte read serves then touch 16 different 16-byte slots of the 256-byte bank line (33 is odd);
+// the V reads are contiguous per row.  Staging writes 256 contiguous bytes per 16 lanes.  Arithmetic is
+// fp32 throughout (fp16 caches are widened when a tile is staged).
 typedef float v16f __attribute__((ext_vector_type(16)));
 
 template <typename T>
 __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(float* q, const T* __restrict__ kc, const T* __restrict__ vc,
                                                              int64_t qL, int64_t H, int64_t maxlen, int64_t kvLen,
                                                              const int32_t* __restrict__ row_token, int qtiles) {
-    constexpr int S = 128, BQ = 128, BK = 32, KS = 130, VS = 136;
+    constexpr int S = 128, BQ = 128, BK = 32, KS = 132, VS = 128;
     __shared__ __align__(16) float ksh[BK * KS];
     __shared__ __align__(16) float vsh[BK * VS];
     __shared__ __align__(16) int tok[BK];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int hf = lane >> 5, c32 = lane & 31;
-    // late query tiles see the most cache rows: they are dealt out first so that they do not form the tail
+    // Late query tiles see the most cache rows.  They are dealt out first, in descending order, so that they do
+    // not form the tail; the early half follows in ASCENDING order: when the whole grid is resident at once (two
+    // workgroups per compute unit), workgroup i and workgroup i + gridDim.x/2 land on the same compute unit,
+    // and the heaviest tile then shares its SIMDs with the lightest, the next with the next lightest, ...
     const int64_t bhs = gridDim.x / qtiles;
-    const int qt = qtiles - 1 - (int)(blockIdx.x / bhs);
+    const int heavy = (qtiles + 1) / 2, slot = (int)(blockIdx.x / bhs);
+    const int qt = slot < heavy ? qtiles - 1 - slot : slot - heavy;
     const int64_t bh = blockIdx.x % bhs, b = bh / H, h = bh % H;
     const int64_t q_lo_wave = (int64_t)qt * BQ + wave * 32;
     const int64_t pq = q_lo_wave + c32;  // this lane's query token
@@ -684,13 +697,12 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(float* q, const T*
     const T* kbase = kc + bh * maxlen * S;
     const T* vbase = vc + bh * maxlen * S;
 
-    // the lane's query row, elements hf, hf+2, hf+4, ... (the k-values its MFMA operand slots cover)
+    // the lane's half of its query row: elements 64*hf .. 64*hf + 63
     float qreg[64];
 #pragma unroll
-    for (int i = 0; i < 32; i++) {
-        const float4 t = *reinterpret_cast<const float4*>(qrow + i * 4);
-        qreg[2 * i] = hf ? t.y : t.x;
-        qreg[2 * i + 1] = hf ? t.w : t.z;
+    for (int i = 0; i < 16; i++) {
+        const float4 t = *reinterpret_cast<const float4*>(qrow + hf * 64 + i * 4);
+        qreg[4 * i] = t.x, qreg[4 * i + 1] = t.y, qreg[4 * i + 2] = t.z, qreg[4 * i + 3] = t.w;
     }
     const float d_scale = 1.0f / sqrtf((float)S);
     float m_run = -FLT_MAX, l_run = 0.0f;
@@ -700,58 +712,91 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(float* q, const T*
 #pragma unroll
         for (int r = 0; r < 16; r++) o[c][r] = 0.0f;
 
-    // staging: every thread moves 16 columns of one row of the K and of the V tile.  The next tile's
-    // global loads are issued before the current tile is computed on and land in registers meanwhile.
-    const int trow = threadIdx.x >> 3, tseg = threadIdx.x & 7;
+    // staging: 16 lanes move 64 contiguous floats of a row (a wave: 4 rows, the workgroup: 16 rows) of the K
+    // and of the V tile, four times over (row halves 0/1, rows +0/+16).  The next tile's global loads are
+    // issued before the current tile is computed on and land in registers meanwhile.
+    const int srow = wave * 4 + (lane >> 4), scol = (lane & 15) * 4;
     float4 kst[4], vst[4];
     int tst = INT_MAX;
 #define LLMOPS_STAGE_LOAD(KV0)                                                                          \
     do {                                                                                                \
-        const int64_t r_ = (KV0) + trow < kvLen ? (KV0) + trow : kvLen - 1;                             \
         _Pragma("unroll") for (int u = 0; u < 4; u++) {                                                 \
-            kst[u] = load4(kbase + r_ * S + tseg * 16 + u * 4);                                         \
-            vst[u] = load4(vbase + r_ * S + tseg * 16 + u * 4);                                         \
+            const int64_t r_ = (KV0) + srow + 16 * (u >> 1) < kvLen ? (KV0) + srow + 16 * (u >> 1) : kvLen - 1; \
+            kst[u] = load4(kbase + r_ * S + (u & 1) * 64 + scol);                                       \
+            vst[u] = load4(vbase + r_ * S + (u & 1) * 64 + scol);                                       \
         }                                                                                               \
         if (threadIdx.x < BK) tst = ((KV0) + threadIdx.x < kvLen) ? row_token[(KV0) + threadIdx.x] : INT_MAX; \
     } while (0)
     LLMOPS_STAGE_LOAD(0);
+    const float* kp = &ksh[c32 * KS + hf * 64];  // + 4j: the operands of steps 4j .. 4j+3
+    const float* vp = &vsh[4 * hf * VS + 4 * c32];  // + (8*(i/4) + i%4) * VS: the operands of step i
     for (int64_t kv0 = 0; kv0 < kvLen; kv0 += BK) {
         __syncthreads();  // the previous tile has been consumed
 #pragma unroll
         for (int u = 0; u < 4; u++) {
-            const int col = tseg * 16 + u * 4;
-            float2* kd = reinterpret_cast<float2*>(&ksh[trow * KS + col]);  // 8-byte aligned (KS even)
-            kd[0] = make_float2(kst[u].x, kst[u].y);
-            kd[1] = make_float2(kst[u].z, kst[u].w);
-            *reinterpret_cast<float4*>(&vsh[trow * VS + col]) = vst[u];
+            const int row = srow + 16 * (u >> 1), col = (u & 1) * 64 + scol;
+            *reinterpret_cast<float4*>(&ksh[row * KS + col]) = kst[u];
+            *reinterpret_cast<float4*>(&vsh[row * VS + col]) = vst[u];
         }
         if (threadIdx.x < BK) tok[threadIdx.x] = tst;
         __syncthreads();
         if (kv0 + BK < kvLen) LLMOPS_STAGE_LOAD(kv0 + BK);
-        // skip the tile if even the wave's last query may not see any of its rows
-        int tmin = tok[c32];
+        // skip the tile if even the wave's last query may not see any of its rows; a tile that every query of the
+        // wave sees whole (the usual case away from the diagonal) needs no masks
+        int tmin = tok[c32], tmax = tmin;
 #pragma unroll
-        for (int off = 16; off > 0; off >>= 1) tmin = min(tmin, __shfl_xor(tmin, off, 64));
+        for (int off = 16; off > 0; off >>= 1) {
+            tmin = min(tmin, __shfl_xor(tmin, off, 64));
+            tmax = max(tmax, __shfl_xor(tmax, off, 64));
+        }
         if (q_lo_wave >= qL || (int64_t)tmin > q_hi_wave) continue;
+        const bool all_visible = (int64_t)tmax <= q_lo_wave && q_lo_wave + 31 < qL;
 
-        v16f sacc;
+        v16f s0, s1;
 #pragma unroll
-        for (int r = 0; r < 16; r++) sacc[r] = 0.0f;
-        const float* kp = &ksh[c32 * KS + hf];
+        for (int r = 0; r < 16; r++) s0[r] = 0.0f, s1[r] = 0.0f;
+        {
+            float4 kk[3];
+            kk[0] = *reinterpret_cast<const float4*>(kp);
+            kk[1] = *reinterpret_cast<const float4*>(kp + 4);
 #pragma unroll
-        for (int i = 0; i < 64; i++) sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(kp[2 * i], qreg[i], sacc, 0, 0, 0);
+            for (int j = 0; j < 16; j++) {
+                if (j + 2 < 16) kk[(j + 2) % 3] = *reinterpret_cast<const float4*>(kp + 4 * (j + 2));
+                __builtin_amdgcn_sched_barrier(0);
+                const float4 a = kk[j % 3];
+                s0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a.x, qreg[4 * j], s0, 0, 0, 0);
+                s1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a.y, qreg[4 * j + 1], s1, 0, 0, 0);
+                s0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a.z, qreg[4 * j + 2], s0, 0, 0, 0);
+                s1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a.w, qreg[4 * j + 3], s1, 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+        // the first two V operands are asked for before the softmax, which hides their latency
+        float4 vv[3];
+        vv[0] = *reinterpret_cast<const float4*>(vp);
+        vv[1] = *reinterpret_cast<const float4*>(vp + VS);
+        v16f sacc = s0 + s1;
 
         // scale, mask (rows written by later tokens of this call, rows beyond kvLen), running max
         float mx = -FLT_MAX;
+        if (all_visible) {  // (the same for the whole wave)
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-            const int4 t4 = *reinterpret_cast<const int4*>(&tok[8 * j + 4 * hf]);
-            const int tt[4] = {t4.x, t4.y, t4.z, t4.w};
+            for (int r = 0; r < 16; r++) {
+                sacc[r] *= d_scale;
+                mx = fmaxf(mx, sacc[r]);
+            }
+        } else {
+            const int pq32 = valid ? (int)pq : INT_MIN;  // (the launcher keeps qL below 2^31)
 #pragma unroll
-            for (int v = 0; v < 4; v++) {
-                const float sv = (valid && (int64_t)tt[v] <= pq) ? sacc[4 * j + v] * d_scale : -FLT_MAX;
-                sacc[4 * j + v] = sv;
-                mx = fmaxf(mx, sv);
+            for (int j = 0; j < 4; j++) {
+                const int4 t4 = *reinterpret_cast<const int4*>(&tok[8 * j + 4 * hf]);
+                const int tt[4] = {t4.x, t4.y, t4.z, t4.w};
+#pragma unroll
+                for (int v = 0; v < 4; v++) {
+                    const float sv = (tt[v] <= pq32) ? sacc[4 * j + v] * d_scale : -FLT_MAX;
+                    sacc[4 * j + v] = sv;
+                    mx = fmaxf(mx, sv);
+                }
             }
         }
         mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
@@ -766,31 +811,39 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(float* q, const T*
         }
         psum += __shfl_xor(psum, 32, 64);
         l_run = l_run * alpha + psum;
+        if (__any(m_new != m_run)) {  // (alpha is exactly 1 for a query whose maximum did not move)
+#pragma unroll
+            for (int c = 0; c < 4; c++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) o[c][r] *= alpha;
+        }
         m_run = m_new;
-#pragma unroll
-        for (int c = 0; c < 4; c++)
-#pragma unroll
-            for (int r = 0; r < 16; r++) o[c][r] *= alpha;
 
         // O^T += V^T P^T; step i of the product takes cache row 8*(i/4) + 4*hf + i%4 of the tile
 #pragma unroll
         for (int i = 0; i < 16; i++) {
-            const float* vp = &vsh[(8 * (i / 4) + 4 * hf + (i % 4)) * VS + c32];
-#pragma unroll
-            for (int c = 0; c < 4; c++) o[c] = __builtin_amdgcn_mfma_f32_32x32x2f32(vp[32 * c], sacc[i], o[c], 0, 0, 0);
+            if (i + 2 < 16) vv[(i + 2) % 3] = *reinterpret_cast<const float4*>(vp + (8 * ((i + 2) / 4) + ((i + 2) % 4)) * VS);
+            __builtin_amdgcn_sched_barrier(0);
+            const float4 a = vv[i % 3];
+            o[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.x, sacc[i], o[0], 0, 0, 0);
+            o[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.y, sacc[i], o[1], 0, 0, 0);
+            o[2] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.z, sacc[i], o[2], 0, 0, 0);
+            o[3] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.w, sacc[i], o[3], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
         }
     }
 
 #undef LLMOPS_STAGE_LOAD
     if (!valid) return;
     const float inv = 1.0f / l_run;
-    // the lane holds columns 32c + 8j + 4*hf + v of its query's output row
+    // register 4j + v of o[c] is column 4*(8j + 4*hf + v) + c of the query's output row
 #pragma unroll
-    for (int c = 0; c < 4; c++)
+    for (int j = 0; j < 4; j++)
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-            const float4 out = make_float4(o[c][4 * j] * inv, o[c][4 * j + 1] * inv, o[c][4 * j + 2] * inv, o[c][4 * j + 3] * inv);
-            *reinterpret_cast<float4*>(qrow + 32 * c + 8 * j + 4 * hf) = out;
+        for (int v = 0; v < 4; v++) {
+            const int r = 4 * j + v;
+            *reinterpret_cast<float4*>(qrow + 4 * (8 * j + 4 * hf + v)) =
+                make_float4(o[0][r] * inv, o[1][r] * inv, o[2][r] * inv, o[3][r] * inv);
         }
 }
 

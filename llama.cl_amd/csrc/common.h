@@ -96,6 +96,32 @@ __device__ __forceinline__ float wave_sum(float v) {
     return v;
 }
 
+// rmsnorm's scale 1/sqrt(mean(x^2) + eps) of one row, computed by a workgroup of 1024 threads that keeps the
+// row in registers (v[i] = floats 4*(1024*i + thread) .. +3, zeros beyond the row).  Every kernel that
+// normalizes whole rows goes through this one function, so that they agree bit for bit.  red: 16 floats of LDS.
+template <int VPT>
+__device__ __forceinline__ float rmsnorm_row_scale(const float* __restrict__ row, int64_t hidden, float eps, float4 (&v)[VPT],
+                                                   float* red) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    float ss = 0.0f;
+#pragma unroll
+    for (int i = 0; i < VPT; i++) {
+        const int64_t e = ((int64_t)i * 1024 + threadIdx.x) * 4;
+        v[i] = e < hidden ? *reinterpret_cast<const float4*>(row + e) : make_float4(0.f, 0.f, 0.f, 0.f);
+        ss = fmaf(v[i].x, v[i].x, ss);
+        ss = fmaf(v[i].y, v[i].y, ss);
+        ss = fmaf(v[i].z, v[i].z, ss);
+        ss = fmaf(v[i].w, v[i].w, ss);
+    }
+    ss = wave_sum(ss);
+    if (lane == 0) red[wave] = ss;
+    __syncthreads();
+    float tot = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 16; i++) tot += red[i];
+    return 1.0f / sqrtf(tot / (float)hidden + eps);
+}
+
 #endif  // __HIPCC__
 
 }  // namespace llmops

@@ -10,6 +10,9 @@ constexpr int kMaxGemvRows = 8;
 
 int launch_quant_x(const float* x, int64_t rows, int64_t K, int group_k, int8_t* xq, float* xd, float* gsum, float2* xsT,
                    bool exact_sum, hipStream_t stream);
+int launch_quant_x_fused(const float* x, int64_t rows, int64_t K, int group_k, const float* norm_w, float eps, bool glu_in,
+                         int8_t* xq, float* xd, float* gsum, float2* xsT, hipStream_t stream);
+int launch_strip_sumsq(const float* y, int64_t rows, int64_t N, float* out, hipStream_t st);
 size_t gemv_workspace_bytes(int64_t rows, int64_t Ng, int64_t Kg, int G);
 int launch_gemv(const uint8_t* w, const int8_t* xq, const float* xd, const float* gs, float* y, float* part,
                 unsigned* counters, int64_t rows, int64_t Ng, int64_t Kg, int G, int64_t N, hipStream_t st);
@@ -84,6 +87,27 @@ static int fc_check_args(const float* x, int64_t rows, int64_t K, const int8_t* 
     return LLMOPS_OK;
 }
 
+// the product for activations that a quantization launch has left in the workspace (more rows than the streaming
+// kernel that quantizes on the fly takes)
+static int fc_product_many_rows(const uint8_t* w, uint8_t* ws, const FcWorkspace& lay, int64_t rows, int64_t Ng, int64_t Kg,
+                                int group_k, int64_t N, const float* residual, float* y, hipStream_t st) {
+    const int8_t* xq = reinterpret_cast<const int8_t*>(ws + lay.off_xq);
+    const float* xd = reinterpret_cast<const float*>(ws + lay.off_xd);
+    const float* gs = reinterpret_cast<const float*>(ws + lay.off_gs);
+    const float2* xst = reinterpret_cast<const float2*>(ws + lay.off_xst);
+    const bool rows_kernel = group_k == 128 && Ng >= 64 && gemm_rows_kernel_enabled();
+    // up to 16 rows are still bound by the weight stream: one strip per workgroup, MFMA inner product
+    // (measured against the tiled kernel: 15 vs 18 us at 16 rows, 11008x4096).  17..32 rows (two row tiles
+    // per wave) only win for tensors of fewer than 256 strips, where the tiled kernel has too few tiles
+    // (us, tiled / streaming: 4096x4096 at 17 rows 20.2 / 9.9, at 32 rows 24.3 / 11.9; 4096x11008 at 24 rows
+    // 22.0 / 15.7; 11008x4096 at 24 rows 19.3 / 18.8; 12288x4096 17.9 / 19.0; 22016x4096 23.0 / 27.4)
+    if (rows_kernel && (rows <= 16 || (rows <= 32 && Ng < 256)))
+        return launch_fc_rows(w, xq, xst, y, rows, Ng, Kg, N, residual, reinterpret_cast<unsigned long long*>(ws + kTicketBytes),
+                              LLMOPS_FC_COUNTER_BYTES - kTicketBytes, st);
+    return launch_gemm(w, xq, xd, gs, xst, y, reinterpret_cast<float*>(ws + lay.off_part), reinterpret_cast<unsigned*>(ws), rows, Ng,
+                       Kg, group_k, N, residual, st);
+}
+
 static int fc_impl(const float* x, int64_t rows, int64_t K, const int8_t* weiq, int64_t Ng, int64_t Kg, int group_k,
                    int64_t N, const float* residual, float* y, void* workspace, size_t workspace_bytes,
                    llmops_stream_t stream) {
@@ -131,15 +155,7 @@ static int fc_impl(const float* x, int64_t rows, int64_t K, const int8_t* weiq, 
     float2* xst = reinterpret_cast<float2*>(ws + lay.off_xst);
     int rc = launch_quant_x(x, rows, K, group_k, xq, xd, gs, xst, false, st);
     if (rc) return rc;
-    // up to 16 rows are still bound by the weight stream: one strip per workgroup, MFMA inner product
-    // (measured against the tiled kernel: 15 vs 18 us at 16 rows, 11008x4096).  17..32 rows (two row tiles
-    // per wave) only win for tensors of fewer than 256 strips, where the tiled kernel has too few tiles
-    // (us, tiled / streaming: 4096x4096 at 17 rows 20.2 / 9.9, at 32 rows 24.3 / 11.9; 4096x11008 at 24 rows
-    // 22.0 / 15.7; 11008x4096 at 24 rows 19.3 / 18.8; 12288x4096 17.9 / 19.0; 22016x4096 23.0 / 27.4)
-    if (rows_kernel && (rows <= 16 || (rows <= 32 && Ng < 256)))
-        return launch_fc_rows(w, xq, xst, y, rows, Ng, Kg, N, residual, reinterpret_cast<unsigned long long*>(ws + kTicketBytes),
-                              LLMOPS_FC_COUNTER_BYTES - kTicketBytes, st);
-    return launch_gemm(w, xq, xd, gs, xst, y, part, counters, rows, Ng, Kg, group_k, N, residual, st);
+    return fc_product_many_rows(w, ws, lay, rows, Ng, Kg, group_k, N, residual, y, st);
 }
 
 extern "C" int llmops_fc_Q4A(const float* x, int64_t rows, int64_t K, const int8_t* weiq, int64_t Ng, int64_t Kg,
@@ -161,7 +177,7 @@ extern "C" int llmops_fc_Q4A_decode(const float* x, int64_t rows, int64_t K, con
                                     void* workspace, size_t workspace_bytes, llmops_stream_t stream) {
     LLMOPS_REQUIRE(valid_group(group_k));
     LLMOPS_REQUIRE(x != nullptr && weiq != nullptr && y != nullptr && workspace != nullptr);
-    LLMOPS_REQUIRE(rows > 0 && rows <= kMaxGemvRows);
+    LLMOPS_REQUIRE(rows > 0);
     LLMOPS_REQUIRE(K > 0 && Ng > 0 && Kg > 0 && K == Kg * group_k);
     LLMOPS_REQUIRE(Ng <= kTicketBytes / 4 && Ng * 64 < ((int64_t)1 << 31));
     LLMOPS_REQUIRE(aligned(weiq, 16) && aligned(workspace, 256) && aligned(x, 8));
@@ -180,6 +196,25 @@ extern "C" int llmops_fc_Q4A_decode(const float* x, int64_t rows, int64_t K, con
     if (workspace_bytes < lay.total)
         return fail(LLMOPS_EWORKSPACE, "fc_Q4A needs %zu workspace bytes, got %zu", lay.total, workspace_bytes);
     uint8_t* ws = reinterpret_cast<uint8_t*>(workspace);
+    if (rows > kMaxGemvRows) {
+        // More rows than the streaming kernel takes: the producer is folded into the quantization launch instead
+        // (its fp32 result never goes through memory), the residual into the product's stores, and the sums of
+        // squares take a launch of their own.  The statistic of the rmsnorm is computed from the row (sumsq_in is
+        // not needed: the launch has the whole row in registers).
+        if (glu == 1) return fail(LLMOPS_EINVAL, "fc_Q4A_decode with more than 8 rows: gate and up stacked (glu 2), not interleaved");
+        hipStream_t st = as_stream(stream);
+        int8_t* xq = reinterpret_cast<int8_t*>(ws + lay.off_xq);
+        float* xd = reinterpret_cast<float*>(ws + lay.off_xd);
+        float* gs = reinterpret_cast<float*>(ws + lay.off_gs);
+        float2* xst = reinterpret_cast<float2*>(ws + lay.off_xst);
+        int rc = (norm_w != nullptr || glu == 2)
+                     ? launch_quant_x_fused(x, rows, K, group_k, norm_w, eps, glu == 2, xq, xd, gs, xst, st)
+                     : launch_quant_x(x, rows, K, group_k, xq, xd, gs, xst, false, st);
+        if (rc) return rc;
+        rc = fc_product_many_rows(reinterpret_cast<const uint8_t*>(weiq), ws, lay, rows, Ng, Kg, group_k, N_out, residual, y, st);
+        if (rc == 0 && sumsq_out != nullptr) rc = launch_strip_sumsq(y, rows, N_out, sumsq_out, st);
+        return rc;
+    }
     return launch_gemv_fused(reinterpret_cast<const uint8_t*>(weiq), x, y, reinterpret_cast<float*>(ws + lay.off_part),
                              reinterpret_cast<unsigned*>(ws), rows, Ng, Kg, group_k, N_out, residual, norm_w, eps, glu,
                              sumsq_in, (int)sumsq_parts, sumsq_out, as_stream(stream));

@@ -14,6 +14,11 @@
 // After every k-group the int32 tile is folded into fp32 accumulators:
 //   f += (d[n]*dx[row]) * float(acc) ; f += m[n]*gsum[row]        (fc_Q4A,
 //   /root/reference/ops/op_fc.hpp:381-412; min term is m * raw group sum).
+// The group-128 kernels with LDS tiles compute the first term as fma(fma(X, d, -B*d), dx, f): their
+// int32 sums start at the bit pattern of the float B = 1.5 * 2^23, so the sum's register, read as a
+// float X, IS B + sum (|sum| <= 128*15*127 < 2^22), and X*d - B*d = sum*d is exact before the fma's
+// one rounding because B*d (2 significant bits times the 11 of an fp16) is itself a float.  Two
+// vector instructions per output element and k-group instead of three (convert, multiply, fma).
 // Result tile layout of the 16x16 MFMAs: lane holds column jj, rows 4*g+v in register v.
 #include "common.h"
 #include "gemv_device.h"
@@ -24,6 +29,9 @@ typedef int v4i __attribute__((ext_vector_type(4)));
 typedef unsigned int v4u __attribute__((ext_vector_type(4)));
 typedef float v2f __attribute__((ext_vector_type(2)));
 typedef float v4f __attribute__((ext_vector_type(4)));
+
+constexpr int kFoldBiasBits = 0x4B400000;  // the float 1.5 * 2^23 ...
+constexpr float kFoldBias = 12582912.0f;   // ... whose low mantissa bits count in units of 1
 
 __device__ __forceinline__ uint32_t lo4(uint32_t w) { return w & 0x0F0F0F0Fu; }
 __device__ __forceinline__ uint32_t hi4(uint32_t w) { return (w >> 4) & 0x0F0F0F0Fu; }
@@ -402,10 +410,13 @@ __global__ __launch_bounds__(256, (RT == 4 ? 2 : (RT == 2 ? 3 : 4))) void fc_gem
         const uint8_t* bblk = &sm.b[buf][strip_l * kBlk128];
         const uint8_t* abase = &sm.a[buf][(wr * (BM / 2) + jj) * kAStride + g * 16];
         v4i acc[RT][4];
+        // the sums start at the bit pattern of 1.5 * 2^23, so that the fold needs no convert instruction
+        // (see fc_gemm_pp_kernel)
+        constexpr int kInit = PARTIALS ? 0 : kFoldBiasBits;
 #pragma unroll
         for (int t = 0; t < RT; t++)
 #pragma unroll
-            for (int c = 0; c < 4; c++) acc[t][c] = v4i{0, 0, 0, 0};
+            for (int c = 0; c < 4; c++) acc[t][c] = v4i{kInit, kInit, kInit, kInit};
 #pragma unroll
         for (int h = 0; h < 2; h++) {
             const uint4 wa = *reinterpret_cast<const uint4*>(bblk + h * 1024 + (2 * g) * kRowBytes + q * 16);
@@ -456,6 +467,7 @@ __global__ __launch_bounds__(256, (RT == 4 ? 2 : (RT == 2 ? 3 : 4))) void fc_gem
             m[1] = f16_bits_to_f32((uint16_t)(mh.x >> 16));
             m[2] = f16_bits_to_f32((uint16_t)(mh.y & 0xFFFFu));
             m[3] = f16_bits_to_f32((uint16_t)(mh.y >> 16));
+            const float nbd[4] = {-kFoldBias * d[0], -kFoldBias * d[1], -kFoldBias * d[2], -kFoldBias * d[3]};
             const int slot4 = (kb - kb0) & 3;
             const bool mine4 = slot4 == g;
 #pragma unroll
@@ -471,7 +483,8 @@ __global__ __launch_bounds__(256, (RT == 4 ? 2 : (RT == 2 ? 3 : 4))) void fc_gem
 #pragma unroll
                 for (int v = 0; v < 4; v++)
 #pragma unroll
-                    for (int c = 0; c < 4; c++) f[t][c][v] = fmaf(d[c] * dxv[v], (float)acc[t][c][v], f[t][c][v]);
+                    for (int c = 0; c < 4; c++)
+                        f[t][c][v] = fmaf(fmaf(__int_as_float(acc[t][c][v]), d[c], nbd[c]), dxv[v], f[t][c][v]);
             }
             if (slot4 == 3 || kb + 1 == kb1) {
 #pragma unroll
@@ -786,7 +799,9 @@ __global__ __launch_bounds__(512, 2) void fc_gemm_pp_kernel(const uint8_t* __res
             for (int t = 0; t < RT; t++) gsr[t] = sm.gs[buf][lrow + t * 16 + jj];
         }
         v4i acc[RT][4];
-        const v4i zero4 = v4i{0, 0, 0, 0};
+        // The int32 sums start at the bit pattern of 1.5 * 2^23: read as a float, bits + sum IS the number
+        // 1.5 * 2^23 + sum (|sum| <= 128 * 15 * 127 < 2^22), so the fold needs no convert instruction.
+        const v4i zero4 = PARTIALS ? v4i{0, 0, 0, 0} : v4i{kFoldBiasBits, kFoldBiasBits, kFoldBiasBits, kFoldBiasBits};
 #define LLMOPS_MMA4(T, H, A)                                                                              \
     _Pragma("unroll") for (int c = 0; c < 4; c++)                                                         \
         acc[T][c] = __builtin_amdgcn_mfma_i32_16x16x64_i8(A, b[H][c], (H) == 0 ? zero4 : acc[T][c], 0, 0, 0)
@@ -818,6 +833,7 @@ __global__ __launch_bounds__(512, 2) void fc_gemm_pp_kernel(const uint8_t* __res
         LLMOPS_MMA4(3, 1, a13);
 #undef LLMOPS_MMA4
         const float d[4] = {d4.x, d4.y, d4.z, d4.w};
+        const float nbd[4] = {-kFoldBias * d4.x, -kFoldBias * d4.y, -kFoldBias * d4.z, -kFoldBias * d4.w};
         if (!PARTIALS) {
             const float m[4] = {m4.x, m4.y, m4.z, m4.w};
             const int slot4 = (kb - kb0) & 3;
@@ -866,10 +882,13 @@ __global__ __launch_bounds__(512, 2) void fc_gemm_pp_kernel(const uint8_t* __res
                 // dx of the 4 rows this lane holds results for: rows lrow + t*16 + 4g + v
                 const float4 x4 = *reinterpret_cast<const float4*>(&sm.dx[buf][lrow + t * 16 + g * 4]);
                 const float dxv[4] = {x4.x, x4.y, x4.z, x4.w};
+                // sum * d in one fma: (bias + sum) * d - bias * d, exact before its single rounding because
+                // bias * d (2 significant bits times the 11 of an fp16) is a float; then one fma with dx
 #pragma unroll
                 for (int v = 0; v < 4; v++)
 #pragma unroll
-                    for (int c = 0; c < 4; c++) f[t][c][v] = fmaf(d[c] * dxv[v], (float)acc[t][c][v], f[t][c][v]);
+                    for (int c = 0; c < 4; c++)
+                        f[t][c][v] = fmaf(fmaf(__int_as_float(acc[t][c][v]), d[c], nbd[c]), dxv[v], f[t][c][v]);
             }
         }
         // the fold is register arithmetic, which the compiler may move across the barrier into the other

@@ -13,25 +13,8 @@ __global__ __launch_bounds__(1024) void rmsnorm_kernel(const float* __restrict__
     __shared__ float red[16];
     const float* row = x + (int64_t)blockIdx.x * hidden;
     float* orow = out + (int64_t)blockIdx.x * hidden;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     float4 v[VPT];
-    float ss = 0.0f;
-#pragma unroll
-    for (int i = 0; i < VPT; i++) {
-        const int64_t e = ((int64_t)i * 1024 + threadIdx.x) * 4;
-        v[i] = e < hidden ? *reinterpret_cast<const float4*>(row + e) : make_float4(0.f, 0.f, 0.f, 0.f);
-        ss = fmaf(v[i].x, v[i].x, ss);
-        ss = fmaf(v[i].y, v[i].y, ss);
-        ss = fmaf(v[i].z, v[i].z, ss);
-        ss = fmaf(v[i].w, v[i].w, ss);
-    }
-    ss = wave_sum(ss);
-    if (lane == 0) red[wave] = ss;
-    __syncthreads();
-    float tot = 0.0f;
-#pragma unroll
-    for (int i = 0; i < 16; i++) tot += red[i];
-    const float rs = 1.0f / sqrtf(tot / (float)hidden + eps);
+    const float rs = rmsnorm_row_scale<VPT>(row, hidden, eps, v, red);
 #pragma unroll
     for (int i = 0; i < VPT; i++) {
         const int64_t e = ((int64_t)i * 1024 + threadIdx.x) * 4;
@@ -174,6 +157,10 @@ __global__ void emb_kernel(float* __restrict__ out, const int64_t* __restrict__ 
 
 using namespace llmops;
 
+namespace llmops {
+int launch_strip_sumsq(const float* y, int64_t rows, int64_t N, float* out, hipStream_t st);
+}
+
 static int rmsnorm_launch(const float* x, float* out, int64_t rows, int64_t hidden, const float* w, float eps,
                           llmops_stream_t stream) {
     LLMOPS_REQUIRE(x != nullptr && out != nullptr && w != nullptr && rows > 0 && hidden > 0 && rows < ((int64_t)1 << 31));
@@ -220,14 +207,17 @@ extern "C" int llmops_silu_mul_interleaved(const float* gate_up, float* out, int
 
 extern "C" int llmops_strip_sumsq(const float* y, int64_t rows, int64_t N, float* out, llmops_stream_t stream) {
     LLMOPS_REQUIRE(y != nullptr && out != nullptr && rows > 0 && N > 0);
-    const int64_t Ng = (N + 31) / 32, threads = rows * Ng * 32;
-    LLMOPS_REQUIRE((threads + 255) / 256 < ((int64_t)1 << 31));
-    strip_sumsq_kernel<<<(unsigned)((threads + 255) / 256), 256, 0, as_stream(stream)>>>(y, rows, N, Ng, out);
-    LLMOPS_LAUNCH_CHECK();
-    return LLMOPS_OK;
+    return launch_strip_sumsq(y, rows, N, out, as_stream(stream));
 }
 
 namespace llmops {
+int launch_strip_sumsq(const float* y, int64_t rows, int64_t N, float* out, hipStream_t st) {
+    const int64_t Ng = (N + 31) / 32, threads = rows * Ng * 32;
+    if ((threads + 255) / 256 >= ((int64_t)1 << 31)) return fail(LLMOPS_EINVAL, "strip_sumsq: too many strips for one launch");
+    strip_sumsq_kernel<<<(unsigned)((threads + 255) / 256), 256, 0, st>>>(y, rows, N, Ng, out);
+    LLMOPS_LAUNCH_CHECK();
+    return LLMOPS_OK;
+}
 int launch_add(float* a, const float* b, int64_t total, hipStream_t st) {
     ibinary_kernel<false><<<(unsigned)((total + 255) / 256), 256, 0, st>>>(a, b, total, total, 0);
     LLMOPS_LAUNCH_CHECK();

@@ -137,7 +137,9 @@ __global__ __launch_bounds__(256) void quant_x_rows_kernel(const float* __restri
 // threads per row): a team reads U*512 contiguous bytes and writes U*128 contiguous bytes of codes, and the 8
 // teams' pairs of one k-group are 64 contiguous bytes -- with one row per workgroup every pair was an 8-byte
 // store into a line of its own, 16 KB from the next.  Codes and scales as in quant_x_rows_kernel.
-template <int U>
+// GLU: x is [rows, 2*Kg*G], a row holding the gate and the up projection side by side, and what is quantized is
+// silu(gate) * up (silu_mul_kernel's expression, so the codes are those of the two launches it replaces).
+template <int U, bool GLU = false>
 __global__ __launch_bounds__(256) void quant_x_tile128_kernel(const float* __restrict__ x, int rows, int Kg, int kparts,
                                                                int8_t* __restrict__ xq, float2* __restrict__ xsT) {
     constexpr int G = 128;
@@ -147,8 +149,22 @@ __global__ __launch_bounds__(256) void quant_x_tile128_kernel(const float* __res
     const bool row_ok = row < rows;
     const int64_t rbase = (int64_t)(row_ok ? row : rows - 1) * Kg;
     float4 v[U];
+    if (GLU) {
+        float4 gt[U], up[U];
 #pragma unroll
-    for (int u = 0; u < U; u++) v[u] = *reinterpret_cast<const float4*>(x + (rbase + min(kb0 + u, Kg - 1)) * G + sub * 4);
+        for (int u = 0; u < U; u++) {
+            const float* p = x + (2 * rbase + min(kb0 + u, Kg - 1)) * G + sub * 4;
+            gt[u] = *reinterpret_cast<const float4*>(p);
+            up[u] = *reinterpret_cast<const float4*>(p + (int64_t)Kg * G);
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++)
+            v[u] = make_float4(silu_times(gt[u].x, up[u].x), silu_times(gt[u].y, up[u].y), silu_times(gt[u].z, up[u].z),
+                               silu_times(gt[u].w, up[u].w));
+    } else {
+#pragma unroll
+        for (int u = 0; u < U; u++) v[u] = *reinterpret_cast<const float4*>(x + (rbase + min(kb0 + u, Kg - 1)) * G + sub * 4);
+    }
 #pragma unroll
     for (int u = 0; u < U; u++) {
         float amax = fmaxf(fmaxf(fabsf(v[u].x), fabsf(v[u].y)), fmaxf(fabsf(v[u].z), fabsf(v[u].w)));
@@ -170,11 +186,99 @@ __global__ __launch_bounds__(256) void quant_x_tile128_kernel(const float* __res
     }
 }
 
+// rmsnorm and the quantization of its result in one pass over the row: one workgroup of 1024 threads per row, the
+// row in registers as in rmsnorm_kernel (same statistic, same expression for the normalized value), and the G/4
+// neighbouring threads that hold a k-group quantize it as quant_x_rows_kernel does (same reduction tree, same
+// codes, scales and sums as rmsnorm_out followed by that kernel).  hidden % G == 0.
+template <int VPT, int G>
+__global__ __launch_bounds__(1024) void rmsnorm_quant_kernel(const float* __restrict__ x, int64_t hidden,
+                                                              const float* __restrict__ w, float eps, int rows, int Kg,
+                                                              int8_t* __restrict__ xq, float* __restrict__ xd,
+                                                              float* __restrict__ gsum, float2* __restrict__ xsT) {
+    constexpr int TPG = G / 4;
+    __shared__ float red[16];
+    const int row = blockIdx.x;
+    float4 v[VPT];
+    const float rs = rmsnorm_row_scale<VPT>(x + (int64_t)row * hidden, hidden, eps, v, red);
+#pragma unroll
+    for (int i = 0; i < VPT; i++) {
+        const int64_t e = ((int64_t)i * 1024 + threadIdx.x) * 4;
+        const bool live = e < hidden;  // the same for all threads of a team (hidden is a whole number of groups)
+        float4 n = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (live) {
+            const float4 ww = *reinterpret_cast<const float4*>(w + e);
+            n = make_float4(v[i].x * rs * ww.x, v[i].y * rs * ww.y, v[i].z * rs * ww.z, v[i].w * rs * ww.w);
+        }
+        float amax = fmaxf(fmaxf(fabsf(n.x), fabsf(n.y)), fmaxf(fabsf(n.z), fabsf(n.w)));
+        float s = (n.x + n.y) + (n.z + n.w);
+#pragma unroll
+        for (int o = TPG / 2; o > 0; o >>= 1) {
+            amax = fmaxf(amax, __shfl_xor(amax, o, 64));
+            s += __shfl_xor(s, o, 64);
+        }
+        const float d = amax / 127.0f;
+        const float id = (d != 0.0f) ? (1.0f / d) : 0.0f;
+        const uint32_t c = ((uint32_t)q8_code(n.x, id) & 0xFFu) | (((uint32_t)q8_code(n.y, id) & 0xFFu) << 8) |
+                           (((uint32_t)q8_code(n.z, id) & 0xFFu) << 16) | (((uint32_t)q8_code(n.w, id) & 0xFFu) << 24);
+        if (live) {
+            *reinterpret_cast<uint32_t*>(xq + (int64_t)row * hidden + e) = c;
+            if ((threadIdx.x % TPG) == 0) {
+                const int64_t kb = e / G;
+                xd[(int64_t)row * Kg + kb] = d;
+                gsum[(int64_t)row * Kg + kb] = s;
+                xsT[kb * rows + row] = make_float2(d, s);
+            }
+        }
+    }
+}
+
 }  // namespace llmops
 
 using namespace llmops;
 
 namespace llmops {
+// Quantization with the producer of the activations folded in (shared with fc.hip): norm_w != nullptr quantizes
+// rmsnorm(x) * norm_w, glu_in quantizes silu(gate) * up of rows [gate | up] of 2K floats; one launch instead of the
+// producer's launch, a round trip of its fp32 result through memory and the quantization launch.  Whole k-groups
+// only; xd and gsum are written with norm_w only (the group-128 product kernels read xsT).
+int launch_quant_x_fused(const float* x, int64_t rows, int64_t K, int group_k, const float* norm_w, float eps, bool glu_in,
+                         int8_t* xq, float* xd, float* gsum, float2* xsT, hipStream_t stream) {
+    const int64_t Kg = K / group_k;
+    if (K != Kg * group_k || !aligned(x, 16) || !aligned(xq, 4) || rows >= ((int64_t)1 << 28))
+        return fail(LLMOPS_EINVAL, "fused quantization: whole k-groups, 16-byte aligned rows, fewer than 2^28 rows");
+    if (norm_w != nullptr) {
+        if (glu_in || K > 16384 || !aligned(norm_w, 16))
+            return fail(LLMOPS_EINVAL, "fused rmsnorm + quantization: rows of at most 16384 floats, 16-byte aligned weights, no glu");
+#define LLMOPS_RQ(VPT)                                                                                                    \
+    do {                                                                                                                  \
+        if (group_k == 32)                                                                                                \
+            rmsnorm_quant_kernel<VPT, 32><<<(unsigned)rows, 1024, 0, stream>>>(x, K, norm_w, eps, (int)rows, (int)Kg, xq, xd, \
+                                                                               gsum, xsT);                                \
+        else                                                                                                              \
+            rmsnorm_quant_kernel<VPT, 128><<<(unsigned)rows, 1024, 0, stream>>>(x, K, norm_w, eps, (int)rows, (int)Kg, xq, xd, \
+                                                                                gsum, xsT);                               \
+    } while (0)
+        if (K <= 4096) LLMOPS_RQ(1);
+        else if (K <= 8192) LLMOPS_RQ(2);
+        else LLMOPS_RQ(4);
+#undef LLMOPS_RQ
+        LLMOPS_LAUNCH_CHECK();
+        return LLMOPS_OK;
+    }
+    if (!glu_in) return fail(LLMOPS_EINVAL, "fused quantization without a producer");
+    const int64_t rblocks = (rows + 7) / 8;
+    if (group_k != 128 || Kg >= ((int64_t)1 << 20) || rblocks * Kg >= ((int64_t)1 << 31))
+        return fail(LLMOPS_EINVAL, "fused silu*up + quantization: group 128 only");
+    if (rblocks * ((Kg + 3) / 4) >= 1024) {
+        const int kparts = (int)((Kg + 3) / 4);
+        quant_x_tile128_kernel<4, true><<<(unsigned)(rblocks * kparts), 256, 0, stream>>>(x, (int)rows, (int)Kg, kparts, xq, xsT);
+    } else {
+        quant_x_tile128_kernel<1, true><<<(unsigned)(rblocks * Kg), 256, 0, stream>>>(x, (int)rows, (int)Kg, (int)Kg, xq, xsT);
+    }
+    LLMOPS_LAUNCH_CHECK();
+    return LLMOPS_OK;
+}
+
 // shared with fc.hip
 int launch_quant_x(const float* x, int64_t rows, int64_t K, int group_k, int8_t* xq, float* xd, float* gsum, float2* xsT,
                    bool exact_sum, hipStream_t stream) {

@@ -243,8 +243,9 @@ def fc_Q4A_decode(input, weiq, N_out, norm=None, residual=None, glu=False, sumsq
     (``attention_rope2_records``), merged as it is loaded.
     want_sumsq=True returns ``(out, sumsq)`` where ``sumsq``
     [B*M, strips] holds the sum of squares of every 32 outputs; passed as ``sumsq_in`` to the FC that
-    rmsnorms ``out`` it saves that FC the pass over the row.  With more than 8 rows the same
-    arithmetic is composed from the separate ops."""
+    rmsnorms ``out`` it saves that FC the pass over the row.  With more than 8 rows the rmsnorm or the
+    silu(gate)*up runs inside the quantization launch (same codes as the separate ops give), the residual inside the
+    product; shapes that launch does not take, and glu=True, are composed from the separate ops."""
     if attn_records is not None:
         # input = the attention output still in chunk records (attention_rope2_records); merged on the way in
         r = attn_records
@@ -285,7 +286,10 @@ def fc_Q4A_decode(input, weiq, N_out, norm=None, residual=None, glu=False, sumsq
         _dev(sumsq_in, torch.float32, 2, "sumsq_in")
         _require(norm is not None and sumsq_in.shape[0] == rows, "sumsq_in.is({B*M, parts}) with norm")
     _require(not (want_sumsq and glu), "no sumsq with glu")
-    if rows > 8:
+    fusable = K % g == 0 and input.data_ptr() % 16 == 0 and (norm is None or (K <= 16384 and norm[0].data_ptr() % 16 == 0)) \
+        and (not glu_in or g == 128)
+    if rows > 8 and (glu or not fusable):
+        # gate and up interleaved on the output side (or a shape the fused quantization does not take): separate ops
         x = input if norm is None else rmsnorm_out(input, norm[0], norm[1])
         if glu_in:
             x = silu_mul(input)

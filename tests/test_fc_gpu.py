@@ -335,6 +335,85 @@ def test_fc_decode_gate_up_input(ops, orc, G, rows, N, K):
         ops.fc_Q4A_decode(dev(gu), dev(pw), N, norm=(torch.ones(K, device="cuda"), 1e-5), glu_in=True)
 
 
+@pytest.mark.parametrize("G", [32, 128])
+@pytest.mark.parametrize("rows", [9, 16, 40, 600])
+@pytest.mark.parametrize("N,K", [(352, 1024), (2048, 4096), (1000, 8192), (96, 11008)])
+def test_fc_decode_many_rows_producer_inside_the_quantization(ops, orc, G, rows, N, K):
+    """fc_Q4A_decode with more than 8 rows: the rmsnorm, or silu(gate)*up, runs inside the quantization launch.
+    The codes are those of the separate ops, so the results are bit-equal to rmsnorm_out / silu_mul followed by
+    fc_Q4A (whose parity with the oracle the other tests hold), with the residual and the sums of squares; and
+    against the oracle directly."""
+    rng = np.random.default_rng(rows + G + N + K)
+    pw = dev(orc.quant_w((rng.standard_normal((N, K)) * 0.02).astype(np.float32), G))
+    res = dev(rng.standard_normal((1, rows, N)).astype(np.float32))
+    strips = -(-N // 32)
+
+    def sums(y):
+        pad = np.zeros((rows, strips * 32))
+        pad[:, :N] = host(y).astype(np.float64).reshape(rows, N)
+        return (pad.reshape(rows, strips, 32) ** 2).sum(-1)
+
+    x = rng.standard_normal((1, rows, K)).astype(np.float32)
+    x[0, 1, :G] = 0.0                # a k-group of zeros: scale 0, codes 0
+    x[0, 2, G:2 * G] *= 1e-30        # tiny values
+    nw = (1.0 + 0.1 * rng.standard_normal(K)).astype(np.float32)
+    if K <= 8192:  # (the oracle's rmsnorm over 600 rows of 11008 adds nothing)
+        two_step = ops.fc_Q4A(ops.rmsnorm_out(dev(x), dev(nw), 1e-5), pw, N)
+        got = ops.fc_Q4A_decode(dev(x), pw, N, norm=(dev(nw), 1e-5))
+        assert torch.equal(got, two_step)
+        if rows <= 40:
+            # the oracle's product on the normalized rows as this library computes them (its rmsnorm and the
+            # oracle's differ by an ulp here and there, which can flip an int8 code: one code is 1e-3 of an
+            # output at K = 1024)
+            xn = host(ops.rmsnorm_out(dev(x), dev(nw), 1e-5))
+            assert max_rel_err(xn, orc.rmsnorm(x, nw, 1e-5)) <= 1e-5
+            assert max_rel_err(host(got), orc.fc(xn, host(pw), N)) <= 1e-5
+        got, ss = ops.fc_Q4A_decode(dev(x), pw, N, norm=(dev(nw), 1e-5), residual=res, want_sumsq=True)
+        assert torch.equal(got, ops.fc_Q4A(ops.rmsnorm_out(dev(x), dev(nw), 1e-5), pw, N, residual=res))
+        want_ss = sums(got)
+        assert host(ss).shape == (rows, strips) and np.abs(host(ss) - want_ss).max() <= 1e-5 * want_ss.max()
+    gu = rng.standard_normal((1, rows, 2 * K)).astype(np.float32)
+    gu[0, 0, :G] = -100.0            # silu underflows to -0.0 * up
+    two_step = ops.fc_Q4A(ops.silu_mul(dev(gu)), pw, N, residual=res)
+    got, ss = ops.fc_Q4A_decode(dev(gu), pw, N, residual=res, want_sumsq=True, glu_in=True)
+    assert torch.equal(got, two_step)
+    want_ss = sums(got)
+    assert np.abs(host(ss) - want_ss).max() <= 1e-5 * want_ss.max()
+    if rows <= 40:
+        act = host(ops.silu_mul(dev(gu)))
+        assert max_rel_err(act, orc.imul(gu[..., K:].copy(), orc.silu(gu[..., :K].copy()))) <= 1e-5
+        assert max_rel_err(host(got), orc.fc(act, host(pw), N) + host(res)) <= 1e-5
+
+
+def test_fc_decode_many_rows_refuses_what_it_cannot_fold(ops, orc):
+    """At the C ABI: interleaved gate/up strips on the output side (glu 1) need the 8-row kernel, and the
+    silu(gate)*up producer needs group 128; both are refused before anything is enqueued (the Python op composes
+    those cases from the separate ops instead)."""
+    from llmops import _lib
+    lib = _lib.load()
+    rng = np.random.default_rng(3)
+    K, F, rows = 256, 64, 12
+    x = dev(rng.standard_normal((rows, 2 * K)).astype(np.float32))
+    y = torch.full((rows, 2 * F), 7.0, device="cuda")
+    for G, glu in ((128, 1), (32, 2)):
+        pw = dev(orc.quant_w((rng.standard_normal((2 * F, K)) * 0.02).astype(np.float32), G))
+        Ng, Kg, _ = pw.shape
+        nbytes = lib.llmops_fc_Q4A_workspace_bytes(rows, K, Ng, Kg, G)
+        ws = torch.zeros(nbytes, dtype=torch.uint8, device="cuda")
+        rc = lib.llmops_fc_Q4A_decode(x.data_ptr(), rows, K, pw.data_ptr(), Ng, Kg, G, F if glu == 1 else 2 * F, None, 0.0,
+                                      None, glu, None, 0, None, y.data_ptr(), ws.data_ptr(), nbytes,
+                                      torch.cuda.current_stream().cuda_stream)
+        assert rc != 0
+        torch.cuda.synchronize()
+        assert bool((y == 7.0).all())
+    # the Python op takes both
+    pg = dev(orc.quant_w((rng.standard_normal((F, K)) * 0.02).astype(np.float32), 128))
+    il = ops.interleave_gate_up(pg, pg)
+    assert ops.fc_Q4A_decode(x[:, :K].reshape(1, rows, K).contiguous(), il, F, glu=True).shape == (1, rows, F)
+    p32 = dev(orc.quant_w((rng.standard_normal((F, K)) * 0.02).astype(np.float32), 32))
+    assert ops.fc_Q4A_decode(x.reshape(1, rows, 2 * K), p32, F, glu_in=True).shape == (1, rows, F)
+
+
 @pytest.mark.parametrize("rows", [1, 2, 4, 5, 8])
 @pytest.mark.parametrize("N,K", [(4096, 11008), (4090, 11008), (3000, 5632)])
 def test_fc_two_k_splits_both_handoffs(ops, orc, rows, N, K):
