@@ -641,44 +641,72 @@ __global__ __launch_bounds__(NWV * 64) void attn_decode_kernel(const int32_t* __
     }
 }
 
-// ---- prefill: tiled attention with fp32 MFMA -------------------------------------------------
+// ---- prefill: tiled attention on the fp16 matrix cores, fp32 values carried as two halves -------
 // Many query tokens share the K and V rows they look at, so the split kernel above (one workgroup
 // per query and chunk) re-reads the cache qL times.  Here a workgroup owns 128 queries of one head
 // (4 waves x 32 queries, ONE QUERY PER LANE PAIR) and walks the cache in tiles of 32 rows that are
-// staged once in LDS:
+// staged once in LDS.
 //
-//   S^T = K_tile * Q^T     v_mfma_f32_32x32x2_f32, 64 steps: in step i the lanes of half hf = lane/32
-//                          cover k = 64*hf + i (which k-values a step sums is free, as long as A and B
-//                          agree).  A = K[kv = lane%32][64*hf + i]: a lane's 64 operands are contiguous
-//                          in the LDS row, so one 16-byte read feeds four steps.  B = the lane's own
-//                          query row, elements 64*hf .. 64*hf+63, kept in 64 registers.  The result puts
-//                          query lane%32 into the lane, 16 cache rows 8j + 4*hf + v each.  Two
-//                          accumulators take alternate steps, so that no MFMA waits for the one before it.
-//   mask, online softmax   per lane, plus one exchange with lane^32 (the other 16 rows of the tile)
-//   O^T += V_tile^T * P^T  16 steps of 4 MFMAs.  B = the lane's 16 probabilities exactly as they sit in
-//                          registers (step i takes cache row 8*(i/4) + 4*hf + i%4).  MFMA c of a step
-//                          owns the output columns 4*m + c, m = 0..31, so A = V[row][4*(lane%32) + c]:
-//                          the four MFMAs' operands are one 16-byte read.
+// Arithmetic.  On this part v_mfma_f32_32x32x2_f32 runs at the vector ALU's rate and keeps the vector ALU
+// busy while it runs (a wave's -- or its SIMD neighbour's -- vector instructions simply add to its time:
+// measured), so an fp32-MFMA kernel pays for the softmax, the staging and the products one after the
+// other.  The fp16 MFMAs are 16 times faster and leave the vector ALU free.  Every fp32 operand x is
+// therefore split into two halves, hi = fp16(x) (rounded toward zero) and lo = fp16(x - hi), whose sum
+// carries 22 bits of x, and a product a*b is computed as hi_a*hi_b + hi_a*lo_b + lo_a*hi_b: three
+// v_mfma_f32_32x32x16_f16 with fp32 accumulation (each half-by-half product is exact in fp32; the dropped
+// lo*lo term is 2^-22 of the product).  Results agree with fp32 arithmetic to about 1e-6 of the largest
+// output, like two fp32 evaluations in different summation orders.  Values beyond the fp16 range
+// (|x| >= 65504) are not representable this way; activations and cache rows of a transformer are far below.
+// An fp16 cache has no low halves: two MFMAs per product.
 //
-// The operand reads run two reads (eight MFMAs) ahead of their use; scheduling fences keep them there
-// (left alone, the compiler issues every read right in front of its first use and the matrix pipe waits
-// out the LDS latency 48 times per tile).  Everything a lane holds (running max, sum, 4 x 16 output
-// values) belongs to its own query, so the rescaling needs no cross-lane traffic, and no probability
-// ever goes through LDS.  Tiles that no query of a wave may see (in-chunk causal mask,
-// ops/op_attn.hpp:1007-1011) are skipped.  K rows are padded to 132 floats: the 16 lanes that one phase
-// of a 16-byte read serves then touch 16 different 16-byte slots of the 256-byte bank line (33 is odd);
-// the V reads are contiguous per row.  Staging writes 256 contiguous bytes per 16 lanes.  Arithmetic is
-// fp32 throughout (fp16 caches are widened when a tile is staged).
+//   S^T = K_tile * Q^T     8 steps of 16 head dims.  A = K[kv = lane%32][16i + 8*hf .. +7]: 16 bytes of the
+//                          row's hi plane (and of its lo plane) in LDS.  B = the lane's own query row, same
+//                          dims, split once into 64 registers.  The result puts query lane%32 into the
+//                          lane, 16 cache rows 8j + 4*hf + v each.  hi*hi goes to one accumulator, the cross
+//                          terms to another.
+//   mask, online softmax   per lane, fp32, plus one exchange with lane^32 (the other 16 rows of the tile)
+//   O^T += V_tile^T * P^T  2 steps of 16 cache rows x 4 blocks of 32 output columns.  B = the lane's 8
+//                          probabilities 8b .. 8b+7 exactly as they sit in registers (rows 8j + 4*hf + v,
+//                          j = 2b, 2b+1), split into halves.  A = V[those 8 rows][column 32c + lane%32]:
+//                          the tile is staged transposed, with the rows of a column permuted so that these
+//                          8 halves are 16 contiguous bytes.
+//
+// Everything a lane holds (running max, sum, 4 x 16 output values) belongs to its own query, so
+// the rescaling needs no cross-lane traffic, and no probability ever goes through LDS.  Tiles that
+// no query of a wave may see (in-chunk causal mask, ops/op_attn.hpp:1007-1011) are skipped.  K rows
+// take 272 bytes per plane and V columns 80, so that the 16 lanes one phase of a 16-byte read serves
+// touch 16 different 16-byte slots of the 256-byte bank line (17 and 5 are odd).
 typedef float v16f __attribute__((ext_vector_type(16)));
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+typedef _Float16 v2h __attribute__((ext_vector_type(2)));
+
+// (a, b) -> packed halves hi and lo with a = hi.x + lo.x, b = hi.y + lo.y to 22 bits
+__device__ __forceinline__ void split2(float a, float b, uint32_t& hi, uint32_t& lo) {
+    const v2h h = __builtin_bit_cast(v2h, __builtin_amdgcn_cvt_pkrtz(a, b));
+    hi = __builtin_bit_cast(uint32_t, h);
+    lo = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(a - (float)h[0], b - (float)h[1]));
+}
+__device__ __forceinline__ uint32_t pack_hi(float a, float b) {
+    return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(a, b));
+}
+union V8hBits {
+    v8h h;
+    uint32_t u[4];
+    uint4 q;
+};
 
 template <typename T>
 __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(float* q, const T* __restrict__ kc, const T* __restrict__ vc,
                                                              int64_t qL, int64_t H, int64_t maxlen, int64_t kvLen,
                                                              const int32_t* __restrict__ row_token, int qtiles) {
-    constexpr int S = 128, BQ = 128, BK = 32, KS = 132, VS = 128;
-    __shared__ __align__(16) float ksh[BK * KS];
-    __shared__ __align__(16) float vsh[BK * VS];
+    constexpr bool LO = sizeof(T) == 4;  // an fp16 cache holds no low halves
+    constexpr int S = 128, BQ = 128, BK = 32, KSB = 272, VSB = 80;
+    __shared__ __align__(16) uint8_t k_hi[BK * KSB];
+    __shared__ __align__(16) uint8_t k_lo[LO ? BK * KSB : 16];
+    __shared__ __align__(16) uint8_t v_hi[S * VSB];
+    __shared__ __align__(16) uint8_t v_lo[LO ? S * VSB : 16];
     __shared__ __align__(16) int tok[BK];
+    __shared__ int tok_range[2];  // smallest and largest token of the tile
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int hf = lane >> 5, c32 = lane & 31;
     // Late query tiles see the most cache rows.  They are dealt out first, in descending order, so that they do
@@ -697,12 +725,16 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(float* q, const T*
     const T* kbase = kc + bh * maxlen * S;
     const T* vbase = vc + bh * maxlen * S;
 
-    // the lane's half of its query row: elements 64*hf .. 64*hf + 63
-    float qreg[64];
+    // the lane's share of its query row as halves: step i covers dims 16i + 8*hf .. +7
+    V8hBits qh[8], ql[8];
 #pragma unroll
-    for (int i = 0; i < 16; i++) {
-        const float4 t = *reinterpret_cast<const float4*>(qrow + hf * 64 + i * 4);
-        qreg[4 * i] = t.x, qreg[4 * i + 1] = t.y, qreg[4 * i + 2] = t.z, qreg[4 * i + 3] = t.w;
+    for (int i = 0; i < 8; i++) {
+        const float4 t0 = *reinterpret_cast<const float4*>(qrow + 16 * i + 8 * hf);
+        const float4 t1 = *reinterpret_cast<const float4*>(qrow + 16 * i + 8 * hf + 4);
+        split2(t0.x, t0.y, qh[i].u[0], ql[i].u[0]);
+        split2(t0.z, t0.w, qh[i].u[1], ql[i].u[1]);
+        split2(t1.x, t1.y, qh[i].u[2], ql[i].u[2]);
+        split2(t1.z, t1.w, qh[i].u[3], ql[i].u[3]);
     }
     const float d_scale = 1.0f / sqrtf((float)S);
     float m_run = -FLT_MAX, l_run = 0.0f;
@@ -712,43 +744,84 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(float* q, const T*
 #pragma unroll
         for (int r = 0; r < 16; r++) o[c][r] = 0.0f;
 
-    // staging: 16 lanes move 64 contiguous floats of a row (a wave: 4 rows, the workgroup: 16 rows) of the K
-    // and of the V tile, four times over (row halves 0/1, rows +0/+16).  The next tile's global loads are
-    // issued before the current tile is computed on and land in registers meanwhile.
-    const int srow = wave * 4 + (lane >> 4), scol = (lane & 15) * 4;
+    // Staging.  K: a thread moves 16 consecutive floats of one row (row = thread/8).  V: a thread moves a
+    // 4 x 4 patch, rows 4g .. 4g+3 (g = thread/32) of columns 4*(thread%32) .. +3, and writes it transposed:
+    // per column 4 halves = 8 bytes at the rows' place in the column's permuted order (cache row r of the tile
+    // sits at position 16*(r/16) + 8*((r/4)%2) + 4*((r%16)/8) + r%4).  The next tile's global loads are issued
+    // before the current tile is computed on and land in registers meanwhile.
+    const int krow = threadIdx.x >> 3, kseg = threadIdx.x & 7;
+    const int vg = threadIdx.x >> 5, vq = threadIdx.x & 31;
+    const int vpos = 16 * (vg >> 2) + 8 * (vg & 1) + 4 * ((vg >> 1) & 1);
     float4 kst[4], vst[4];
     int tst = INT_MAX;
 #define LLMOPS_STAGE_LOAD(KV0)                                                                          \
     do {                                                                                                \
+        const int64_t rk_ = (KV0) + krow < kvLen ? (KV0) + krow : kvLen - 1;                            \
         _Pragma("unroll") for (int u = 0; u < 4; u++) {                                                 \
-            const int64_t r_ = (KV0) + srow + 16 * (u >> 1) < kvLen ? (KV0) + srow + 16 * (u >> 1) : kvLen - 1; \
-            kst[u] = load4(kbase + r_ * S + (u & 1) * 64 + scol);                                       \
-            vst[u] = load4(vbase + r_ * S + (u & 1) * 64 + scol);                                       \
+            const int64_t rv_ = (KV0) + 4 * vg + u < kvLen ? (KV0) + 4 * vg + u : kvLen - 1;            \
+            kst[u] = load4(kbase + rk_ * S + kseg * 16 + u * 4);                                        \
+            vst[u] = load4(vbase + rv_ * S + vq * 4);                                                   \
         }                                                                                               \
         if (threadIdx.x < BK) tst = ((KV0) + threadIdx.x < kvLen) ? row_token[(KV0) + threadIdx.x] : INT_MAX; \
     } while (0)
     LLMOPS_STAGE_LOAD(0);
-    const float* kp = &ksh[c32 * KS + hf * 64];  // + 4j: the operands of steps 4j .. 4j+3
-    const float* vp = &vsh[4 * hf * VS + 4 * c32];  // + (8*(i/4) + i%4) * VS: the operands of step i
+    const uint8_t* kp_hi = &k_hi[c32 * KSB + 16 * hf];  // + 32 i
+    const uint8_t* kp_lo = &k_lo[LO ? c32 * KSB + 16 * hf : 0];
+    const uint8_t* vp_hi = &v_hi[c32 * VSB + 16 * hf];  // + 32 c * VSB + 32 b
+    const uint8_t* vp_lo = &v_lo[LO ? c32 * VSB + 16 * hf : 0];
     for (int64_t kv0 = 0; kv0 < kvLen; kv0 += BK) {
         __syncthreads();  // the previous tile has been consumed
+        {
+            uint32_t hi[8], lo[8];
 #pragma unroll
-        for (int u = 0; u < 4; u++) {
-            const int row = srow + 16 * (u >> 1), col = (u & 1) * 64 + scol;
-            *reinterpret_cast<float4*>(&ksh[row * KS + col]) = kst[u];
-            *reinterpret_cast<float4*>(&vsh[row * VS + col]) = vst[u];
+            for (int u = 0; u < 4; u++) {
+                split2(kst[u].x, kst[u].y, hi[2 * u], lo[2 * u]);
+                split2(kst[u].z, kst[u].w, hi[2 * u + 1], lo[2 * u + 1]);
+            }
+            uint4* dh = reinterpret_cast<uint4*>(&k_hi[krow * KSB + kseg * 32]);
+            dh[0] = make_uint4(hi[0], hi[1], hi[2], hi[3]);
+            dh[1] = make_uint4(hi[4], hi[5], hi[6], hi[7]);
+            if (LO) {
+                uint4* dl = reinterpret_cast<uint4*>(&k_lo[krow * KSB + kseg * 32]);
+                dl[0] = make_uint4(lo[0], lo[1], lo[2], lo[3]);
+                dl[1] = make_uint4(lo[4], lo[5], lo[6], lo[7]);
+            }
+            // V patch: column j of the patch is (vst[0..3])[j]
+            const float vx[4][4] = {{vst[0].x, vst[0].y, vst[0].z, vst[0].w},
+                                    {vst[1].x, vst[1].y, vst[1].z, vst[1].w},
+                                    {vst[2].x, vst[2].y, vst[2].z, vst[2].w},
+                                    {vst[3].x, vst[3].y, vst[3].z, vst[3].w}};
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                uint32_t h0, l0, h1, l1;
+                split2(vx[0][j], vx[1][j], h0, l0);
+                split2(vx[2][j], vx[3][j], h1, l1);
+                *reinterpret_cast<uint2*>(&v_hi[(4 * vq + j) * VSB + vpos * 2]) = make_uint2(h0, h1);
+                if (LO) *reinterpret_cast<uint2*>(&v_lo[(4 * vq + j) * VSB + vpos * 2]) = make_uint2(l0, l1);
+            }
         }
-        if (threadIdx.x < BK) tok[threadIdx.x] = tst;
+        if (wave == 0) {
+            // the tile's token range, once for all waves: DPP steps inside the rows of 16 lanes, the two rows that
+            // hold tokens (lanes 0..31) combined through scalar registers
+            int mn = tst, mx = tst;
+#define LLMOPS_DPP_MINMAX(CTRL)                                                  \
+    mn = min(mn, __builtin_amdgcn_update_dpp(mn, mn, CTRL, 0xF, 0xF, false)); \
+    mx = max(mx, __builtin_amdgcn_update_dpp(mx, mx, CTRL, 0xF, 0xF, false))
+            LLMOPS_DPP_MINMAX(0xB1);   // quad_perm [1,0,3,2]
+            LLMOPS_DPP_MINMAX(0x4E);   // quad_perm [2,3,0,1]
+            LLMOPS_DPP_MINMAX(0x141);  // row_half_mirror
+            LLMOPS_DPP_MINMAX(0x140);  // row_mirror
+#undef LLMOPS_DPP_MINMAX
+            const int lo = min(__builtin_amdgcn_readlane(mn, 0), __builtin_amdgcn_readlane(mn, 16));
+            const int hi = max(__builtin_amdgcn_readlane(mx, 0), __builtin_amdgcn_readlane(mx, 16));
+            if (lane < BK) tok[lane] = tst;
+            if (lane == 0) tok_range[0] = lo, tok_range[1] = hi;
+        }
         __syncthreads();
         if (kv0 + BK < kvLen) LLMOPS_STAGE_LOAD(kv0 + BK);
         // skip the tile if even the wave's last query may not see any of its rows; a tile that every query of the
         // wave sees whole (the usual case away from the diagonal) needs no masks
-        int tmin = tok[c32], tmax = tmin;
-#pragma unroll
-        for (int off = 16; off > 0; off >>= 1) {
-            tmin = min(tmin, __shfl_xor(tmin, off, 64));
-            tmax = max(tmax, __shfl_xor(tmax, off, 64));
-        }
+        const int tmin = tok_range[0], tmax = tok_range[1];
         if (q_lo_wave >= qL || (int64_t)tmin > q_hi_wave) continue;
         const bool all_visible = (int64_t)tmax <= q_lo_wave && q_lo_wave + 31 < qL;
 
@@ -756,25 +829,27 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(float* q, const T*
 #pragma unroll
         for (int r = 0; r < 16; r++) s0[r] = 0.0f, s1[r] = 0.0f;
         {
-            float4 kk[3];
-            kk[0] = *reinterpret_cast<const float4*>(kp);
-            kk[1] = *reinterpret_cast<const float4*>(kp + 4);
+            // operand reads run two steps ahead of the MFMAs that use them
+            v8h ah[3], al[3];
+            ah[0] = *reinterpret_cast<const v8h*>(kp_hi);
+            ah[1] = *reinterpret_cast<const v8h*>(kp_hi + 32);
+            if (LO) {
+                al[0] = *reinterpret_cast<const v8h*>(kp_lo);
+                al[1] = *reinterpret_cast<const v8h*>(kp_lo + 32);
+            }
 #pragma unroll
-            for (int j = 0; j < 16; j++) {
-                if (j + 2 < 16) kk[(j + 2) % 3] = *reinterpret_cast<const float4*>(kp + 4 * (j + 2));
+            for (int i = 0; i < 8; i++) {
+                if (i + 2 < 8) {
+                    ah[(i + 2) % 3] = *reinterpret_cast<const v8h*>(kp_hi + 32 * (i + 2));
+                    if (LO) al[(i + 2) % 3] = *reinterpret_cast<const v8h*>(kp_lo + 32 * (i + 2));
+                }
                 __builtin_amdgcn_sched_barrier(0);
-                const float4 a = kk[j % 3];
-                s0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a.x, qreg[4 * j], s0, 0, 0, 0);
-                s1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a.y, qreg[4 * j + 1], s1, 0, 0, 0);
-                s0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a.z, qreg[4 * j + 2], s0, 0, 0, 0);
-                s1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a.w, qreg[4 * j + 3], s1, 0, 0, 0);
+                s0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah[i % 3], qh[i].h, s0, 0, 0, 0);
+                s1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah[i % 3], ql[i].h, s1, 0, 0, 0);
+                if (LO) s1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(al[i % 3], qh[i].h, s1, 0, 0, 0);
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
-        // the first two V operands are asked for before the softmax, which hides their latency
-        float4 vv[3];
-        vv[0] = *reinterpret_cast<const float4*>(vp);
-        vv[1] = *reinterpret_cast<const float4*>(vp + VS);
         v16f sacc = s0 + s1;
 
         // scale, mask (rows written by later tokens of this call, rows beyond kvLen), running max
@@ -819,31 +894,39 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(float* q, const T*
         }
         m_run = m_new;
 
-        // O^T += V^T P^T; step i of the product takes cache row 8*(i/4) + 4*hf + i%4 of the tile
+        // O^T += V^T P^T: step b takes the lane's probabilities 8b .. 8b+7 (cache rows 8j + 4*hf + v, j = 2b, 2b+1)
 #pragma unroll
-        for (int i = 0; i < 16; i++) {
-            if (i + 2 < 16) vv[(i + 2) % 3] = *reinterpret_cast<const float4*>(vp + (8 * ((i + 2) / 4) + ((i + 2) % 4)) * VS);
-            __builtin_amdgcn_sched_barrier(0);
-            const float4 a = vv[i % 3];
-            o[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.x, sacc[i], o[0], 0, 0, 0);
-            o[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.y, sacc[i], o[1], 0, 0, 0);
-            o[2] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.z, sacc[i], o[2], 0, 0, 0);
-            o[3] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.w, sacc[i], o[3], 0, 0, 0);
-            __builtin_amdgcn_sched_barrier(0);
+        for (int bb = 0; bb < 2; bb++) {
+            V8hBits ph, pl;
+#pragma unroll
+            for (int e = 0; e < 4; e++) split2(sacc[8 * bb + 2 * e], sacc[8 * bb + 2 * e + 1], ph.u[e], pl.u[e]);
+            v8h ah[4], al[4];
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+                ah[c] = *reinterpret_cast<const v8h*>(vp_hi + 32 * c * VSB + 32 * bb);
+                if (LO) al[c] = *reinterpret_cast<const v8h*>(vp_lo + 32 * c * VSB + 32 * bb);
+            }
+#pragma unroll
+            for (int c = 0; c < 4; c++) o[c] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah[c], ph.h, o[c], 0, 0, 0);
+#pragma unroll
+            for (int c = 0; c < 4; c++) o[c] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah[c], pl.h, o[c], 0, 0, 0);
+            if (LO) {
+#pragma unroll
+                for (int c = 0; c < 4; c++) o[c] = __builtin_amdgcn_mfma_f32_32x32x16_f16(al[c], ph.h, o[c], 0, 0, 0);
+            }
         }
     }
 
 #undef LLMOPS_STAGE_LOAD
     if (!valid) return;
     const float inv = 1.0f / l_run;
-    // register 4j + v of o[c] is column 4*(8j + 4*hf + v) + c of the query's output row
+    // the lane holds columns 32c + 8j + 4*hf + v of its query's output row
 #pragma unroll
-    for (int j = 0; j < 4; j++)
+    for (int c = 0; c < 4; c++)
 #pragma unroll
-        for (int v = 0; v < 4; v++) {
-            const int r = 4 * j + v;
-            *reinterpret_cast<float4*>(qrow + 4 * (8 * j + 4 * hf + v)) =
-                make_float4(o[0][r] * inv, o[1][r] * inv, o[2][r] * inv, o[3][r] * inv);
+        for (int j = 0; j < 4; j++) {
+            const float4 out = make_float4(o[c][4 * j] * inv, o[c][4 * j + 1] * inv, o[c][4 * j + 2] * inv, o[c][4 * j + 3] * inv);
+            *reinterpret_cast<float4*>(qrow + 32 * c + 8 * j + 4 * hf) = out;
         }
 }
 
