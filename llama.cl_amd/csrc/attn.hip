@@ -644,8 +644,13 @@ __global__ __launch_bounds__(NWV * 64) void attn_decode_kernel(const int32_t* __
 // ---- prefill: tiled attention on the fp16 matrix cores, fp32 values carried as two halves -------
 // Many query tokens share the K and V rows they look at, so the split kernel above (one workgroup
 // per query and chunk) re-reads the cache qL times.  Here a workgroup owns 128 queries of one head
-// (4 waves x 32 queries, ONE QUERY PER LANE PAIR) and walks the cache in tiles of 32 rows that are
-// staged once in LDS.
+// and walks the cache in tiles of 32 rows that are staged once in LDS.  It has two sets of 4 waves
+// (32 queries per wave, ONE QUERY PER LANE PAIR): both sets hold the same queries, set 0 takes the even
+// tiles and set 1 the odd ones, each with its own online softmax, and the two results are merged through
+// LDS at the end.  (A tile's chain -- stage, products, softmax, products -- is a sequence of latencies
+// that one wave per SIMD cannot hide, and under the causal mask the last query tile of a head has 16
+// times the tiles of the first; two sets halve the longest chain.)  Query tiles are dealt out from the
+// last to the first, one workgroup per compute unit at a time.
 //
 // Arithmetic.  On this part v_mfma_f32_32x32x2_f32 runs at the vector ALU's rate and keeps the vector ALU
 // busy while it runs (a wave's -- or its SIMD neighbour's -- vector instructions simply add to its time:
@@ -695,33 +700,46 @@ union V8hBits {
     uint4 q;
 };
 
+// One tile in LDS (fp16 planes, the tile's tokens); each wave set has two of them; the merge at the end reuses the memory
+template <bool LO>
+struct PrefillSmem {
+    static constexpr int S = 128, BK = 32, KSB = 272, VSB = 80;
+    uint8_t k_hi[BK * KSB];
+    uint8_t k_lo[LO ? BK * KSB : 16];
+    uint8_t v_hi[S * VSB];
+    uint8_t v_lo[LO ? S * VSB : 16];
+    int tok[BK];
+    int tok_range[4];  // smallest and largest token of the tile
+};
+constexpr size_t kPrefillMergeBytes = (size_t)66 * 256 * sizeof(float);  // set 1's (max, sum, 64 outputs) per lane
+template <bool LO>
+constexpr size_t prefill_smem_bytes() {
+    return 4 * sizeof(PrefillSmem<LO>) > kPrefillMergeBytes ? 4 * sizeof(PrefillSmem<LO>) : kPrefillMergeBytes;
+}
+
 template <typename T>
-__global__ __launch_bounds__(256, 2) void attn_prefill_kernel(float* q, const T* __restrict__ kc, const T* __restrict__ vc,
-                                                             int64_t qL, int64_t H, int64_t maxlen, int64_t kvLen,
-                                                             const int32_t* __restrict__ row_token, int qtiles) {
+__global__ __launch_bounds__(512) void attn_prefill_kernel(float* q, const T* __restrict__ kc, const T* __restrict__ vc,
+                                                          int64_t qL, int64_t H, int64_t maxlen, int64_t kvLen,
+                                                          const int32_t* __restrict__ row_token, int qtiles) {
     constexpr bool LO = sizeof(T) == 4;  // an fp16 cache holds no low halves
     constexpr int S = 128, BQ = 128, BK = 32, KSB = 272, VSB = 80;
-    __shared__ __align__(16) uint8_t k_hi[BK * KSB];
-    __shared__ __align__(16) uint8_t k_lo[LO ? BK * KSB : 16];
-    __shared__ __align__(16) uint8_t v_hi[S * VSB];
-    __shared__ __align__(16) uint8_t v_lo[LO ? S * VSB : 16];
-    __shared__ __align__(16) int tok[BK];
-    __shared__ int tok_range[2];  // smallest and largest token of the tile
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    extern __shared__ __align__(16) uint8_t smem_raw[];
+    const int lane = threadIdx.x & 63, wave8 = threadIdx.x >> 6;
+    const int set = wave8 >> 2, wave = wave8 & 3, tid = threadIdx.x & 255;  // (wave, tid: within the set)
+    // two tile buffers per set, used alternately: while a tile is multiplied the next one is written
+    PrefillSmem<LO>* const sm2 = reinterpret_cast<PrefillSmem<LO>*>(smem_raw) + 2 * set;
     const int hf = lane >> 5, c32 = lane & 31;
-    // Late query tiles see the most cache rows.  They are dealt out first, in descending order, so that they do
-    // not form the tail; the early half follows in ASCENDING order: when the whole grid is resident at once (two
-    // workgroups per compute unit), workgroup i and workgroup i + gridDim.x/2 land on the same compute unit,
-    // and the heaviest tile then shares its SIMDs with the lightest, the next with the next lightest, ...
+    // late query tiles see the most cache rows: they are dealt out first so that they do not form the tail
     const int64_t bhs = gridDim.x / qtiles;
-    const int heavy = (qtiles + 1) / 2, slot = (int)(blockIdx.x / bhs);
-    const int qt = slot < heavy ? qtiles - 1 - slot : slot - heavy;
+    const int qt = qtiles - 1 - (int)(blockIdx.x / bhs);
     const int64_t bh = blockIdx.x % bhs, b = bh / H, h = bh % H;
-    const int64_t q_lo_wave = (int64_t)qt * BQ + wave * 32;
-    const int64_t pq = q_lo_wave + c32;  // this lane's query token
-    const bool valid = pq < qL;
-    const int64_t q_hi_wave = (q_lo_wave + 31 < qL ? q_lo_wave + 31 : qL - 1);
-    float* qrow = q + ((b * qL + (valid ? pq : qL - 1)) * H + h) * S;
+    // (32-bit arithmetic from here on: the launcher keeps qL and kvLen below 2^31 and a head's cache plane below 4 GiB)
+    const int qLi = (int)qL, kvLeni = (int)kvLen;
+    const int q_lo_wave = qt * BQ + wave * 32;
+    const int pq = q_lo_wave + c32;  // this lane's query token
+    const bool valid = pq < qLi;
+    const int q_hi_wave = min(q_lo_wave + 31, qLi - 1);
+    float* qrow = q + ((b * qL + (valid ? pq : qLi - 1)) * H + h) * S;
     const T* kbase = kc + bh * maxlen * S;
     const T* vbase = vc + bh * maxlen * S;
 
@@ -749,81 +767,102 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(float* q, const T*
     // per column 4 halves = 8 bytes at the rows' place in the column's permuted order (cache row r of the tile
     // sits at position 16*(r/16) + 8*((r/4)%2) + 4*((r%16)/8) + r%4).  The next tile's global loads are issued
     // before the current tile is computed on and land in registers meanwhile.
-    const int krow = threadIdx.x >> 3, kseg = threadIdx.x & 7;
-    const int vg = threadIdx.x >> 5, vq = threadIdx.x & 31;
+    const int krow = tid >> 3, kseg = tid & 7;
+    const int vg = tid >> 5, vq = tid & 31;
     const int vpos = 16 * (vg >> 2) + 8 * (vg & 1) + 4 * ((vg >> 1) & 1);
     float4 kst[4], vst[4];
     int tst = INT_MAX;
 #define LLMOPS_STAGE_LOAD(KV0)                                                                          \
     do {                                                                                                \
-        const int64_t rk_ = (KV0) + krow < kvLen ? (KV0) + krow : kvLen - 1;                            \
+        const uint32_t rk_ = (uint32_t)min((KV0) + krow, kvLeni - 1);                                   \
         _Pragma("unroll") for (int u = 0; u < 4; u++) {                                                 \
-            const int64_t rv_ = (KV0) + 4 * vg + u < kvLen ? (KV0) + 4 * vg + u : kvLen - 1;            \
-            kst[u] = load4(kbase + rk_ * S + kseg * 16 + u * 4);                                        \
-            vst[u] = load4(vbase + rv_ * S + vq * 4);                                                   \
+            const uint32_t rv_ = (uint32_t)min((KV0) + 4 * vg + u, kvLeni - 1);                         \
+            kst[u] = load4(kbase + (rk_ * (uint32_t)S + (uint32_t)(kseg * 16 + u * 4)));               \
+            vst[u] = load4(vbase + (rv_ * (uint32_t)S + (uint32_t)(vq * 4)));                           \
         }                                                                                               \
-        if (threadIdx.x < BK) tst = ((KV0) + threadIdx.x < kvLen) ? row_token[(KV0) + threadIdx.x] : INT_MAX; \
+        if (tid < BK) tst = ((KV0) + tid < kvLeni) ? row_token[(KV0) + tid] : INT_MAX;                  \
     } while (0)
-    LLMOPS_STAGE_LOAD(0);
-    const uint8_t* kp_hi = &k_hi[c32 * KSB + 16 * hf];  // + 32 i
-    const uint8_t* kp_lo = &k_lo[LO ? c32 * KSB + 16 * hf : 0];
-    const uint8_t* vp_hi = &v_hi[c32 * VSB + 16 * hf];  // + 32 c * VSB + 32 b
-    const uint8_t* vp_lo = &v_lo[LO ? c32 * VSB + 16 * hf : 0];
-    for (int64_t kv0 = 0; kv0 < kvLen; kv0 += BK) {
-        __syncthreads();  // the previous tile has been consumed
-        {
-            uint32_t hi[8], lo[8];
+    // The last cache row that any query of the workgroup may see bounds the walk (rows of later tokens and rows
+    // beyond it are masked anyway; without the bound an early query tile would stage, barrier by barrier, all the
+    // tiles that only later tiles need).
+    int kv_end;
+    {
+        const int q_hi_wg = min((qt + 1) * BQ, qLi) - 1;
+        int last = -1;
+        for (int r = tid; r < kvLeni; r += 256)
+            if (row_token[r] <= q_hi_wg) last = r;  // (r grows: the last hit is the largest; each set scans all rows)
 #pragma unroll
-            for (int u = 0; u < 4; u++) {
-                split2(kst[u].x, kst[u].y, hi[2 * u], lo[2 * u]);
-                split2(kst[u].z, kst[u].w, hi[2 * u + 1], lo[2 * u + 1]);
-            }
-            uint4* dh = reinterpret_cast<uint4*>(&k_hi[krow * KSB + kseg * 32]);
-            dh[0] = make_uint4(hi[0], hi[1], hi[2], hi[3]);
-            dh[1] = make_uint4(hi[4], hi[5], hi[6], hi[7]);
-            if (LO) {
-                uint4* dl = reinterpret_cast<uint4*>(&k_lo[krow * KSB + kseg * 32]);
-                dl[0] = make_uint4(lo[0], lo[1], lo[2], lo[3]);
-                dl[1] = make_uint4(lo[4], lo[5], lo[6], lo[7]);
-            }
-            // V patch: column j of the patch is (vst[0..3])[j]
-            const float vx[4][4] = {{vst[0].x, vst[0].y, vst[0].z, vst[0].w},
-                                    {vst[1].x, vst[1].y, vst[1].z, vst[1].w},
-                                    {vst[2].x, vst[2].y, vst[2].z, vst[2].w},
-                                    {vst[3].x, vst[3].y, vst[3].z, vst[3].w}};
-#pragma unroll
-            for (int j = 0; j < 4; j++) {
-                uint32_t h0, l0, h1, l1;
-                split2(vx[0][j], vx[1][j], h0, l0);
-                split2(vx[2][j], vx[3][j], h1, l1);
-                *reinterpret_cast<uint2*>(&v_hi[(4 * vq + j) * VSB + vpos * 2]) = make_uint2(h0, h1);
-                if (LO) *reinterpret_cast<uint2*>(&v_lo[(4 * vq + j) * VSB + vpos * 2]) = make_uint2(l0, l1);
-            }
-        }
-        if (wave == 0) {
-            // the tile's token range, once for all waves: DPP steps inside the rows of 16 lanes, the two rows that
-            // hold tokens (lanes 0..31) combined through scalar registers
-            int mn = tst, mx = tst;
-#define LLMOPS_DPP_MINMAX(CTRL)                                                  \
-    mn = min(mn, __builtin_amdgcn_update_dpp(mn, mn, CTRL, 0xF, 0xF, false)); \
-    mx = max(mx, __builtin_amdgcn_update_dpp(mx, mx, CTRL, 0xF, 0xF, false))
-            LLMOPS_DPP_MINMAX(0xB1);   // quad_perm [1,0,3,2]
-            LLMOPS_DPP_MINMAX(0x4E);   // quad_perm [2,3,0,1]
-            LLMOPS_DPP_MINMAX(0x141);  // row_half_mirror
-            LLMOPS_DPP_MINMAX(0x140);  // row_mirror
-#undef LLMOPS_DPP_MINMAX
-            const int lo = min(__builtin_amdgcn_readlane(mn, 0), __builtin_amdgcn_readlane(mn, 16));
-            const int hi = max(__builtin_amdgcn_readlane(mx, 0), __builtin_amdgcn_readlane(mx, 16));
-            if (lane < BK) tok[lane] = tst;
-            if (lane == 0) tok_range[0] = lo, tok_range[1] = hi;
-        }
+        for (int off = 32; off > 0; off >>= 1) last = max(last, __shfl_xor(last, off, 64));
+        int* const red = sm2[1].tok;  // (the second buffer is first written at the end of the loop's first pass)
+        if (lane == 0) red[wave] = last;
         __syncthreads();
-        if (kv0 + BK < kvLen) LLMOPS_STAGE_LOAD(kv0 + BK);
+        kv_end = max(max(red[0], red[1]), max(red[2], red[3])) + 1;
+    }
+    if (kv_end <= 0) kv_end = 1;  // no row is visible to anybody (cannot happen: a token sees its own row)
+    // Writing a staged tile: halves of K row-major, halves of V transposed, the tile's tokens and their range.
+#define LLMOPS_STAGE_STORE(SM)                                                                                  \
+    do {                                                                                                        \
+        uint32_t hi_[8], lo_[8];                                                                                \
+        _Pragma("unroll") for (int u = 0; u < 4; u++) {                                                         \
+            split2(kst[u].x, kst[u].y, hi_[2 * u], lo_[2 * u]);                                                 \
+            split2(kst[u].z, kst[u].w, hi_[2 * u + 1], lo_[2 * u + 1]);                                         \
+        }                                                                                                       \
+        uint4* dh_ = reinterpret_cast<uint4*>(&(SM).k_hi[krow * KSB + kseg * 32]);                              \
+        dh_[0] = make_uint4(hi_[0], hi_[1], hi_[2], hi_[3]);                                                    \
+        dh_[1] = make_uint4(hi_[4], hi_[5], hi_[6], hi_[7]);                                                    \
+        if (LO) {                                                                                               \
+            uint4* dl_ = reinterpret_cast<uint4*>(&(SM).k_lo[krow * KSB + kseg * 32]);                          \
+            dl_[0] = make_uint4(lo_[0], lo_[1], lo_[2], lo_[3]);                                                \
+            dl_[1] = make_uint4(lo_[4], lo_[5], lo_[6], lo_[7]);                                                \
+        }                                                                                                       \
+        /* V patch: column j of the patch is (vst[0..3])[j] */                                                  \
+        const float vx_[4][4] = {{vst[0].x, vst[0].y, vst[0].z, vst[0].w},                                      \
+                                 {vst[1].x, vst[1].y, vst[1].z, vst[1].w},                                      \
+                                 {vst[2].x, vst[2].y, vst[2].z, vst[2].w},                                      \
+                                 {vst[3].x, vst[3].y, vst[3].z, vst[3].w}};                                     \
+        _Pragma("unroll") for (int j = 0; j < 4; j++) {                                                         \
+            uint32_t h0_, l0_, h1_, l1_;                                                                        \
+            split2(vx_[0][j], vx_[1][j], h0_, l0_);                                                             \
+            split2(vx_[2][j], vx_[3][j], h1_, l1_);                                                             \
+            *reinterpret_cast<uint2*>(&(SM).v_hi[(4 * vq + j) * VSB + vpos * 2]) = make_uint2(h0_, h1_);        \
+            if (LO) *reinterpret_cast<uint2*>(&(SM).v_lo[(4 * vq + j) * VSB + vpos * 2]) = make_uint2(l0_, l1_); \
+        }                                                                                                       \
+        if (wave == 0) {                                                                                        \
+            /* the tile's token range, once for all waves: DPP steps inside the rows of 16 lanes, the two rows */ \
+            /* that hold tokens (lanes 0..31) combined through scalar registers */                              \
+            int mn_ = tst, mx_ = tst;                                                                           \
+            LLMOPS_DPP_MINMAX(0xB1);  /* quad_perm [1,0,3,2] */                                                 \
+            LLMOPS_DPP_MINMAX(0x4E);  /* quad_perm [2,3,0,1] */                                                 \
+            LLMOPS_DPP_MINMAX(0x141); /* row_half_mirror */                                                     \
+            LLMOPS_DPP_MINMAX(0x140); /* row_mirror */                                                          \
+            const int lo2_ = min(__builtin_amdgcn_readlane(mn_, 0), __builtin_amdgcn_readlane(mn_, 16));        \
+            const int hi2_ = max(__builtin_amdgcn_readlane(mx_, 0), __builtin_amdgcn_readlane(mx_, 16));        \
+            if (lane < BK) (SM).tok[lane] = tst;                                                                \
+            if (lane == 0) (SM).tok_range[0] = lo2_, (SM).tok_range[1] = hi2_;                                  \
+        }                                                                                                       \
+    } while (0)
+#define LLMOPS_DPP_MINMAX(CTRL)                                                      \
+    mn_ = min(mn_, __builtin_amdgcn_update_dpp(mn_, mn_, CTRL, 0xF, 0xF, false)); \
+    mx_ = max(mx_, __builtin_amdgcn_update_dpp(mx_, mx_, CTRL, 0xF, 0xF, false))
+    // Set 0 walks the tiles 0, 2, 4, ..., set 1 the tiles 1, 3, 5, ...: both make the same number of passes.  One
+    // barrier per pass: behind it the pass's buffer is complete and nobody reads the other buffer any more, which
+    // the pass then fills -- after its own products -- from the registers that the loads of the pass before filled.
+    LLMOPS_STAGE_LOAD(set * BK);
+    LLMOPS_STAGE_STORE(sm2[0]);
+    if (2 * BK < kv_end) LLMOPS_STAGE_LOAD(set * BK + 2 * BK);
+    for (int kv_pair = 0, pass = 0; kv_pair < kv_end; kv_pair += 2 * BK, pass++) {
+        PrefillSmem<LO>& sm = sm2[pass & 1];
+        const uint8_t* kp_hi = &sm.k_hi[c32 * KSB + 16 * hf];  // + 32 i
+        const uint8_t* kp_lo = &sm.k_lo[LO ? c32 * KSB + 16 * hf : 0];
+        const uint8_t* vp_hi = &sm.v_hi[c32 * VSB + 16 * hf];  // + 32 c * VSB + 32 b
+        const uint8_t* vp_lo = &sm.v_lo[LO ? c32 * VSB + 16 * hf : 0];
+        const int* tok = sm.tok;
+        __syncthreads();
         // skip the tile if even the wave's last query may not see any of its rows; a tile that every query of the
         // wave sees whole (the usual case away from the diagonal) needs no masks
-        const int tmin = tok_range[0], tmax = tok_range[1];
-        if (q_lo_wave >= qL || (int64_t)tmin > q_hi_wave) continue;
-        const bool all_visible = (int64_t)tmax <= q_lo_wave && q_lo_wave + 31 < qL;
+        const int tmin = sm.tok_range[0], tmax = sm.tok_range[1];
+        if (q_lo_wave < qLi && tmin <= q_hi_wave) {
+        const bool all_visible = tmax <= q_lo_wave && q_lo_wave + 31 < qLi;
 
         v16f s0, s1;
 #pragma unroll
@@ -861,7 +900,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(float* q, const T*
                 mx = fmaxf(mx, sacc[r]);
             }
         } else {
-            const int pq32 = valid ? (int)pq : INT_MIN;  // (the launcher keeps qL below 2^31)
+            const int pq32 = valid ? pq : INT_MIN;
 #pragma unroll
             for (int j = 0; j < 4; j++) {
                 const int4 t4 = *reinterpret_cast<const int4*>(&tok[8 * j + 4 * hf]);
@@ -874,7 +913,10 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(float* q, const T*
                 }
             }
         }
-        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        {  // the other half of the lane pair (lane ^ 32) holds the other 16 rows of the query's tile
+            const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(mx), __float_as_uint(mx), false, false);
+            mx = fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1]));
+        }
         const float m_new = fmaxf(m_run, mx);
         const float alpha = expf(m_run - m_new);  // 0 on the first visible tile, 1 while nothing is visible
         float psum = 0.0f;
@@ -884,7 +926,10 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(float* q, const T*
             sacc[r] = pv;
             psum += pv;
         }
-        psum += __shfl_xor(psum, 32, 64);
+        {
+            const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(psum), __float_as_uint(psum), false, false);
+            psum = __uint_as_float(sw[0]) + __uint_as_float(sw[1]);
+        }
         l_run = l_run * alpha + psum;
         if (__any(m_new != m_run)) {  // (alpha is exactly 1 for a query whose maximum did not move)
 #pragma unroll
@@ -915,10 +960,40 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(float* q, const T*
                 for (int c = 0; c < 4; c++) o[c] = __builtin_amdgcn_mfma_f32_32x32x16_f16(al[c], ph.h, o[c], 0, 0, 0);
             }
         }
+        }  // (tile visible to the wave)
+        if (kv_pair + 2 * BK < kv_end) {
+            LLMOPS_STAGE_STORE(sm2[(pass + 1) & 1]);
+            if (kv_pair + 4 * BK < kv_end) LLMOPS_STAGE_LOAD(kv_pair + set * BK + 4 * BK);
+        }
     }
 
+#undef LLMOPS_STAGE_STORE
+#undef LLMOPS_DPP_MINMAX
 #undef LLMOPS_STAGE_LOAD
-    if (!valid) return;
+    // Merge of the two sets: lane by lane (same query, same columns in both).  Set 1 leaves its running maximum, its
+    // sum and its 64 outputs in LDS, value r of lane l of wave w at float r*256 + w*64 + l.
+    __syncthreads();  // every wave is done with its tile
+    float* mrg = reinterpret_cast<float*>(smem_raw) + wave * 64 + lane;
+    if (set == 1) {
+        mrg[0] = m_run;
+        mrg[256] = l_run;
+#pragma unroll
+        for (int c = 0; c < 4; c++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) mrg[(2 + 16 * c + r) * 256] = o[c][r];
+    }
+    __syncthreads();
+    if (set == 1 || !valid) return;
+    {
+        const float m1 = mrg[0], l1 = mrg[256];
+        const float mm = fmaxf(m_run, m1);
+        const float a0 = expf(m_run - mm), a1 = expf(m1 - mm);  // (a set that saw no row has sum 0 and outputs 0)
+        l_run = l_run * a0 + l1 * a1;
+#pragma unroll
+        for (int c = 0; c < 4; c++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) o[c][r] = o[c][r] * a0 + mrg[(2 + 16 * c + r) * 256] * a1;
+    }
     const float inv = 1.0f / l_run;
     // the lane holds columns 32c + 8j + 4*hf + v of its query's output row
 #pragma unroll
@@ -1104,8 +1179,17 @@ static int attention_impl(float* q, float* k, const float* v, int64_t B, int64_t
     LLMOPS_LAUNCH_CHECK();
     if (qL >= g_prefill_min_tokens) {
         // enough query tokens to share K/V tiles: the MFMA kernel reads the cache once per 128 queries
+        if (maxlen * S * (int64_t)sizeof(T) >= ((int64_t)1 << 32))
+            return fail(LLMOPS_EINVAL, "attention over 32 or more query tokens: a head's cache plane must be below 4 GiB");
         const int qtiles = (int)((qL + 127) / 128);
-        attn_prefill_kernel<T><<<(unsigned)(B * H * qtiles), 256, 0, st>>>(q, kc, vc, qL, H, maxlen, kvLen, row_token, qtiles);
+        constexpr size_t smem = prefill_smem_bytes<!kHalfCache>();
+        static bool configured = false;  // opt in to more than 64 KiB of dynamic LDS once per kernel
+        if (!configured) {
+            LLMOPS_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_prefill_kernel<T>),
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+            configured = true;
+        }
+        attn_prefill_kernel<T><<<(unsigned)(B * H * qtiles), 512, smem, st>>>(q, kc, vc, qL, H, maxlen, kvLen, row_token, qtiles);
         LLMOPS_LAUNCH_CHECK();
         return LLMOPS_OK;
     }
