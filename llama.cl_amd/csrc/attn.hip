@@ -922,7 +922,9 @@ __global__ __launch_bounds__(512) void attn_prefill_kernel(float* q, const T* __
         float psum = 0.0f;
 #pragma unroll
         for (int r = 0; r < 16; r++) {
-            const float pv = (sacc[r] == -FLT_MAX) ? 0.0f : expf(sacc[r] - m_new);
+            // e^x as 2^(x * log2 e) on the exponential unit: x <= 0, and wherever the result matters (|x| < 20)
+            // the product's rounding moves it by less than 1e-6 of itself
+            const float pv = (sacc[r] == -FLT_MAX) ? 0.0f : __builtin_amdgcn_exp2f((sacc[r] - m_new) * 1.44269504088896341f);
             sacc[r] = pv;
             psum += pv;
         }

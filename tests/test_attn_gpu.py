@@ -321,6 +321,34 @@ def _prefill_case(ops, orc, rng, past, qL, maxlen, half, heads, H=32, S=128):
     assert np.isfinite(out).all()
 
 
+@pytest.mark.parametrize("scale_q,scale_kv", [(1.0, 1.0), (4.0, 0.25), (1e-3, 1e-3), (0.05, 300.0)])
+def test_attention_prefill_two_halves_arithmetic_over_a_wide_range(ops, orc, scale_q, scale_kv):
+    """The prompt kernel carries fp32 operands as two fp16 halves (22 bits) and multiplies them on the fp16
+    matrix cores.  Inputs whose magnitudes are far from 1 -- sharp softmaxes (large q*k), values whose low halves
+    fall into the fp16 denormals (1e-3), cache rows in the hundreds, a few outliers 50 times the rest -- stay
+    within the contract of 1e-3 of the largest output; what is observed is asserted: 1e-5, as for inputs of
+    order 1, except where logits of magnitude ~100 meet cache values up to 6e4 (the last case: the 2^-22 of every
+    product then shows in the exponent of the softmax, observed 3e-5)."""
+    rng = np.random.default_rng(11)
+    B, H, S, qL, past, maxlen, half = 1, 4, 128, 200, 90, 512, 64
+    inv_freq = (1.0 / (10000.0 ** (np.arange(0, 2 * half, 2, dtype=np.float32) / np.float32(2 * half)))).astype(np.float32)
+    cache = (rng.standard_normal((2, B, H, maxlen, S)) * scale_kv).astype(np.float32)
+    q = (rng.standard_normal((B, qL, H * S)) * scale_q).astype(np.float32)
+    k = (rng.standard_normal((B, qL, H * S)) * scale_kv).astype(np.float32)
+    v = (rng.standard_normal((B, qL, H * S)) * scale_kv).astype(np.float32)
+    for t in (q, k, v):
+        t[0, ::17, ::29] *= 50.0  # outliers
+    cache[:, 0, :, ::13, ::31] *= 50.0
+    slots = ((past + np.arange(qL)) % maxlen).astype(np.int32)
+    g = dict(q=q, k=k, v=v, cache=cache, inv_freq=inv_freq, slots=slots, position_id=past, layer_id=0)
+    out, k_rot, cache_after = run_attention(ops, g)
+    want, k_ref, cache_ref = orc.attention(q, k, v, inv_freq, cache, slots, past, 0)
+    assert np.isfinite(out).all()
+    err = max_rel_err(out, want)
+    assert err <= 1e-3
+    assert err <= (1e-4 if scale_kv > 100 else 1e-5), err
+
+
 @pytest.mark.parametrize("past,qL,half", [(0, 1022, 32), (0, 1023, 32), (0, 1024, 32), (0, 1025, 32), (0, 1026, 32),
                                           (0, 1024, 64), (0, 2048, 32), (0, 2048, 64), (0, 128, 64), (0, 512, 64)])
 def test_attention_prefill_at_the_reference_sweep_sizes(ops, orc, past, qL, half):
