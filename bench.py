@@ -371,6 +371,23 @@ def decode_step(torch, stream, kv_len=2048, reps=50, warm=10):
                 model.forward(ids, kv.cache, slots, kv_len - 1)
             torch.cuda.synchronize()
             eager_ms = (time.perf_counter() - t0) / 5 * 1e3
+        if name == "fp32_kv":
+            # the prompt pass of the same model: kv_len tokens at position 0 through all layers and the lm_head
+            # (rows > 8: rmsnorm / silu*up inside the quantization launches, MFMA GEMMs, tiled attention), op by op
+            with torch.cuda.stream(stream):
+                pids = torch.zeros(1, kv_len, dtype=torch.int64, device="cuda")
+                pslots = torch.arange(kv_len, dtype=torch.int32, device="cuda")
+                model.forward(pids, kv.cache, pslots, 0)
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                for _ in range(3):
+                    model.forward(pids, kv.cache, pslots, 0)
+                torch.cuda.synchronize()
+                pms = (time.perf_counter() - t0) / 3 * 1e3
+            out["prefill_step"] = {"tokens": kv_len, "ms": round(pms, 3), "tokens_per_s": round(kv_len / pms * 1e3, 0),
+                                   "what": "prompt of kv_len tokens, batch 1, fp32 KV cache, logits for every token"}
+            del pids, pslots
+            kv.cache.normal_()
         kv_bytes = 2 * LLAMA_7B["layer_num"] * LLAMA_7B["head_num"] * kv_len * LLAMA_7B["head_size"] * kv.cache.element_size()
         fc = model.fc_weight_size()
         out[name] = {"ms_per_token": round(ms, 4), "ms_per_token_eager": round(eager_ms, 3),

@@ -162,6 +162,15 @@ int llmops_fc_Q4A_decode(const float* x, int64_t rows, int64_t K, const int8_t* 
                          const float* sumsq_in, int64_t sumsq_parts, float* sumsq_out, float* y, void* workspace,
                          size_t workspace_bytes, llmops_stream_t stream);
 
+/* llmops_fc_Q4A_decode for more than 8 rows whose result is wanted as out_parts dense matrices, y laid out
+ * [out_parts][rows][N_out / out_parts] (Ng % out_parts == 0, N_out == Ng*32): the strips of part p are strips
+ * p*Ng/out_parts .. of weiq.  A q|k|v projection over weights stacked along N (chatllama/main.py:347-349 runs three
+ * FCs on the same input) thus leaves q, k and v as the three dense [rows, H*S] matrices the attention op takes,
+ * with one quantization of the input.  norm_w / eps / glu (0 or 2) as above; no residual, no sums of squares. */
+int llmops_fc_Q4A_decode_parts(const float* x, int64_t rows, int64_t K, const int8_t* weiq, int64_t Ng, int64_t Kg,
+                               int group_k, int64_t N_out, const float* norm_w, float eps, int glu, int64_t out_parts,
+                               float* y, void* workspace, size_t workspace_bytes, llmops_stream_t stream);
+
 /* fc_Q4A (one row, group 128) on the output of llmops_attention_rope_decode_records: the o projection of a decode
  * step (chatllama/main.py:353-355) with the merge of the attention chunks (ops/op_attn.hpp:1012-1025 computes the
  * same softmax-weighted sum in one piece) folded into the FC's input side.  K = H*128 = Kg*128; residual and

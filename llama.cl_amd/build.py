@@ -37,7 +37,7 @@ def sources():
 # s_waitcnt pairs (a register spilled between the two would be saved before its data has arrived); the
 # one-row group-128 decode kernels are written to fit the 64 registers that two 16-wave workgroups per
 # CU leave each wave, and scratch traffic in their loop costs what the rewrite gained.
-NO_SPILL = ["fc_gemm_pp_kernelILb0E", "fc_gemv_fused_kernelILi128ELi1E"]
+NO_SPILL = ["fc_gemm_pp_kernelILb0E", "fc_gemv_fused_kernelILi128ELi1E", "attn_prefill_kernel"]
 
 
 def check_spills(remarks):

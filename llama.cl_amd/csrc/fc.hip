@@ -171,10 +171,10 @@ extern "C" int llmops_fc_Q4A_residual(const float* x, int64_t rows, int64_t K, c
     return fc_impl(x, rows, K, weiq, Ng, Kg, group_k, N, residual, y, workspace, workspace_bytes, stream);
 }
 
-extern "C" int llmops_fc_Q4A_decode(const float* x, int64_t rows, int64_t K, const int8_t* weiq, int64_t Ng, int64_t Kg,
-                                    int group_k, int64_t N_out, const float* norm_w, float eps, const float* residual,
-                                    int glu, const float* sumsq_in, int64_t sumsq_parts, float* sumsq_out, float* y,
-                                    void* workspace, size_t workspace_bytes, llmops_stream_t stream) {
+static int fc_decode_impl(const float* x, int64_t rows, int64_t K, const int8_t* weiq, int64_t Ng, int64_t Kg, int group_k,
+                          int64_t N_out, const float* norm_w, float eps, const float* residual, int glu,
+                          const float* sumsq_in, int64_t sumsq_parts, float* sumsq_out, float* y, int64_t out_parts,
+                          void* workspace, size_t workspace_bytes, llmops_stream_t stream) {
     LLMOPS_REQUIRE(valid_group(group_k));
     LLMOPS_REQUIRE(x != nullptr && weiq != nullptr && y != nullptr && workspace != nullptr);
     LLMOPS_REQUIRE(rows > 0);
@@ -192,6 +192,10 @@ extern "C" int llmops_fc_Q4A_decode(const float* x, int64_t rows, int64_t K, con
     if (sumsq_in != nullptr) LLMOPS_REQUIRE(norm_w != nullptr && sumsq_parts > 0 && sumsq_parts <= 65536);
     if (sumsq_out != nullptr) LLMOPS_REQUIRE(glu != 1);
     if (glu == 2) LLMOPS_REQUIRE(norm_w == nullptr && sumsq_in == nullptr);
+    LLMOPS_REQUIRE(out_parts >= 1);
+    if (out_parts > 1)
+        LLMOPS_REQUIRE(glu != 1 && residual == nullptr && sumsq_out == nullptr && (Ng % out_parts) == 0 &&
+                       N_out == Ng * kGroupN);
     const FcWorkspace lay = fc_layout(rows, Ng, Kg, group_k);
     if (workspace_bytes < lay.total)
         return fail(LLMOPS_EWORKSPACE, "fc_Q4A needs %zu workspace bytes, got %zu", lay.total, workspace_bytes);
@@ -211,13 +215,39 @@ extern "C" int llmops_fc_Q4A_decode(const float* x, int64_t rows, int64_t K, con
                      ? launch_quant_x_fused(x, rows, K, group_k, norm_w, eps, glu == 2, xq, xd, gs, xst, st)
                      : launch_quant_x(x, rows, K, group_k, xq, xd, gs, xst, false, st);
         if (rc) return rc;
+        if (out_parts > 1) {
+            // y is [out_parts][rows][N_out / out_parts]: one product per slice of strips on the same quantized rows
+            // (q, k and v of a fused q|k|v tensor come out as three dense matrices instead of one to be cut up)
+            const int64_t ngp = Ng / out_parts, np = N_out / out_parts;
+            for (int64_t p = 0; p < out_parts && rc == 0; p++)
+                rc = fc_product_many_rows(reinterpret_cast<const uint8_t*>(weiq) + p * ngp * Kg * block_bytes(group_k), ws, lay,
+                                          rows, ngp, Kg, group_k, np, nullptr, y + p * rows * np, st);
+            return rc;
+        }
         rc = fc_product_many_rows(reinterpret_cast<const uint8_t*>(weiq), ws, lay, rows, Ng, Kg, group_k, N_out, residual, y, st);
         if (rc == 0 && sumsq_out != nullptr) rc = launch_strip_sumsq(y, rows, N_out, sumsq_out, st);
         return rc;
     }
+    LLMOPS_REQUIRE(out_parts == 1);  // (up to 8 rows: a slice of a row is as good as a row of its own)
     return launch_gemv_fused(reinterpret_cast<const uint8_t*>(weiq), x, y, reinterpret_cast<float*>(ws + lay.off_part),
                              reinterpret_cast<unsigned*>(ws), rows, Ng, Kg, group_k, N_out, residual, norm_w, eps, glu,
                              sumsq_in, (int)sumsq_parts, sumsq_out, as_stream(stream));
+}
+
+extern "C" int llmops_fc_Q4A_decode(const float* x, int64_t rows, int64_t K, const int8_t* weiq, int64_t Ng, int64_t Kg,
+                                    int group_k, int64_t N_out, const float* norm_w, float eps, const float* residual,
+                                    int glu, const float* sumsq_in, int64_t sumsq_parts, float* sumsq_out, float* y,
+                                    void* workspace, size_t workspace_bytes, llmops_stream_t stream) {
+    return fc_decode_impl(x, rows, K, weiq, Ng, Kg, group_k, N_out, norm_w, eps, residual, glu, sumsq_in, sumsq_parts, sumsq_out, y,
+                          1, workspace, workspace_bytes, stream);
+}
+
+extern "C" int llmops_fc_Q4A_decode_parts(const float* x, int64_t rows, int64_t K, const int8_t* weiq, int64_t Ng, int64_t Kg,
+                                          int group_k, int64_t N_out, const float* norm_w, float eps, int glu, int64_t out_parts,
+                                          float* y, void* workspace, size_t workspace_bytes, llmops_stream_t stream) {
+    LLMOPS_REQUIRE(rows > kMaxGemvRows);
+    return fc_decode_impl(x, rows, K, weiq, Ng, Kg, group_k, N_out, norm_w, eps, nullptr, glu, nullptr, 0, nullptr, y, out_parts,
+                          workspace, workspace_bytes, stream);
 }
 
 static int fc_decode_attn(const float* rec_stats, const float* rec_outs, int64_t chunks, int64_t H, const int8_t* weiq,

@@ -232,7 +232,7 @@ def interleave_gate_up(gate_packed, up_packed):
 
 
 def fc_Q4A_decode(input, weiq, N_out, norm=None, residual=None, glu=False, sumsq_in=None, want_sumsq=False,
-                  glu_in=False, attn_records=None):
+                  glu_in=False, attn_records=None, out_parts=1):
     """Extension: fc_Q4A with its neighbours of the decode step folded in (one launch for B*M <= 8).
 
     norm=(weight, eps): input is rmsnorm'ed first;  residual: added to the result;
@@ -241,6 +241,8 @@ def fc_Q4A_decode(input, weiq, N_out, norm=None, residual=None, glu=False, sumsq
     over the gate and up weights stacked along N leaves behind) and the FC runs on silu(gate)*up.
     attn_records=...: ``input`` is None and the FC's input is the output of decode attention still in chunk records
     (``attention_rope2_records``), merged as it is loaded.
+    out_parts=p (more than 8 rows, plain or norm FC): the result comes as p dense tensors [p, B, M, N_out/p] (part i =
+    columns i*N_out/p ..), e.g. q, k and v of a fused q|k|v projection, instead of one tensor to be cut up and copied.
     want_sumsq=True returns ``(out, sumsq)`` where ``sumsq``
     [B*M, strips] holds the sum of squares of every 32 outputs; passed as ``sumsq_in`` to the FC that
     rmsnorms ``out`` it saves that FC the pass over the row.  With more than 8 rows the rmsnorm or the
@@ -288,6 +290,9 @@ def fc_Q4A_decode(input, weiq, N_out, norm=None, residual=None, glu=False, sumsq
     _require(not (want_sumsq and glu), "no sumsq with glu")
     fusable = K % g == 0 and input.data_ptr() % 16 == 0 and (norm is None or (K <= 16384 and norm[0].data_ptr() % 16 == 0)) \
         and (not glu_in or g == 128)
+    if out_parts != 1 and (rows <= 8 or glu or not fusable):
+        whole = fc_Q4A_decode(input, weiq, N_out, norm=norm, glu_in=glu_in, sumsq_in=sumsq_in)
+        return torch.stack([c.contiguous() for c in whole.chunk(out_parts, dim=-1)])
     if rows > 8 and (glu or not fusable):
         # gate and up interleaved on the output side (or a shape the fused quantization does not take): separate ops
         x = input if norm is None else rmsnorm_out(input, norm[0], norm[1])
@@ -308,6 +313,15 @@ def fc_Q4A_decode(input, weiq, N_out, norm=None, residual=None, glu=False, sumsq
         return out
     lib = _lib.load()
     ws = _workspace(input.device, lib.llmops_fc_Q4A_workspace_bytes(rows, K, Ng, Kg, g))
+    if out_parts != 1:
+        _require(rows > 8 and not glu and residual is None and not want_sumsq and Ng % out_parts == 0 and N_out == Ng * 32,
+                 "out_parts: more than 8 rows, whole strips per part, no residual, no sumsq")
+        out = torch.empty((out_parts, B, M, N_out // out_parts), dtype=torch.float32, device=input.device)
+        _lib.check(lib.llmops_fc_Q4A_decode_parts(_ptr(input), rows, K, _ptr(weiq), Ng, Kg, g, N_out,
+                                                  _ptr(norm[0]) if norm is not None else None,
+                                                  float(norm[1]) if norm is not None else 0.0, 2 if glu_in else 0, out_parts,
+                                                  _ptr(out), _ptr(ws), ws.numel(), _stream(input)))
+        return out
     out = torch.empty((B, M, N_out), dtype=torch.float32, device=input.device)
     sumsq = torch.empty((rows, Ng), dtype=torch.float32, device=input.device) if want_sumsq else None
     _lib.check(lib.llmops_fc_Q4A_decode(_ptr(input), rows, K, _ptr(weiq), Ng, Kg, g, N_out,

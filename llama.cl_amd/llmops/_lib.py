@@ -29,6 +29,8 @@ SIGNATURES = {
                                        c_ptr]),
     "llmops_fc_Q4A_decode": (c_int, [c_ptr, c_i64, c_i64, c_ptr, c_i64, c_i64, c_int, c_i64, c_ptr, c_f32, c_ptr, c_int, c_ptr,
                                      c_i64, c_ptr, c_ptr, c_ptr, c_size, c_ptr]),
+    "llmops_fc_Q4A_decode_parts": (c_int, [c_ptr, c_i64, c_i64, c_ptr, c_i64, c_i64, c_int, c_i64, c_ptr, c_f32, c_int, c_i64,
+                                           c_ptr, c_ptr, c_size, c_ptr]),
     "llmops_fc_Q4A_decode_attn": (c_int, [c_ptr, c_ptr, c_i64, c_i64, c_ptr, c_i64, c_i64, c_i64, c_ptr, c_ptr, c_ptr, c_ptr,
                                           c_size, c_ptr]),
     "llmops_fc_Q4A_prequantized": (c_int, [c_ptr, c_ptr, c_ptr, c_i64, c_ptr, c_i64, c_i64, c_int, c_i64, c_ptr, c_ptr,

@@ -195,11 +195,16 @@ class LlamaDecoder:
         projections, rope + cache update inside the attention kernel."""
         H, F = self.configs["hidden_size"], self.configs["intermediate_size"]
         n1, n2 = ops["input_layernorm"], ops["post_attention_layernorm"]
-        qkv = llmops.fc_Q4A_decode(hidden_states, ops["qkv_proj"].weight, 3 * H, norm=(n1.weight, n1.eps), sumsq_in=sumsq)
-        q, k, v = qkv[..., :H], qkv[..., H:2 * H], qkv[..., 2 * H:]
-        if not q.is_contiguous():  # more than one token: the op needs dense [B,qL,H*S] tensors
-            q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
-        if qkv.shape[0] * qkv.shape[1] == 1 and self.merge_in_o_proj and llmops.attention_records_supported(kv_cache) \
+        rows = hidden_states.shape[0] * hidden_states.shape[1]
+        many = rows > 8  # a prompt or a batch: the sums of squares are not handed on (the norms read their rows)
+        if many:  # q, k and v as three dense [B,qL,H*S] tensors straight from the product
+            q, k, v = llmops.fc_Q4A_decode(hidden_states, ops["qkv_proj"].weight, 3 * H, norm=(n1.weight, n1.eps), out_parts=3)
+        else:
+            qkv = llmops.fc_Q4A_decode(hidden_states, ops["qkv_proj"].weight, 3 * H, norm=(n1.weight, n1.eps), sumsq_in=sumsq)
+            q, k, v = qkv[..., :H], qkv[..., H:2 * H], qkv[..., 2 * H:]
+            if not q.is_contiguous():  # more than one token: the op needs dense [B,qL,H*S] tensors
+                q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+        if rows == 1 and self.merge_in_o_proj and llmops.attention_records_supported(kv_cache) \
                 and llmops.group_k_of(ops["o_proj"].weight) == 128 and self.inv_freq.shape[0] % 4 == 0:
             # one token: attention leaves its split-KV chunk records and the o projection merges them on its way in
             recs = llmops.attention_rope2_records(q, k, v, self.inv_freq, kv_cache, kv_cache_slots, position_id, i)
@@ -207,14 +212,21 @@ class LlamaDecoder:
                                                    attn_records=recs)
         else:
             llmops.attention_rope2(q, k, v, self.inv_freq, kv_cache, kv_cache_slots, position_id, i)
-            attn_output, ss = llmops.fc_Q4A_decode(q, ops["o_proj"].weight, H, residual=hidden_states, want_sumsq=True)
+            if many:
+                attn_output, ss = llmops.fc_Q4A_decode(q, ops["o_proj"].weight, H, residual=hidden_states), None
+            else:
+                attn_output, ss = llmops.fc_Q4A_decode(q, ops["o_proj"].weight, H, residual=hidden_states, want_sumsq=True)
         if self.stacked_gate_up:
             gate_up = llmops.fc_Q4A_decode(attn_output, ops["gate_up_proj"].weight, 2 * F, norm=(n2.weight, n2.eps),
                                            sumsq_in=ss)
+            if many:
+                return llmops.fc_Q4A_decode(gate_up, ops["down_proj"].weight, H, residual=attn_output, glu_in=True), None
             return llmops.fc_Q4A_decode(gate_up, ops["down_proj"].weight, H, residual=attn_output, want_sumsq=True,
                                         glu_in=True)
         act = llmops.fc_Q4A_decode(attn_output, ops["gate_up_proj"].weight, F, norm=(n2.weight, n2.eps), glu=True,
                                    sumsq_in=ss)
+        if many:
+            return llmops.fc_Q4A_decode(act, ops["down_proj"].weight, H, residual=attn_output), None
         return llmops.fc_Q4A_decode(act, ops["down_proj"].weight, H, residual=attn_output, want_sumsq=True)
 
     def capture_decode(self, kv_cache, slot, position_id, stream=None):

@@ -385,6 +385,28 @@ def test_fc_decode_many_rows_producer_inside_the_quantization(ops, orc, G, rows,
         assert max_rel_err(host(got), orc.fc(act, host(pw), N) + host(res)) <= 1e-5
 
 
+@pytest.mark.parametrize("G", [32, 128])
+@pytest.mark.parametrize("rows", [9, 40, 600])
+def test_fc_decode_many_rows_result_in_dense_parts(ops, orc, G, rows):
+    """out_parts: the columns of a fused q|k|v projection come out as three dense tensors, bit-equal to the slices
+    of the one-tensor result (same quantized rows, same product kernels on a third of the strips each)."""
+    rng = np.random.default_rng(rows + G)
+    K, N = 1024, 3 * 352
+    pw = dev(orc.quant_w((rng.standard_normal((N, K)) * 0.02).astype(np.float32), G))
+    x = dev(rng.standard_normal((1, rows, K)).astype(np.float32))
+    nw = dev((1.0 + 0.1 * rng.standard_normal(K)).astype(np.float32))
+    whole = ops.fc_Q4A_decode(x, pw, N, norm=(nw, 1e-5))
+    parts = ops.fc_Q4A_decode(x, pw, N, norm=(nw, 1e-5), out_parts=3)
+    assert parts.shape == (3, 1, rows, 352) and parts.is_contiguous()
+    for i in range(3):
+        # (a third of the strips may be cut into tiles and k-splits differently from the whole: fp32 summation order)
+        assert max_rel_err(host(parts[i]), host(whole[..., 352 * i:352 * (i + 1)])) <= 1e-5
+    plain = ops.fc_Q4A_decode(x, pw, N, out_parts=3)
+    assert max_rel_err(host(plain[1]), host(ops.fc_Q4A(x, pw, N)[..., 352:704])) <= 1e-5
+    with pytest.raises(RuntimeError):
+        ops.fc_Q4A_decode(x, pw, N, out_parts=4)  # 33 strips do not divide by 4
+
+
 def test_fc_decode_many_rows_refuses_what_it_cannot_fold(ops, orc):
     """At the C ABI: interleaved gate/up strips on the output side (glu 1) need the 8-row kernel, and the
     silu(gate)*up producer needs group 128; both are refused before anything is enqueued (the Python op composes
