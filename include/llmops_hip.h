@@ -216,9 +216,13 @@ size_t llmops_attention_workspace_bytes(int64_t B, int64_t qL, int64_t H, int64_
  * on fp16-rounded K/V); slots int32 [qL] (device).  Effects: q,k rotated in place (k stays
  * rotated), k,v rows written to cache[2*layer_id+{0,1}, b, h, slots[p], :], and q overwritten by
  * softmax((q.K^T)/sqrt(S) with in-chunk causal mask via slots) . V over
- * kvLen = min(position_id+qL, maxlen) cache rows.  One query token (qL == 1, the decode form) needs
- * maxlen*S*sizeof(cache element) < 4 GiB (LLMOPS_EINVAL otherwise); more than 65535 heads in all (B*H) are served
- * by the general kernels (three launches instead of two). */
+ * kvLen = min(position_id+qL, maxlen) cache rows.  One query token (qL == 1, the decode form) and 32 or more
+ * (the tiled prompt kernel, S == 128) need maxlen*S*sizeof(cache element) < 4 GiB (LLMOPS_EINVAL otherwise); more
+ * than 65535 heads in all (B*H) with one query token are served by the general kernels (three launches instead
+ * of two).  Arithmetic: fp32 throughout, except that the tiled prompt kernel multiplies on the fp16 matrix cores
+ * with every fp32 operand carried as two fp16 halves (22 bits, fp32 accumulation): its results agree with fp32
+ * evaluation to about 1e-6 of the largest output (tests assert 1e-5; the contract is 1e-3), and q, k, v and cache
+ * values must lie inside the fp16 range (|x| < 65504) there. */
 int llmops_attention_rope(float* q, float* k, const float* v, int64_t B, int64_t qL, int64_t H, int64_t S,
                           const float* inv_freq, int64_t half, void* kv_cache, int cache_dtype,
                           int64_t planes, int64_t maxlen, const int32_t* slots, int position_id,
