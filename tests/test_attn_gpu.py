@@ -169,6 +169,26 @@ def test_attention_prefill_tiled_vs_oracle(ops, orc, cache_dtype):
             assert np.abs(cache_after - cache_ref).max() <= 1e-5
 
 
+@pytest.mark.parametrize("order", ["reversed", "shuffled"])
+def test_attention_prefill_tiled_with_slots_in_any_order(ops, orc, order):
+    """The tiled prompt kernel finds what a query may see from the slot -> token map alone: the chunk's rows are
+    written to slots in reversed / shuffled order among rows of earlier context (so the tile with the chunk's last
+    tokens comes first, tiles mix visible and masked rows, and the last row a query tile may see is not where a
+    prompt written front to back would have it)."""
+    rng = np.random.default_rng(21 + len(order))
+    B, H, S, maxlen, past, qL = 1, 2, 128, 400, 100, 260
+    inv_freq = (1.0 / (10000.0 ** (np.arange(0, S, 2, dtype=np.float32) / np.float32(S)))).astype(np.float32)
+    cache = rng.standard_normal((2, B, H, maxlen, S)).astype(np.float32)
+    free = np.arange(past, past + qL)
+    slots = (free[::-1] if order == "reversed" else rng.permutation(free)).astype(np.int32)
+    q, k, v = (rng.standard_normal((B, qL, H * S)).astype(np.float32) for _ in range(3))
+    g = dict(q=q, k=k, v=v, cache=cache, inv_freq=inv_freq, slots=slots, position_id=past, layer_id=0)
+    out, k_rot, cache_after = run_attention(ops, g)
+    want, k_ref, cache_ref = orc.attention(q, k, v, inv_freq, cache, slots, past, 0)
+    assert max_rel_err(out, want) <= 1e-5
+    assert np.abs(cache_after - cache_ref).max() <= 1e-5
+
+
 def _attend_cache(orc, q, inv_freq, cache, slots, past, maxlen):
     """fp64 attention of the rotated queries over a finished cache with the reference's in-chunk mask."""
     B, qL, HS = q.shape
