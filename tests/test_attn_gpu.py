@@ -497,7 +497,6 @@ def test_attention_records_merged_by_the_o_projection(ops, orc, cache_dtype, max
             # (3) outputs
             yf, ss = ops.fc_Q4A_decode(None, wq, N, residual=dev(res), want_sumsq=True, attn_records=recs)
             assert np.array_equal(host(yf)[0], host(y) + res[0])            # production build == dump build (+ residual)
-            print("records-vs-unfused", cache_dtype, maxlen, kv, dev_pos, max_rel_err(host(yf), host(want_y)), max_rel_err(host(ss), host(want_ss)))
             assert max_rel_err(host(yf), host(want_y)) <= 1e-2, (kv, dev_pos)
             assert max_rel_err(host(ss), host(want_ss)) <= 2e-2
         if cache_dtype == torch.float32 and kv in (257, 2048):              # and the oracle's two ops
