@@ -113,6 +113,12 @@ __device__ __forceinline__ float4 load4(const __half* p) {
     return make_float4(fa.x, fa.y, fb.x, fb.y);
 }
 
+__device__ __forceinline__ float2 load2(const float* p) { return *reinterpret_cast<const float2*>(p); }
+__device__ __forceinline__ float2 load2(const __half* p) {
+    const uint32_t u = *reinterpret_cast<const uint32_t*>(p);
+    return __half22float2(*reinterpret_cast<const __half2*>(&u));
+}
+
 // Per-chunk record in the workspace: [max, sum, out[S]]
 // Workgroup = 4 waves; wave w owns rows w*PW .. w*PW+PW-1 of the chunk (C = 4*PW rows);
 // lane = 32*hf + e: row parity hf, elements 4e..4e+3 (S == 128).
@@ -762,23 +768,26 @@ __global__ __launch_bounds__(512) void attn_prefill_kernel(float* q, const T* __
 #pragma unroll
         for (int r = 0; r < 16; r++) o[c][r] = 0.0f;
 
-    // Staging.  K: a thread moves 16 consecutive floats of one row (row = thread/8).  V: a thread moves a
-    // 4 x 4 patch, rows 4g .. 4g+3 (g = thread/32) of columns 4*(thread%32) .. +3, and writes it transposed:
-    // per column 4 halves = 8 bytes at the rows' place in the column's permuted order (cache row r of the tile
-    // sits at position 16*(r/16) + 8*((r/4)%2) + 4*((r%16)/8) + r%4).  The next tile's global loads are issued
-    // before the current tile is computed on and land in registers meanwhile.
+    // Staging.  K: a thread moves 16 consecutive floats of one row (row = thread/8).  V is written transposed,
+    // cache row r of the tile at position 16*(r/16) + 8*((r/4)%2) + 4*((r%16)/8) + r%4 of its column: a thread
+    // moves the 8 rows that share an aligned run of 8 positions (rows 16b + 4h + w and 16b + 8 + 4h + w, w = 0..3;
+    // (b, h) = the thread's wave) of two neighbouring columns, so that a column's share is one 16-byte store.
+    // (Four rows of four columns per thread meant 8-byte stores 320 bytes apart: eight lanes on every bank.)
+    // The next tile's global loads are issued before the current tile is computed on and land in registers
+    // meanwhile.
     const int krow = tid >> 3, kseg = tid & 7;
-    const int vg = tid >> 5, vq = tid & 31;
-    const int vpos = 16 * (vg >> 2) + 8 * (vg & 1) + 4 * ((vg >> 1) & 1);
-    float4 kst[4], vst[4];
+    const int vb = wave >> 1, vh = wave & 1, vcp = lane;  // rows 16*vb + 8*(e/4) + 4*vh + e%4, columns 2*vcp, 2*vcp+1
+    float4 kst[4];
+    float2 vst[8];
     int tst = INT_MAX;
 #define LLMOPS_STAGE_LOAD(KV0)                                                                          \
     do {                                                                                                \
         const uint32_t rk_ = (uint32_t)min((KV0) + krow, kvLeni - 1);                                   \
-        _Pragma("unroll") for (int u = 0; u < 4; u++) {                                                 \
-            const uint32_t rv_ = (uint32_t)min((KV0) + 4 * vg + u, kvLeni - 1);                         \
+        _Pragma("unroll") for (int u = 0; u < 4; u++)                                                   \
             kst[u] = load4(kbase + (rk_ * (uint32_t)S + (uint32_t)(kseg * 16 + u * 4)));               \
-            vst[u] = load4(vbase + (rv_ * (uint32_t)S + (uint32_t)(vq * 4)));                           \
+        _Pragma("unroll") for (int e = 0; e < 8; e++) {                                                 \
+            const uint32_t rv_ = (uint32_t)min((KV0) + 16 * vb + 8 * (e >> 2) + 4 * vh + (e & 3), kvLeni - 1); \
+            vst[e] = load2(vbase + (rv_ * (uint32_t)S + (uint32_t)(vcp * 2)));                          \
         }                                                                                               \
         if (tid < BK) tst = ((KV0) + tid < kvLeni) ? row_token[(KV0) + tid] : INT_MAX;                  \
     } while (0)
@@ -815,17 +824,17 @@ __global__ __launch_bounds__(512) void attn_prefill_kernel(float* q, const T* __
             dl_[0] = make_uint4(lo_[0], lo_[1], lo_[2], lo_[3]);                                                \
             dl_[1] = make_uint4(lo_[4], lo_[5], lo_[6], lo_[7]);                                                \
         }                                                                                                       \
-        /* V patch: column j of the patch is (vst[0..3])[j] */                                                  \
-        const float vx_[4][4] = {{vst[0].x, vst[0].y, vst[0].z, vst[0].w},                                      \
-                                 {vst[1].x, vst[1].y, vst[1].z, vst[1].w},                                      \
-                                 {vst[2].x, vst[2].y, vst[2].z, vst[2].w},                                      \
-                                 {vst[3].x, vst[3].y, vst[3].z, vst[3].w}};                                     \
-        _Pragma("unroll") for (int j = 0; j < 4; j++) {                                                         \
-            uint32_t h0_, l0_, h1_, l1_;                                                                        \
-            split2(vx_[0][j], vx_[1][j], h0_, l0_);                                                             \
-            split2(vx_[2][j], vx_[3][j], h1_, l1_);                                                             \
-            *reinterpret_cast<uint2*>(&(SM).v_hi[(4 * vq + j) * VSB + vpos * 2]) = make_uint2(h0_, h1_);        \
-            if (LO) *reinterpret_cast<uint2*>(&(SM).v_lo[(4 * vq + j) * VSB + vpos * 2]) = make_uint2(l0_, l1_); \
+        {                                                                                                       \
+            uint32_t h_[2][4], l_[2][4]; /* [column][pair of rows] */                                           \
+            _Pragma("unroll") for (int e2 = 0; e2 < 4; e2++) {                                                  \
+                split2(vst[2 * e2].x, vst[2 * e2 + 1].x, h_[0][e2], l_[0][e2]);                                 \
+                split2(vst[2 * e2].y, vst[2 * e2 + 1].y, h_[1][e2], l_[1][e2]);                                 \
+            }                                                                                                   \
+            _Pragma("unroll") for (int j = 0; j < 2; j++) {                                                     \
+                const int at_ = (2 * vcp + j) * VSB + (16 * vb + 8 * vh) * 2;                                   \
+                *reinterpret_cast<uint4*>(&(SM).v_hi[at_]) = make_uint4(h_[j][0], h_[j][1], h_[j][2], h_[j][3]); \
+                if (LO) *reinterpret_cast<uint4*>(&(SM).v_lo[at_]) = make_uint4(l_[j][0], l_[j][1], l_[j][2], l_[j][3]); \
+            }                                                                                                   \
         }                                                                                                       \
         if (wave == 0) {                                                                                        \
             /* the tile's token range, once for all waves: DPP steps inside the rows of 16 lanes, the two rows */ \
