@@ -33,11 +33,16 @@ def sources():
     return sorted(glob.glob(os.path.join(CSRC, "*.hip")) + glob.glob(os.path.join(CSRC, "*.cpp")))
 
 
-# Kernels that must compile without VGPR spills: the 256-row GEMM reads LDS with hand-placed ds_read /
-# s_waitcnt pairs (a register spilled between the two would be saved before its data has arrived); the
-# one-row group-128 decode kernels are written to fit the 64 registers that two 16-wave workgroups per
-# CU leave each wave, and scratch traffic in their loop costs what the rewrite gained.
-NO_SPILL = ["fc_gemm_pp_kernelILb0E", "fc_gemv_fused_kernelILi128ELi1E", "attn_prefill_kernel"]
+# Kernels that must compile without VGPR spills: the one-row group-128 decode kernels are written to fit
+# the 64 registers that two 16-wave workgroups per CU leave each wave, and scratch traffic in their loop
+# costs what the rewrite gained; the prompt attention kernel likewise (a reload in its loop waits for the
+# next tile's loads).
+NO_SPILL = ["fc_gemv_fused_kernelILi128ELi1E", "attn_prefill_kernel"]
+# Kernels that may park a few registers around rarely-run code but whose main loop must be free of spill
+# code: the 256-row GEMM reads LDS there with hand-placed ds_read / s_waitcnt pairs (a register spilled
+# between the two would be saved before its data has arrived).  Checked in the device assembly: no scratch
+# instruction between the kernel's first and last instruction of the kind that marks the loop.
+NO_SPILL_IN_LOOP = {"fc_gemm_pp_kernelILb0E": "v_mfma_i32_16x16x64_i8"}
 
 
 def check_spills(remarks):
@@ -52,8 +57,28 @@ def check_spills(remarks):
                 raise RuntimeError(f"{name} spills {spilled} VGPRs; this kernel must not spill (see NO_SPILL)")
 
 
+def check_loop_spills(asm_path):
+    """asm_path: the device assembly of one source (kept by -save-temps); returns the kernels it has checked"""
+    with open(asm_path) as fh:
+        lines = fh.read().splitlines()
+    seen = []
+    for key, marker in NO_SPILL_IN_LOOP.items():
+        # a function starts at a line "<mangled name>:" in column 0
+        starts = [i for i, l in enumerate(lines) if l[:1] not in (" ", "\t", ".", ";", "") and key in l.split(":")[0] and ":" in l]
+        for a in starts:
+            seen.append(key)
+            b = next((j for j in range(a, len(lines)) if lines[j].startswith(".Lfunc_end")), len(lines))
+            marks = [j for j in range(a, b) if marker in lines[j]]
+            if not marks:
+                raise RuntimeError(f"{key}: no {marker} found in {asm_path}; the loop check cannot tell where the loop is")
+            bad = [j for j in range(marks[0], marks[-1] + 1) if "scratch_" in lines[j]]
+            if bad:
+                raise RuntimeError(f"{key} has spill code inside its main loop ({lines[bad[0]].strip()}); see NO_SPILL_IN_LOOP")
+    return seen
+
+
 def _compile(src, obj):
-    cmd = [HIPCC] + [f for f in FLAGS if f != "-shared"] + ["-Rpass-analysis=kernel-resource-usage", "-c", "-o", obj, src]
+    cmd = [HIPCC] + [f for f in FLAGS if f != "-shared"] + ["-Rpass-analysis=kernel-resource-usage", "-save-temps=obj", "-c", "-o", obj, src]
     proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     return src, proc.returncode, proc.stdout.splitlines()
 
@@ -97,6 +122,12 @@ def build(verbose=False, jobs=None):
             if log.strip():
                 logs.append(log)
         check_spills(remarks)
+        checked = []
+        for asm in glob.glob(os.path.join(objdir, "*-hip-amdgcn-amd-amdhsa-gfx950.s")):
+            checked += check_loop_spills(asm)
+        missing = sorted(set(NO_SPILL_IN_LOOP) - set(checked))
+        if missing:
+            raise RuntimeError(f"kernels named in NO_SPILL_IN_LOOP were not found in the device assembly: {missing}")
         link = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", OUT] + objs
         proc = subprocess.run(link, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
         if proc.returncode != 0:

@@ -282,6 +282,120 @@ __device__ __forceinline__ v2f buf_ld_pair(buffer_rsrc r, uint32_t voff, uint32_
     return v2f{__uint_as_float(t.x), __uint_as_float(t.y)};
 }
 
+// ---- the min term of a tile on the fp16 matrix cores -------------------------------------------------
+// sum over k-groups of m[column][kg] * gsum[row][kg] is a product with K = number of k-groups.  It is
+// taken out of the k-group loop and computed once per tile, 32 k-groups per MFMA, with fp32 accumulation:
+// gsum = hi + lo (hi = gsum rounded toward zero to fp16, lo = the rest: 22 significant bits in all), m as
+// it is stored (fp16), two MFMAs per 16x16 tile.  (The fp32 MFMA that did this inside the loop stalls the
+// vector ALU for its whole duration; the fp16 one runs beside vector work.)  That is good for a row's eight
+// k-groups in one lane if the largest |gsum| among them lies in [1/8, 60000]: below that lo falls into fp16's
+// subnormals and the row could lose bits relative to its own size, above it hi overflows.  Zeros are exact.
+// When a lane of the wave does not qualify, the wave takes the round with fp32 MFMAs instead (four k-groups
+// each, exact products): the slow path, there for correctness on any input.
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+typedef _Float16 v2h __attribute__((ext_vector_type(2)));
+union Halves8 {
+    v8h h;
+    uint32_t u[4];
+};
+
+// What a lane fetches for one round of 32 k-groups (k32 .. k32+31, those below kb1): for its eight k-groups
+// kgs .. kgs+7 the group sums of its row in each of RT row tiles (32 contiguous bytes of the [row][kg] matrix, which
+// start on a 4-byte boundary only) and the mins of its four columns.  kgs is k32 + 8g unless that would read past
+// the end of a row: then it is Kg - 8, and the slots below k32 + 8g do not count (min_term_add).
+struct __attribute__((packed, aligned(4))) Float4U {
+    float v[4];
+};
+template <int RT>
+struct MinTermRound {
+    Float4U ga[RT][2];
+    uint2 mb[8];
+};
+// roff[t] = Kg * the lane's row of row tile t (clamped to the matrix); strip: its strip (clamped); q: its column
+// quad.  Rows and strip count from wherever gs and weiq point (the matrix, or the workgroup's tile of it): offsets
+// from there must fit 32 bits.
+template <int RT>
+__device__ __forceinline__ void min_term_fetch(MinTermRound<RT>& r, const float* __restrict__ gs, const int (&roff)[RT],
+                                               const uint8_t* __restrict__ weiq, int Kg, int kgs, int strip, int q) {
+    // (a uniform base and a 32-bit byte offset per lane: one address register per load, not two)
+    const uint8_t* gb = reinterpret_cast<const uint8_t*>(gs);
+#pragma unroll
+    for (int t = 0; t < RT; t++) {
+        const uint32_t off = (uint32_t)(roff[t] + kgs) * 4u;
+        r.ga[t][0] = *reinterpret_cast<const Float4U*>(gb + off);
+        r.ga[t][1] = *reinterpret_cast<const Float4U*>(gb + off + 16u);
+    }
+    const uint32_t moff = (uint32_t)((strip * Kg + kgs) * kBlk128 + 2112 + q * 8);
+#pragma unroll
+    for (int i = 0; i < 8; i++) r.mb[i] = *reinterpret_cast<const uint2*>(weiq + (moff + (uint32_t)(i * kBlk128)));
+}
+// f[t][c] += the round's part of the min term; operand layout of the 16x16x32 MFMA: A lane (row = lane & 15,
+// k = 8 * (lane >> 4) + i), B lane (column = lane & 15, same k), D as the int8 MFMAs' (row 4g+v, column = lane & 15).
+// Slot i of the lane is k-group kgs + i and counts if it lies in [lo, kb1).  FIRST: f = instead of f += (the
+// accumulators then do not exist yet while the operands are fetched and examined).
+template <int RT, bool FIRST>
+__device__ __forceinline__ void min_term_add(v4f (&f)[RT][4], const MinTermRound<RT>& r, int kgs, int lo, int kb1) {
+    const v4f zero = {0.f, 0.f, 0.f, 0.f};
+    // (the slot tests are repeated where the values are used -- behind an empty asm statement, or the compiler
+    // keeps the 8 * RT masked values of the first pass in registers, which do not fit beside the accumulators,
+    // the operands and what the k-group loop keeps across this prologue)
+#define LLMOPS_GSUM(T, I) ((kgs + (I) >= lo && kgs + (I) < kb1) ? r.ga[T][(I) >> 2].v[(I) & 3] : 0.0f)
+    // (tested per lane, i.e. per row and eight k-groups, which is stricter than per row and needs no exchange)
+    bool rows_fit = true;
+#pragma unroll
+    for (int t = 0; t < RT; t++) {
+        float big = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 8; i++) big = fmaxf(big, fabsf(LLMOPS_GSUM(t, i)));
+        rows_fit = rows_fit && (big == 0.0f || (big >= 0.125f && big <= 60000.0f));
+    }
+    asm volatile("" : "+v"(lo));
+    if (__all(rows_fit)) {
+        Halves8 m[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const uint2 e = r.mb[2 * j], o = r.mb[2 * j + 1];
+            m[0].u[j] = __builtin_amdgcn_perm(o.x, e.x, 0x05040100u);
+            m[1].u[j] = __builtin_amdgcn_perm(o.x, e.x, 0x07060302u);
+            m[2].u[j] = __builtin_amdgcn_perm(o.y, e.y, 0x05040100u);
+            m[3].u[j] = __builtin_amdgcn_perm(o.y, e.y, 0x07060302u);
+        }
+#pragma unroll
+        for (int t = 0; t < RT; t++) {
+            Halves8 ah, al;
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const float e = LLMOPS_GSUM(t, 2 * j), o = LLMOPS_GSUM(t, 2 * j + 1);
+                const v2h h = __builtin_bit_cast(v2h, __builtin_amdgcn_cvt_pkrtz(e, o));
+                ah.u[j] = __builtin_bit_cast(uint32_t, h);
+                al.u[j] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(e - (float)h[0], o - (float)h[1]));
+            }
+#pragma unroll
+            for (int c = 0; c < 4; c++)
+                f[t][c] = __builtin_amdgcn_mfma_f32_16x16x32_f16(al.h, m[c].h, FIRST ? zero : f[t][c], 0, 0, 0);
+#pragma unroll
+            for (int c = 0; c < 4; c++) f[t][c] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ah.h, m[c].h, f[t][c], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);  // one row tile's halves at a time: registers
+        }
+    } else {
+        // slot i of the four lanes (row or column, g = 0..3) is one 16x16x4 product: k = g
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const float mc[4] = {f16_bits_to_f32((uint16_t)(r.mb[i].x & 0xFFFFu)), f16_bits_to_f32((uint16_t)(r.mb[i].x >> 16)),
+                                 f16_bits_to_f32((uint16_t)(r.mb[i].y & 0xFFFFu)), f16_bits_to_f32((uint16_t)(r.mb[i].y >> 16))};
+#pragma unroll
+            for (int t = 0; t < RT; t++) {
+                const float a = LLMOPS_GSUM(t, i);
+#pragma unroll
+                for (int c = 0; c < 4; c++)
+                    f[t][c] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, mc[c], (FIRST && i == 0) ? zero : f[t][c], 0, 0, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);  // one slot's operands at a time: registers, not speed, matter here
+        }
+    }
+#undef LLMOPS_GSUM
+}
+
 template <int RT>
 struct GemmSmem {
     static constexpr int BM = RT * 32;
@@ -571,7 +685,12 @@ __global__ __launch_bounds__(256, (RT == 4 ? 2 : (RT == 2 ? 3 : 4))) void fc_gem
 //   The fold is register arithmetic and the MFMAs have no side effects, so the compiler is free to
 //   move either across a barrier into the other phase (it did: the fold ended up next to the same
 //   group's MFMAs).  Empty asm statements that name the accumulators as operands pin them.
-// Measured per k-group (2048 x 11008 x 4096, cycles of the shader clock): matrix-core side ~1500
+//   The min term is not in the loop: the accumulators start at it (min_term_add above), formed from
+//   the [row][kg] group sums and the blocks' mins before the first k-group -- by group 0 while group 1
+//   unpacks the first k-group's weights, by group 1 in the phase it has to wait anyway.  In the loop
+//   it was 16 fp32 MFMAs per four k-groups and wave, each of which holds up the vector ALU of its SIMD
+//   for its 32 cycles (2048 rows: 11008 x 4096 187 -> 181 us, 4096 x 11008 164 -> 159 us).
+// Measured per k-group with the min term still in the loop (2048 x 11008 x 4096, cycles of the shader clock): matrix-core side ~1500
 // (operand reads 450, 32 MFMAs with the copies between them 1000), fold side ~1350-1900 (the fold
 // itself 1350: the vector ALU is shared with the other group's MFMA issue; unpacking the weights on
 // group 0 adds the wait for their fetch), barriers ~400; 4000 per k-group against ~4700 for the
@@ -581,10 +700,8 @@ struct GemmPPSmem {
     static constexpr int BM = 256;
     uint8_t a[2][BM * 128];
     uint8_t bu[2][4 * kBuStrip];            // unpacked weights: [strip][h][c][g][q][16], strips padded
-    float d[2][4 * 32];                     // weight scale, min per strip column
-    float m[2][4 * 32];
+    float d[2][4 * 32];                     // weight scale per strip column
     float dx[2][BM];
-    float gs[2][BM];
 };
 
 __device__ __forceinline__ uint32_t lds_off(const void* p) {
@@ -662,7 +779,7 @@ __global__ __launch_bounds__(512, 2) void fc_gemm_pp_kernel(const uint8_t* __res
         const int key = (r + ((r >> 3) & 1)) & 7;
         aoff[i] = (uint32_t)(min(rows - 1, row0 + r) * (int)Kp + (((lane & 7) ^ key) * 16));
     }
-    // scales: waves 0,1 copy dx of rows 64*w4 + lane, waves 2,3 the group sums of rows 64*(w4-2) + lane
+    // activation scales: waves 0,1 of a group copy dx of rows 64*w4 + lane
     const int xr = (w4 & 1) * 64 + lane;
     const int64_t xrow = min(rows - 1, row0 + xr);
     const uint8_t* xbase = nullptr;
@@ -671,21 +788,21 @@ __global__ __launch_bounds__(512, 2) void fc_gemm_pp_kernel(const uint8_t* __res
     if (!PARTIALS) {
         if (xsT) {
             xbase = reinterpret_cast<const uint8_t*>(xsT);
-            xoff = (uint32_t)((xrow * 2 + (w4 >> 1)) * 4);
+            xoff = (uint32_t)(xrow * 8);
             xstep = (int64_t)rows * 8;
         } else {
-            xbase = reinterpret_cast<const uint8_t*>((w4 >> 1) ? gs : xd);
+            xbase = reinterpret_cast<const uint8_t*>(xd);
             xoff = (uint32_t)(xrow * Kg * 4);
             xstep = 4;
         }
     }
     const uint32_t lds_a = lds_off(&sm.a[0][0]);
-    const uint32_t lds_x = (w4 >> 1) ? lds_off(&sm.gs[0][0]) : lds_off(&sm.dx[0][0]);
+    const uint32_t lds_x = lds_off(&sm.dx[0][0]);
 #define LLMOPS_COPY_A(KB, BUF, I)                                                                                  \
     copy16_to_lds(xq + (int64_t)(KB) * 128, aoff[I], lds_a + (BUF) * (BM * 128) + (grp * GM + (w4 * 4 + (I)) * 8) * 128)
 #define LLMOPS_COPY_X(KB, BUF)                                                                                     \
     do {                                                                                                           \
-        if (!PARTIALS) copy4_to_lds(xbase + (int64_t)(KB) * xstep, xoff, lds_x + (BUF) * (BM * 4) + (grp * GM + (w4 & 1) * 64) * 4); \
+        if (!PARTIALS && w4 < 2) copy4_to_lds(xbase + (int64_t)(KB) * xstep, xoff, lds_x + (BUF) * (BM * 4) + (grp * GM + w4 * 64) * 4); \
     } while (0)
 #define LLMOPS_COPY(KB, BUF)                                                                                       \
     do {                                                                                                           \
@@ -693,9 +810,10 @@ __global__ __launch_bounds__(512, 2) void fc_gemm_pp_kernel(const uint8_t* __res
         LLMOPS_COPY_X(KB, BUF);                                                                                    \
     } while (0)
 
-    // weights (group 0): thread t of the group takes the 16-byte chunks t and t + 256 of the tile's
-    // 512 (chunk = strip (2 bits) | k8-row (4 bits) | column quad (3 bits)); its first 32 threads also
-    // the 32 chunks of fp16 scales (strip (2 bits) | d or m (1 bit) | column octet (2 bits))
+    // weights (group 0; group 1 for the first k-group, while group 0 has the min term to compute): thread t
+    // of the group takes the 16-byte chunks t and t + 256 of the tile's 512 (chunk = strip (2 bits) | k8-row
+    // (4 bits) | column quad (3 bits)); its first 16 threads also the 16 chunks of fp16 scales d (strip
+    // (2 bits) | column octet (2 bits))
     const int gtid = tid & 255;
     uint32_t boff[2];
     int bdst[2];
@@ -706,21 +824,21 @@ __global__ __launch_bounds__(512, 2) void fc_gemm_pp_kernel(const uint8_t* __res
         // [strip][h = r>>3][c][g = (r&7)>>1][q4][8 * (r&1)]; c adds 512 bytes
         bdst[i] = st * kBuStrip + ((((r >> 3) * 4) * 4 + ((r & 7) >> 1)) * 8 + q4) * 16 + (r & 1) * 8;
     }
-    const int sst = (gtid >> 3) & 3, spart = gtid & 7;
+    const int sst = (gtid >> 2) & 3, spart = gtid & 3;
     const uint32_t soff = (uint32_t)(min(Ng - 1, strip0 + sst) * Kg * kBlk128 + 2048 + spart * 16);
     v4u rb[2], rs = {0u, 0u, 0u, 0u};
-#define LLMOPS_FETCH_B(KB)                                                                                 \
+#define LLMOPS_FETCH_B(KB, WHO)                                                                            \
     do {                                                                                                   \
-        if (grp == 0) {                                                                                    \
+        if (grp == (WHO)) {                                                                                \
             const uint8_t* wkb = weiq + (int64_t)(KB) * kBlk128;                                           \
             rb[0] = *reinterpret_cast<const v4u*>(wkb + boff[0]);                                          \
             rb[1] = *reinterpret_cast<const v4u*>(wkb + boff[1]);                                          \
-            if (gtid < 32) rs = *reinterpret_cast<const v4u*>(wkb + soff);                                 \
+            if (gtid < 16) rs = *reinterpret_cast<const v4u*>(wkb + soff);                                 \
         }                                                                                                  \
     } while (0)
-#define LLMOPS_STASH_B(BUF)                                                                                \
+#define LLMOPS_STASH_B(BUF, WHO)                                                                           \
     do {                                                                                                   \
-        if (grp == 0) {                                                                                    \
+        if (grp == (WHO)) {                                                                                \
             _Pragma("unroll") for (int i = 0; i < 2; i++)                                                  \
                 _Pragma("unroll") for (int c = 0; c < 4; c++) {                                            \
                     uint2 u;                                                                               \
@@ -728,8 +846,8 @@ __global__ __launch_bounds__(512, 2) void fc_gemm_pp_kernel(const uint8_t* __res
                     u.y = hi4(rb[i][c]);                                                                   \
                     *reinterpret_cast<uint2*>(&sm.bu[BUF][bdst[i] + c * 512]) = u;                         \
                 }                                                                                          \
-            if (gtid < 32) {                                                                               \
-                float* dstf = (spart < 4 ? sm.d[BUF] : sm.m[BUF]) + sst * 32 + (spart & 3) * 8;            \
+            if (gtid < 16) {                                                                               \
+                float* dstf = sm.d[BUF] + sst * 32 + spart * 8;                                            \
                 float4 lo, hi;                                                                             \
                 lo.x = f16_bits_to_f32((uint16_t)(rs[0] & 0xFFFFu));                                       \
                 lo.y = f16_bits_to_f32((uint16_t)(rs[0] >> 16));                                           \
@@ -746,27 +864,50 @@ __global__ __launch_bounds__(512, 2) void fc_gemm_pp_kernel(const uint8_t* __res
     } while (0)
 
     v4f f[RT][4];
-#pragma unroll
-    for (int t = 0; t < RT; t++)
-#pragma unroll
-        for (int c = 0; c < 4; c++) f[t][c] = v4f{0.f, 0.f, 0.f, 0.f};
-    float gk[RT], mk[4];  // min term, four k-groups at a time by fp32 MFMA (see the kernel above)
-#pragma unroll
-    for (int t = 0; t < RT; t++) gk[t] = 0.0f;
-#pragma unroll
-    for (int c = 0; c < 4; c++) mk[c] = 0.0f;
-
-    if (kb0 < kb1) {
-        LLMOPS_COPY(kb0, 0);
-        LLMOPS_FETCH_B(kb0);
-        LLMOPS_STASH_B(0);
-    }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-    if (grp == 1) __syncthreads();  // group 1 runs one phase behind group 0
-
     const int strip_l = wc * 2 + sp;          // strip (0..3) of the tile this lane's B operands come from
     const int lrow = grp * GM + wr * 64;      // first tile row of this wave
+
+    // The accumulators start at the tile's min term (min_term_add).  Its operands are asked for ahead of the first
+    // k-group's; group 0 forms it while group 1 unpacks the first k-group's weights, group 1 in the phase it
+    // has to wait anyway (it runs one phase behind group 0).  A second and third round of 32 k-groups are
+    // fetched while the round before is being added.
+    MinTermRound<RT> mt;
+    int mroff[RT];
+#pragma unroll
+    for (int t = 0; t < RT; t++) mroff[t] = min(rows - 1, row0 + wr * 64 + t * 16 + jj) * Kg;
+    const int mstrip = min(Ng - 1, strip0 + strip_l);
+    if (kb0 < kb1) {
+        LLMOPS_COPY(kb0, 0);
+        LLMOPS_FETCH_B(kb0, 1);
+    }
+    __builtin_amdgcn_sched_barrier(0);  // the first k-group's operands are asked for first
+    if (!PARTIALS && kb0 < kb1) min_term_fetch<RT>(mt, gs, mroff, weiq, Kg, min(kb0 + 8 * g, Kg - 8), mstrip, q);
+#define LLMOPS_MIN_TERM()                                                                                  \
+    do {                                                                                                   \
+        if (!PARTIALS && kb0 < kb1) {                                                                      \
+            min_term_add<RT, true>(f, mt, min(kb0 + 8 * g, Kg - 8), kb0 + 8 * g, kb1);                     \
+            for (int k32 = kb0 + 32; k32 < kb1; k32 += 32) {                                               \
+                min_term_fetch<RT>(mt, gs, mroff, weiq, Kg, min(k32 + 8 * g, Kg - 8), mstrip, q);          \
+                min_term_add<RT, false>(f, mt, min(k32 + 8 * g, Kg - 8), k32 + 8 * g, kb1);                \
+            }                                                                                              \
+        } else {                                                                                           \
+            _Pragma("unroll") for (int t = 0; t < RT; t++)                                                 \
+                _Pragma("unroll") for (int c = 0; c < 4; c++) f[t][c] = v4f{0.f, 0.f, 0.f, 0.f};           \
+        }                                                                                                  \
+    } while (0)
+    // (s_waitcnt through the builtin, so that the compiler knows that no load of this prologue is pending in
+    // the k-group loop: left to its own bookkeeping it assumes that a further round may have been asked for and
+    // waits for "it" -- in fact for the k-group's asynchronous copies -- where the loop reuses the registers)
+    constexpr int kVmcnt0 = 0x0F70;  // vmcnt(0), the other counters left alone
+    if (grp == 1) {
+        if (kb0 < kb1) LLMOPS_STASH_B(0, 1);
+        __builtin_amdgcn_s_waitcnt(kVmcnt0);
+        __syncthreads();  // group 0 arrives here with its min term done ...
+    }
+    LLMOPS_MIN_TERM();
+    __builtin_amdgcn_s_waitcnt(kVmcnt0);
+    __syncthreads();  // ... by this one; for group 1 it is the barrier that puts it one phase behind group 0
+#undef LLMOPS_MIN_TERM
     // A operand of row tile t, k half h: row lrow + 16t + jj, chunk 4h + g, swizzled by the row's low bits
     const int akey = (jj + (jj >> 3)) & 7;
     const uint32_t a_rd0 = lds_a + (lrow + jj) * 128 + (((0 + g) ^ akey) * 16);
@@ -792,12 +933,6 @@ __global__ __launch_bounds__(512, 2) void fc_gemm_pp_kernel(const uint8_t* __res
 #pragma unroll
             for (int c = 0; c < 4; c++) b[h][c] = *reinterpret_cast<const v4i*>(&sm.bu[buf][b_rd + (h * 4 + c) * 512]);
         const float4 d4 = *reinterpret_cast<const float4*>(&sm.d[buf][strip_l * 32 + q * 4]);
-        const float4 m4 = *reinterpret_cast<const float4*>(&sm.m[buf][strip_l * 32 + q * 4]);
-        float gsr[RT];
-        if (!PARTIALS) {
-#pragma unroll
-            for (int t = 0; t < RT; t++) gsr[t] = sm.gs[buf][lrow + t * 16 + jj];
-        }
         v4i acc[RT][4];
         // The int32 sums start at the bit pattern of 1.5 * 2^23: read as a float, bits + sum IS the number
         // 1.5 * 2^23 + sum (|sum| <= 128 * 15 * 127 < 2^22), so the fold needs no convert instruction.
@@ -826,7 +961,7 @@ __global__ __launch_bounds__(512, 2) void fc_gemm_pp_kernel(const uint8_t* __res
         if (more) LLMOPS_COPY_X(kb + 1, buf ^ 1);
         lds_ready<2, PARTIALS>(a11);
         LLMOPS_MMA4(1, 1, a11);
-        if (more) LLMOPS_FETCH_B(kb + 1);
+        if (more) LLMOPS_FETCH_B(kb + 1, 0);
         lds_ready<1, PARTIALS>(a12);
         LLMOPS_MMA4(2, 1, a12);
         lds_ready<0, PARTIALS>(a13);
@@ -834,25 +969,6 @@ __global__ __launch_bounds__(512, 2) void fc_gemm_pp_kernel(const uint8_t* __res
 #undef LLMOPS_MMA4
         const float d[4] = {d4.x, d4.y, d4.z, d4.w};
         const float nbd[4] = {-kFoldBias * d4.x, -kFoldBias * d4.y, -kFoldBias * d4.z, -kFoldBias * d4.w};
-        if (!PARTIALS) {
-            const float m[4] = {m4.x, m4.y, m4.z, m4.w};
-            const int slot4 = (kb - kb0) & 3;
-            const bool mine4 = slot4 == g;
-#pragma unroll
-            for (int c = 0; c < 4; c++) mk[c] = mine4 ? m[c] : mk[c];
-#pragma unroll
-            for (int t = 0; t < RT; t++) gk[t] = mine4 ? gsr[t] : gk[t];
-            if (slot4 == 3 || kb + 1 == kb1) {
-#pragma unroll
-                for (int t = 0; t < RT; t++) {
-#pragma unroll
-                    for (int c = 0; c < 4; c++) f[t][c] = __builtin_amdgcn_mfma_f32_16x16x4f32(gk[t], mk[c], f[t][c], 0, 0, 0);
-                    gk[t] = 0.0f;
-                }
-#pragma unroll
-                for (int c = 0; c < 4; c++) mk[c] = 0.0f;
-            }
-        }
         asm volatile("" : "+v"(acc[0][0]), "+v"(acc[0][1]), "+v"(acc[0][2]), "+v"(acc[0][3]), "+v"(acc[1][0]),
                           "+v"(acc[1][1]), "+v"(acc[1][2]), "+v"(acc[1][3]), "+v"(acc[2][0]), "+v"(acc[2][1]),
                           "+v"(acc[2][2]), "+v"(acc[2][3]), "+v"(acc[3][0]), "+v"(acc[3][1]), "+v"(acc[3][2]),
@@ -896,7 +1012,7 @@ __global__ __launch_bounds__(512, 2) void fc_gemm_pp_kernel(const uint8_t* __res
         asm volatile("" : "+v"(f[0][0]), "+v"(f[0][1]), "+v"(f[0][2]), "+v"(f[0][3]), "+v"(f[1][0]), "+v"(f[1][1]),
                           "+v"(f[1][2]), "+v"(f[1][3]), "+v"(f[2][0]), "+v"(f[2][1]), "+v"(f[2][2]), "+v"(f[2][3]),
                           "+v"(f[3][0]), "+v"(f[3][1]), "+v"(f[3][2]), "+v"(f[3][3]));
-        if (kb + 1 < kb1) LLMOPS_STASH_B(buf ^ 1);
+        if (kb + 1 < kb1) LLMOPS_STASH_B(buf ^ 1, 0);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's copies for the next k-group have landed
         __syncthreads();
     }
@@ -1048,7 +1164,7 @@ static GemmPlan plan_gemm(int64_t rows, int64_t Ng, int64_t Kg, int G) {
     double best = 0.0;
     for (int i = 0; i < 4; i++) {
         if (g_gemm_rt > 0 && kRT[i] != g_gemm_rt) continue;
-        if (kRT[i] == 8 && (!small || (g_gemm_rt != 8 && rows < g_gemm_pp_min_rows))) continue;
+        if (kRT[i] == 8 && (!small || Kg < 8 || (g_gemm_rt != 8 && rows < g_gemm_pp_min_rows))) continue;
         const int64_t bm = kRows[i], slots = 256 * kWgPerCu[i];
         const int64_t tiles = ((Ng + 3) / 4) * ((rows + bm - 1) / bm);
         const int64_t s_floor = slots / tiles, s_ceil = (slots + tiles - 1) / tiles;

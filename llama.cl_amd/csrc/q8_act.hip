@@ -141,7 +141,8 @@ __global__ __launch_bounds__(256) void quant_x_rows_kernel(const float* __restri
 // silu(gate) * up (silu_mul_kernel's expression, so the codes are those of the two launches it replaces).
 template <int U, bool GLU = false>
 __global__ __launch_bounds__(256) void quant_x_tile128_kernel(const float* __restrict__ x, int rows, int Kg, int kparts,
-                                                               int8_t* __restrict__ xq, float2* __restrict__ xsT) {
+                                                               int8_t* __restrict__ xq, float* __restrict__ gsum,
+                                                               float2* __restrict__ xsT) {
     constexpr int G = 128;
     const int sub = threadIdx.x & 31, team = threadIdx.x >> 5;
     const int rb = blockIdx.x / kparts, kp = blockIdx.x - rb * kparts;
@@ -181,7 +182,10 @@ __global__ __launch_bounds__(256) void quant_x_tile128_kernel(const float* __res
         const int kb = kb0 + u;
         if (row_ok && kb < Kg) {
             *reinterpret_cast<uint32_t*>(xq + (rbase + kb) * G + sub * 4) = c;
-            if (sub == 0) xsT[(int64_t)kb * rows + row] = make_float2(d, s);
+            if (sub == 0) {
+                xsT[(int64_t)kb * rows + row] = make_float2(d, s);
+                gsum[rbase + kb] = s;  // [row][kg] as well: the 256-row product kernel reads a row's sums eight at a time
+            }
         }
     }
 }
@@ -240,7 +244,7 @@ namespace llmops {
 // Quantization with the producer of the activations folded in (shared with fc.hip): norm_w != nullptr quantizes
 // rmsnorm(x) * norm_w, glu_in quantizes silu(gate) * up of rows [gate | up] of 2K floats; one launch instead of the
 // producer's launch, a round trip of its fp32 result through memory and the quantization launch.  Whole k-groups
-// only; xd and gsum are written with norm_w only (the group-128 product kernels read xsT).
+// only; xd is written with norm_w only (the group-128 product kernels read xsT and gsum).
 int launch_quant_x_fused(const float* x, int64_t rows, int64_t K, int group_k, const float* norm_w, float eps, bool glu_in,
                          int8_t* xq, float* xd, float* gsum, float2* xsT, hipStream_t stream) {
     const int64_t Kg = K / group_k;
@@ -271,9 +275,9 @@ int launch_quant_x_fused(const float* x, int64_t rows, int64_t K, int group_k, c
         return fail(LLMOPS_EINVAL, "fused silu*up + quantization: group 128 only");
     if (rblocks * ((Kg + 3) / 4) >= 1024) {
         const int kparts = (int)((Kg + 3) / 4);
-        quant_x_tile128_kernel<4, true><<<(unsigned)(rblocks * kparts), 256, 0, stream>>>(x, (int)rows, (int)Kg, kparts, xq, xsT);
+        quant_x_tile128_kernel<4, true><<<(unsigned)(rblocks * kparts), 256, 0, stream>>>(x, (int)rows, (int)Kg, kparts, xq, gsum, xsT);
     } else {
-        quant_x_tile128_kernel<1, true><<<(unsigned)(rblocks * Kg), 256, 0, stream>>>(x, (int)rows, (int)Kg, (int)Kg, xq, xsT);
+        quant_x_tile128_kernel<1, true><<<(unsigned)(rblocks * Kg), 256, 0, stream>>>(x, (int)rows, (int)Kg, (int)Kg, xq, gsum, xsT);
     }
     LLMOPS_LAUNCH_CHECK();
     return LLMOPS_OK;
@@ -286,13 +290,13 @@ int launch_quant_x(const float* x, int64_t rows, int64_t K, int group_k, int8_t*
     const int64_t items = rows * Kg;
     if (!exact_sum && xsT != nullptr && group_k == 128 && K == Kg * group_k && aligned(x, 16) && aligned(xq, 4) &&
         rows < ((int64_t)1 << 28) && Kg < ((int64_t)1 << 20) && ((rows + 7) / 8) * Kg < ((int64_t)1 << 31)) {  // (the grid)
-        // the group-128 prefill kernels read only the codes and the transposed pairs: xd and gsum stay unwritten
+        // the group-128 prefill kernels read only the codes, the transposed pairs and the sums: xd stays unwritten
         const int64_t rblocks = (rows + 7) / 8;
         if (rblocks * ((Kg + 3) / 4) >= 1024) {  // enough workgroups with four k-groups per team
             const int kparts = (int)((Kg + 3) / 4);
-            quant_x_tile128_kernel<4><<<(unsigned)(rblocks * kparts), 256, 0, stream>>>(x, (int)rows, (int)Kg, kparts, xq, xsT);
+            quant_x_tile128_kernel<4><<<(unsigned)(rblocks * kparts), 256, 0, stream>>>(x, (int)rows, (int)Kg, kparts, xq, gsum, xsT);
         } else {
-            quant_x_tile128_kernel<1><<<(unsigned)(rblocks * Kg), 256, 0, stream>>>(x, (int)rows, (int)Kg, (int)Kg, xq, xsT);
+            quant_x_tile128_kernel<1><<<(unsigned)(rblocks * Kg), 256, 0, stream>>>(x, (int)rows, (int)Kg, (int)Kg, xq, gsum, xsT);
         }
         LLMOPS_LAUNCH_CHECK();
         return LLMOPS_OK;

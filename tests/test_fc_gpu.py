@@ -569,6 +569,40 @@ def test_fc_prefill_every_tiling_vs_oracle(ops, orc, tiling, rows, N, K):
     assert np.array_equal(ye, (xe.astype(np.float64) @ we.astype(np.float64).T).astype(np.float32).reshape(1, rows, N))
 
 
+@pytest.mark.parametrize("split", [0, 3])
+@pytest.mark.parametrize("K", [1024, 5120, 11008])
+def test_fc_prefill_min_term_at_any_activation_scale(ops, orc, K, split):
+    """The 256-row kernel forms the min term sum_kg m * gsum once per tile from fp16 halves of the group
+    sums, 32 k-groups per MFMA, and falls back to fp32 MFMAs for a round in which some row's sums are too
+    small or too large for that.  Rows of ordinary, tiny, huge and zero activations side by side, k-group
+    counts of one round exactly-not (8), a short second round (40) and a short third (86), with and
+    without split-K (splits that start off a multiple of 8): every ROW to 1e-5 of its own largest
+    output, which is what the fallback exists for."""
+    from llmops import _lib
+    lib = _lib.load()
+    rows, N = 300, 1056
+    rng = np.random.default_rng(K + split)
+    x = rng.standard_normal((1, rows, K)).astype(np.float32)
+    x[0, 100:200] *= 1e-4      # group sums far below 1/8
+    x[0, 200:290] *= 3000.0    # group sums beyond fp16
+    x[0, 290:] = 0.0
+    x[0, 5, 128:256] = 0.0     # a zero k-group inside an ordinary row
+    w = (rng.standard_normal((N, K)) * 0.02).astype(np.float32)
+    pw = orc.quant_w(w, 128)
+    want = orc.fc(x, pw, N)
+    lib.llmops_test_gemm_set_tuning(8)
+    lib.llmops_test_gemm_set_split(split)
+    try:
+        got = host(ops.fc_Q4A(dev(x), dev(pw), N))
+    finally:
+        lib.llmops_test_gemm_set_tuning(0)
+        lib.llmops_test_gemm_set_split(0)
+    scale = np.abs(want[0]).max(axis=1)
+    err = np.abs(got[0] - want[0]).max(axis=1)
+    assert np.all(err[290:] == 0.0)
+    assert np.all(err[:290] <= 1e-5 * scale[:290]), (err[:290] / scale[:290]).max()
+
+
 @pytest.mark.parametrize("rows", [9, 12, 16])
 @pytest.mark.parametrize("N,K", [(2070, 1024), (4096, 4096)])
 def test_fc_rows_9_to_16_streaming_mfma(ops, orc, rows, N, K):
