@@ -574,9 +574,9 @@ def test_fc_prefill_every_tiling_vs_oracle(ops, orc, tiling, rows, N, K):
 def test_fc_prefill_min_term_at_any_activation_scale(ops, orc, K, split):
     """The 256-row kernel forms the min term sum_kg m * gsum once per tile from fp16 halves of the group
     sums, 32 k-groups per MFMA, and falls back to fp32 MFMAs for a round in which some row's sums are too
-    small or too large for that.  Rows of ordinary, tiny, huge and zero activations side by side, k-group
-    counts of one round exactly-not (8), a short second round (40) and a short third (86), with and
-    without split-K (splits that start off a multiple of 8): every ROW to 1e-5 of its own largest
+    small or too large for that.  Rows of ordinary, tiny, huge and zero activations side by side; 8
+    k-groups (a quarter of one MFMA's 32), 40 (a short second batch of 32) and 86 (a short third), with
+    and without split-K (splits that start off a multiple of 8): every ROW to 1e-5 of its own largest
     output, which is what the fallback exists for."""
     from llmops import _lib
     lib = _lib.load()
