@@ -48,6 +48,11 @@ void llmops_test_gemm_set_reduce(int in_kernel);
  * compared bit for bit. */
 void llmops_test_gemm_set_split(int splits);
 
+/* prefill GEMM: what the planner chooses for a product of `rows` rows with a packed tensor of Ng strips x Kg
+ * k-groups (host arithmetic only, no launch): the row-tile factor (1, 2, 4: 32, 64, 128 rows per workgroup of
+ * the four-wave kernel; 8: the 256-row kernel) and the split-K factor.  Reads the knobs above. */
+int llmops_test_gemm_plan(int64_t rows, int64_t Ng, int64_t Kg, int group_k, int* row_tile_factor, int* splits);
+
 /* weight-streaming MFMA kernel (3..16 rows, 17..32 for tensors of fewer than 256 strips): two workgroups per strip with half of K each for tensors of
  * fewer than 256 strips (default on; 0 switches it off, for comparisons and tests) */
 void llmops_test_fc_rows_set_split(int on);

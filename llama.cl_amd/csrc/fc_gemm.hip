@@ -1170,7 +1170,16 @@ static GemmPlan plan_gemm(int64_t rows, int64_t Ng, int64_t Kg, int G) {
         const int64_t s_floor = slots / tiles, s_ceil = (slots + tiles - 1) / tiles;
         // (a third candidate where the machine would take more: the most splits the product kernel still adds itself)
         const int64_t s_cap = 12 * (int64_t)g_gemm_fused_reduce;
-        for (int64_t s_try : {s_floor, s_ceil, (s_cap > 0 && s_cap < s_floor && kRT[i] != 8) ? s_cap : s_floor}) {
+        // Below the 256-row kernel's range a workgroup's run of k-groups is short and what a workgroup costs before
+        // and after it decides: every split factor the kernel can finish itself is tried, a workgroup counts as
+        // its run plus 3 k-groups, and a split as 2.0 * bm / Kg (measured: sweeps of every tiling x 1..12 splits at
+        // 24..256 rows on 4096^2, 11008|12288|22016 x 4096 and 4096 x 11008; the choices made this way are 1.4 %
+        // slower on average than the best measured one, against 5 % -- up to 27 % at 24..64 rows -- before).
+        const bool few_rows = rows < g_gemm_pp_min_rows && g_gemm_fused_reduce && kRT[i] != 8;
+        const int n_try = few_rows ? 12 : 3;
+        for (int it = 0; it < n_try; it++) {
+            const int64_t s_try = few_rows ? it + 1
+                                           : (it == 0 ? s_floor : (it == 1 ? s_ceil : ((s_cap > 0 && s_cap < s_floor && kRT[i] != 8) ? s_cap : s_floor)));
             GemmPlan q = p;
             q.RT = kRT[i];
             int64_t S = s_try < 1 ? 1 : (s_try > Kg ? Kg : s_try);
@@ -1178,14 +1187,14 @@ static GemmPlan plan_gemm(int64_t rows, int64_t Ng, int64_t Kg, int G) {
             q.kb_per_split = (int)((Kg + S - 1) / S);
             q.S = (int)((Kg + q.kb_per_split - 1) / q.kb_per_split);
             const int64_t rounds = (tiles * q.S + slots - 1) / slots;
-            double cost = (double)rounds * (double)(bm * kWgPerCu[i]) / kEff[i] * (double)q.kb_per_split / (double)Kg;
+            double cost = (double)rounds * (double)(bm * kWgPerCu[i]) / kEff[i] * (double)(q.kb_per_split + (few_rows ? 3 : 0)) / (double)Kg;
             // Split-K is not free.  In the unit of this estimate (rows x share of K; about 0.014 us x Kg) the last
             // split of a tile to arrive adds S tiles of bm rows at ~150 GB/s (0.24 * S * bm / Kg); a second launch
             // over the partial sums costs 8-11 us whatever the shape (800 / Kg: the price at which the measured
             // choices came out best; 4096x11008 at 40-64 rows 24-25.5 -> 21-21.8 us against 570 / Kg).
             if (q.S > 1) {
                 const bool in_kernel = g_gemm_fused_reduce && q.S <= 12 * g_gemm_fused_reduce && kRT[i] != 8;
-                cost += in_kernel ? 0.24 * (double)q.S * (double)bm / (double)Kg : 800.0 / (double)Kg;
+                cost += in_kernel ? (few_rows ? 2.0 : 0.24) * (double)q.S * (double)bm / (double)Kg : 800.0 / (double)Kg;
             }
             if (best == 0.0 || cost < best) {
                 best = cost;
@@ -1342,6 +1351,14 @@ extern "C" void llmops_test_gemm_set_tuning(int rows_per_wave_tile) {
 }
 extern "C" void llmops_test_gemm_set_split(int splits) {
     if (llmops::test_hooks_enabled(__func__)) llmops::g_gemm_force_split = splits < 0 ? 0 : splits;
+}
+extern "C" int llmops_test_gemm_plan(int64_t rows, int64_t Ng, int64_t Kg, int group_k, int* row_tile_factor, int* splits) {
+    LLMOPS_TEST_HOOK();
+    if (rows < 1 || Ng < 1 || Kg < 1 || (group_k != 32 && group_k != 128) || !row_tile_factor || !splits) return LLMOPS_EINVAL;
+    const llmops::GemmPlan p = llmops::plan_gemm(rows, Ng, Kg, group_k);
+    *row_tile_factor = p.RT;
+    *splits = p.S;
+    return LLMOPS_OK;
 }
 extern "C" void llmops_test_gemm_set_reduce(int in_kernel) {
     if (llmops::test_hooks_enabled(__func__)) llmops::g_gemm_fused_reduce = in_kernel < 0 ? 0 : in_kernel;

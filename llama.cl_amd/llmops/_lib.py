@@ -65,6 +65,7 @@ SIGNATURES = {
     "llmops_test_gemm_set_tuning": (None, [c_int]),
     "llmops_test_gemm_set_reduce": (None, [c_int]),
     "llmops_test_gemm_set_split": (None, [c_int]),
+    "llmops_test_gemm_plan": (c_int, [c_i64, c_i64, c_i64, c_int, c_ptr, c_ptr]),
     "llmops_test_fc_set_row_routing": (None, [c_int, c_int]),
     "llmops_test_fc_rows_set_split": (None, [c_int]),
     "llmops_test_attn_set_decode_plan": (None, [c_int]),

@@ -103,6 +103,37 @@ def test_test_hooks_are_refused_unless_the_process_asks_for_them():
     assert "test hooks are switched off" in out.stderr
 
 
+def test_gemm_planner_choices(lib):
+    """The prefill GEMM's planner is host arithmetic: what it chooses for the shapes its rules were measured
+    on (row-tile factor 1, 2, 4 = 32, 64, 128 rows per workgroup, 8 = the 256-row kernel; split-K factor),
+    and that every plan covers K exactly once."""
+    i64, ci = ctypes.c_int64, ctypes.c_int
+
+    def plan(rows, N, K, G=128):
+        rt, S = ci(0), ci(0)
+        assert lib.llmops_test_gemm_plan(i64(rows), i64((N + 31) // 32), i64((K + G - 1) // G), G, ctypes.byref(rt),
+                                         ctypes.byref(S)) == 0
+        return rt.value, S.value
+
+    # many rows: the 256-row kernel, no split where the tiles fill the machine
+    assert plan(2048, 11008, 4096) == (8, 1)
+    assert plan(2048, 4096, 11008) == (8, 1)
+    assert plan(2048, 4096, 512)[0] != 8          # fewer than 8 k-groups: its min-term prologue reads 8 at a time
+    # few rows: 32-row tiles and as many splits as still leave runs of 4 k-groups (not 11 runs of 3)
+    assert plan(32, 11008, 4096) == (1, 8)
+    assert plan(64, 11008, 4096) == (1, 5)
+    assert plan(128, 11008, 4096) == (2, 4)
+    assert plan(128, 4096, 11008) == (1, 8)
+    for rows in (17, 24, 40, 100, 255, 256, 300, 512, 1000, 4096):
+        for N, K in ((4096, 4096), (11008, 4096), (4096, 11008), (352, 640), (22016, 4096), (64, 128)):
+            rt, S = plan(rows, N, K)
+            Kg = (K + 127) // 128
+            assert rt in (1, 2, 4, 8) and 1 <= S <= Kg
+            per = (Kg + S - 1) // S
+            assert (Kg + per - 1) // per == S     # S splits of `per` k-groups, the last possibly short, none empty
+    assert lib.llmops_test_gemm_plan(i64(0), i64(1), i64(1), 128, None, None) != 0
+
+
 def test_python_ops_refuse_host_tensors():
     """The product path has no CPU fallback: host tensors raise instead of being computed elsewhere."""
     import torch
