@@ -696,7 +696,8 @@ def test_quant_x_short_last_group(ops, orc, G, rows, K):
 
 
 @pytest.mark.parametrize("G", [32, 128])
-@pytest.mark.parametrize("rows,N,K", [(1, 4096, 4100), (2, 100, 1001), (8, 352, 333), (17, 96, 1001), (300, 160, 700)])
+@pytest.mark.parametrize("rows,N,K", [(1, 4096, 4100), (2, 100, 1001), (8, 352, 333), (17, 96, 1001), (300, 160, 700),
+                                      (300, 160, 1100), (300, 160, 5000)])
 def test_fc_short_last_group(ops, orc, G, rows, N, K):
     """fc_Q4A with K not a multiple of the group size, on the kernels of few and of many rows, with and without
     the residual epilogue, against the oracle (whose tail handling is pinned by the reference build)."""
@@ -709,6 +710,29 @@ def test_fc_short_last_group(ops, orc, G, rows, N, K):
     want = orc.fc(x, pw, N)
     assert max_rel_err(host(ops.fc_Q4A(dev(x), dev(pw), N)), want) <= 1e-5
     assert max_rel_err(host(ops.fc_Q4A(dev(x), dev(pw), N, residual=dev(res))), want + res) <= 1e-5
+
+
+@pytest.mark.parametrize("rows,N,K", [(300, 160, 1100), (300, 160, 5000), (513, 352, 4100)])
+def test_fc_256_row_kernel_short_last_group(ops, orc, rows, N, K):
+    """The 256-row kernel (forced) on a K that is not a whole number of k-groups: its min-term prologue reads a
+    row's group sums eight at a time from rows of 9, 40 and 33 floats (4-byte aligned only), the last k-group
+    is zero padded by the quantization."""
+    from llmops import _lib
+    lib = _lib.load()
+    rng = np.random.default_rng(rows + N + K)
+    w = (rng.standard_normal((N, K)) * 0.02).astype(np.float32)
+    pw = orc.quant_w(w, 128)
+    x = rng.standard_normal((1, rows, K)).astype(np.float32)
+    res = rng.standard_normal((1, rows, N)).astype(np.float32)
+    want = orc.fc(x, pw, N)
+    lib.llmops_test_gemm_set_tuning(8)
+    try:
+        got = host(ops.fc_Q4A(dev(x), dev(pw), N))
+        got_res = host(ops.fc_Q4A(dev(x), dev(pw), N, residual=dev(res)))
+    finally:
+        lib.llmops_test_gemm_set_tuning(0)
+    assert max_rel_err(got, want) <= 1e-5
+    assert max_rel_err(got_res, want + res) <= 1e-5
 
 
 @pytest.mark.parametrize("rows,N,K", [(1, 4096, 4096), (2, 4096, 11008), (1, 1000, 2048), (5, 352, 512), (40, 4096, 4096)])
