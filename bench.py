@@ -41,7 +41,7 @@ MEASURED_TRAFFIC_PROFILE = "profiles/fc_gemv_fused_kernel__hbm_traffic_pmc.md"
 PROFILE_SOURCES = {
     "profiles/fc_gemv_fused_kernel__hbm_traffic_pmc.md": (("fc_gemv.hip", "gemv_device.h"), "13290cb794320013"),
     "profiles/fc_gemv_fused_kernel__vector_alu_pmc.md": (("fc_gemv.hip", "gemv_device.h"), "13290cb794320013"),
-    "profiles/fc_gemm_kernels__prefill_g128_pmc.md": (("fc_gemm.hip", "fc_rows.hip", "q8_act.hip"), "c8fa3b8f3b5b2f94"),
+    "profiles/fc_gemm_kernels__prefill_g128_pmc.md": (("fc_gemm.hip", "fc_rows.hip", "q8_act.hip"), "e8ede7feb8d88665"),
     "profiles/attn_prefill_kernel__prompt_2048_pmc.md": (("attn.hip",), "08562b1e2698a706"),
 }
 MEASURED_TRAFFIC_KERNEL_SHA16 = PROFILE_SOURCES[MEASURED_TRAFFIC_PROFILE][1]
